@@ -1,0 +1,23 @@
+// Glue between the C entry points and launch_map: checks, early exits, launch bracket.
+#pragma once
+
+#include "dispatch.hpp"
+#include "map.hpp"
+#include "ops.hpp"
+
+namespace hmr {
+
+// Runs an elementwise entry point: prepares the call from `descs` (nullptr = constant), returns
+// early for empty tensors, and launches through `pick`, which returns false when there is no
+// kernel for the dtypes/op.
+template <class Pick>
+hmr_status run_map(hmr_context_t ctx, const char *what, int count, const hmr_tensor_desc *const *descs,
+                   const uint64_t *bits, Pick pick) {
+    MapCall call;
+    if (hmr_status s = prepare_map(call, count, descs, bits)) return s;
+    if (call.n == 0) return HMR_OK;
+    call.compute_units = ctx->compute_units;
+    return launch_on(ctx, what, [&](hipStream_t stream) { return pick(call, stream); });
+}
+
+}  // namespace hmr

@@ -1,0 +1,510 @@
+// The elementwise engine: out[i] = f(in0[i], in1[i], in2[i]) over strided operands.
+//
+// Replaces the reference's three generic kernels (ref: csrc/elementwise.hip:412-551 and
+// csrc/kernel.hpp:83-103, which index every element of every broadcast with int64 div/mod).
+// Two kernels, picked on the host from the operands' merged dimensions:
+//
+//  map_rows_kernel   every operand walks its innermost dimension with stride 1 or 0. A lane owns
+//                    V consecutive elements of a row, V = 16 bytes of the narrowest operand, so
+//                    every operand moves in 128-bit accesses (wider operands take several). The
+//                    outer dimensions are resolved once per V elements with 32-bit multiply-shift
+//                    division; a contiguous tensor is the one-dimensional case with no division
+//                    at all. Stride-0 operands (bias rows, per-row scales, scalars) are read once
+//                    per lane-tile and replicated in registers. Each lane runs U tiles per pass,
+//                    loads first, stores after, to keep >= 64 bytes per operand in flight.
+//  map_any_kernel    anything else (transposed, every-other, overflowing 32 bits ...): one
+//                    element per lane per step, 32-bit multiply-shift indexing when every offset
+//                    fits, int64 otherwise.
+//
+// A functor F describes one op:
+//   static constexpr int N;           number of inputs (1..3)
+//   using Out, In0, In1, In2;         storage types (unused inputs: hmr::Unused)
+//   __device__ Out operator()(In0, In1, In2) const;
+// Inputs may also be kernel-argument constants (hmr_binary_constant, hmr_where_constant,
+// hmr_fill), which cost no memory traffic.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <string>
+
+#include "common.hpp"
+#include "elem.hpp"
+
+namespace hmr {
+
+constexpr int kBlock = 256;      // 4 waves of 64
+constexpr int kFastDims = 6;     // merged dimensions the 32-bit kernels take
+constexpr int kMaxOperands = 4;  // output + 3 inputs
+
+struct Unused {};
+
+// ---- host-side view of one call ----------------------------------------------------------------
+
+// The operands of a call after this library's own dimension merge (callers merge too, but the
+// contract only promises same sizes). Operand 0 is the output.
+struct MapCall {
+    int nops = 0;  // operands including the output
+    int64_t n = 0;
+    int ndim = 0;
+    int64_t size[HMR_MAX_DIMS];
+    int64_t stride[kMaxOperands][HMR_MAX_DIMS];
+    char *ptr[kMaxOperands];         // address of element (0,..,0); nullptr for a constant
+    int elem_size[kMaxOperands];
+    uint64_t cbits[kMaxOperands];
+    bool is_const[kMaxOperands];
+    int compute_units = 256;
+};
+
+// Validates one description (ref: csrc/kernel.hpp:62-78): dtype and rank in range, no negative
+// size or stride. Leaves the element count in n.
+hmr_status check_desc(const hmr_tensor_desc &d, int64_t &n);
+
+// Builds the call for `descs[0..count)` (descs[k] == nullptr marks a constant with bits[k]):
+// checks that all have the output's sizes, then drops size-1 dimensions and joins neighbours
+// that are contiguous with each other in every operand.
+hmr_status prepare_map(MapCall &call, int count, const hmr_tensor_desc *const *descs, const uint64_t *bits);
+
+// ---- device-side argument blocks ------------------------------------------------------------------
+
+// x / d for 0 <= x < 2^31 and 1 <= d < 2^31 as (x * mul) >> (32 + shift): round-up method.
+struct FastDiv {
+    uint32_t div;
+    uint32_t mul;
+    uint32_t shift;
+};
+
+inline FastDiv make_fastdiv(uint32_t d) {
+    FastDiv f{d, 0, 0};
+    uint32_t s = 0;
+    while ((1ull << s) < d) ++s;  // ceil(log2 d)
+    uint64_t m = ((1ull << 32) * ((1ull << s) - d)) / d + 1;
+    f.mul = static_cast<uint32_t>(m);
+    f.shift = s;
+    return f;
+}
+
+__device__ __forceinline__ uint32_t divide(uint32_t x, const FastDiv &f) {
+    // floor(x * (2^32 + mul) / 2^(32 + shift)); t <= x < 2^31, so the sum cannot wrap.
+    uint32_t t = __umulhi(x, f.mul);
+    return (t + x) >> f.shift;
+}
+
+template <int NOPS>
+struct RowsArgs {
+    char *ptr[NOPS];
+    uint64_t cbits[NOPS];
+    uint32_t const_mask;   // bit k: operand k is a constant
+    uint32_t bcast_mask;   // bit k: operand k has inner stride 0
+    int64_t n;             // elements
+    uint32_t inner;        // size of the innermost dimension
+    int32_t nouter;        // outer dimensions (0 for contiguous)
+    FastDiv div[kFastDims - 1];            // outer dims, innermost first
+    int32_t ostride[NOPS][kFastDims - 1];  // their strides, same order, in elements
+    FastDiv inner_div;
+};
+
+template <int NOPS, class Idx>
+struct AnyArgs {
+    char *ptr[NOPS];
+    uint64_t cbits[NOPS];
+    uint32_t const_mask;
+    int32_t ndim;
+    int64_t n;
+    static constexpr int kDims = std::is_same_v<Idx, uint32_t> ? kFastDims : HMR_MAX_DIMS;
+    FastDiv div[std::is_same_v<Idx, uint32_t> ? kFastDims : 1];  // innermost first (32-bit only)
+    int64_t size64[std::is_same_v<Idx, uint32_t> ? 1 : HMR_MAX_DIMS];
+    std::conditional_t<std::is_same_v<Idx, uint32_t>, int32_t, int64_t> stride[NOPS][kDims];  // innermost first
+};
+
+// ---- register tiles ---------------------------------------------------------------------------------
+
+template <class T, int V>
+__device__ __forceinline__ void load_tile(const char *p, T (&r)[V]) {
+    constexpr int bytes = V * static_cast<int>(sizeof(T));
+    if constexpr (bytes % 16 == 0) {
+#pragma unroll
+        for (int i = 0; i < bytes / 16; ++i) {
+            uint4 w = reinterpret_cast<const uint4 *>(p)[i];
+            __builtin_memcpy(reinterpret_cast<char *>(r) + 16 * i, &w, 16);
+        }
+    } else if constexpr (bytes == 8) {
+        uint2 w = *reinterpret_cast<const uint2 *>(p);
+        __builtin_memcpy(r, &w, 8);
+    } else if constexpr (bytes == 4) {
+        uint32_t w = *reinterpret_cast<const uint32_t *>(p);
+        __builtin_memcpy(r, &w, 4);
+    } else if constexpr (bytes == 2) {
+        uint16_t w = *reinterpret_cast<const uint16_t *>(p);
+        __builtin_memcpy(r, &w, 2);
+    } else {
+        static_assert(bytes == 1, "tile size");
+        __builtin_memcpy(r, p, 1);
+    }
+}
+
+template <class T, int V>
+__device__ __forceinline__ void store_tile(char *p, const T (&r)[V]) {
+    constexpr int bytes = V * static_cast<int>(sizeof(T));
+    if constexpr (bytes % 16 == 0) {
+#pragma unroll
+        for (int i = 0; i < bytes / 16; ++i) {
+            uint4 w;
+            __builtin_memcpy(&w, reinterpret_cast<const char *>(r) + 16 * i, 16);
+            reinterpret_cast<uint4 *>(p)[i] = w;
+        }
+    } else if constexpr (bytes == 8) {
+        uint2 w;
+        __builtin_memcpy(&w, r, 8);
+        *reinterpret_cast<uint2 *>(p) = w;
+    } else if constexpr (bytes == 4) {
+        uint32_t w;
+        __builtin_memcpy(&w, r, 4);
+        *reinterpret_cast<uint32_t *>(p) = w;
+    } else if constexpr (bytes == 2) {
+        uint16_t w;
+        __builtin_memcpy(&w, r, 2);
+        *reinterpret_cast<uint16_t *>(p) = w;
+    } else {
+        static_assert(bytes == 1, "tile size");
+        __builtin_memcpy(p, r, 1);
+    }
+}
+
+template <class T>
+__device__ __forceinline__ T from_cbits(uint64_t bits) {
+    if constexpr (std::is_same_v<T, Unused>) {
+        return Unused{};
+    } else {
+        T v;
+        __builtin_memcpy(&v, &bits, sizeof(T));
+        return v;
+    }
+}
+
+template <class T>
+constexpr int size_or_zero() {
+    if constexpr (std::is_same_v<T, Unused>) return 0;
+    else return static_cast<int>(sizeof(T));
+}
+
+template <class F>
+struct MapTraits {
+    static constexpr int N = F::N;
+    static constexpr int so = static_cast<int>(sizeof(typename F::Out));
+    static constexpr int s0 = size_or_zero<typename F::In0>();
+    static constexpr int s1 = size_or_zero<typename F::In1>();
+    static constexpr int s2 = size_or_zero<typename F::In2>();
+    static constexpr int cmin(int a, int b) { return (b != 0 && b < a) ? b : a; }
+    static constexpr int cmax(int a, int b) { return b > a ? b : a; }
+    static constexpr int narrow = cmin(cmin(cmin(so, s0), s1), s2);
+    static constexpr int wide = cmax(cmax(cmax(so, s0), s1), s2);
+    // Elements per lane-tile: 16 bytes of the narrowest operand.
+    static constexpr int V = 16 / narrow;
+    // Tiles per lane per pass: aim at 64 bytes of the widest operand in flight.
+    static constexpr int U = (V * wide >= 64) ? 1 : 64 / (V * wide);
+};
+
+template <class F>
+__device__ __forceinline__ typename F::Out apply(const F &f, typename F::In0 a, typename F::In1 b,
+                                                 typename F::In2 c) {
+    if constexpr (F::N == 1) return f(a);
+    else if constexpr (F::N == 2) return f(a, b);
+    else return f(a, b, c);
+}
+
+// Reads the tile of input K (operand K+1) at element offset `off`.
+template <class T, int V>
+__device__ __forceinline__ void read_input(T (&r)[V], const char *base, uint64_t cbits, bool is_const, bool bcast,
+                                           int64_t off, bool full, int valid) {
+    if constexpr (std::is_same_v<T, Unused>) {
+        return;
+    } else {
+        if (is_const) {
+            T v = from_cbits<T>(cbits);
+#pragma unroll
+            for (int i = 0; i < V; ++i) r[i] = v;
+        } else if (bcast) {
+            T v = *reinterpret_cast<const T *>(base + off * static_cast<int64_t>(sizeof(T)));
+#pragma unroll
+            for (int i = 0; i < V; ++i) r[i] = v;
+        } else if (full) {
+            load_tile<T, V>(base + off * static_cast<int64_t>(sizeof(T)), r);
+        } else {
+            const T *p = reinterpret_cast<const T *>(base + off * static_cast<int64_t>(sizeof(T)));
+#pragma unroll
+            for (int i = 0; i < V; ++i) {
+                if (i < valid) r[i] = p[i];
+            }
+        }
+    }
+}
+
+// FLAT: one dimension (contiguous / scalar-broadcast operands); its last tile may be ragged.
+// Otherwise the innermost size is a multiple of V and rows never straddle a tile.
+template <class F, bool FLAT>
+__global__ void __launch_bounds__(kBlock) map_rows_kernel(RowsArgs<F::N + 1> a) {
+    using T = MapTraits<F>;
+    constexpr int V = T::V, U = T::U, N = F::N;
+    using Out = typename F::Out;
+    using A = typename F::In0;
+    using B = typename F::In1;
+    using C = typename F::In2;
+    const F f{};
+    const int64_t tiles = (a.n + V - 1) / V;
+    const bool c0 = a.const_mask & 2u, c1 = a.const_mask & 4u, c2 = a.const_mask & 8u;
+    const bool b0 = a.bcast_mask & 2u, b1 = a.bcast_mask & 4u, b2 = a.bcast_mask & 8u;
+    for (int64_t t0 = static_cast<int64_t>(blockIdx.x) * (U * kBlock) + threadIdx.x; t0 < tiles;
+         t0 += static_cast<int64_t>(gridDim.x) * (U * kBlock)) {
+        A ra[U][V];
+        B rb[U][V];
+        C rc[U][V];
+        using Off = std::conditional_t<FLAT, int64_t, uint32_t>;
+        Off oo[U];
+        int valid[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            int64_t t = t0 + static_cast<int64_t>(u) * kBlock;
+            valid[u] = 0;
+            if (t < tiles) {
+                int64_t e = t * V;
+                int64_t rem = a.n - e;
+                valid[u] = rem >= V ? V : static_cast<int>(rem);
+                Off off[4];
+                if constexpr (FLAT) {
+                    off[0] = e;
+                    off[1] = b0 ? 0 : e;
+                    off[2] = b1 ? 0 : e;
+                    off[3] = b2 ? 0 : e;
+                } else {
+                    uint32_t e32 = static_cast<uint32_t>(e);
+                    uint32_t row = divide(e32, a.inner_div);
+                    uint32_t col = e32 - row * a.inner;
+                    off[0] = col;
+                    off[1] = b0 ? 0 : col;
+                    off[2] = b1 ? 0 : col;
+                    off[3] = b2 ? 0 : col;
+                    for (int d = 0; d < a.nouter; ++d) {
+                        uint32_t q = divide(row, a.div[d]);
+                        uint32_t idx = row - q * a.div[d].div;
+                        row = q;
+                        off[0] += idx * static_cast<uint32_t>(a.ostride[0][d]);
+                        if constexpr (N >= 1) off[1] += idx * static_cast<uint32_t>(a.ostride[1][d]);
+                        if constexpr (N >= 2) off[2] += idx * static_cast<uint32_t>(a.ostride[2][d]);
+                        if constexpr (N >= 3) off[3] += idx * static_cast<uint32_t>(a.ostride[3][d]);
+                    }
+                }
+                oo[u] = off[0];
+                bool full = valid[u] == V;
+                read_input<A, V>(ra[u], a.ptr[1], a.cbits[1], c0, b0, off[1], full, valid[u]);
+                if constexpr (N >= 2) read_input<B, V>(rb[u], a.ptr[2], a.cbits[2], c1, b1, off[2], full, valid[u]);
+                if constexpr (N >= 3) read_input<C, V>(rc[u], a.ptr[3], a.cbits[3], c2, b2, off[3], full, valid[u]);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (valid[u] == 0) continue;
+            Out ro[V];
+#pragma unroll
+            for (int i = 0; i < V; ++i) ro[i] = apply(f, ra[u][i], rb[u][i], rc[u][i]);
+            char *po = a.ptr[0] + static_cast<int64_t>(oo[u]) * static_cast<int64_t>(sizeof(Out));
+            if (valid[u] == V) {
+                store_tile<Out, V>(po, ro);
+            } else {
+#pragma unroll
+                for (int i = 0; i < V; ++i) {
+                    if (i < valid[u]) reinterpret_cast<Out *>(po)[i] = ro[i];
+                }
+            }
+        }
+    }
+}
+
+template <class T, class Idx>
+__device__ __forceinline__ T read_one(const char *base, uint64_t cbits, bool is_const, Idx off) {
+    if constexpr (std::is_same_v<T, Unused>) {
+        return Unused{};
+    } else {
+        if (is_const) return from_cbits<T>(cbits);
+        return *reinterpret_cast<const T *>(base + static_cast<int64_t>(off) * static_cast<int64_t>(sizeof(T)));
+    }
+}
+
+template <class F, class Idx>
+__global__ void __launch_bounds__(kBlock) map_any_kernel(AnyArgs<F::N + 1, Idx> a) {
+    constexpr int N = F::N;
+    using Out = typename F::Out;
+    const F f{};
+    const bool c0 = a.const_mask & 2u, c1 = a.const_mask & 4u, c2 = a.const_mask & 8u;
+    using Off = std::conditional_t<std::is_same_v<Idx, uint32_t>, uint32_t, int64_t>;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; i < a.n;
+         i += static_cast<int64_t>(gridDim.x) * kBlock) {
+        Off off[4] = {0, 0, 0, 0};
+        if constexpr (std::is_same_v<Idx, uint32_t>) {
+            uint32_t rest = static_cast<uint32_t>(i);
+            for (int d = 0; d < a.ndim; ++d) {
+                uint32_t q = divide(rest, a.div[d]);
+                uint32_t idx = rest - q * a.div[d].div;
+                rest = q;
+#pragma unroll
+                for (int k = 0; k <= N; ++k) off[k] += idx * static_cast<uint32_t>(a.stride[k][d]);
+            }
+        } else {
+            int64_t rest = i;
+            for (int d = 0; d < a.ndim; ++d) {
+                int64_t q = rest / a.size64[d];
+                int64_t idx = rest - q * a.size64[d];
+                rest = q;
+#pragma unroll
+                for (int k = 0; k <= N; ++k) off[k] += idx * a.stride[k][d];
+            }
+        }
+        typename F::In0 x = read_one<typename F::In0, Off>(a.ptr[1], a.cbits[1], c0, off[1]);
+        typename F::In1 y{};
+        typename F::In2 z{};
+        if constexpr (N >= 2) y = read_one<typename F::In1, Off>(a.ptr[2], a.cbits[2], c1, off[2]);
+        if constexpr (N >= 3) z = read_one<typename F::In2, Off>(a.ptr[3], a.cbits[3], c2, off[3]);
+        Out r = apply(f, x, y, z);
+        *reinterpret_cast<Out *>(a.ptr[0] + static_cast<int64_t>(off[0]) * static_cast<int64_t>(sizeof(Out))) = r;
+    }
+}
+
+// ---- host-side launch -----------------------------------------------------------------------------
+
+inline unsigned grid_for(int64_t work_items, int64_t per_block) {
+    int64_t blocks = work_items / per_block + (work_items % per_block != 0);
+    const int64_t cap = int64_t{1} << 22;
+    if (blocks < 1) blocks = 1;
+    return static_cast<unsigned>(blocks < cap ? blocks : cap);
+}
+
+// Largest element offset (exclusive bound - 1) operand k can reach.
+inline bool fits_32(const MapCall &c) {
+    if (c.n >= (int64_t{1} << 31)) return false;
+    for (int k = 0; k < c.nops; ++k) {
+        if (c.is_const[k]) continue;
+        __int128 reach = 0;
+        for (int d = 0; d < c.ndim; ++d) reach += static_cast<__int128>(c.size[d] - 1) * c.stride[k][d];
+        if (reach >= (int64_t{1} << 31)) return false;
+    }
+    return true;
+}
+
+// Which kernel a call takes: 0 contiguous rows kernel, 1 rows kernel with outer dims, 2 any/32, 3 any/64.
+template <class F>
+int pick_variant(const MapCall &c) {
+    using T = MapTraits<F>;
+    constexpr int sizes[4] = {T::so, T::s0, T::s1, T::s2};
+    if (c.ndim > kFastDims || !fits_32(c)) return c.ndim <= 1 && c.n < (int64_t{1} << 62) ? -1 : 3;
+    if (c.ndim == 0) return 0;
+    const int last = c.ndim - 1;
+    bool rows = c.stride[0][last] == 1;
+    for (int k = 1; rows && k < c.nops; ++k) {
+        if (c.is_const[k]) continue;
+        rows = c.stride[k][last] == 1 || c.stride[k][last] == 0;
+    }
+    if (rows) {
+        // Every vector access must be aligned: base pointers and (for outer dims) row starts.
+        bool aligned = true;
+        for (int k = 0; aligned && k < c.nops; ++k) {
+            if (c.is_const[k] || c.stride[k][last] == 0) continue;
+            int chunk = T::V * sizes[k] < 16 ? T::V * sizes[k] : 16;
+            aligned = reinterpret_cast<uintptr_t>(c.ptr[k]) % chunk == 0;
+            for (int d = 0; aligned && d < last; ++d) {
+                aligned = (c.stride[k][d] * sizes[k]) % chunk == 0;
+            }
+        }
+        if (aligned && c.ndim == 1) return 0;
+        if (aligned && c.size[last] % T::V == 0) return 1;
+    }
+    return 2;
+}
+
+template <class F>
+void launch_map(const MapCall &c, hipStream_t stream) {
+    using T = MapTraits<F>;
+    constexpr int NOPS = F::N + 1;
+    int variant = pick_variant<F>(c);
+    if (variant == -1) {
+        // One huge contiguous dimension (>= 2^31 elements): the FLAT rows kernel indexes in 64 bits.
+        bool ok = c.ndim == 0 || c.stride[0][0] == 1;
+        for (int k = 1; ok && k < c.nops; ++k) ok = c.is_const[k] || c.stride[k][0] == 1 || c.stride[k][0] == 0;
+        constexpr int sizes[4] = {T::so, T::s0, T::s1, T::s2};
+        for (int k = 0; ok && k < c.nops; ++k) {
+            if (c.is_const[k] || (c.ndim == 1 && c.stride[k][0] == 0)) continue;
+            int chunk = T::V * sizes[k] < 16 ? T::V * sizes[k] : 16;
+            ok = reinterpret_cast<uintptr_t>(c.ptr[k]) % chunk == 0;
+        }
+        variant = ok ? 0 : 3;
+    }
+    if (variant <= 1) {
+        RowsArgs<NOPS> a{};
+        a.n = c.n;
+        a.const_mask = 0;
+        a.bcast_mask = 0;
+        const int last = c.ndim - 1;
+        for (int k = 0; k < NOPS; ++k) {
+            a.ptr[k] = c.ptr[k];
+            a.cbits[k] = c.cbits[k];
+            if (c.is_const[k]) a.const_mask |= 1u << k;
+            else if (c.ndim == 0 || c.stride[k][last] == 0) a.bcast_mask |= k == 0 ? 0u : 1u << k;
+        }
+        int64_t tiles = (c.n + T::V - 1) / T::V;
+        unsigned grid = grid_for(tiles, int64_t{T::U} * kBlock);
+        if (variant == 0) {
+            a.inner = static_cast<uint32_t>(c.n < (int64_t{1} << 31) ? c.n : 0);
+            a.nouter = 0;
+            hipLaunchKernelGGL((map_rows_kernel<F, true>), dim3(grid), dim3(kBlock), 0, stream, a);
+        } else {
+            a.inner = static_cast<uint32_t>(c.size[last]);
+            a.inner_div = make_fastdiv(a.inner);
+            a.nouter = last;
+            for (int d = 0; d < last; ++d) {
+                int src = last - 1 - d;  // innermost outer dimension first
+                a.div[d] = make_fastdiv(static_cast<uint32_t>(c.size[src]));
+                for (int k = 0; k < NOPS; ++k) {
+                    a.ostride[k][d] = c.is_const[k] ? 0 : static_cast<int32_t>(c.stride[k][src]);
+                }
+            }
+            hipLaunchKernelGGL((map_rows_kernel<F, false>), dim3(grid), dim3(kBlock), 0, stream, a);
+        }
+        return;
+    }
+    unsigned grid = grid_for(c.n, kBlock);
+    if (variant == 2) {
+        AnyArgs<NOPS, uint32_t> a{};
+        a.n = c.n;
+        a.ndim = c.ndim;
+        a.const_mask = 0;
+        for (int k = 0; k < NOPS; ++k) {
+            a.ptr[k] = c.ptr[k];
+            a.cbits[k] = c.cbits[k];
+            if (c.is_const[k]) a.const_mask |= 1u << k;
+        }
+        for (int d = 0; d < c.ndim; ++d) {
+            int src = c.ndim - 1 - d;
+            a.div[d] = make_fastdiv(static_cast<uint32_t>(c.size[src]));
+            for (int k = 0; k < NOPS; ++k) a.stride[k][d] = c.is_const[k] ? 0 : static_cast<int32_t>(c.stride[k][src]);
+        }
+        hipLaunchKernelGGL((map_any_kernel<F, uint32_t>), dim3(grid), dim3(kBlock), 0, stream, a);
+    } else {
+        AnyArgs<NOPS, int64_t> a{};
+        a.n = c.n;
+        a.ndim = c.ndim;
+        a.const_mask = 0;
+        for (int k = 0; k < NOPS; ++k) {
+            a.ptr[k] = c.ptr[k];
+            a.cbits[k] = c.cbits[k];
+            if (c.is_const[k]) a.const_mask |= 1u << k;
+        }
+        for (int d = 0; d < c.ndim; ++d) {
+            int src = c.ndim - 1 - d;
+            a.size64[d] = c.size[src];
+            for (int k = 0; k < NOPS; ++k) a.stride[k][d] = c.is_const[k] ? 0 : c.stride[k][src];
+        }
+        hipLaunchKernelGGL((map_any_kernel<F, int64_t>), dim3(grid), dim3(kBlock), 0, stream, a);
+    }
+}
+
+}  // namespace hmr

@@ -1,0 +1,336 @@
+// The op functors of the elementwise engine. Each mirrors one arm of homura's CPU kernels
+// (ref: src/backend/cpu/mod.rs:336-507, 573-577; src/backend/cpu/num.rs:109-219): float ops widen
+// to the computation type (f32 for F16/BF16/F32, f64 for F64), compute, and round once; integer
+// ops wrap.
+//
+// Transcendental accuracy. The CPU calls the host libm in the computation type. Here:
+//   F32 tensors   evaluate the function in f64 and round to f32. That is the correctly rounded
+//                 f32 value except within ~2^-29 of a rounding boundary, which is also what a good
+//                 libm returns, so results agree to the last bit nearly everywhere and to 1 ulp
+//                 otherwise.
+//   F16/BF16      evaluate in f32; an f32-ulp difference can only flip the final rounding to the
+//                 16-bit type by one ulp. GELU is the exception: 1 + erf(z) cancels for z << 0, so
+//                 erf is always evaluated in f64 and rounded to f32 exactly as the CPU does
+//                 (ref: src/backend/cpu/num.rs:30-33).
+//   F64           the device library's f64 functions.
+// The surrounding arithmetic (1/(1+e), 0.5*x*(1+t), ...) is done in the computation type in the
+// CPU's order, so it contributes no difference of its own.
+#pragma once
+
+#include "elem.hpp"
+#include "map.hpp"
+
+namespace hmr {
+
+// ---- math in the evaluation type ---------------------------------------------------------------
+
+template <class T>
+struct Eval {  // halves and their f32 computation type: evaluate in f32
+    using E = float;
+};
+template <>
+struct Eval<float> {
+    using E = double;
+};
+template <>
+struct Eval<double> {
+    using E = double;
+};
+
+__device__ __forceinline__ float m_exp(float x) { return expf(x); }
+__device__ __forceinline__ double m_exp(double x) { return exp(x); }
+__device__ __forceinline__ float m_log(float x) { return logf(x); }
+__device__ __forceinline__ double m_log(double x) { return log(x); }
+__device__ __forceinline__ float m_log1p(float x) { return log1pf(x); }
+__device__ __forceinline__ double m_log1p(double x) { return log1p(x); }
+__device__ __forceinline__ float m_sin(float x) { return sinf(x); }
+__device__ __forceinline__ double m_sin(double x) { return sin(x); }
+__device__ __forceinline__ float m_cos(float x) { return cosf(x); }
+__device__ __forceinline__ double m_cos(double x) { return cos(x); }
+__device__ __forceinline__ float m_tanh(float x) { return tanhf(x); }
+__device__ __forceinline__ double m_tanh(double x) { return tanh(x); }
+__device__ __forceinline__ float m_pow(float x, float y) { return powf(x, y); }
+__device__ __forceinline__ double m_pow(double x, double y) { return pow(x, y); }
+__device__ __forceinline__ float m_sqrt(float x) { return sqrtf(x); }  // correctly rounded
+__device__ __forceinline__ double m_sqrt(double x) { return sqrt(x); }
+__device__ __forceinline__ float m_abs(float x) { return fabsf(x); }
+__device__ __forceinline__ double m_abs(double x) { return fabs(x); }
+
+// fn evaluated for a value of computation type C that belongs to storage type T.
+#define HMR_EVAL1(NAME, FN)                                            \
+    template <class T>                                                 \
+    __device__ __forceinline__ typename Comp<T>::C NAME(typename Comp<T>::C x) { \
+        using E = typename Eval<T>::E;                                 \
+        return static_cast<typename Comp<T>::C>(FN(static_cast<E>(x))); \
+    }
+HMR_EVAL1(e_exp, m_exp)
+HMR_EVAL1(e_log, m_log)
+HMR_EVAL1(e_log1p, m_log1p)
+HMR_EVAL1(e_sin, m_sin)
+HMR_EVAL1(e_cos, m_cos)
+HMR_EVAL1(e_tanh, m_tanh)
+#undef HMR_EVAL1
+
+template <class T>
+__device__ __forceinline__ typename Comp<T>::C e_pow(typename Comp<T>::C x, typename Comp<T>::C y) {
+    using E = typename Eval<T>::E;
+    return static_cast<typename Comp<T>::C>(m_pow(static_cast<E>(x), static_cast<E>(y)));
+}
+
+// erf of a computation-type value: always through f64 (see the header comment).
+__device__ __forceinline__ float e_erf(float x) { return static_cast<float>(erf(static_cast<double>(x))); }
+__device__ __forceinline__ double e_erf(double x) { return erf(x); }
+
+// ---- unary ------------------------------------------------------------------------------------------
+
+template <int OP, class T>
+struct UnaryFloat {
+    static constexpr int N = 1;
+    using Out = T;
+    using In0 = T;
+    using In1 = Unused;
+    using In2 = Unused;
+    using C = typename Comp<T>::C;
+    __device__ __forceinline__ Out operator()(T v) const {
+        const C x = Comp<T>::up(v);
+        const C one = C(1), zero = C(0), half = C(0.5);
+        C r;
+        if constexpr (OP == HMR_UNARY_NEG) r = -x;
+        else if constexpr (OP == HMR_UNARY_ABS) r = m_abs(x);
+        else if constexpr (OP == HMR_UNARY_SIGN) r = x > zero ? one : (x < zero ? -one : zero);
+        else if constexpr (OP == HMR_UNARY_RELU) r = (x != x || x > zero) ? x : zero;
+        else if constexpr (OP == HMR_UNARY_EXP) r = e_exp<T>(x);
+        else if constexpr (OP == HMR_UNARY_LOG) r = e_log<T>(x);
+        else if constexpr (OP == HMR_UNARY_SQRT) r = m_sqrt(x);
+        else if constexpr (OP == HMR_UNARY_RSQRT) r = one / m_sqrt(x);
+        else if constexpr (OP == HMR_UNARY_RECIPROCAL) r = one / x;
+        else if constexpr (OP == HMR_UNARY_SIN) r = e_sin<T>(x);
+        else if constexpr (OP == HMR_UNARY_COS) r = e_cos<T>(x);
+        else if constexpr (OP == HMR_UNARY_ERF) r = e_erf(x);
+        else if constexpr (OP == HMR_UNARY_TANH) r = e_tanh<T>(x);
+        else if constexpr (OP == HMR_UNARY_SIGMOID) r = one / (one + e_exp<T>(-x));
+        else if constexpr (OP == HMR_UNARY_LOG_SIGMOID) {
+            C mn = (x != x || x < zero) ? x : zero;
+            r = mn - e_log1p<T>(e_exp<T>(-m_abs(x)));
+        } else if constexpr (OP == HMR_UNARY_SILU) r = x / (one + e_exp<T>(-x));
+        else if constexpr (OP == HMR_UNARY_GELU) {
+            const C k = static_cast<C>(0.70710678118654752440);
+            r = half * x * (one + e_erf(x * k));
+        } else {
+            static_assert(OP == HMR_UNARY_GELU_TANH, "unary op");
+            const C k = static_cast<C>(__builtin_sqrt(2.0 / 3.14159265358979323846));  // as the CPU: f64 sqrt(2/pi), then to C
+            const C c = static_cast<C>(0.044715);
+            r = half * x * (one + e_tanh<T>(k * (x + c * x * x * x)));
+        }
+        return Comp<T>::down(r);
+    }
+};
+
+template <int OP, class T>
+struct UnaryInt {
+    static constexpr int N = 1;
+    using Out = T;
+    using In0 = T;
+    using In1 = Unused;
+    using In2 = Unused;
+    __device__ __forceinline__ T operator()(T x) const {
+        using U = std::make_unsigned_t<T>;
+        if constexpr (OP == HMR_UNARY_NEG) return bits_as<T>(static_cast<U>(U(0) - static_cast<U>(x)));
+        else if constexpr (OP == HMR_UNARY_ABS) {
+            if constexpr (std::is_unsigned_v<T>) return x;
+            else return x < 0 ? bits_as<T>(static_cast<U>(U(0) - static_cast<U>(x))) : x;
+        } else if constexpr (OP == HMR_UNARY_RELU) return x > T(0) ? x : T(0);
+        else {
+            static_assert(OP == HMR_UNARY_SIGN, "integer unary op");
+            return x > T(0) ? T(1) : (x < T(0) ? static_cast<T>(-1) : T(0));
+        }
+    }
+};
+
+template <class T>
+struct LogicalNot {
+    static constexpr int N = 1;
+    using Out = bool_t;
+    using In0 = T;
+    using In1 = Unused;
+    using In2 = Unused;
+    __device__ __forceinline__ bool_t operator()(T x) const {
+        return bool_t{static_cast<uint8_t>(!Conv<T>::to_bool(x))};
+    }
+};
+
+// Moves elements of one size unchanged (same-dtype copies, fills, Sign of a bool tensor).
+template <class W>
+struct Move {
+    static constexpr int N = 1;
+    using Out = W;
+    using In0 = W;
+    using In1 = Unused;
+    using In2 = Unused;
+    __device__ __forceinline__ W operator()(W x) const { return x; }
+};
+
+template <class D, class S>
+struct Convert {
+    static constexpr int N = 1;
+    using Out = D;
+    using In0 = S;
+    using In1 = Unused;
+    using In2 = Unused;
+    __device__ __forceinline__ D operator()(S x) const { return convert<D, S>(x); }
+};
+
+// ---- binary -----------------------------------------------------------------------------------------
+
+// Value a comparison looks at: halves compare as floats, bools as 0/1.
+template <class T>
+__device__ __forceinline__ auto cmp_value(T x) {
+    if constexpr (std::is_same_v<T, f16_t>) return f16_widen(x);
+    else if constexpr (std::is_same_v<T, bf16_t>) return bf16_up(x);
+    else if constexpr (std::is_same_v<T, bool_t>) return x.v;
+    else return x;
+}
+
+template <int OP, class T>
+struct Compare {
+    static constexpr int N = 2;
+    using Out = bool_t;
+    using In0 = T;
+    using In1 = T;
+    using In2 = Unused;
+    __device__ __forceinline__ bool_t operator()(T a, T b) const {
+        auto x = cmp_value(a);
+        auto y = cmp_value(b);
+        bool r;
+        if constexpr (OP == HMR_BINARY_GREATER) r = x > y;
+        else if constexpr (OP == HMR_BINARY_GREATER_EQUAL) r = x >= y;
+        else if constexpr (OP == HMR_BINARY_LESS) r = x < y;
+        else if constexpr (OP == HMR_BINARY_LESS_EQUAL) r = x <= y;
+        else if constexpr (OP == HMR_BINARY_EQUAL) r = x == y;
+        else r = x != y;
+        return bool_t{static_cast<uint8_t>(r)};
+    }
+};
+
+// AND: LogicalAnd, bool Mul/Minimum, bool BitwiseAnd. OR: LogicalOr, bool Add/Maximum.
+template <bool AND>
+struct BoolBinary {
+    static constexpr int N = 2;
+    using Out = bool_t;
+    using In0 = bool_t;
+    using In1 = bool_t;
+    using In2 = Unused;
+    __device__ __forceinline__ bool_t operator()(bool_t a, bool_t b) const {
+        bool x = a.v != 0, y = b.v != 0;
+        return bool_t{static_cast<uint8_t>(AND ? (x && y) : (x || y))};
+    }
+};
+
+template <class T>
+__device__ __forceinline__ T wrapping_mul(T a, T b) {
+    using U = std::make_unsigned_t<T>;
+    using W = std::conditional_t<sizeof(T) == 8, uint64_t, uint32_t>;
+    return bits_as<T>(static_cast<U>(static_cast<W>(static_cast<U>(a)) * static_cast<W>(static_cast<U>(b))));
+}
+
+// ref: src/backend/cpu/num.rs:160-187
+template <class T>
+__device__ __forceinline__ T int_pow(T base, T exp) {
+    int64_t e = static_cast<int64_t>(exp);
+    if (e < 0) {
+        int64_t b = static_cast<int64_t>(base);
+        if (b == 1) return T(1);
+        if (b == -1) return (e % 2 == 0) ? T(1) : base;
+        return T(0);
+    }
+    T result = 1;
+    uint64_t k = static_cast<uint64_t>(e);
+    while (k > 0) {
+        if (k & 1) result = wrapping_mul(result, base);
+        base = wrapping_mul(base, base);
+        k >>= 1;
+    }
+    return result;
+}
+
+template <int OP, class T>
+struct IntBinary {
+    static constexpr int N = 2;
+    using Out = T;
+    using In0 = T;
+    using In1 = T;
+    using In2 = Unused;
+    __device__ __forceinline__ T operator()(T a, T b) const {
+        using U = std::make_unsigned_t<T>;
+        if constexpr (OP == HMR_BINARY_ADD) return bits_as<T>(static_cast<U>(static_cast<U>(a) + static_cast<U>(b)));
+        else if constexpr (OP == HMR_BINARY_SUB) return bits_as<T>(static_cast<U>(static_cast<U>(a) - static_cast<U>(b)));
+        else if constexpr (OP == HMR_BINARY_MUL) return wrapping_mul(a, b);
+        else if constexpr (OP == HMR_BINARY_POW) return int_pow(a, b);
+        else if constexpr (OP == HMR_BINARY_MAXIMUM) return a > b ? a : b;
+        else if constexpr (OP == HMR_BINARY_MINIMUM) return a < b ? a : b;
+        else {
+            static_assert(OP == HMR_BINARY_BITWISE_AND, "integer binary op");
+            return static_cast<T>(a & b);
+        }
+    }
+};
+
+// A and B may differ from T (mixed-dtype extension): both are converted exactly to T's
+// computation type, which is what a separate cast kernel followed by the op would produce.
+template <int OP, class T, class A = T, class B = T>
+struct FloatBinary {
+    static constexpr int N = 2;
+    using Out = T;
+    using In0 = A;
+    using In1 = B;
+    using In2 = Unused;
+    using C = typename Comp<T>::C;
+    __device__ __forceinline__ T operator()(A a, B b) const {
+        const C x = static_cast<C>(Comp<A>::up(a));
+        const C y = static_cast<C>(Comp<B>::up(b));
+        C r;
+        if constexpr (OP == HMR_BINARY_ADD) r = x + y;
+        else if constexpr (OP == HMR_BINARY_SUB) r = x - y;
+        else if constexpr (OP == HMR_BINARY_MUL) r = x * y;
+        else if constexpr (OP == HMR_BINARY_DIV) r = x / y;
+        else if constexpr (OP == HMR_BINARY_POW) r = e_pow<T>(x, y);
+        else if constexpr (OP == HMR_BINARY_MAXIMUM) r = (x != x || x > y) ? x : y;
+        else {
+            static_assert(OP == HMR_BINARY_MINIMUM, "float binary op");
+            r = (x != x || x < y) ? x : y;
+        }
+        return Comp<T>::down(r);
+    }
+};
+
+// hmr_binary_scalar: the scalar stays in the computation type (it travels as a kernel constant
+// holding the bits of a C value in input 1). MODE 0: a*s, 1: a/s, 2: s/a.
+template <int MODE, class T>
+struct ScalarBinary {
+    static constexpr int N = 2;
+    using Out = T;
+    using In0 = T;
+    using In1 = typename Comp<T>::C;
+    using In2 = Unused;
+    using C = typename Comp<T>::C;
+    __device__ __forceinline__ T operator()(T a, C s) const {
+        const C x = Comp<T>::up(a);
+        if constexpr (MODE == 0) return Comp<T>::down(x * s);
+        else if constexpr (MODE == 1) return Comp<T>::down(x / s);
+        else return Comp<T>::down(s / x);
+    }
+};
+
+// ---- where --------------------------------------------------------------------------------------------
+
+template <class W>
+struct Select {
+    static constexpr int N = 3;
+    using Out = W;
+    using In0 = bool_t;
+    using In1 = W;
+    using In2 = W;
+    __device__ __forceinline__ W operator()(bool_t c, W x, W y) const { return c.v ? x : y; }
+};
+
+}  // namespace hmr

@@ -1,0 +1,81 @@
+/*
+ * cpu_backend.h -- the kernel interface a CPU backend offers to the host layer's dispatch.
+ *
+ * homura dispatches every tensor kernel on the device of its operands
+ * (ref: src/backend/mod.rs:44-55, 298-534): `Device::Cpu` goes to `cpu::<kernel>`,
+ * `Device::Rocm(i)` to `rocm::<kernel>`. This library ships the ROCm arm only. The CPU arm is a
+ * table of function pointers with the signatures of the reference's CPU kernels
+ * (ref: src/backend/cpu/mod.rs:28-38) that a process may register at run time; without one,
+ * every kernel on a CPU tensor fails with "no CPU backend is registered". Nothing in this
+ * package provides such a table.
+ *
+ * Tensors are described un-merged, exactly as the CPU kernels of the reference receive them
+ * (shape + strides + offset in elements); the backend does its own loop-nest planning.
+ */
+#ifndef HOMURA_CPU_BACKEND_H
+#define HOMURA_CPU_BACKEND_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct hcb_tensor {
+    void *data;             /* first byte of the storage */
+    int64_t offset;         /* of element (0,..,0), in elements */
+    int32_t dtype;          /* HMR_BOOL .. HMR_F64 */
+    int32_t ndim;
+    const int64_t *shape;   /* ndim entries */
+    const int64_t *strides; /* ndim entries, in elements, >= 0 */
+} hcb_tensor;
+
+/* homura's Scalar (ref: src/dtype.rs:285-293). */
+#define HCB_SCALAR_BOOL 0
+#define HCB_SCALAR_INT 1
+#define HCB_SCALAR_FLOAT 2
+typedef struct hcb_scalar {
+    int32_t kind;
+    int32_t reserved;
+    int64_t i; /* value for BOOL (0/1) and INT */
+    double f;  /* value for FLOAT */
+} hcb_scalar;
+
+/*
+ * Every kernel returns 0, or nonzero where the reference's CPU kernel would panic; the text of
+ * that panic is then available from last_error() until the thread's next call.
+ * All operands of one call have the same shape (inputs already expanded by the caller).
+ */
+typedef struct hcb_backend {
+    const char *name;
+    const char *(*last_error)(void);
+    /* ref: src/backend/cpu/mod.rs:315-332 */
+    int (*copy)(const hcb_tensor *dst, const hcb_tensor *src);
+    int (*fill)(const hcb_tensor *dst, hcb_scalar value);
+    /* ref: src/backend/cpu/mod.rs:336-507 */
+    int (*unary)(int32_t op, const hcb_tensor *out, const hcb_tensor *src);
+    int (*binary)(int32_t op, const hcb_tensor *out, const hcb_tensor *a, const hcb_tensor *b);
+    int (*binary_constant)(int32_t op, const hcb_tensor *out, const hcb_tensor *a,
+                           hcb_scalar value, int32_t constant_first);
+    int (*binary_scalar)(int32_t op, const hcb_tensor *out, const hcb_tensor *a, double s,
+                         int32_t scalar_first);
+    /* ref: src/backend/cpu/mod.rs:573-600; a NULL branch is the constant beside it */
+    int (*where_)(const hcb_tensor *out, const hcb_tensor *cond, const hcb_tensor *x,
+                  const hcb_tensor *y);
+    int (*where_constant)(const hcb_tensor *out, const hcb_tensor *cond, const hcb_tensor *x,
+                          hcb_scalar x_value, const hcb_tensor *y, hcb_scalar y_value);
+    /* ref: src/backend/cpu/reduce.rs:92-225; mask has src->ndim entries (1 = reduced) */
+    int (*reduce)(int32_t op, const hcb_tensor *out, const hcb_tensor *src, const uint8_t *mask);
+    int (*var)(const hcb_tensor *out, const hcb_tensor *src, const uint8_t *mask,
+               double correction, int32_t take_sqrt);
+    int (*arg_reduce)(const hcb_tensor *values, const hcb_tensor *indices, const hcb_tensor *src,
+                      int32_t dim, int32_t is_max);
+    /* ref: src/backend/cpu/misc.rs:15-51 */
+    int (*softmax)(const hcb_tensor *out, const hcb_tensor *src, int32_t dim, int32_t log);
+} hcb_backend;
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* HOMURA_CPU_BACKEND_H */

@@ -1,0 +1,304 @@
+/*
+ * homura_rocm.h -- C ABI of the gfx950 (MI355X, CDNA4, wave64) build of homura's ROCm layer.
+ *
+ * This header is a drop-in for the reference's csrc/homura_rocm.h for the tensor elementwise,
+ * broadcast, copy/convert, reduction and softmax entry points, plus the plumbing those need
+ * (contexts, memory, error text). Every declaration names the reference declaration it replaces
+ * as `ref: csrc/homura_rocm.h:<line>`; signatures, struct layouts and enumerator values are the
+ * same, so the Rust bindings in src/backend/rocm/ffi.rs bind to this library unchanged.
+ *
+ * Calling conventions (ref: csrc/homura_rocm.h:1-15):
+ *  - plain C, <stdint.h>/<stddef.h> only;
+ *  - every entry point returns an hmr_status; after a failure hmr_last_error() holds a message
+ *    that belongs to the calling thread and lives until that thread calls the library again;
+ *  - no C++ exception leaves the library;
+ *  - an entry point that uses a device makes it current for the calling thread and puts the
+ *    previous device back before it returns;
+ *  - enumerations travel as int32_t.
+ *
+ * Entry points of the reference that belong to other kernel families (gemm, indexing, pooling,
+ * random, fused optimiser steps ...) are declared in homura_rocm_unbuilt.h and exported as
+ * stubs that fail with HMR_INVALID, so that the reference crate still links.
+ */
+#ifndef HOMURA_ROCM_H
+#define HOMURA_ROCM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- status ------------------------------------------------- ref: csrc/homura_rocm.h:26-40 */
+#define HMR_OK 0
+#define HMR_OUT_OF_MEMORY 1 /* a device allocation found no memory */
+#define HMR_INVALID 2       /* bad argument, unsupported GPU, unsupported dtype/op pair */
+#define HMR_HIP_ERROR 3     /* the HIP runtime reported an error */
+#define HMR_INTERNAL_ERROR 4 /* a failure inside the library (e.g. a C++ exception) */
+
+typedef int32_t hmr_status;
+
+/* Text of the calling thread's most recent failure ("" when it has had none). */
+const char *hmr_last_error(void);
+
+/* ---- devices ------------------------------------------------ ref: csrc/homura_rocm.h:42-64 */
+#define HMR_NAME_LEN 256
+#define HMR_ARCH_LEN 64
+
+typedef struct hmr_device_properties {
+    char name[HMR_NAME_LEN]; /* marketing name */
+    char arch[HMR_ARCH_LEN]; /* "gfx950": gcnArchName without the ":sramecc+:xnack-" features */
+    /* hipDeviceProp_t::multiProcessorCount. On CDNA this IS the number of compute units (256
+     * on MI355X); the reference's doubling for RDNA work-group processors does not apply. */
+    int32_t multiprocessor_count;
+    int32_t warp_size; /* 64 on gfx950 */
+    uint64_t total_memory;
+} hmr_device_properties;
+
+/* Visible devices; 0 with HMR_OK when there is no device or no driver. */
+hmr_status hmr_device_count(int32_t *count);
+hmr_status hmr_device_properties_get(int32_t device, hmr_device_properties *out);
+hmr_status hmr_mem_get_info(int32_t device, uint64_t *free_bytes, uint64_t *total_bytes);
+
+/* ---- contexts ----------------------------------------------- ref: csrc/homura_rocm.h:66-79 */
+/* One per device: owns the non-blocking stream every kernel of that device is queued on. */
+typedef struct hmr_context *hmr_context_t;
+
+/* Fails with HMR_INVALID unless the GPU is one the library was built for (gfx950) and runs
+ * 64-lane wavefronts; then creates the stream and runs a probe kernel on it. Leaves nothing
+ * allocated on failure. */
+hmr_status hmr_context_create(int32_t device, hmr_context_t *out);
+hmr_status hmr_context_destroy(hmr_context_t ctx);
+/* Blocks until the context's stream is idle. */
+hmr_status hmr_context_synchronize(hmr_context_t ctx);
+
+/* ---- memory ------------------------------------------------- ref: csrc/homura_rocm.h:81-100 */
+/* hipMalloc / hipFree on `device`; running out of memory is HMR_OUT_OF_MEMORY and is not left
+ * behind as HIP's sticky last error. The caller's caching allocator sits on top of these. */
+hmr_status hmr_malloc(int32_t device, uint64_t nbytes, void **out);
+hmr_status hmr_free(int32_t device, void *ptr);
+/* Stream-ordered byte fill. */
+hmr_status hmr_memset(hmr_context_t ctx, void *ptr, uint8_t value, uint64_t nbytes);
+/* Stream-ordered copies to/from pageable host memory; they return once the bytes have moved. */
+hmr_status hmr_copy_to_host(hmr_context_t ctx, void *dst, const void *src, uint64_t nbytes);
+hmr_status hmr_copy_from_host(hmr_context_t ctx, void *dst, const void *src, uint64_t nbytes);
+
+/* ---- element types ------------------------------------------ ref: csrc/homura_rocm.h:102-113 */
+/* Numbered as homura's DType. BOOL is one byte holding 0 or 1; F16/BF16 are raw 16-bit patterns. */
+#define HMR_BOOL 0
+#define HMR_U8 1
+#define HMR_I8 2
+#define HMR_I16 3
+#define HMR_I32 4
+#define HMR_I64 5
+#define HMR_F16 6
+#define HMR_BF16 7
+#define HMR_F32 8
+#define HMR_F64 9
+
+/* ---- tensor descriptions ------------------------------------ ref: csrc/homura_rocm.h:115-130 */
+#define HMR_MAX_DIMS 25
+
+/* Element (i_0 .. i_{ndim-1}) lives at data[offset + sum_k i_k * strides[k]], counted in
+ * elements of `dtype`. ndim == 0 describes one element. The caller merges dimensions first
+ * (size-1 dims dropped, neighbours that are contiguous in every operand joined). 424 bytes. */
+typedef struct hmr_tensor_desc {
+    void *data;
+    int64_t offset;
+    int32_t dtype;
+    int32_t ndim;
+    int64_t sizes[HMR_MAX_DIMS];
+    int64_t strides[HMR_MAX_DIMS];
+} hmr_tensor_desc;
+
+/* ---- copy / convert / fill ---------------------------------- ref: csrc/homura_rocm.h:132-146 */
+/* dst[i] = cast(src[i]) with homura's Element::to_element rules (src/dtype.rs:171-277): float
+ * sources go through f64; halves are rounded through f32; float->int truncates, saturates to
+ * i64 and wraps; NaN payloads follow the CPU's conversions. Same ndim/sizes; src strides may
+ * be 0. Equal dtypes move the bytes. */
+hmr_status hmr_copy(hmr_context_t ctx, const hmr_tensor_desc *dst, const hmr_tensor_desc *src);
+/* Every element of dst = the element whose little-endian bytes are the low bytes of `bits`. */
+hmr_status hmr_fill(hmr_context_t ctx, const hmr_tensor_desc *dst, uint64_t bits);
+/* hipMemcpyAsync device->device of non-overlapping ranges on the context's device. */
+hmr_status hmr_copy_device(hmr_context_t ctx, void *dst, const void *src, uint64_t nbytes);
+
+/* ---- elementwise -------------------------------------------- ref: csrc/homura_rocm.h:148-263 */
+/*
+ * Results are those of homura's CPU backend (src/backend/cpu/mod.rs:336-600): F16/BF16/F32 are
+ * computed in f32 and F64 in f64 with one rounding to the dtype, integers wrap. Operands share
+ * ndim and sizes; input strides may be 0; the output's elements are distinct and either do not
+ * overlap an input or are that input (in place). HMR_INVALID for an op the dtype has no rule for.
+ */
+#define HMR_UNARY_NEG 0
+#define HMR_UNARY_ABS 1
+#define HMR_UNARY_SIGN 2
+#define HMR_UNARY_RELU 3
+#define HMR_UNARY_EXP 4
+#define HMR_UNARY_LOG 5
+#define HMR_UNARY_SQRT 6
+#define HMR_UNARY_RSQRT 7
+#define HMR_UNARY_RECIPROCAL 8
+#define HMR_UNARY_SIN 9
+#define HMR_UNARY_COS 10
+#define HMR_UNARY_ERF 11
+#define HMR_UNARY_TANH 12
+#define HMR_UNARY_SIGMOID 13
+#define HMR_UNARY_LOG_SIGMOID 14
+#define HMR_UNARY_SILU 15
+#define HMR_UNARY_GELU 16
+#define HMR_UNARY_GELU_TANH 17
+#define HMR_UNARY_LOGICAL_NOT 18
+
+#define HMR_BINARY_ADD 0
+#define HMR_BINARY_SUB 1
+#define HMR_BINARY_MUL 2
+#define HMR_BINARY_DIV 3
+#define HMR_BINARY_POW 4
+#define HMR_BINARY_MAXIMUM 5
+#define HMR_BINARY_MINIMUM 6
+#define HMR_BINARY_GREATER 7
+#define HMR_BINARY_GREATER_EQUAL 8
+#define HMR_BINARY_LESS 9
+#define HMR_BINARY_LESS_EQUAL 10
+#define HMR_BINARY_EQUAL 11
+#define HMR_BINARY_NOT_EQUAL 12
+#define HMR_BINARY_LOGICAL_AND 13
+#define HMR_BINARY_LOGICAL_OR 14
+/* Extension (the reference has no bitwise op, ref: src/ops/mod.rs:68-85): two's-complement `&`
+ * on integer dtypes, logical and on BOOL; floats are HMR_INVALID. Appended, nothing renumbered. */
+#define HMR_BINARY_BITWISE_AND 15
+
+/* ref :202  out = op(src). LOGICAL_NOT writes BOOL, everything else src's dtype. */
+hmr_status hmr_unary(hmr_context_t ctx, int32_t op, const hmr_tensor_desc *out,
+                     const hmr_tensor_desc *src);
+
+/* ref :206  out = op(a, b). Comparisons and logical ops write BOOL.
+ * Extension: when a and b are floating point dtypes that differ, each is first converted
+ * (exactly) to out's dtype, which must be their promotion; this folds the reference's separate
+ * cast kernel (ref: src/ops/mod.rs:177-195) into the op and yields the same bits. */
+hmr_status hmr_binary(hmr_context_t ctx, int32_t op, const hmr_tensor_desc *out,
+                      const hmr_tensor_desc *a, const hmr_tensor_desc *b);
+
+/* ref :212  hmr_binary with the other operand equal to the constant whose bytes are the low
+ * bytes of `bits` (an element of a's dtype); op(c, a) when constant_first. */
+hmr_status hmr_binary_constant(hmr_context_t ctx, int32_t op, const hmr_tensor_desc *out,
+                               const hmr_tensor_desc *a, uint64_t bits, int32_t constant_first);
+
+/* ref :217  MUL and DIV only, float `a`: a*s, a/s or (scalar_first) s/a with `s` rounded to the
+ * computation type, not to the dtype (f16/bf16 keep an f32 scalar). */
+hmr_status hmr_binary_scalar(hmr_context_t ctx, int32_t op, const hmr_tensor_desc *out,
+                             const hmr_tensor_desc *a, double s, int32_t scalar_first);
+
+/* ref :247  out = cond ? x : y, cond BOOL, x and y of out's dtype. */
+hmr_status hmr_where(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_tensor_desc *cond,
+                     const hmr_tensor_desc *x, const hmr_tensor_desc *y);
+
+/* ref :253  hmr_where where a NULL branch stands for the constant x_bits / y_bits. */
+hmr_status hmr_where_constant(hmr_context_t ctx, const hmr_tensor_desc *out,
+                              const hmr_tensor_desc *cond, const hmr_tensor_desc *x,
+                              uint64_t x_bits, const hmr_tensor_desc *y, uint64_t y_bits);
+
+/* ---- reductions --------------------------------------------- ref: csrc/homura_rocm.h:297-346 */
+/*
+ * `kept`: the kept dimensions with the SOURCE's strides, data, offset, dtype; `red`: the reduced
+ * dimensions with the source's strides (same dtype). Outputs are contiguous over kept's sizes.
+ * The fold order depends only on sizes and strides, so results repeat from run to run. Plans
+ * that cut the reduced range across workgroups stage partial results in `workspace`, whose size
+ * hmr_reduce_workspace reports (var = 1 for hmr_var); NULL is fine when that is 0.
+ */
+#define HMR_REDUCE_SUM 0
+#define HMR_REDUCE_PROD 1
+#define HMR_REDUCE_MEAN 2
+#define HMR_REDUCE_MAX 3
+#define HMR_REDUCE_MIN 4
+#define HMR_REDUCE_ALL 5
+#define HMR_REDUCE_ANY 6
+
+/* ref :315 */
+hmr_status hmr_reduce_workspace(const hmr_tensor_desc *kept, const hmr_tensor_desc *red,
+                                int32_t var, int64_t *bytes);
+
+/* ref :321  cpu::reduce (src/backend/cpu/reduce.rs:92-131): float SUM/PROD/MEAN accumulate in
+ * f64; integer and bool SUM/PROD wrap in i64 and write I64; MAX/MIN keep the dtype (first NaN
+ * wins, then the first of equals) and need a nonempty range; ALL/ANY write BOOL (U8 for U8). */
+hmr_status hmr_reduce(hmr_context_t ctx, int32_t op, const hmr_tensor_desc *out,
+                      const hmr_tensor_desc *kept, const hmr_tensor_desc *red, void *workspace,
+                      int64_t workspace_bytes);
+
+/* ref :327  cpu::var (src/backend/cpu/reduce.rs:135-170): f64 variance about the f64 mean,
+ * divided by max(0, n - correction); NaN for n == 0; sqrt of it with take_sqrt. */
+hmr_status hmr_var(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_tensor_desc *kept,
+                   const hmr_tensor_desc *red, double correction, int32_t take_sqrt,
+                   void *workspace, int64_t workspace_bytes);
+
+/* ref :333  cpu::arg_reduce (src/backend/cpu/reduce.rs:175-225): I64 index along the single
+ * reduced dimension of the max (min) and, when `values` is not NULL, the value itself. */
+hmr_status hmr_arg_reduce(hmr_context_t ctx, const hmr_tensor_desc *values,
+                          const hmr_tensor_desc *indices, const hmr_tensor_desc *kept,
+                          const hmr_tensor_desc *red, int32_t is_max, void *workspace,
+                          int64_t workspace_bytes);
+
+/* ref :341-346  cpu::softmax (src/backend/cpu/misc.rs:15-51) over rows of n elements:
+ * `out_rows` / `src_rows` describe the remaining dimensions, row elements are out_stride /
+ * src_stride apart. */
+hmr_status hmr_softmax_workspace(const hmr_tensor_desc *src_rows, int64_t n, int64_t src_stride,
+                                 int64_t *bytes);
+hmr_status hmr_softmax(hmr_context_t ctx, const hmr_tensor_desc *out_rows,
+                       const hmr_tensor_desc *src_rows, int64_t n, int64_t out_stride,
+                       int64_t src_stride, int32_t log, void *workspace,
+                       int64_t workspace_bytes);
+
+/* ---- build facts and ABI self-description ------------------- ref: csrc/homura_rocm.h:589-610 */
+/* ';'-separated offload architectures compiled in ("gfx950"). */
+const char *hmr_built_archs(void);
+
+typedef struct hmr_abi_info {
+    uint32_t abi_info_size;
+    uint32_t properties_size;
+    uint32_t properties_align;
+    uint32_t properties_offsets[5];
+    int32_t status_values[5];
+    int32_t name_len;
+    int32_t arch_len;
+    uint32_t desc_size;
+    uint32_t desc_align;
+    uint32_t desc_offsets[6];
+    int32_t dtype_values[10];
+    int32_t max_dims;
+    uint32_t gemm_desc_size;
+    uint32_t gemm_desc_align;
+} hmr_abi_info;
+
+/* Sizes, alignments, field offsets and enumerator values as this library was compiled. */
+void hmr_abi_check(hmr_abi_info *out);
+
+/* ---- test hooks ("not part of the supported interface") ----- ref: csrc/homura_rocm.h:612-666 */
+/* Per calling thread: the next n stream creations / context creations after the probe /
+ * property queries / data operations fail (data operations fail before queueing anything, as
+ * out of memory when out_of_memory != 0, else as an invalid handle). */
+void hmr_test_fail_stream_create(int32_t n);
+void hmr_test_fail_after_probe(int32_t n);
+void hmr_test_fail_properties(int32_t n);
+void hmr_test_fail_data(int32_t n, int32_t out_of_memory);
+/* The plan this library picks. The numbers describe THIS design and are not the reference's:
+ *   group  = lanes that cooperate on one output (1, 64 = one wave, or the workgroup size),
+ *   splits = workgroup slices the reduced range is cut into (>1 means a second pass),
+ *   chunk  = reduced elements per slice. */
+hmr_status hmr_test_reduce_plan(const hmr_tensor_desc *kept, const hmr_tensor_desc *red,
+                                int64_t *group, int64_t *splits, int64_t *chunk);
+/*   split = 0 (rows are never cut: one wave or one workgroup owns a row),
+ *   group = lanes per row, cache = row elements a lane keeps in registers (0: the row is
+ *   streamed twice instead). */
+hmr_status hmr_test_softmax_plan(const hmr_tensor_desc *src_rows, int64_t n, int64_t src_stride,
+                                 int32_t *split, int32_t *group, int32_t *cache);
+int32_t hmr_test_live_streams(void);
+hmr_status hmr_test_current_device(int32_t *device);
+hmr_status hmr_test_set_current_device(int32_t device);
+hmr_status hmr_test_fail(const char *message);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* HOMURA_ROCM_H */
