@@ -1,0 +1,236 @@
+#!/usr/bin/env python3
+"""Throughput of homura's elementwise / broadcast / reduction path on one MI355X.
+
+A step is one pass of the hot path over one batch of BASELINE.json configs[1]: the bf16 broadcast
+chain  ((x[8,2048,4096] + bias[4096]) * scale[8,2048,1]) + residual_f32[8,2048,4096]  through the
+C++ host layer (type promotion, broadcasting, output allocation) and the C ABI, three kernel
+launches. `value` is algorithmic bytes per step / time per step with every input resident in HBM.
+
+The same JSON line carries
+  roofline      the dominant kernel of the step (the bf16 + f32 -> f32 add), timed on its own with
+                HIP events on the stream it is launched on;
+  cpu_baseline  the CPU oracle (a port of homura's single-threaded CPU backend) timed on one host
+                core on the same workload;
+  ops           achieved GB/s and fraction of the 8 TB/s HBM peak for every op of every BASELINE
+                config (--ops none to skip), algorithmic bytes as in BASELINE.md section 3.
+
+usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--ops all|none]
+"""
+import argparse
+import ctypes
+import json
+import math
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+METRIC = "achieved HBM GB/s & % of MI355X peak per op; speedup vs host-CPU reference"
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--ops", choices=["all", "none"], default="all")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU: this path has no cross-GPU step (every box has one GPU); got --gpus {args.gpus}",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import homura_amd
+    from tests.support import DT, GPU, NP, from_f64, normal, tensor, uniform, words
+
+    h = homura_amd.load_host()
+    hip = ctypes.CDLL("libamdhip64.so")
+    stream = ctypes.c_void_p(h.stream_handle(GPU))
+
+    def event():
+        e = ctypes.c_void_p()
+        assert hip.hipEventCreate(ctypes.byref(e)) == 0
+        return e
+
+    def timed(fn, iters, warmup):
+        """Average milliseconds per call of fn over `iters` calls, by HIP events on the kernels' stream."""
+        for _ in range(warmup):
+            fn()
+        h.synchronize(GPU)
+        a, b = event(), event()
+        assert hip.hipEventRecord(a, stream) == 0
+        for _ in range(iters):
+            fn()
+        assert hip.hipEventRecord(b, stream) == 0
+        assert hip.hipEventSynchronize(b) == 0
+        h.synchronize(GPU)
+        ms = ctypes.c_float()
+        assert hip.hipEventElapsedTime(ctypes.byref(ms), a, b) == 0
+        hip.hipEventDestroy(a)
+        hip.hipEventDestroy(b)
+        return ms.value / iters
+
+    # ---- configs[1]: the broadcast + promotion chain --------------------------------------------------
+    B, S, H = 8, 2048, 4096
+    N = B * S * H
+    host_x = from_f64(normal(0x5EED0001, N), DT.BF16)
+    host_bias = from_f64(normal(0x5EED0002, H, 0.0, 0.02), DT.BF16)
+    host_scale = from_f64(uniform(0x5EED0003, B * S, 0.5, 1.5), DT.BF16)
+    host_res = from_f64(normal(0x5EED0004, N), DT.F32)
+    x = tensor(host_x, DT.BF16, [B, S, H], GPU)
+    bias = tensor(host_bias, DT.BF16, [H], GPU)
+    scale = tensor(host_scale, DT.BF16, [B, S, 1], GPU)
+    residual = tensor(host_res, DT.F32, [B, S, H], GPU)
+
+    def chain():
+        return x.add(bias).mul(scale).add(residual)
+
+    chain_bytes = (4 * N + 2 * H) + (4 * N + 2 * B * S) + 10 * N  # BASELINE.md section 3, promotion fused
+    ms_step = timed(chain, args.steps, args.warmup)
+    value = chain_bytes / (ms_step * 1e-3) / 1e9
+
+    # The dominant kernel: bf16 + f32 -> f32 (10 bytes per element).
+    t2 = x.add(bias).mul(scale)
+    ms_add = timed(lambda: t2.add(residual), max(args.steps, 20), 3)
+    add_bytes = 10 * N
+    achieved = add_bytes / (ms_add * 1e-3) / 1e9
+    roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "kernel": "map_rows_kernel<FloatBinary<ADD, f32, bf16, f32>> (bf16 + f32 -> f32)",
+                "algorithmic_bytes_per_launch": add_bytes, "us_per_launch": round(ms_add * 1e3, 2)}
+
+    # ---- every op of every config ------------------------------------------------------------------------
+    ops = []
+    if args.ops == "all":
+        ops = per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP, x, bias, scale, residual, t2)
+
+    # ---- CPU baseline: the oracle on one host core, same workload ------------------------------------------
+    cpu = None
+    if not args.no_cpu:
+        from tests import oracle
+
+        h.register_cpu_backend(oracle.backend_address())
+        cx = tensor(host_x, DT.BF16, [B, S, H])
+        cb = tensor(host_bias, DT.BF16, [H])
+        cs = tensor(host_scale, DT.BF16, [B, S, 1])
+        cr = tensor(host_res, DT.F32, [B, S, H])
+        t0 = time.perf_counter()
+        cx.add(cb).mul(cs).add(cr)
+        dt = time.perf_counter() - t0
+        # The CPU path follows the reference: the bf16 intermediate is cast to f32 by a separate copy.
+        cpu = {"value": round(chain_bytes / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+               "host_cores_available": os.cpu_count(),
+               "sample": "one full pass of configs[1] (67 108 864 elements per op), C++ port of homura's "
+                         "single-threaded CPU backend, g++ -O2 -ffp-contract=off",
+               "seconds": round(dt, 3), "gpu_speedup": round(value / (chain_bytes / dt / 1e9), 1)}
+
+    line = {
+        "metric": METRIC, "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16+f32", "data": "synthetic",
+        "config": {"workload": "configs[1]: ((x_bf16[8,2048,4096] + bias_bf16[4096]) * scale_bf16[8,2048,1]) + "
+                               "residual_f32[8,2048,4096] -> f32; 3 kernel launches per step",
+                   "algorithmic_bytes_per_step": chain_bytes, "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+                   "seeds": "SplitMix64 0x5EED0001..4"},
+        "roofline": roofline, "cpu_baseline": cpu, "ops": ops,
+    }
+    print(json.dumps(line))
+
+
+def per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP, x, bias, scale, residual, t2):
+    """[{cfg, op, bytes, us, gbs, frac}] for the ops of BASELINE configs 1-5."""
+    rows = []
+
+    def add(cfg, op, nbytes, fns, iters=20):
+        """fns: one callable, or several over disjoint buffers that are cycled so that a working set
+        smaller than the 256 MB Infinity Cache is read from HBM every time."""
+        fns = fns if isinstance(fns, list) else [fns]
+        k = [0]
+
+        def call():
+            fns[k[0] % len(fns)]()
+            k[0] += 1
+
+        ms = timed(call, iters, 3)
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        rows.append({"cfg": cfg, "op": op, "bytes": nbytes, "us": round(ms * 1e3, 2), "gbs": round(gbs, 1),
+                     "frac": round(gbs / HBM_PEAK_GBS, 4)})
+
+    N = x.num_elements()
+    # cfg 1: f32 add [4096, 4096], four disjoint buffer sets (805 MB in rotation).
+    n1 = 4096 * 4096
+    sets = []
+    for i in range(4):
+        a = tensor(uniform(0x5EED0100 + 2 * i, n1, -1.0, 1.0).astype(np.float32), DT.F32, [4096, 4096], GPU)
+        b = tensor(uniform(0x5EED0101 + 2 * i, n1, -1.0, 1.0).astype(np.float32), DT.F32, [4096, 4096], GPU)
+        sets.append((a, b))
+    add(1, "add f32 [4096,4096] (HBM-resident, rotating buffers)", 12 * n1, [lambda a=a, b=b: a.add(b) for a, b in sets], 40)
+    a0, b0 = sets[0]
+    add(1, "add f32 [4096,4096] (same buffers, Infinity-Cache-resident)", 12 * n1, lambda: a0.add(b0), 40)
+    del sets
+    # cfg 2: the three steps.
+    t1 = x.add(bias)
+    add(2, "x_bf16 + bias_bf16[4096] (inner broadcast)", 4 * N + 2 * 4096, lambda: x.add(bias))
+    add(2, "t_bf16 * scale_bf16[8,2048,1] (row broadcast)", 4 * N + 2 * 8 * 2048, lambda: t1.mul(scale))
+    add(2, "t_bf16 + residual_f32 -> f32 (promotion fused)", 10 * N, lambda: t2.add(residual))
+    h.set_fused_promotion(False)
+    add(2, "t_bf16 + residual_f32 -> f32 (reference style: cast kernel + add, 2 launches)", 18 * N,
+        lambda: t2.add(residual))
+    h.set_fused_promotion(True)
+    del t1
+    # cfg 3: reductions of f32 [16384, 4096] and of its bf16 copy.
+    R, C = 16384, 4096
+    xf = residual.reshape([R, C])
+    add(3, "sum dim=-1 f32", 4 * N + 4 * R, lambda: xf.sum_dim(-1, False))
+    add(3, "mean dim=-1 f32", 4 * N + 4 * R, lambda: xf.mean_dim(-1, False))
+    add(3, "amax dim=-1 f32 (max_dim: values + i64 indices)", 4 * N + 12 * R, lambda: xf.max_dim(-1, False))
+    add(3, "var(unbiased) dim=-1 f32", 4 * N + 4 * R, lambda: xf.var_dim(-1, 1, False))
+    add(3, "sum dim=0 f32", 4 * N + 4 * C, lambda: xf.sum_dim(0, False))
+    add(3, "mean dim=0 f32", 4 * N + 4 * C, lambda: xf.mean_dim(0, False))
+    add(3, "amax dim=0 f32 (max_dim: values + i64 indices)", 4 * N + 12 * C, lambda: xf.max_dim(0, False))
+    add(3, "var(unbiased) dim=0 f32", 4 * N + 4 * C, lambda: xf.var_dim(0, 1, False))
+    add(3, "sum over all elements f32", 4 * N + 4, lambda: xf.sum())
+    xb = xf.to(DT.BF16)
+    add(3, "sum dim=-1 bf16", 2 * N + 2 * R, lambda: xb.sum_dim(-1, False))
+    del xb
+    # cfg 4: permuted bf16 unary; int64 ops.
+    p = tensor(from_f64(normal(0x5EED0400, N, 0.0, 2.0), DT.BF16), DT.BF16, [8, 2048, 32, 128], GPU).permute([0, 2, 1, 3])
+    add(4, "silu bf16 [8,2048,32,128].permute(0,2,1,3) -> contiguous", 4 * N, lambda: p.silu())
+    add(4, "gelu(erf) bf16, same view", 4 * N, lambda: p.gelu())
+    del p
+    w1 = words(0x5EED0401, N)
+    w2 = words(0x5EED0402, N)
+    ia = tensor(((w1 % np.uint64(2001)).astype(np.int64) - 1000), DT.I64, [8, 2048, 4096], GPU)
+    ib = tensor(((w2 % np.uint64(2001)).astype(np.int64) - 1000), DT.I64, [8, 2048, 4096], GPU)
+    del w1, w2
+    add(4, "bitwise_and i64", 24 * N, lambda: ia.bitwise_and(ib))
+    add(4, "greater i64 -> bool", 17 * N, lambda: ia.greater(ib))
+    mask = ia.greater(ib)
+    add(4, "where(mask, a, b) i64", 25 * N, lambda: h.where_(mask, ia, ib))
+    del ia, ib, mask
+    # cfg 5a: bf16 logits [4096, 32000].
+    n5a = 4096 * 32000
+    logits = tensor(from_f64(normal(0x5EED0500, n5a, 0.0, 3.0), DT.BF16), DT.BF16, [4096, 32000], GPU)
+    add(5, "softmax bf16 [4096,32000]", 4 * n5a, lambda: logits.softmax(-1))
+    add(5, "log_softmax bf16 [4096,32000]", 4 * n5a, lambda: logits.log_softmax(-1))
+    del logits
+    # cfg 5b: causal f32 scores [32, 2048, 2048].
+    n5b = 32 * 2048 * 2048
+    s = normal(0x5EED0501, n5b).astype(np.float32).reshape(32, 2048, 2048)
+    s[:, np.triu_indices(2048, 1)[0], np.triu_indices(2048, 1)[1]] = -np.inf
+    scores = tensor(s, DT.F32, [32, 2048, 2048], GPU)
+    del s
+    add(5, "softmax f32 [32,2048,2048] causal", 8 * n5b, lambda: scores.softmax(-1))
+    add(5, "log_softmax f32 [32,2048,2048] causal", 8 * n5b, lambda: scores.log_softmax(-1))
+    return rows
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,271 @@
+// Reduction plans and the entry points hmr_reduce_workspace, hmr_reduce, hmr_var, hmr_arg_reduce,
+// hmr_test_reduce_plan (ref: csrc/homura_rocm.h:297-336, csrc/reduce.hip:133-170, 432-517).
+#include "reduce_plan.hpp"
+
+namespace hmr {
+namespace {
+
+// Merges a description's dimensions by its strides (size-1 dropped, contiguous neighbours joined)
+// into a Walk, innermost first. Returns the element count (0 when a size is 0).
+int64_t build_walk(const hmr_tensor_desc &d, Walk &w) {
+    int64_t size[HMR_MAX_DIMS], stride[HMR_MAX_DIMS];
+    int n = 0;
+    int64_t count = 1;
+    for (int i = 0; i < d.ndim; ++i) count *= d.sizes[i];
+    w.ndim = 0;
+    if (count == 0) return 0;
+    for (int i = 0; i < d.ndim; ++i) {
+        if (d.sizes[i] == 1) continue;
+        int64_t prod = 0;
+        if (n > 0 && !__builtin_mul_overflow(d.strides[i], d.sizes[i], &prod) && prod == stride[n - 1]) {
+            size[n - 1] *= d.sizes[i];
+            stride[n - 1] = d.strides[i];
+        } else {
+            size[n] = d.sizes[i];
+            stride[n] = d.strides[i];
+            ++n;
+        }
+    }
+    w.ndim = n;
+    for (int i = 0; i < n; ++i) {
+        w.size[i] = size[n - 1 - i];
+        w.stride[i] = stride[n - 1 - i];
+    }
+    return count;
+}
+
+int64_t ceil_div(int64_t a, int64_t b) { return a / b + (a % b != 0); }
+
+int64_t clamp64(int64_t v, int64_t lo, int64_t hi) { return v < lo ? lo : (v > hi ? hi : v); }
+
+// Cuts nred into at most `want` slices of a multiple of `quantum` elements.
+void cut(ReducePlan &p, int64_t want, int64_t quantum) {
+    int64_t nred = p.args.nred;
+    if (want <= 1 || nred <= quantum) {
+        p.splits = 1;
+        p.chunk = nred;
+        return;
+    }
+    int64_t chunk = ceil_div(ceil_div(nred, want), quantum) * quantum;
+    p.chunk = chunk;
+    p.splits = ceil_div(nred, chunk);
+    if (p.splits <= 1) {
+        p.splits = 1;
+        p.chunk = nred;
+    }
+}
+
+}  // namespace
+
+hmr_status plan_reduction(const hmr_tensor_desc *out, const hmr_tensor_desc &kept, const hmr_tensor_desc &red,
+                          ReducePlan &p) {
+    int64_t n = 0;
+    if (hmr_status s = check_desc(kept, n)) return s;
+    if (hmr_status s = check_desc(red, n)) return s;
+    if (red.dtype != kept.dtype) return fail(HMR_INVALID, "reduction descriptions differ");
+    if (out != nullptr) {
+        if (hmr_status s = check_desc(*out, n)) return s;
+        bool same = out->ndim == kept.ndim;
+        int64_t stride = 1;
+        for (int k = kept.ndim - 1; same && k >= 0; --k) {
+            same = out->sizes[k] == kept.sizes[k] && (out->sizes[k] == 1 || out->strides[k] == stride);
+            stride *= kept.sizes[k];
+        }
+        if (!same) return fail(HMR_INVALID, "a reduction's output is not contiguous with its sizes");
+    }
+    const int elem = dtype_size(kept.dtype);
+    ReduceArgs &a = p.args;
+    a.src = static_cast<const char *>(kept.data) + kept.offset * elem;
+    a.nout = build_walk(kept, a.kept);
+    a.nred = build_walk(red, a.red);
+    a.partials = nullptr;
+    p.kind = ReduceKind::Any;
+    p.group = 1;
+    p.splits = 1;
+    p.chunk = a.nred;
+    p.rstride = 0;
+    p.inner = 0;
+    if (a.nout == 0 || a.nred == 0) return HMR_OK;  // nothing to read: one lane per output writes the identity
+
+    const bool base_aligned = reinterpret_cast<uintptr_t>(a.src) % 16 == 0;
+    auto strides_aligned = [&](const Walk &w, int from) {
+        for (int d = from; d < w.ndim; ++d) {
+            if ((w.stride[d] * elem) % 16 != 0) return false;
+        }
+        return true;
+    };
+    const bool red_contiguous = a.red.ndim == 1 && a.red.stride[0] == 1;
+    const int vec = 16 / elem;
+
+    // Rows: one contiguous run per output.
+    if (red_contiguous && a.nred >= 256 && base_aligned && strides_aligned(a.kept, 0)) {
+        p.kind = ReduceKind::Rows;
+        if (a.nout * kWave >= kTargetLanes / 2 || a.nred <= 2048) {
+            p.group = kWave;
+        } else {
+            p.group = kBlock;
+            if (a.nout * kBlock < kTargetLanes / 2) cut(p, ceil_div(2 * kTargetLanes, a.nout * kBlock), 4096);
+        }
+        return HMR_OK;
+    }
+    // Cols: a contiguous run of outputs, one strided reduced dimension.
+    if (a.red.ndim == 1 && a.kept.ndim >= 1 && a.kept.stride[0] == 1 && a.kept.size[0] >= 32 && base_aligned &&
+        (a.red.stride[0] * elem) % 16 == 0 && strides_aligned(a.kept, 1)) {
+        p.kind = ReduceKind::Cols;
+        p.group = kBlock / kWave;
+        p.rstride = a.red.stride[0];
+        p.inner = a.kept.size[0];
+        // The kernel walks the outer kept dimensions only.
+        for (int d = 1; d < a.kept.ndim; ++d) {
+            a.kept.size[d - 1] = a.kept.size[d];
+            a.kept.stride[d - 1] = a.kept.stride[d];
+        }
+        a.kept.ndim -= 1;
+        int64_t tiles = ceil_div(p.inner, int64_t{kWave} * vec) * (a.nout / p.inner);
+        cut(p, ceil_div(8 * 256, tiles), 16);
+        return HMR_OK;
+    }
+    // Any layout.
+    p.group = a.nred <= 32 ? 1 : (a.nred <= 4096 ? kWave : kBlock);
+    if (a.nout * p.group < kTargetLanes / 2 && a.nred > 4096) {
+        cut(p, ceil_div(kTargetLanes, a.nout * p.group), 1024);
+    }
+    return HMR_OK;
+}
+
+int64_t means_bytes(const ReducePlan &p, bool var) {
+    if (!var || p.args.nout == 0) return 0;
+    return (p.args.nout * 8 + 255) / 256 * 256;
+}
+
+int64_t partial_bytes(const ReducePlan &p) { return p.splits > 1 ? p.splits * p.args.nout * kPartialBytes : 0; }
+
+namespace {
+
+// Checks the workspace and returns where the partials start.
+hmr_status take_workspace(const ReducePlan &p, bool var, void *workspace, int64_t bytes, void *&partials) {
+    int64_t need = means_bytes(p, var) + partial_bytes(p);
+    if (need > 0 && (workspace == nullptr || bytes < need)) {
+        return fail(HMR_INVALID, "a reduction's workspace is too small");
+    }
+    partials = need > 0 ? static_cast<char *>(workspace) + means_bytes(p, var) : nullptr;
+    return HMR_OK;
+}
+
+void *element0(const hmr_tensor_desc &d) { return static_cast<char *>(d.data) + d.offset * dtype_size(d.dtype); }
+
+bool is_float(int d) { return d >= HMR_F16 && d <= HMR_F64; }
+
+}  // namespace
+}  // namespace hmr
+
+using hmr::guarded;
+
+extern "C" {
+
+hmr_status hmr_reduce_workspace(const hmr_tensor_desc *kept, const hmr_tensor_desc *red, int32_t var,
+                                int64_t *bytes) {
+    return guarded([&] {
+        hmr::ReducePlan p;
+        if (hmr_status s = hmr::plan_reduction(nullptr, *kept, *red, p)) return s;
+        *bytes = hmr::means_bytes(p, var != 0) + hmr::partial_bytes(p);
+        return HMR_OK;
+    });
+}
+
+hmr_status hmr_test_reduce_plan(const hmr_tensor_desc *kept, const hmr_tensor_desc *red, int64_t *group,
+                                int64_t *splits, int64_t *chunk) {
+    return guarded([&] {
+        hmr::ReducePlan p;
+        if (hmr_status s = hmr::plan_reduction(nullptr, *kept, *red, p)) return s;
+        *group = p.group;
+        *splits = p.splits;
+        *chunk = p.chunk;
+        return HMR_OK;
+    });
+}
+
+hmr_status hmr_reduce(hmr_context_t ctx, int32_t op, const hmr_tensor_desc *out, const hmr_tensor_desc *kept,
+                      const hmr_tensor_desc *red, void *workspace, int64_t workspace_bytes) {
+    return guarded([&] {
+        hmr::ReducePlan p;
+        if (hmr_status s = hmr::plan_reduction(out, *kept, *red, p)) return s;
+        void *partials = nullptr;
+        if (hmr_status s = hmr::take_workspace(p, false, workspace, workspace_bytes, partials)) return s;
+        if (p.args.nout == 0) return HMR_OK;
+        if ((op == HMR_REDUCE_MAX || op == HMR_REDUCE_MIN) && p.args.nred == 0) {
+            return hmr::fail(HMR_INVALID, "reduction over an empty dimension");
+        }
+        return hmr::launch_on(ctx, "reduce", [&](hipStream_t stream) {
+            const int dtype = kept->dtype;
+            void *o = hmr::element0(*out);
+            switch (op) {
+                case HMR_REDUCE_SUM:
+                case HMR_REDUCE_PROD:
+                case HMR_REDUCE_MEAN:
+                    if (hmr::is_float(dtype)) {
+                        if (out->dtype != dtype) return false;
+                        return hmr::launch_float_reduce(op, dtype, p, partials, o, stream);
+                    }
+                    if (op == HMR_REDUCE_MEAN || out->dtype != HMR_I64) return false;
+                    return hmr::launch_int_reduce(op, dtype, p, partials, o, stream);
+                case HMR_REDUCE_MAX:
+                case HMR_REDUCE_MIN:
+                    if (out->dtype != dtype) return false;
+                    return hmr::launch_extreme_reduce(op == HMR_REDUCE_MAX, dtype, p, partials, o, nullptr, stream);
+                case HMR_REDUCE_ALL:
+                case HMR_REDUCE_ANY:
+                    if (out->dtype != (dtype == HMR_U8 ? HMR_U8 : HMR_BOOL)) return false;
+                    return hmr::launch_truth_reduce(op, dtype, p, partials, o, stream);
+                default: return false;
+            }
+        });
+    });
+}
+
+hmr_status hmr_var(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_tensor_desc *kept,
+                   const hmr_tensor_desc *red, double correction, int32_t take_sqrt, void *workspace,
+                   int64_t workspace_bytes) {
+    return guarded([&] {
+        hmr::ReducePlan p;
+        if (hmr_status s = hmr::plan_reduction(out, *kept, *red, p)) return s;
+        void *partials = nullptr;
+        if (hmr_status s = hmr::take_workspace(p, true, workspace, workspace_bytes, partials)) return s;
+        if (p.args.nout == 0) return HMR_OK;
+        return hmr::launch_on(ctx, "var", [&](hipStream_t stream) {
+            if (out->dtype != kept->dtype || !hmr::is_float(kept->dtype)) return false;
+            double *means = static_cast<double *>(workspace);
+            double divisor = static_cast<double>(p.args.nred) - correction;
+            divisor = divisor > 0.0 ? divisor : 0.0;
+            if (!hmr::launch_mean_pass(kept->dtype, p, partials, means, stream)) return false;
+            return hmr::launch_deviation_pass(kept->dtype, p, partials, means, hmr::element0(*out), divisor,
+                                              take_sqrt != 0, stream);
+        });
+    });
+}
+
+hmr_status hmr_arg_reduce(hmr_context_t ctx, const hmr_tensor_desc *values, const hmr_tensor_desc *indices,
+                          const hmr_tensor_desc *kept, const hmr_tensor_desc *red, int32_t is_max, void *workspace,
+                          int64_t workspace_bytes) {
+    return guarded([&] {
+        hmr::ReducePlan p;
+        if (hmr_status s = hmr::plan_reduction(indices, *kept, *red, p)) return s;
+        if (values != nullptr) {
+            hmr::ReducePlan q;
+            if (hmr_status s = hmr::plan_reduction(values, *kept, *red, q)) return s;
+        }
+        void *partials = nullptr;
+        if (hmr_status s = hmr::take_workspace(p, false, workspace, workspace_bytes, partials)) return s;
+        if (p.args.nred == 0) return hmr::fail(HMR_INVALID, "arg reduction of an empty dimension");
+        if (p.args.nout == 0) return HMR_OK;
+        return hmr::launch_on(ctx, "arg_reduce", [&](hipStream_t stream) {
+            if (indices->dtype != HMR_I64) return false;
+            if (values != nullptr && values->dtype != kept->dtype) return false;
+            return hmr::launch_extreme_reduce(is_max != 0, kept->dtype, p, partials,
+                                              values ? hmr::element0(*values) : nullptr, hmr::element0(*indices),
+                                              stream);
+        });
+    });
+}
+
+}  // extern "C"

@@ -1,0 +1,563 @@
+// Storage, the device dispatch of every kernel, and the ROCm host side that turns tensors into
+// hmr_tensor_desc's and calls the C ABI. See homura.hpp for the map to the reference's files.
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <mutex>
+
+#include "homura.hpp"
+#include "homura_rocm.h"
+#include "homura_rocm_ext.h"
+
+namespace homura {
+
+namespace {
+
+// ---- the C ABI: status -> Error (ref: src/backend/rocm/mod.rs:55-75) ------------------------------
+
+void expect(hmr_status s) {
+    if (s == HMR_OK) return;
+    std::string message = hmr_last_error();
+    if (s == HMR_OUT_OF_MEMORY) throw Error("ROCm out of memory: " + message);
+    throw Error(message);
+}
+
+// ---- contexts: one per device, created on first use (ref: src/backend/rocm/context.rs:137-210) ----
+
+struct DeviceState {
+    hmr_context_t ctx = nullptr;
+    std::recursive_mutex exec;  // makes one op's kernel submissions atomic
+    std::mutex alloc;
+    std::multimap<size_t, void *> cache;  // freed blocks by size, reused in stream order
+};
+
+std::mutex g_registry;
+std::map<int, std::unique_ptr<DeviceState>> g_devices;
+
+DeviceState &device_state(int index) {
+    std::lock_guard<std::mutex> lock(g_registry);
+    auto it = g_devices.find(index);
+    if (it != g_devices.end()) return *it->second;
+    auto st = std::make_unique<DeviceState>();
+    expect(hmr_context_create(index, &st->ctx));
+    return *(g_devices[index] = std::move(st));
+}
+
+// Runs `f(ctx)` inside the device's execution lock.
+template <class F>
+void exec(const TensorData &on, F f) {
+    DeviceState &st = device_state(on.device().index);
+    std::lock_guard<std::recursive_mutex> lock(st.exec);
+    f(st.ctx);
+}
+
+// ---- a minimal caching allocator over hmr_malloc (ref: src/backend/caching.rs:1-13) ---------------
+// Every kernel of a device runs on its one stream, so a freed block may be handed out again at once:
+// work already queued on it finishes before anything queued later touches it.
+
+size_t round_block(size_t nbytes) {
+    const size_t q = nbytes < (1u << 20) ? 512 : (2u << 20);
+    return (nbytes + q - 1) / q * q;
+}
+
+void *device_alloc(int index, size_t block) {
+    DeviceState &st = device_state(index);
+    {
+        std::lock_guard<std::mutex> lock(st.alloc);
+        auto it = st.cache.find(block);
+        if (it != st.cache.end()) {
+            void *p = it->second;
+            st.cache.erase(it);
+            return p;
+        }
+    }
+    void *p = nullptr;
+    hmr_status s = hmr_malloc(index, block, &p);
+    if (s == HMR_OUT_OF_MEMORY) {
+        // Release the cache and try once more, as the reference's allocator does.
+        {
+            std::lock_guard<std::recursive_mutex> run(st.exec);
+            expect(hmr_context_synchronize(st.ctx));
+            std::lock_guard<std::mutex> lock(st.alloc);
+            for (auto &kv : st.cache) expect(hmr_free(index, kv.second));
+            st.cache.clear();
+        }
+        s = hmr_malloc(index, block, &p);
+    }
+    expect(s);
+    return p;
+}
+
+void device_release(int index, size_t block, void *p) {
+    DeviceState &st = device_state(index);
+    std::lock_guard<std::mutex> lock(st.alloc);
+    st.cache.emplace(block, p);
+}
+
+const hcb_backend *g_cpu = nullptr;
+
+const hcb_backend &cpu_backend(const char *kernel) {
+    if (!g_cpu) {
+        throw Error(std::string(kernel) + ": no CPU backend is registered; this library only runs kernels on ROCm "
+                                          "tensors");
+    }
+    return *g_cpu;
+}
+
+void cpu_check(int rc) {
+    if (rc != 0) throw Error(g_cpu->last_error());
+}
+
+hcb_tensor cpu_desc(const TensorData &t) {
+    return hcb_tensor{t.storage->ptr(),          t.layout.offset,       static_cast<int32_t>(t.dtype),
+                      static_cast<int32_t>(t.layout.shape.size()), t.layout.shape.data(), t.layout.strides.data()};
+}
+
+hcb_scalar cpu_scalar(Scalar s) {
+    hcb_scalar c{};
+    c.kind = s.kind == Scalar::K::Bool ? HCB_SCALAR_BOOL : (s.kind == Scalar::K::Int ? HCB_SCALAR_INT : HCB_SCALAR_FLOAT);
+    c.i = s.i;
+    c.f = s.f;
+    return c;
+}
+
+void check_shape(const TensorData &out, const TensorData &in) {
+    if (out.layout.shape != in.layout.shape) throw Error("kernel operands must have the same shape");
+}
+
+// ---- descriptions (ref: src/backend/rocm/copy.rs:59-119) ----------------------------------------------
+
+constexpr size_t kMaxDims = HMR_MAX_DIMS;
+
+hmr_tensor_desc desc_with_dims(const char *kernel, const TensorData &t, int64_t offset,
+                               const std::vector<MergedDim> &dims, size_t operand) {
+    if (dims.size() > kMaxDims) {
+        throw Error(std::string(kernel) + " on ROCm supports at most " + std::to_string(kMaxDims) +
+                    " dimensions that can't be merged, got " + std::to_string(dims.size()));
+    }
+    hmr_tensor_desc d;
+    std::memset(&d, 0, sizeof d);
+    d.data = t.storage->ptr();
+    d.offset = offset;
+    d.dtype = static_cast<int32_t>(t.dtype);
+    d.ndim = static_cast<int32_t>(dims.size());
+    for (size_t j = 0; j < dims.size(); ++j) {
+        d.sizes[j] = dims[j].size;
+        d.strides[j] = dims[j].strides[operand];
+    }
+    return d;
+}
+
+// The descriptions of operands of one shape, merged together; false when they have no elements.
+bool descs(const char *kernel, const std::vector<const TensorData *> &ops, std::vector<hmr_tensor_desc> &out) {
+    std::vector<const Strides *> strides;
+    for (const TensorData *t : ops) strides.push_back(&t->layout.strides);
+    auto dims = merge_dims(ops[0]->layout.shape, strides);
+    if (!dims) return false;
+    out.clear();
+    for (size_t k = 0; k < ops.size(); ++k) out.push_back(desc_with_dims(kernel, *ops[k], ops[k]->layout.offset, *dims, k));
+    return true;
+}
+
+Strides walk_strides(const Layout &l) {
+    return l.num_elements() == 0 ? Strides(l.strides.size(), 0) : l.strides;
+}
+
+// ref: src/backend/rocm/reduce.rs:32-103
+struct Reduction {
+    std::vector<MergedDim> dims;  // merged kept dims: strides[0] of the outputs, [1] of the source
+    hmr_tensor_desc kept, red;
+};
+
+bool describe(const char *kernel, const TensorData &src, const std::vector<bool> &mask, Reduction &r) {
+    const Layout &l = src.layout;
+    Strides strides = walk_strides(l);
+    Shape kept_shape, red_shape;
+    Strides kept_strides, red_strides;
+    for (size_t i = 0; i < l.shape.size(); ++i) {
+        if (mask[i]) {
+            red_shape.push_back(l.shape[i]);
+            red_strides.push_back(strides[i]);
+        } else {
+            kept_shape.push_back(l.shape[i]);
+            kept_strides.push_back(strides[i]);
+        }
+    }
+    Strides out_strides = contiguous_strides(kept_shape);
+    auto dims = merge_dims(kept_shape, {&out_strides, &kept_strides});
+    if (!dims) return false;
+    r.dims = *dims;
+    std::vector<MergedDim> red_dims;
+    if (auto rd = merge_dims(red_shape, {&red_strides})) red_dims = *rd;
+    else red_dims = {MergedDim{0, {0}}};  // nothing to fold
+    std::vector<MergedDim> src_dims;
+    for (const MergedDim &d : r.dims) src_dims.push_back(MergedDim{d.size, {d.strides[1]}});
+    r.kept = desc_with_dims(kernel, src, l.offset, src_dims, 0);
+    r.red = desc_with_dims(kernel, src, 0, red_dims, 0);
+    return true;
+}
+
+hmr_tensor_desc output_desc(const char *kernel, const Reduction &r, const TensorData &out) {
+    if (!out.layout.is_contiguous()) throw Error(std::string("internal error: ") + kernel + " into a strided tensor");
+    std::vector<MergedDim> dims;
+    for (const MergedDim &d : r.dims) dims.push_back(MergedDim{d.size, {d.strides[0]}});
+    return desc_with_dims(kernel, out, out.layout.offset, dims, 0);
+}
+
+// A workspace of `bytes` bytes on `device`, allocated before the execution lock is taken.
+std::shared_ptr<Storage> workspace(int64_t bytes, Device device) {
+    if (bytes <= 0) return nullptr;
+    return std::make_shared<Storage>(device, static_cast<size_t>(bytes));
+}
+
+// ref: src/backend/rocm/reduce.rs:222-263
+bool lines(const char *kernel, const TensorData &out, const TensorData &src, size_t dim, hmr_tensor_desc &o,
+           hmr_tensor_desc &s, int64_t &n, int64_t &so, int64_t &si) {
+    const Layout &ls = src.layout, &lo = out.layout;
+    check_shape(out, src);
+    if (ls.num_elements() == 0) return false;
+    Shape other_shape;
+    Strides other_out, other_src;
+    for (size_t d = 0; d < ls.shape.size(); ++d) {
+        if (d == dim) continue;
+        other_shape.push_back(ls.shape[d]);
+        other_out.push_back(lo.strides[d]);
+        other_src.push_back(ls.strides[d]);
+    }
+    if (ls.shape.empty()) {
+        n = 1;
+        so = si = 0;
+    } else {
+        n = ls.shape[dim];
+        so = lo.strides[dim];
+        si = ls.strides[dim];
+    }
+    auto dims = merge_dims(other_shape, {&other_out, &other_src});
+    if (!dims) return false;
+    o = desc_with_dims(kernel, out, lo.offset, *dims, 0);
+    s = desc_with_dims(kernel, src, ls.offset, *dims, 1);
+    return true;
+}
+
+}  // namespace
+
+// ---- Storage ---------------------------------------------------------------------------------------------
+
+Storage::Storage(Device device, size_t nbytes) : device_(device), nbytes_(nbytes) {
+    if (device.kind == Device::K::Cpu) {
+        block_ = (nbytes + 63) / 64 * 64 + 64;
+        ptr_ = std::aligned_alloc(64, block_);
+        if (!ptr_) throw Error("host allocation failed");
+    } else {
+        block_ = round_block(nbytes == 0 ? 1 : nbytes);
+        ptr_ = device_alloc(device.index, block_);
+    }
+}
+
+Storage::~Storage() {
+    if (!ptr_) return;
+    if (device_.kind == Device::K::Cpu) std::free(ptr_);
+    else device_release(device_.index, block_, ptr_);
+}
+
+void register_cpu_backend(const hcb_backend *table) { g_cpu = table; }
+
+void empty_cache() {
+    std::lock_guard<std::mutex> lock(g_registry);
+    for (auto &kv : g_devices) {
+        DeviceState &st = *kv.second;
+        std::lock_guard<std::recursive_mutex> run(st.exec);
+        expect(hmr_context_synchronize(st.ctx));
+        std::lock_guard<std::mutex> a(st.alloc);
+        for (auto &b : st.cache) expect(hmr_free(kv.first, b.second));
+        st.cache.clear();
+    }
+}
+
+void synchronize(Device device) {
+    if (device.kind != Device::K::Rocm) return;
+    DeviceState &st = device_state(device.index);
+    std::lock_guard<std::recursive_mutex> run(st.exec);
+    expect(hmr_context_synchronize(st.ctx));
+}
+
+void *stream_handle(Device device) {
+    if (device.kind != Device::K::Rocm) throw Error("stream_handle: not a ROCm device");
+    void *s = nullptr;
+    expect(hmr_ext_stream(device_state(device.index).ctx, &s));
+    return s;
+}
+
+// ---- dispatch ------------------------------------------------------------------------------------------------
+
+namespace backend {
+
+namespace {
+bool on_cpu(const TensorData &t) { return t.device().kind == Device::K::Cpu; }
+}  // namespace
+
+void copy(const TensorData &dst, const TensorData &src_in) {
+    if (dst.device() != src_in.device()) throw Error("internal error: copy between devices");
+    TensorData src = src_in.expand_to(dst.layout.shape);
+    if (on_cpu(dst)) {
+        hcb_tensor d = cpu_desc(dst), s = cpu_desc(src);
+        cpu_check(cpu_backend("copy").copy(&d, &s));
+        return;
+    }
+    std::vector<hmr_tensor_desc> ds;
+    if (!descs("copy", {&dst, &src}, ds)) return;
+    auto flat = [](const hmr_tensor_desc &x) { return x.ndim == 0 || (x.ndim == 1 && x.strides[0] == 1); };
+    exec(dst, [&](hmr_context_t ctx) {
+        if (dst.dtype == src.dtype && flat(ds[0]) && flat(ds[1])) {
+            size_t size = size_in_bytes(dst.dtype);
+            expect(hmr_copy_device(ctx, static_cast<char *>(ds[0].data) + ds[0].offset * size,
+                                   static_cast<const char *>(ds[1].data) + ds[1].offset * size,
+                                   static_cast<uint64_t>(dst.layout.num_elements()) * size));
+        } else {
+            expect(hmr_copy(ctx, &ds[0], &ds[1]));
+        }
+    });
+}
+
+void fill(const TensorData &dst, Scalar value) {
+    if (on_cpu(dst)) {
+        hcb_tensor d = cpu_desc(dst);
+        cpu_check(cpu_backend("fill").fill(&d, cpu_scalar(value)));
+        return;
+    }
+    std::vector<hmr_tensor_desc> ds;
+    if (!descs("fill", {&dst}, ds)) return;
+    uint64_t bits = scalar_bits(value, dst.dtype);
+    exec(dst, [&](hmr_context_t ctx) { expect(hmr_fill(ctx, &ds[0], bits)); });
+}
+
+void unary(UnaryOp op, const TensorData &out, const TensorData &src) {
+    check_shape(out, src);
+    if (on_cpu(out)) {
+        hcb_tensor o = cpu_desc(out), s = cpu_desc(src);
+        cpu_check(cpu_backend("unary").unary(static_cast<int32_t>(op), &o, &s));
+        return;
+    }
+    std::vector<hmr_tensor_desc> ds;
+    if (!descs("unary", {&out, &src}, ds)) return;
+    exec(out, [&](hmr_context_t ctx) { expect(hmr_unary(ctx, static_cast<int32_t>(op), &ds[0], &ds[1])); });
+}
+
+void binary(BinaryOp op, const TensorData &out, const TensorData &a, const TensorData &b) {
+    check_shape(out, a);
+    check_shape(out, b);
+    if (on_cpu(out)) {
+        hcb_tensor o = cpu_desc(out), x = cpu_desc(a), y = cpu_desc(b);
+        cpu_check(cpu_backend("binary").binary(static_cast<int32_t>(op), &o, &x, &y));
+        return;
+    }
+    std::vector<hmr_tensor_desc> ds;
+    if (!descs("binary", {&out, &a, &b}, ds)) return;
+    exec(out, [&](hmr_context_t ctx) { expect(hmr_binary(ctx, static_cast<int32_t>(op), &ds[0], &ds[1], &ds[2])); });
+}
+
+void binary_constant(BinaryOp op, const TensorData &out, const TensorData &a, Scalar value, bool constant_first) {
+    check_shape(out, a);
+    if (on_cpu(out)) {
+        hcb_tensor o = cpu_desc(out), x = cpu_desc(a);
+        cpu_check(cpu_backend("binary_constant")
+                      .binary_constant(static_cast<int32_t>(op), &o, &x, cpu_scalar(value), constant_first));
+        return;
+    }
+    uint64_t bits = scalar_bits(value, a.dtype);
+    std::vector<hmr_tensor_desc> ds;
+    if (!descs("binary_constant", {&out, &a}, ds)) return;
+    exec(out, [&](hmr_context_t ctx) {
+        expect(hmr_binary_constant(ctx, static_cast<int32_t>(op), &ds[0], &ds[1], bits, constant_first));
+    });
+}
+
+void binary_scalar(BinaryOp op, const TensorData &out, const TensorData &a, double s, bool scalar_first) {
+    check_shape(out, a);
+    if (on_cpu(out)) {
+        hcb_tensor o = cpu_desc(out), x = cpu_desc(a);
+        cpu_check(cpu_backend("binary_scalar").binary_scalar(static_cast<int32_t>(op), &o, &x, s, scalar_first));
+        return;
+    }
+    std::vector<hmr_tensor_desc> ds;
+    if (!descs("binary_scalar", {&out, &a}, ds)) return;
+    exec(out, [&](hmr_context_t ctx) {
+        expect(hmr_binary_scalar(ctx, static_cast<int32_t>(op), &ds[0], &ds[1], s, scalar_first));
+    });
+}
+
+void where_(const TensorData &out, const TensorData &cond, const TensorData &x, const TensorData &y) {
+    check_shape(out, cond);
+    check_shape(out, x);
+    check_shape(out, y);
+    if (on_cpu(out)) {
+        hcb_tensor o = cpu_desc(out), c = cpu_desc(cond), a = cpu_desc(x), b = cpu_desc(y);
+        cpu_check(cpu_backend("where_").where_(&o, &c, &a, &b));
+        return;
+    }
+    std::vector<hmr_tensor_desc> ds;
+    if (!descs("where_", {&out, &cond, &x, &y}, ds)) return;
+    exec(out, [&](hmr_context_t ctx) { expect(hmr_where(ctx, &ds[0], &ds[1], &ds[2], &ds[3])); });
+}
+
+void where_constant(const TensorData &out, const TensorData &cond, Branch x, Branch y) {
+    check_shape(out, cond);
+    if (x.tensor && y.tensor) return where_(out, cond, *x.tensor, *y.tensor);
+    if (on_cpu(out)) {
+        hcb_tensor o = cpu_desc(out), c = cpu_desc(cond), a{}, b{};
+        if (x.tensor) a = cpu_desc(*x.tensor);
+        if (y.tensor) b = cpu_desc(*y.tensor);
+        cpu_check(cpu_backend("where_constant")
+                      .where_constant(&o, &c, x.tensor ? &a : nullptr, cpu_scalar(x.constant), y.tensor ? &b : nullptr,
+                                      cpu_scalar(y.constant)));
+        return;
+    }
+    uint64_t xb = x.tensor ? 0 : scalar_bits(x.constant, out.dtype);
+    uint64_t yb = y.tensor ? 0 : scalar_bits(y.constant, out.dtype);
+    std::vector<const TensorData *> ops = {&out, &cond};
+    if (x.tensor) {
+        check_shape(out, *x.tensor);
+        ops.push_back(x.tensor);
+    }
+    if (y.tensor) {
+        check_shape(out, *y.tensor);
+        ops.push_back(y.tensor);
+    }
+    std::vector<hmr_tensor_desc> ds;
+    if (!descs("where_constant", ops, ds)) return;
+    const hmr_tensor_desc *xd = x.tensor ? &ds[2] : nullptr;
+    const hmr_tensor_desc *yd = y.tensor ? &ds[2] : nullptr;
+    exec(out, [&](hmr_context_t ctx) { expect(hmr_where_constant(ctx, &ds[0], &ds[1], xd, xb, yd, yb)); });
+}
+
+void reduce(ReduceOp op, const TensorData &out, const TensorData &src, const std::vector<bool> &mask) {
+    if (on_cpu(out)) {
+        hcb_tensor o = cpu_desc(out), s = cpu_desc(src);
+        std::vector<uint8_t> m(mask.begin(), mask.end());
+        cpu_check(cpu_backend("reduce").reduce(static_cast<int32_t>(op), &o, &s, m.data()));
+        return;
+    }
+    Reduction r;
+    if (!describe("reduce", src, mask, r)) return;
+    hmr_tensor_desc o = output_desc("reduce", r, out);
+    int64_t bytes = 0;
+    expect(hmr_reduce_workspace(&r.kept, &r.red, 0, &bytes));
+    auto ws = workspace(bytes, src.device());
+    exec(out, [&](hmr_context_t ctx) {
+        expect(hmr_reduce(ctx, static_cast<int32_t>(op), &o, &r.kept, &r.red, ws ? ws->ptr() : nullptr, bytes));
+    });
+}
+
+void var(const TensorData &out, const TensorData &src, const std::vector<bool> &mask, double correction,
+         bool take_sqrt) {
+    if (on_cpu(out)) {
+        hcb_tensor o = cpu_desc(out), s = cpu_desc(src);
+        std::vector<uint8_t> m(mask.begin(), mask.end());
+        cpu_check(cpu_backend("var").var(&o, &s, m.data(), correction, take_sqrt));
+        return;
+    }
+    Reduction r;
+    if (!describe("var", src, mask, r)) return;
+    hmr_tensor_desc o = output_desc("var", r, out);
+    int64_t bytes = 0;
+    expect(hmr_reduce_workspace(&r.kept, &r.red, 1, &bytes));
+    auto ws = workspace(bytes, src.device());
+    exec(out, [&](hmr_context_t ctx) {
+        expect(hmr_var(ctx, &o, &r.kept, &r.red, correction, take_sqrt, ws ? ws->ptr() : nullptr, bytes));
+    });
+}
+
+void arg_reduce(const TensorData *values, const TensorData &indices, const TensorData &src, size_t dim,
+                bool is_max) {
+    if (on_cpu(indices)) {
+        hcb_tensor v{}, i = cpu_desc(indices), s = cpu_desc(src);
+        if (values) v = cpu_desc(*values);
+        cpu_check(cpu_backend("arg_reduce").arg_reduce(values ? &v : nullptr, &i, &s, static_cast<int32_t>(dim), is_max));
+        return;
+    }
+    size_t nd = src.layout.shape.size();
+    std::vector<bool> mask(nd, false);
+    if (nd > 0) {
+        mask[dim] = true;
+        if (src.layout.shape[dim] <= 0) throw Error("cannot compute the arg reduction of an empty dimension");
+    }
+    Reduction r;
+    if (!describe("arg_reduce", src, mask, r)) return;
+    hmr_tensor_desc i = output_desc("arg_reduce", r, indices);
+    hmr_tensor_desc v{};
+    if (values) v = output_desc("arg_reduce", r, *values);
+    int64_t bytes = 0;
+    expect(hmr_reduce_workspace(&r.kept, &r.red, 0, &bytes));
+    auto ws = workspace(bytes, src.device());
+    exec(indices, [&](hmr_context_t ctx) {
+        expect(hmr_arg_reduce(ctx, values ? &v : nullptr, &i, &r.kept, &r.red, is_max, ws ? ws->ptr() : nullptr, bytes));
+    });
+}
+
+void softmax(const TensorData &out, const TensorData &src, size_t dim, bool log) {
+    if (on_cpu(out)) {
+        hcb_tensor o = cpu_desc(out), s = cpu_desc(src);
+        cpu_check(cpu_backend("softmax").softmax(&o, &s, static_cast<int32_t>(dim), log));
+        return;
+    }
+    hmr_tensor_desc o, s;
+    int64_t n = 0, so = 0, si = 0;
+    if (!lines("softmax", out, src, dim, o, s, n, so, si)) return;
+    int64_t bytes = 0;
+    expect(hmr_softmax_workspace(&s, n, si, &bytes));
+    auto ws = workspace(bytes, src.device());
+    exec(out, [&](hmr_context_t ctx) {
+        expect(hmr_softmax(ctx, &o, &s, n, so, si, log, ws ? ws->ptr() : nullptr, bytes));
+    });
+}
+
+void upload(const TensorData &dst, const TensorData &src) {
+    if (!src.layout.is_contiguous() || !dst.layout.is_contiguous() || !on_cpu(src) || on_cpu(dst)) {
+        throw Error("internal error: upload needs a contiguous CPU source and a contiguous ROCm destination");
+    }
+    size_t size = size_in_bytes(dst.dtype);
+    size_t nbytes = static_cast<size_t>(src.layout.num_elements()) * size;
+    if (nbytes == 0) return;
+    exec(dst, [&](hmr_context_t ctx) {
+        expect(hmr_copy_from_host(ctx, static_cast<char *>(dst.storage->ptr()) + dst.layout.offset * size,
+                                  static_cast<const char *>(src.storage->ptr()) + src.layout.offset * size, nbytes));
+    });
+}
+
+void download(const TensorData &dst, const TensorData &src) {
+    if (!src.layout.is_contiguous() || !dst.layout.is_contiguous() || on_cpu(src) || !on_cpu(dst)) {
+        throw Error("internal error: download needs a contiguous ROCm source and a contiguous CPU destination");
+    }
+    size_t size = size_in_bytes(dst.dtype);
+    size_t nbytes = static_cast<size_t>(src.layout.num_elements()) * size;
+    if (nbytes == 0) return;
+    exec(src, [&](hmr_context_t ctx) {
+        expect(hmr_copy_to_host(ctx, static_cast<char *>(dst.storage->ptr()) + dst.layout.offset * size,
+                                static_cast<const char *>(src.storage->ptr()) + src.layout.offset * size, nbytes));
+    });
+}
+
+}  // namespace backend
+
+// ---- plan hooks ------------------------------------------------------------------------------------------------
+
+ReducePlanInfo rocm_reduce_plan(const Tensor &src, const std::vector<int64_t> &dims) {
+    std::vector<bool> mask = dims_mask(dims, src.num_dims());
+    Reduction r;
+    if (!describe("test", src.data(), mask, r)) throw Error("reduction without outputs");
+    ReducePlanInfo p{};
+    expect(hmr_test_reduce_plan(&r.kept, &r.red, &p.group, &p.splits, &p.chunk));
+    return p;
+}
+
+SoftmaxPlanInfo rocm_softmax_plan(const Tensor &src, int64_t dim) {
+    size_t d = normalize_dim(dim, src.num_dims());
+    hmr_tensor_desc o, s;
+    int64_t n = 0, so = 0, si = 0;
+    if (!lines("test", src.data(), src.data(), d, o, s, n, so, si)) throw Error("softmax without elements");
+    int32_t split = 0, group = 0, cache = 0;
+    expect(hmr_test_softmax_plan(&s, n, si, &split, &group, &cache));
+    return SoftmaxPlanInfo{split != 0, group, cache};
+}
+
+}  // namespace homura

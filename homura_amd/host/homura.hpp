@@ -1,0 +1,346 @@
+// homura.hpp -- the host side of homura's tensor elementwise / broadcast / reduction path, in
+// C++ (the reference's host side is Rust; no Rust toolchain exists where this is built).
+//
+// It mirrors, name for name, the part of the reference that sits between user code and the C ABI:
+//   dtype rules      promote_types, ResultType, can_cast, Scalar      ref: src/dtype.rs:279-535
+//   shape algebra    broadcast_shapes, contiguous_strides, dims_mask,
+//                    compute_view_strides, infer_size                 ref: src/shape.rs:520-742
+//   Layout / views   expand_to, permute, transpose, narrow, select... ref: src/tensor/mod.rs:83-170,
+//                                                                          src/tensor/view.rs
+//   ops front end    binary_op, where_/select, unary_op, reduce_op,
+//                    arg_op, var_op, softmax_op, cast_data            ref: src/ops/{binary,unary,reduce,composite,mod}.rs
+//   dispatch         backend::<kernel> by device                      ref: src/backend/mod.rs:298-534
+//   ROCm host        merge_dims, descs, workspaces, exec lock, status
+//                    -> error                                         ref: src/backend/rocm/{copy,elementwise,reduce,context,mod}.rs
+// Where the reference panics, this code throws homura::Error with the reference's message.
+// Autograd, in-place ops and the Meta device are outside this path and absent.
+#pragma once
+
+#include <cstdint>
+#include <memory>
+#include <optional>
+#include <stdexcept>
+#include <string>
+#include <variant>
+#include <vector>
+
+#include "cpu_backend.h"
+
+namespace homura {
+
+struct Error : std::runtime_error {
+    using std::runtime_error::runtime_error;
+};
+
+// ---- dtype ------------------------------------------------------------------------------------------
+
+enum class DType : int32_t { Bool = 0, U8, I8, I16, I32, I64, F16, BF16, F32, F64 };
+enum class Kind { Bool, Int, Float };
+
+Kind kind_of(DType d);
+inline bool is_floating_point(DType d) { return kind_of(d) == Kind::Float; }
+inline bool is_integral(DType d) { return kind_of(d) == Kind::Int; }
+size_t size_in_bytes(DType d);
+const char *name_of(DType d);
+
+DType default_dtype();
+void set_default_dtype(DType d);  // floating point dtypes only
+
+struct Scalar {
+    enum class K { Bool, Int, Float } kind;
+    int64_t i = 0;
+    double f = 0.0;
+    static Scalar of_bool(bool v) { return Scalar{K::Bool, v ? 1 : 0, 0.0}; }
+    static Scalar of_int(int64_t v) { return Scalar{K::Int, v, 0.0}; }
+    static Scalar of_float(double v) { return Scalar{K::Float, 0, v}; }
+    double to_f64() const;
+    int64_t to_i64() const;
+    bool to_bool() const;
+    DType dtype() const;  // default float dtype / I64 / Bool
+    // The value as a scalar of `dtype` if it fits (fill_, masked_fill): ref src/dtype.rs:334-374.
+    std::optional<Scalar> checked_to(DType dtype) const;
+    std::string str() const;
+};
+
+DType promote_types(DType a, DType b);
+bool can_cast(DType from, DType to);
+
+class ResultType {
+  public:
+    ResultType &tensor(DType dtype, size_t num_dims);
+    ResultType &scalar(Scalar s);
+    DType result() const;
+
+  private:
+    std::optional<DType> dim_, zero_dim_, scalar_;
+};
+
+// `value` converted to `dtype` as the CPU's fill converts it, little-endian in the low bytes
+// (ref: src/backend/rocm/copy.rs:253-270).
+uint64_t scalar_bits(Scalar value, DType dtype);
+
+// ---- shapes -------------------------------------------------------------------------------------------
+
+using Shape = std::vector<int64_t>;
+using Strides = std::vector<int64_t>;
+
+std::string shape_str(const Shape &s);
+size_t normalize_dim(int64_t dim, size_t num_dims);
+std::vector<bool> dims_mask(const std::vector<int64_t> &dims, size_t num_dims);
+Strides contiguous_strides(const Shape &shape);
+bool is_contiguous(const Shape &shape, const Strides &strides);
+bool is_expandable_to(const Shape &shape, const Shape &desired);
+Shape broadcast_shapes(const Shape &a, const Shape &b);
+Shape infer_size(const std::vector<int64_t> &spec, int64_t num_elements);
+std::optional<Strides> compute_view_strides(const Shape &old_shape, const Strides &old_strides, const Shape &new_shape);
+
+// One merged dimension: its size and its stride in each operand (ref: src/backend/rocm/copy.rs:28-57).
+struct MergedDim {
+    int64_t size;
+    std::vector<int64_t> strides;
+};
+// nullopt for an empty shape.
+std::optional<std::vector<MergedDim>> merge_dims(const Shape &shape, const std::vector<const Strides *> &strides);
+
+// ---- devices, storage, layout -----------------------------------------------------------------------
+
+struct Device {
+    enum class K { Cpu, Rocm } kind = K::Cpu;
+    int index = 0;
+    static Device cpu() { return Device{K::Cpu, 0}; }
+    static Device rocm(int i) { return Device{K::Rocm, i}; }
+    bool operator==(const Device &o) const { return kind == o.kind && index == o.index; }
+    bool operator!=(const Device &o) const { return !(*this == o); }
+    std::string str() const;
+};
+
+class Storage {
+  public:
+    Storage(Device device, size_t nbytes);  // uninitialised; throws Error / OutOfMemory
+    ~Storage();
+    Storage(const Storage &) = delete;
+    Storage &operator=(const Storage &) = delete;
+    Device device() const { return device_; }
+    void *ptr() const { return ptr_; }
+    size_t nbytes() const { return nbytes_; }
+
+  private:
+    Device device_;
+    void *ptr_ = nullptr;
+    size_t nbytes_ = 0;
+    size_t block_ = 0;
+};
+
+struct Layout {
+    Shape shape;
+    Strides strides;
+    int64_t offset = 0;
+    static Layout contiguous(Shape shape);
+    int64_t num_elements() const;
+    bool is_contiguous() const { return homura::is_contiguous(shape, strides); }
+    Layout expand_to(const Shape &target) const;  // ref: src/tensor/mod.rs:139-170
+    Layout select(size_t dim, int64_t index) const;
+};
+
+struct TensorData {
+    std::shared_ptr<Storage> storage;
+    Layout layout;
+    DType dtype = DType::F32;
+    Device device() const { return storage->device(); }
+    TensorData expand_to(const Shape &shape) const;
+};
+
+// Registers the kernels that run on Device::Cpu tensors (see cpu_backend.h). nullptr unregisters.
+void register_cpu_backend(const hcb_backend *table);
+// Returns device memory cached by the allocator to the driver.
+void empty_cache();
+// Waits for everything queued on the device's stream.
+void synchronize(Device device);
+// Whether a half tensor combined with an F32 tensor is widened inside the binary kernel (default)
+// or, as the reference does, by a separate cast kernel first. Both give the same bits.
+void set_fused_promotion(bool on);
+// The hipStream_t of the device's context (for harnesses that record their own events).
+void *stream_handle(Device device);
+
+// ---- Tensor ---------------------------------------------------------------------------------------------
+
+class Tensor;
+using Operand = std::variant<Tensor, Scalar>;
+
+enum class UnaryOp : int32_t {
+    Neg = 0, Abs, Sign, Relu, Exp, Log, Sqrt, Rsqrt, Reciprocal, Sin, Cos, Erf, Tanh, Sigmoid, LogSigmoid,
+    Silu, Gelu, GeluTanh, LogicalNot
+};
+enum class BinaryOp : int32_t {
+    Add = 0, Sub, Mul, Div, Pow, Maximum, Minimum, Greater, GreaterEqual, Less, LessEqual, Equal, NotEqual,
+    LogicalAnd, LogicalOr, BitwiseAnd
+};
+enum class ReduceOp : int32_t { Sum = 0, Prod, Mean, Max, Min, All, Any };
+enum class GeluApproximate { None, Tanh };
+
+struct ValuesAndIndices;
+
+class Tensor {
+  public:
+    Tensor() = default;
+    explicit Tensor(TensorData d) : d_(std::move(d)) {}
+
+    // Creation. `bytes` holds num_elements * size_in_bytes(dtype) bytes in row-major order.
+    static Tensor from_bytes(const void *bytes, DType dtype, const Shape &shape, Device device = Device::cpu());
+    static Tensor uninit_on(const Shape &shape, DType dtype, Device device);
+    static Tensor full(const Shape &shape, Scalar value, DType dtype, Device device);
+
+    const TensorData &data() const { return d_; }
+    const Shape &shape() const { return d_.layout.shape; }
+    const Strides &stride() const { return d_.layout.strides; }
+    int64_t storage_offset() const { return d_.layout.offset; }
+    DType dtype() const { return d_.dtype; }
+    Device device() const { return d_.device(); }
+    size_t num_dims() const { return d_.layout.shape.size(); }
+    int64_t num_elements() const { return d_.layout.num_elements(); }
+    bool is_contiguous() const { return d_.layout.is_contiguous(); }
+
+    // The elements in row-major order (moves to the host; waits for the device).
+    std::vector<uint8_t> to_bytes() const;
+
+    Tensor to(DType dtype) const;
+    Tensor to(Device device) const;
+    Tensor contiguous() const;
+
+    // Views (ref: src/tensor/view.rs).
+    Tensor reshape(const std::vector<int64_t> &spec) const;
+    Tensor permute(const std::vector<int64_t> &dims) const;
+    Tensor transpose(int64_t dim0, int64_t dim1) const;
+    Tensor expand(const std::vector<int64_t> &spec) const;
+    Tensor unsqueeze(int64_t dim) const;
+    Tensor narrow(int64_t dim, int64_t start, int64_t length) const;
+    Tensor select(int64_t dim, int64_t index) const;
+    Tensor flatten(int64_t start_dim, int64_t end_dim) const;
+
+    // Unary (ref: src/ops/unary.rs).
+    Tensor unary(UnaryOp op) const;
+    Tensor neg() const { return unary(UnaryOp::Neg); }
+    Tensor abs() const { return unary(UnaryOp::Abs); }
+    Tensor sign() const { return unary(UnaryOp::Sign); }
+    Tensor relu() const { return unary(UnaryOp::Relu); }
+    Tensor exp() const { return unary(UnaryOp::Exp); }
+    Tensor log() const { return unary(UnaryOp::Log); }
+    Tensor sqrt() const { return unary(UnaryOp::Sqrt); }
+    Tensor rsqrt() const { return unary(UnaryOp::Rsqrt); }
+    Tensor reciprocal() const { return unary(UnaryOp::Reciprocal); }
+    Tensor sin() const { return unary(UnaryOp::Sin); }
+    Tensor cos() const { return unary(UnaryOp::Cos); }
+    Tensor erf() const { return unary(UnaryOp::Erf); }
+    Tensor tanh() const { return unary(UnaryOp::Tanh); }
+    Tensor sigmoid() const { return unary(UnaryOp::Sigmoid); }
+    Tensor log_sigmoid() const { return unary(UnaryOp::LogSigmoid); }
+    Tensor silu() const { return unary(UnaryOp::Silu); }
+    Tensor gelu(GeluApproximate a = GeluApproximate::None) const {
+        return unary(a == GeluApproximate::None ? UnaryOp::Gelu : UnaryOp::GeluTanh);
+    }
+    Tensor logical_not() const { return unary(UnaryOp::LogicalNot); }
+
+    // Binary with broadcasting and type promotion (ref: src/ops/binary.rs).
+    Tensor binary(BinaryOp op, const Operand &other) const;
+    Tensor add(const Operand &o) const { return binary(BinaryOp::Add, o); }
+    Tensor sub(const Operand &o) const { return binary(BinaryOp::Sub, o); }
+    Tensor mul(const Operand &o) const { return binary(BinaryOp::Mul, o); }
+    Tensor div(const Operand &o) const { return binary(BinaryOp::Div, o); }
+    Tensor pow(const Operand &o) const { return binary(BinaryOp::Pow, o); }
+    Tensor maximum(const Operand &o) const { return binary(BinaryOp::Maximum, o); }
+    Tensor minimum(const Operand &o) const { return binary(BinaryOp::Minimum, o); }
+    Tensor greater(const Operand &o) const { return binary(BinaryOp::Greater, o); }
+    Tensor greater_equal(const Operand &o) const { return binary(BinaryOp::GreaterEqual, o); }
+    Tensor less(const Operand &o) const { return binary(BinaryOp::Less, o); }
+    Tensor less_equal(const Operand &o) const { return binary(BinaryOp::LessEqual, o); }
+    Tensor equal(const Operand &o) const { return binary(BinaryOp::Equal, o); }
+    Tensor not_equal(const Operand &o) const { return binary(BinaryOp::NotEqual, o); }
+    Tensor logical_and(const Operand &o) const { return binary(BinaryOp::LogicalAnd, o); }
+    Tensor logical_or(const Operand &o) const { return binary(BinaryOp::LogicalOr, o); }
+    Tensor bitwise_and(const Operand &o) const { return binary(BinaryOp::BitwiseAnd, o); }  // extension
+    Tensor clamp(const Operand &min, const Operand &max) const { return maximum(min).minimum(max); }
+    Tensor clamp_min(const Operand &min) const { return maximum(min); }
+    Tensor clamp_max(const Operand &max) const { return minimum(max); }
+    Tensor masked_fill(const Tensor &mask, const Operand &value) const;
+
+    // Reductions (ref: src/ops/reduce.rs).
+    Tensor sum() const;
+    Tensor sum_dim(const std::vector<int64_t> &dims, bool keepdim) const;
+    Tensor sum_to_size(const Shape &size) const;
+    Tensor mean() const;
+    Tensor mean_dim(const std::vector<int64_t> &dims, bool keepdim) const;
+    Tensor prod() const;
+    Tensor prod_dim(int64_t dim, bool keepdim) const;
+    Tensor max() const;
+    Tensor min() const;
+    ValuesAndIndices max_dim(int64_t dim, bool keepdim) const;
+    ValuesAndIndices min_dim(int64_t dim, bool keepdim) const;
+    Tensor argmax() const;
+    Tensor argmin() const;
+    Tensor argmax_dim(int64_t dim, bool keepdim) const;
+    Tensor argmin_dim(int64_t dim, bool keepdim) const;
+    Tensor var(int64_t correction) const;
+    Tensor var_dim(const std::vector<int64_t> &dims, int64_t correction, bool keepdim) const;
+    Tensor std(int64_t correction) const;
+    Tensor std_dim(const std::vector<int64_t> &dims, int64_t correction, bool keepdim) const;
+    Tensor all() const;
+    Tensor any() const;
+    Tensor all_dim(const std::vector<int64_t> &dims, bool keepdim) const;
+    Tensor any_dim(const std::vector<int64_t> &dims, bool keepdim) const;
+
+    // ref: src/ops/composite.rs:10-27
+    Tensor softmax(int64_t dim) const;
+    Tensor log_softmax(int64_t dim) const;
+
+  private:
+    TensorData d_;
+};
+
+struct ValuesAndIndices {
+    Tensor values;
+    Tensor indices;
+};
+
+// op(lhs, rhs); at least one operand is a tensor (ref: src/ops/binary.rs:68-143).
+Tensor binary_op(BinaryOp op, const Operand &lhs, const Operand &rhs);
+// torch.where (ref: src/ops/binary.rs:152-176).
+Tensor where_(const Tensor &condition, const Operand &x, const Operand &y);
+
+// ---- backend dispatch (ref: src/backend/mod.rs:298-534) ---------------------------------------------
+
+namespace backend {
+struct Branch {
+    const TensorData *tensor = nullptr;  // else the constant
+    Scalar constant{};
+};
+void copy(const TensorData &dst, const TensorData &src);
+void fill(const TensorData &dst, Scalar value);
+void unary(UnaryOp op, const TensorData &out, const TensorData &src);
+void binary(BinaryOp op, const TensorData &out, const TensorData &a, const TensorData &b);
+void binary_constant(BinaryOp op, const TensorData &out, const TensorData &a, Scalar value, bool constant_first);
+void binary_scalar(BinaryOp op, const TensorData &out, const TensorData &a, double s, bool scalar_first);
+void where_(const TensorData &out, const TensorData &cond, const TensorData &x, const TensorData &y);
+void where_constant(const TensorData &out, const TensorData &cond, Branch x, Branch y);
+void reduce(ReduceOp op, const TensorData &out, const TensorData &src, const std::vector<bool> &mask);
+void var(const TensorData &out, const TensorData &src, const std::vector<bool> &mask, double correction,
+         bool take_sqrt);
+void arg_reduce(const TensorData *values, const TensorData &indices, const TensorData &src, size_t dim,
+                bool is_max);
+void softmax(const TensorData &out, const TensorData &src, size_t dim, bool log);
+// Host <-> device and device <-> host transfers of contiguous data of one dtype.
+void upload(const TensorData &dst, const TensorData &src);
+void download(const TensorData &dst, const TensorData &src);
+}  // namespace backend
+
+// The plan the library reports for a reduction / softmax of `src` (test hook).
+struct ReducePlanInfo {
+    int64_t group, splits, chunk;
+};
+ReducePlanInfo rocm_reduce_plan(const Tensor &src, const std::vector<int64_t> &dims);
+struct SoftmaxPlanInfo {
+    bool split;
+    int32_t group, cache;
+};
+SoftmaxPlanInfo rocm_softmax_plan(const Tensor &src, int64_t dim);
+
+}  // namespace homura

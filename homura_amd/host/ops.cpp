@@ -1,0 +1,453 @@
+// The ops front end: argument checks, type promotion, broadcasting, output allocation and the
+// call into the backend. See homura.hpp for the map to the reference's files.
+#include <cstring>
+
+#include "homura.hpp"
+
+namespace homura {
+
+namespace {
+
+bool g_fused_promotion = true;
+
+// ---- helpers of src/ops/mod.rs ---------------------------------------------------------------------------
+
+Device common_device(const std::vector<const TensorData *> &tensors) {
+    std::optional<Device> device;
+    for (const TensorData *t : tensors) {
+        if (!device) device = t->device();
+        else if (*device != t->device()) {
+            throw Error("Expected all tensors to be on the same device, but found at least two devices, " +
+                        device->str() + " and " + t->device().str() + "!");
+        }
+    }
+    if (!device) throw Error("expected at least one tensor");
+    return *device;
+}
+
+TensorData uninit_data(const Shape &shape, DType dtype, Device device) {
+    Layout l = Layout::contiguous(shape);
+    size_t nbytes = static_cast<size_t>(l.num_elements()) * size_in_bytes(dtype);
+    return TensorData{std::make_shared<Storage>(device, nbytes), l, dtype};
+}
+
+// `data` converted to `dtype` (a copy only when the dtype differs): ref src/ops/mod.rs:175-195.
+TensorData cast_data(const TensorData &data, DType dtype) {
+    if (data.dtype == dtype) return data;
+    TensorData out = uninit_data(data.layout.shape, dtype, data.device());
+    backend::copy(out, data);
+    return out;
+}
+
+TensorData clone_data(const TensorData &data) {
+    TensorData out = uninit_data(data.layout.shape, data.dtype, data.device());
+    backend::copy(out, data);
+    return out;
+}
+
+TensorData reshape_data(const TensorData &data, const Shape &shape) {
+    const Layout &l = data.layout;
+    if (auto st = compute_view_strides(l.shape, l.strides, shape)) {
+        return TensorData{data.storage, Layout{shape, *st, l.offset}, data.dtype};
+    }
+    TensorData c = clone_data(data);
+    c.layout = Layout::contiguous(shape);
+    return c;
+}
+
+TensorData scalar_data(Scalar value, DType dtype, Device device) {
+    TensorData out = uninit_data({}, dtype, device);
+    backend::fill(out, value);
+    return out;
+}
+
+Scalar fill_value(Scalar value, DType dtype) {
+    if (auto v = value.checked_to(dtype)) return *v;
+    throw Error(std::string("value cannot be converted to type ") + name_of(dtype) + " without overflow");
+}
+
+// ---- Resolved operands (ref: src/ops/binary.rs:12-61) -----------------------------------------------
+
+struct Resolved {
+    std::optional<TensorData> tensor;
+    Scalar scalar{};
+    explicit Resolved(const Operand &o) {
+        if (std::holds_alternative<Tensor>(o)) tensor = std::get<Tensor>(o).data();
+        else scalar = std::get<Scalar>(o);
+    }
+    void add_to(ResultType &rt) const {
+        if (tensor) rt.tensor(tensor->dtype, tensor->layout.shape.size());
+        else rt.scalar(scalar);
+    }
+    bool is_bool() const { return tensor ? tensor->dtype == DType::Bool : scalar.kind == Scalar::K::Bool; }
+    Shape shape() const { return tensor ? tensor->layout.shape : Shape{}; }
+    TensorData materialize(DType dtype, Device device, const Shape &shape) const {
+        if (tensor) return cast_data(*tensor, dtype).expand_to(shape);
+        return scalar_data(scalar, dtype, device).expand_to(shape);
+    }
+};
+
+const char *unary_debug_name(UnaryOp op) {
+    static const char *names[] = {"Neg", "Abs", "Sign", "Relu", "Exp", "Log", "Sqrt", "Rsqrt", "Reciprocal", "Sin",
+                                  "Cos", "Erf", "Tanh", "Sigmoid", "LogSigmoid", "Silu", "Gelu", "GeluTanh",
+                                  "LogicalNot"};
+    return names[static_cast<int>(op)];
+}
+
+bool is_comparison(BinaryOp op) { return op >= BinaryOp::Greater && op <= BinaryOp::NotEqual; }
+
+// [`where_`] with the result's dtype given (ref: src/ops/binary.rs:178-216).
+Tensor select_op(const Tensor &condition, const Operand &x_operand, const Operand &y_operand, DType dtype) {
+    TensorData cond = condition.data();
+    Resolved x(x_operand), y(y_operand);
+    std::vector<const TensorData *> devices = {&cond};
+    if (x.tensor) devices.push_back(&*x.tensor);
+    if (y.tensor) devices.push_back(&*y.tensor);
+    Device device = common_device(devices);
+    Shape shape = broadcast_shapes(broadcast_shapes(cond.layout.shape, x.shape()), y.shape());
+    TensorData out = uninit_data(shape, dtype, device);
+    TensorData c = cond.expand_to(shape);
+    if (x.tensor && y.tensor) {
+        backend::where_(out, c, x.materialize(dtype, device, shape), y.materialize(dtype, device, shape));
+    } else {
+        std::optional<TensorData> xd, yd;
+        if (x.tensor) xd = x.materialize(dtype, device, shape);
+        if (y.tensor) yd = y.materialize(dtype, device, shape);
+        backend::Branch bx{xd ? &*xd : nullptr, x.scalar}, by{yd ? &*yd : nullptr, y.scalar};
+        backend::where_constant(out, c, bx, by);
+    }
+    return Tensor(out);
+}
+
+Shape reduced_shape(const Shape &shape, const std::vector<bool> &mask, bool keepdim) {
+    Shape out;
+    for (size_t d = 0; d < shape.size(); ++d) {
+        if (!mask[d]) out.push_back(shape[d]);
+        else if (keepdim) out.push_back(1);
+    }
+    return out;
+}
+
+// ref: src/ops/reduce.rs:55-90
+Tensor reduce_op(ReduceOp op, const Tensor &x, const std::vector<int64_t> &dims, bool keepdim, const char *name) {
+    const TensorData &src = x.data();
+    DType dtype = src.dtype;
+    std::vector<bool> mask = dims_mask(dims, src.layout.shape.size());
+    DType out_dtype = dtype;
+    if ((op == ReduceOp::Sum || op == ReduceOp::Prod) && !is_floating_point(dtype)) out_dtype = DType::I64;
+    else if (op == ReduceOp::Mean && !is_floating_point(dtype)) {
+        throw Error(std::string(name) + "(): could not infer output dtype. Input dtype must be either a floating "
+                                        "point or complex dtype. Got: " + name_of(dtype));
+    } else if ((op == ReduceOp::All || op == ReduceOp::Any) && dtype != DType::U8) out_dtype = DType::Bool;
+    bool reduces_empty = false;
+    for (size_t d = 0; d < mask.size(); ++d) reduces_empty = reduces_empty || (mask[d] && src.layout.shape[d] == 0);
+    if ((op == ReduceOp::Max || op == ReduceOp::Min) && reduces_empty) {
+        throw Error(std::string(name) + "(): Expected reduction dim to be specified for input.numel() == 0. Specify "
+                                        "the reduction dim with the 'dim' argument.");
+    }
+    TensorData out = uninit_data(reduced_shape(src.layout.shape, mask, keepdim), out_dtype, src.device());
+    backend::reduce(op, out, src, mask);
+    return Tensor(out);
+}
+
+// ref: src/ops/reduce.rs:92-135
+std::pair<std::optional<Tensor>, Tensor> arg_op(const Tensor &x, std::optional<int64_t> dim_in, bool keepdim,
+                                                bool is_max, bool values, const char *name) {
+    TensorData src = x.data();
+    int64_t dim = 0;
+    if (dim_in) {
+        dim = *dim_in;
+    } else {
+        src = reshape_data(src, Shape{src.layout.num_elements()});
+        keepdim = false;
+    }
+    size_t nd = src.layout.shape.size();
+    size_t d = normalize_dim(dim, nd);
+    int64_t size = nd == 0 ? 1 : src.layout.shape[d];
+    if (size == 0) {
+        throw Error(std::string(name) + "(): Expected reduction dim " + std::to_string(d) + " to have non-zero size.");
+    }
+    std::vector<bool> mask(nd, false);
+    if (nd > 0) mask[d] = true;
+    Shape shape = reduced_shape(src.layout.shape, mask, keepdim);
+    std::optional<TensorData> vals;
+    if (values) vals = uninit_data(shape, src.dtype, src.device());
+    TensorData indices = uninit_data(shape, DType::I64, src.device());
+    backend::arg_reduce(vals ? &*vals : nullptr, indices, src, d, is_max);
+    return {vals ? std::optional<Tensor>(Tensor(*vals)) : std::nullopt, Tensor(indices)};
+}
+
+// ref: src/ops/reduce.rs:137-156
+Tensor var_op(const Tensor &x, const std::vector<int64_t> &dims, int64_t correction, bool keepdim, bool take_sqrt) {
+    const TensorData &src = x.data();
+    if (!is_floating_point(src.dtype)) {
+        throw Error(std::string("std and var only support floating point dtypes, got ") + name_of(src.dtype));
+    }
+    std::vector<bool> mask = dims_mask(dims, src.layout.shape.size());
+    TensorData out = uninit_data(reduced_shape(src.layout.shape, mask, keepdim), src.dtype, src.device());
+    backend::var(out, src, mask, static_cast<double>(correction), take_sqrt);
+    return Tensor(out);
+}
+
+// ref: src/ops/composite.rs:10-27
+Tensor softmax_op(const Tensor &x, int64_t dim, bool log) {
+    const TensorData &src = x.data();
+    if (!is_floating_point(src.dtype)) {
+        throw Error(std::string(log ? "log_softmax" : "softmax") + " is not implemented for " + name_of(src.dtype) +
+                    " tensors");
+    }
+    size_t d = normalize_dim(dim, src.layout.shape.size());
+    TensorData out = uninit_data(src.layout.shape, src.dtype, src.device());
+    backend::softmax(out, src, d, log);
+    return Tensor(out);
+}
+
+}  // namespace
+
+void set_fused_promotion(bool on) { g_fused_promotion = on; }
+
+// ---- creation and movement ------------------------------------------------------------------------------
+
+Tensor Tensor::uninit_on(const Shape &shape, DType dtype, Device device) { return Tensor(uninit_data(shape, dtype, device)); }
+
+Tensor Tensor::from_bytes(const void *bytes, DType dtype, const Shape &shape, Device device) {
+    TensorData host = uninit_data(shape, dtype, Device::cpu());
+    size_t nbytes = static_cast<size_t>(host.layout.num_elements()) * size_in_bytes(dtype);
+    if (nbytes) std::memcpy(host.storage->ptr(), bytes, nbytes);
+    Tensor t(host);
+    return device == Device::cpu() ? t : t.to(device);
+}
+
+Tensor Tensor::full(const Shape &shape, Scalar value, DType dtype, Device device) {
+    TensorData out = uninit_data(shape, dtype, device);
+    backend::fill(out, fill_value(value, dtype));
+    return Tensor(out);
+}
+
+Tensor Tensor::contiguous() const {
+    if (d_.layout.is_contiguous()) return *this;
+    return Tensor(clone_data(d_));
+}
+
+Tensor Tensor::to(DType dtype) const {
+    if (dtype == d_.dtype) return *this;
+    return Tensor(cast_data(d_, dtype));
+}
+
+Tensor Tensor::to(Device device) const {
+    if (device == d_.device()) return *this;
+    // A contiguous copy on the source device, then the transfer (device to device goes through
+    // host memory, ref: src/backend/mod.rs:250-252).
+    Tensor src = contiguous();
+    if (d_.device().kind == Device::K::Rocm && device.kind == Device::K::Rocm) return src.to(Device::cpu()).to(device);
+    TensorData out = uninit_data(src.shape(), d_.dtype, device);
+    if (device.kind == Device::K::Rocm) backend::upload(out, src.data());
+    else backend::download(out, src.data());
+    return Tensor(out);
+}
+
+std::vector<uint8_t> Tensor::to_bytes() const {
+    Tensor host = to(Device::cpu()).contiguous();
+    size_t size = size_in_bytes(d_.dtype);
+    size_t nbytes = static_cast<size_t>(host.num_elements()) * size;
+    std::vector<uint8_t> out(nbytes);
+    if (nbytes) {
+        std::memcpy(out.data(), static_cast<const char *>(host.data().storage->ptr()) + host.storage_offset() * size,
+                    nbytes);
+    }
+    return out;
+}
+
+// ---- unary (ref: src/ops/unary.rs:17-57) ---------------------------------------------------------------
+
+Tensor Tensor::unary(UnaryOp op) const {
+    const TensorData &src = d_;
+    DType dtype = src.dtype;
+    DType compute;
+    switch (op) {
+        case UnaryOp::LogicalNot: compute = dtype; break;
+        case UnaryOp::Neg:
+            if (dtype == DType::Bool) {
+                throw Error("Negation, the `-` operator, on a bool tensor is not supported. If you are trying to "
+                            "invert a mask, use `logical_not()` instead.");
+            }
+            compute = dtype;
+            break;
+        case UnaryOp::Abs:
+        case UnaryOp::Relu:
+            if (dtype == DType::Bool) throw Error(std::string(unary_debug_name(op)) + " is not supported for bool tensors");
+            compute = dtype;
+            break;
+        case UnaryOp::Sign: compute = dtype; break;
+        case UnaryOp::Silu:
+        case UnaryOp::Gelu:
+        case UnaryOp::GeluTanh:
+        case UnaryOp::LogSigmoid:
+            if (!is_floating_point(dtype)) {
+                throw Error(std::string(unary_debug_name(op)) + " is not implemented for " + name_of(dtype) + " tensors");
+            }
+            compute = dtype;
+            break;
+        default: compute = is_floating_point(dtype) ? dtype : default_dtype(); break;
+    }
+    DType out_dtype = op == UnaryOp::LogicalNot ? DType::Bool : compute;
+    TensorData out = uninit_data(src.layout.shape, out_dtype, src.device());
+    backend::unary(op, out, cast_data(src, compute));
+    return Tensor(out);
+}
+
+// ---- binary (ref: src/ops/binary.rs:68-143) -------------------------------------------------------------
+
+Tensor binary_op(BinaryOp op, const Operand &lhs, const Operand &rhs) {
+    Resolved a(lhs), b(rhs);
+    std::vector<const TensorData *> tensors;
+    if (a.tensor) tensors.push_back(&*a.tensor);
+    if (b.tensor) tensors.push_back(&*b.tensor);
+    Device device = common_device(tensors);
+    ResultType rt;
+    a.add_to(rt);
+    b.add_to(rt);
+    DType common = rt.result();
+    DType compute = common;
+    if (op == BinaryOp::Div && !is_floating_point(common)) compute = default_dtype();
+    else if (op == BinaryOp::LogicalAnd || op == BinaryOp::LogicalOr) compute = DType::Bool;
+    if (op == BinaryOp::Sub) {
+        if (a.is_bool() && b.is_bool()) {
+            throw Error("Subtraction, the `-` operator, with two bool tensors is not supported. Use `not_equal()` "
+                        "(logical xor) instead.");
+        }
+        if (a.is_bool() || b.is_bool()) {
+            throw Error("Subtraction, the `-` operator, with a bool tensor is not supported. If you are trying to "
+                        "invert a mask, use `logical_not()` instead.");
+        }
+    }
+    if (compute == DType::Bool && op == BinaryOp::Pow) throw Error("pow is not supported for bool tensors");
+    if (is_integral(compute) && op == BinaryOp::Pow && !b.tensor && b.scalar.to_i64() < 0) {
+        throw Error("Integers to negative integer powers are not allowed.");
+    }
+    if (op == BinaryOp::BitwiseAnd && is_floating_point(compute)) {
+        throw Error(std::string("bitwise_and is not implemented for ") + name_of(compute) + " tensors");
+    }
+    DType out_dtype = (is_comparison(op) || op == BinaryOp::LogicalAnd || op == BinaryOp::LogicalOr) ? DType::Bool : compute;
+    Shape shape = broadcast_shapes(a.shape(), b.shape());
+    TensorData out = uninit_data(shape, out_dtype, device);
+    bool keeps_scalar = (op == BinaryOp::Mul || op == BinaryOp::Div) && (compute == DType::F16 || compute == DType::BF16);
+    if (a.tensor && b.tensor) {
+        // On ROCm the library's hmr_binary accepts a half operand next to an F32 one and widens it
+        // inside the kernel (exactly, so the bits are those of cast-then-op); the reference would
+        // first write an F32 copy of the half tensor (cast_data) and read it back.
+        auto half = [](DType d) { return d == DType::F16 || d == DType::BF16; };
+        bool arithmetic = op == BinaryOp::Add || op == BinaryOp::Sub || op == BinaryOp::Mul || op == BinaryOp::Div;
+        bool mixed = (half(a.tensor->dtype) && b.tensor->dtype == DType::F32) ||
+                     (a.tensor->dtype == DType::F32 && half(b.tensor->dtype));
+        if (g_fused_promotion && device.kind == Device::K::Rocm && compute == DType::F32 && arithmetic && mixed) {
+            backend::binary(op, out, a.tensor->expand_to(shape), b.tensor->expand_to(shape));
+        } else {
+            backend::binary(op, out, a.materialize(compute, device, shape), b.materialize(compute, device, shape));
+        }
+    } else {
+        bool scalar_first = !a.tensor;
+        const Resolved &t = scalar_first ? b : a;
+        Scalar s = scalar_first ? a.scalar : b.scalar;
+        TensorData td = t.materialize(compute, device, shape);
+        if (keeps_scalar) backend::binary_scalar(op, out, td, s.to_f64(), scalar_first);
+        else backend::binary_constant(op, out, td, s, scalar_first);
+    }
+    return Tensor(out);
+}
+
+Tensor Tensor::binary(BinaryOp op, const Operand &other) const { return binary_op(op, Operand(*this), other); }
+
+Tensor where_(const Tensor &condition, const Operand &x, const Operand &y) {
+    if (condition.dtype() != DType::Bool) {
+        throw Error(std::string("where expected condition to be a boolean tensor, but got a tensor with dtype ") +
+                    name_of(condition.dtype()));
+    }
+    ResultType rt;
+    Resolved(x).add_to(rt);
+    Resolved(y).add_to(rt);
+    return select_op(condition, x, y, rt.result());
+}
+
+// ref: src/ops/binary.rs:430-470
+Tensor Tensor::masked_fill(const Tensor &mask, const Operand &value) const {
+    if (mask.dtype() != DType::Bool) {
+        throw Error(std::string("masked_fill only supports boolean masks, but got mask with dtype ") + name_of(mask.dtype()));
+    }
+    if (std::holds_alternative<Scalar>(value)) {
+        return select_op(mask, Operand(fill_value(std::get<Scalar>(value), dtype())), Operand(*this), dtype());
+    }
+    const Tensor &t = std::get<Tensor>(value);
+    if (t.num_dims() != 0) {
+        throw Error("masked_fill only supports a 0-dimensional value tensor, but got tensor with " +
+                    std::to_string(t.num_dims()) + " dimension(s).");
+    }
+    return select_op(mask, Operand(t.to(dtype())), Operand(*this), dtype());
+}
+
+// ---- reductions (ref: src/ops/reduce.rs:175-405) --------------------------------------------------------
+
+Tensor Tensor::sum() const { return reduce_op(ReduceOp::Sum, *this, {}, false, "sum"); }
+Tensor Tensor::sum_dim(const std::vector<int64_t> &dims, bool keepdim) const {
+    return reduce_op(ReduceOp::Sum, *this, dims, keepdim, "sum");
+}
+
+Tensor Tensor::sum_to_size(const Shape &size) const {
+    const Shape &shape = d_.layout.shape;
+    if (!is_expandable_to(size, shape)) {
+        throw Error("size {" + shape_str(size) + "} is not expandable to size {" + shape_str(shape) + "}.");
+    }
+    size_t lead = shape.size() - size.size();
+    std::vector<int64_t> dims;
+    for (size_t d = 0; d < shape.size(); ++d) {
+        if (d < lead || (size[d - lead] == 1 && shape[d] != 1)) dims.push_back(static_cast<int64_t>(d));
+    }
+    if (dims.empty()) return *this;
+    Tensor summed = reduce_op(ReduceOp::Sum, *this, dims, true, "sum");
+    return Tensor(reshape_data(summed.data(), size));
+}
+
+Tensor Tensor::mean() const { return reduce_op(ReduceOp::Mean, *this, {}, false, "mean"); }
+Tensor Tensor::mean_dim(const std::vector<int64_t> &dims, bool keepdim) const {
+    return reduce_op(ReduceOp::Mean, *this, dims, keepdim, "mean");
+}
+Tensor Tensor::prod() const { return reduce_op(ReduceOp::Prod, *this, {}, false, "prod"); }
+Tensor Tensor::prod_dim(int64_t dim, bool keepdim) const { return reduce_op(ReduceOp::Prod, *this, {dim}, keepdim, "prod"); }
+Tensor Tensor::max() const { return reduce_op(ReduceOp::Max, *this, {}, false, "max"); }
+Tensor Tensor::min() const { return reduce_op(ReduceOp::Min, *this, {}, false, "min"); }
+
+ValuesAndIndices Tensor::max_dim(int64_t dim, bool keepdim) const {
+    auto r = arg_op(*this, dim, keepdim, true, true, "max");
+    return ValuesAndIndices{*r.first, r.second};
+}
+ValuesAndIndices Tensor::min_dim(int64_t dim, bool keepdim) const {
+    auto r = arg_op(*this, dim, keepdim, false, true, "min");
+    return ValuesAndIndices{*r.first, r.second};
+}
+Tensor Tensor::argmax() const { return arg_op(*this, std::nullopt, false, true, false, "argmax").second; }
+Tensor Tensor::argmin() const { return arg_op(*this, std::nullopt, false, false, false, "argmin").second; }
+Tensor Tensor::argmax_dim(int64_t dim, bool keepdim) const { return arg_op(*this, dim, keepdim, true, false, "argmax").second; }
+Tensor Tensor::argmin_dim(int64_t dim, bool keepdim) const { return arg_op(*this, dim, keepdim, false, false, "argmin").second; }
+
+Tensor Tensor::var(int64_t correction) const { return var_op(*this, {}, correction, false, false); }
+Tensor Tensor::var_dim(const std::vector<int64_t> &dims, int64_t correction, bool keepdim) const {
+    return var_op(*this, dims, correction, keepdim, false);
+}
+Tensor Tensor::std(int64_t correction) const { return var_op(*this, {}, correction, false, true); }
+Tensor Tensor::std_dim(const std::vector<int64_t> &dims, int64_t correction, bool keepdim) const {
+    return var_op(*this, dims, correction, keepdim, true);
+}
+
+Tensor Tensor::all() const { return reduce_op(ReduceOp::All, *this, {}, false, "all"); }
+Tensor Tensor::any() const { return reduce_op(ReduceOp::Any, *this, {}, false, "any"); }
+Tensor Tensor::all_dim(const std::vector<int64_t> &dims, bool keepdim) const {
+    return reduce_op(ReduceOp::All, *this, dims, keepdim, "all");
+}
+Tensor Tensor::any_dim(const std::vector<int64_t> &dims, bool keepdim) const {
+    return reduce_op(ReduceOp::Any, *this, dims, keepdim, "any");
+}
+
+Tensor Tensor::softmax(int64_t dim) const { return softmax_op(*this, dim, false); }
+Tensor Tensor::log_softmax(int64_t dim) const { return softmax_op(*this, dim, true); }
+
+}  // namespace homura

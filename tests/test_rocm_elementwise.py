@@ -1,0 +1,315 @@
+"""Elementwise kernels on the GPU against the CPU oracle, through the host layer and the C ABI.
+Modelled on the reference's tests/rocm_elementwise.rs: the bitwise class for IEEE operations,
+integers, comparisons, logic and data selection; ulp bounds for the transcendental functions."""
+import math
+import threading
+
+import numpy as np
+import pytest
+
+from tests import oracle
+from tests.support import (DT, DTYPES, FLOATS, GPU, INTS, NP, VIEWS, array, assert_bitwise, bits, check_within, from_f64,
+                           h, large_layouts, layouts, tensor, to_f64, uniform, values, words)
+
+pytestmark = pytest.mark.gpu
+h.register_cpu_backend(oracle.backend_address())
+
+
+def float_tensor(v, dtype):
+    return tensor(from_f64(v, dtype), dtype)
+
+
+def near_zero(n, seed):
+    """Magnitudes below 2^-10 down to the subnormals of every float dtype (ref: rocm_elementwise.rs:30-46)."""
+    w = words(seed, n)
+    e = -10 - (w % np.uint64(1070)).astype(np.int64)
+    m = 1.0 + (w >> np.uint64(20)).astype(np.float64) / float(1 << 44)
+    s = np.where((w & np.uint64(1 << 12)) != 0, -1.0, 1.0)
+    v = s * np.ldexp(m, np.maximum(e, -1074))
+    return np.concatenate([v, [0.0, -0.0, 5.96e-8, 1e-40, -1e-45, math.ldexp(1.0, -1074)]])
+
+
+def domains(dtype, tails, seed):
+    d = [(p.name, p.cpu) for p in layouts(dtype, seed)]
+    for r in (1.0, 10.0, 100.0):
+        d.append((f"uniform +-{r}", float_tensor(uniform(seed + 1, 4096, -r, r), dtype)))
+    d.append(("near zero", float_tensor(near_zero(2048, seed + 2), dtype)))
+    d.append(("tails", float_tensor(np.array(tails, dtype=np.float64), dtype)))
+    return d
+
+
+IEEE_UNARY = ["neg", "abs", "sign", "relu", "sqrt", "rsqrt", "reciprocal", "logical_not"]
+
+
+def test_ieee_unary_ops_are_bitwise():
+    for dtype in DTYPES:
+        for p in layouts(dtype, 1):
+            for name in IEEE_UNARY:
+                if dtype == DT.Bool and name in ("neg", "abs", "relu"):
+                    continue
+                assert_bitwise(getattr(p.gpu, name)(), getattr(p.cpu, name)(), f"{name} {dtype} {p.name}")
+    for p in large_layouts(DT.F32, 2):
+        assert_bitwise(p.gpu.sqrt(), p.cpu.sqrt(), p.name)
+        assert_bitwise(p.gpu.neg(), p.cpu.neg(), p.name)
+    for p in large_layouts(DT.BF16, 3):
+        assert_bitwise(p.gpu.abs(), p.cpu.abs(), p.name)
+
+
+# (name, op, k of the reference's bound k*u*m + ulp, tails)
+TRANSCENDENTAL = [
+    ("exp", 2.0, [88.7, 88.72, 88.73, -87.3, -103.9, -104.0, 709.7, 709.8, -745.1, 11.09, -17.3]),
+    ("log", 2.0, [1e-300, 1e300, 1.0 + 1e-7]),
+    ("sin", 2.0, [math.pi, 1e6, 1e20, 355.0]),
+    ("cos", 2.0, [math.pi / 2, 1e6, 1e20, 33.0]),
+    ("tanh", 2.0, [9.0, 20.0, -20.0, 1e-5]),
+    ("erf", 2.0, [5.9, 6.0, 6.1, -7.0, 1.49999, 1.5, 1.50001, 3.0]),
+    ("sigmoid", 4.0, [-30.0, -88.0, -104.0, 30.0, 40.0, -745.0]),
+    ("silu", 4.0, [-30.0, -88.0, -104.0, 30.0, 40.0, -745.0]),
+    ("log_sigmoid", 6.0, [-30.0, -31.0, -1e4, 30.0, 31.0, 40.0, 1e4]),
+    ("gelu", 4.0, [-10.0, -10.5, -12.0, -30.0, 10.0]),
+    ("gelu_tanh", 4.0, [-10.0, -10.5, -12.0, -30.0, 10.0]),
+]
+
+
+def magnitude(name, x, y):
+    """Size of the largest intermediate at input x with CPU result y (ref: rocm_elementwise.rs:203-232)."""
+    with np.errstate(all="ignore"):
+        if name == "silu":
+            return np.abs(x) / (1.0 + np.exp(-x))
+        if name == "log_sigmoid":
+            return np.abs(np.minimum(x, 0.0)) + np.log1p(np.exp(-np.abs(x)))
+        if name == "gelu":
+            erf = np.array([oracle.lib().orc_erf(float(v) * math.sqrt(0.5)) for v in x])
+            return 0.5 * np.abs(x) * (1.0 + np.abs(erf))
+        if name == "gelu_tanh":
+            k = math.sqrt(2.0 / math.pi)
+            return 0.5 * np.abs(x) * (1.0 + np.abs(np.tanh(k * (x + 0.044715 * x * x * x))))
+        return np.abs(y)
+
+
+# Ops whose f32 / half results must sit within ONE ulp of the output dtype of the oracle's, with no
+# further allowance. The others (tanh, log_sigmoid, gelu_tanh) go through glibc functions whose own
+# error exceeds half an ulp, so they are held to the reference's bound k*u*m + ulp instead.
+ONE_ULP = {"exp", "log", "sin", "cos", "erf", "sigmoid", "silu", "gelu"}
+
+
+@pytest.mark.parametrize("name,k,tails", TRANSCENDENTAL, ids=[t[0] for t in TRANSCENDENTAL])
+def test_transcendental_unary_ops_stay_within_the_bounds(name, k, tails):
+    for dtype in FLOATS:
+        u = 2.0 ** -53 if dtype == DT.F64 else 2.0 ** -24
+        differ = total = worst = 0
+        for what, x in domains(dtype, tails, 11):
+            cpu = getattr(x, name)()
+            gpu = getattr(x.to(GPU), name)()
+            if name in ONE_ULP and dtype != DT.F64:
+                extra = 0.0
+            else:
+                xs = to_f64(array(x.contiguous()).reshape(-1), dtype)
+                ys = to_f64(array(cpu).reshape(-1), dtype)
+                with np.errstate(all="ignore"):
+                    extra = np.nan_to_num(k * u * magnitude(name, xs, ys), nan=0.0, posinf=0.0)
+            d, m = check_within(gpu, cpu, extra=extra, max_ulp=1, what=f"{name} {dtype} {what}")
+            differ += d
+            worst = max(worst, m)
+            total += cpu.num_elements()
+        print(f"ulp {name:<12} {dtype}: max {worst} ulp, {differ} of {total} elements differ")
+
+
+@pytest.mark.parametrize("dtype", [DT.BF16, DT.F16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("name", ["silu", "gelu", "exp", "sigmoid", "erf", "log", "tanh", "gelu_tanh"])
+def test_half_unary_ops_over_every_input(name, dtype):
+    """All 65 536 bit patterns of a 16-bit dtype: at most one ulp from the oracle, NaN to NaN."""
+    x = tensor(np.arange(65536, dtype=np.uint16), dtype)
+    cpu = getattr(x, name)()
+    gpu = getattr(x.to(GPU), name)()
+    differ, worst = check_within(gpu, cpu, extra=0.0, max_ulp=1, what=f"{name} {dtype} exhaustive")
+    print(f"exhaustive {name} {dtype}: {differ} of 65536 differ, max {worst} ulp")
+
+
+BINARY_FLOAT = ["add", "sub", "mul", "div", "maximum", "minimum"]
+BINARY_INT = ["add", "sub", "mul", "maximum", "minimum", "pow", "bitwise_and"]
+BINARY_BOOL = ["add", "mul", "maximum", "minimum", "bitwise_and"]
+COMPARE = ["greater", "greater_equal", "less", "less_equal", "equal", "not_equal"]
+
+
+def ops_for(dtype):
+    if dtype == DT.Bool:
+        return BINARY_BOOL
+    return BINARY_INT if dtype in INTS else BINARY_FLOAT
+
+
+def test_ieee_binary_ops_comparisons_and_logic_are_bitwise():
+    for dtype in DTYPES:
+        a, b = layouts(dtype, 21), layouts(dtype, 22)
+        for p, q in zip(a, b):
+            for name in ops_for(dtype) + COMPARE + ["logical_and", "logical_or"]:
+                assert_bitwise(getattr(p.gpu, name)(q.gpu), getattr(p.cpu, name)(q.cpu), f"{name} {dtype} {p.name}")
+    # Operands of different layouts and broadcasting between them.
+    for dtype in (DT.F32, DT.BF16, DT.I64, DT.Bool):
+        x = tensor(values(dtype, 35, 5), dtype, [7, 5])
+        y = tensor(values(dtype, 35, 6), dtype, [5, 7])
+        row = tensor(values(dtype, 5, 7), dtype, [5])
+        col = tensor(values(dtype, 7, 8), dtype, [7, 1])
+        for name in ops_for(dtype)[:3] + COMPARE[:2]:
+            for l, r, what in ((x, y.transpose(0, 1), "transposed rhs"), (x, row, "row"), (x, col, "column"),
+                               (col, row, "outer"), (row, x, "row lhs")):
+                gpu = getattr(l.to(GPU), name)(r.to(GPU))
+                assert_bitwise(gpu, getattr(l, name)(r), f"{name} {dtype} {what}")
+    for p, q in zip(large_layouts(DT.F32, 23), large_layouts(DT.F32, 24)):
+        assert_bitwise(p.gpu.add(q.gpu), p.cpu.add(q.cpu), f"add {p.name}")
+        assert_bitwise(p.gpu.div(q.gpu), p.cpu.div(q.cpu), f"div {p.name}")
+
+
+def test_float_pow_stays_within_one_ulp():
+    for dtype in FLOATS:
+        base = float_tensor(np.abs(uniform(31, 4096, 0.0, 20.0)), dtype)
+        expo = float_tensor(uniform(32, 4096, -4.0, 4.0), dtype)
+        cpu = base.pow(expo)
+        gpu = base.to(GPU).pow(expo.to(GPU))
+        d, m = check_within(gpu, cpu, extra=0.0, max_ulp=1 if dtype != DT.F64 else 2, what=f"pow {dtype}")
+        print(f"ulp pow {dtype}: max {m} ulp, {d} differ")
+
+
+def test_type_promotion_matches_the_cpu_front_end():
+    """Mixed dtypes, zero-dim tensors and scalars: the same result dtype and bits on both devices."""
+    cases = [(DT.BF16, DT.F32), (DT.F16, DT.F32), (DT.I32, DT.F16), (DT.U8, DT.I8), (DT.Bool, DT.I64), (DT.I64, DT.F64),
+             (DT.F16, DT.BF16), (DT.I16, DT.I64)]
+    for da, db in cases:
+        a = tensor(values(da, 24, 41), da, [4, 6])
+        b = tensor(values(db, 6, 42), db, [6])
+        for name in ("add", "mul", "div", "less"):
+            cpu = getattr(a, name)(b)
+            gpu = getattr(a.to(GPU), name)(b.to(GPU))
+            assert_bitwise(gpu, cpu, f"{name} {da}x{db}")
+        zero_dim = tensor(values(db, 70, 43)[60:61], db, [])
+        assert_bitwise(a.to(GPU).add(zero_dim.to(GPU)), a.add(zero_dim), f"zero-dim {da}x{db}")
+    for dtype in DTYPES:
+        a = tensor(values(dtype, 40, 44), dtype, [5, 8])
+        for s in (2.5, -3, True):
+            for name in ("add", "mul", "div", "greater_equal", "rsub", "rdiv"):
+                if dtype == DT.Bool and name in ("rsub",):
+                    continue
+                if name == "rsub" and isinstance(s, bool):
+                    continue
+                try:
+                    cpu = getattr(a, name)(s)
+                except h.HomuraError as e:
+                    with pytest.raises(h.HomuraError) as g:
+                        getattr(a.to(GPU), name)(s)
+                    assert str(g.value) == str(e)
+                    continue
+                assert_bitwise(getattr(a.to(GPU), name)(s), cpu, f"{name} {dtype} scalar {s!r}")
+
+
+def test_half_scalar_products_keep_the_scalar_in_f32():
+    """ref: tests/tensor_api.rs:686-701: 7*(1/3) etc. for f16 and bf16."""
+    third = 1.0 / 3.0
+    for dtype, prod, quot, summ, diff in ((DT.F16, 2.333984375, 0.047607421875, 7.33203125, 6.66796875),
+                                          (DT.BF16, 2.328125, None, 7.34375, 6.65625)):
+        seven = float_tensor([7.0], dtype).to(GPU)
+        t3 = float_tensor([third], dtype).to(GPU)
+        assert to_f64(array(seven.mul(third)), dtype)[0] == prod
+        if quot is not None:
+            assert to_f64(array(t3.div(7.0)), dtype)[0] == quot
+        assert to_f64(array(seven.add(third)), dtype)[0] == summ
+        assert to_f64(array(seven.sub(third)), dtype)[0] == diff
+
+
+def test_where_and_masked_fill_move_exact_bits():
+    for dtype in DTYPES:
+        xs, ys = layouts(dtype, 51), layouts(dtype, 52)
+        conds = layouts(DT.Bool, 53)
+        for c, x, y in zip(conds, xs, ys):
+            assert_bitwise(h.where_(c.gpu, x.gpu, y.gpu), h.where_(c.cpu, x.cpu, y.cpu), f"where {dtype} {c.name}")
+            for s in (2.5, 7, False):
+                try:
+                    cpu = h.where_(c.cpu, x.cpu, s)
+                except h.HomuraError:
+                    continue
+                assert_bitwise(h.where_(c.gpu, x.gpu, s), cpu, f"where {dtype} scalar y {c.name}")
+                assert_bitwise(h.where_(c.gpu, s, y.gpu), h.where_(c.cpu, s, y.cpu), f"where {dtype} scalar x {c.name}")
+            assert_bitwise(h.where_(c.gpu, 1.5, -2), h.where_(c.cpu, 1.5, -2), f"where constants {c.name}")
+            fill = 3 if dtype != DT.Bool else True
+            assert_bitwise(x.gpu.masked_fill(c.gpu, fill), x.cpu.masked_fill(c.cpu, fill), f"masked_fill {dtype} {c.name}")
+    # Broadcast mask (the causal-mask pattern): mask [n, n] over scores [b, n, n].
+    n = 33
+    scores = tensor(values(DT.F32, 3 * n * n, 54), DT.F32, [3, n, n])
+    mask = tensor((np.arange(n)[None, :] > np.arange(n)[:, None]).astype(np.uint8), DT.Bool, [n, n])
+    assert_bitwise(scores.to(GPU).masked_fill(mask.to(GPU), -math.inf), scores.masked_fill(mask, -math.inf), "causal mask")
+
+
+def test_tails_and_alignments():
+    """Every start offset and length around the vector widths, so that the aligned 128-bit path, the
+    ragged last tile and the unaligned fallback all run (ref: rocm_elementwise.rs:801-824)."""
+    for dtype in (DT.F32, DT.BF16, DT.I64, DT.Bool, DT.I16):
+        base_a = tensor(values(dtype, 200, 61), dtype, [200])
+        base_b = tensor(values(dtype, 200, 62), dtype, [200])
+        ga, gb = base_a.to(GPU), base_b.to(GPU)
+        name = "add" if dtype != DT.Bool else "maximum"
+        for off in range(0, 18):
+            for length in list(range(0, 20)) + [31, 32, 33, 64, 65, 127, 128, 129]:
+                cpu = getattr(base_a.narrow(0, off, length), name)(base_b.narrow(0, 17 - off, length))
+                gpu = getattr(ga.narrow(0, off, length), name)(gb.narrow(0, 17 - off, length))
+                assert_bitwise(gpu, cpu, f"{dtype} offset {off} length {length}")
+    # Rows of a 2-D view: inner length not a multiple of the vector width, and unaligned rows.
+    for dtype in (DT.F32, DT.BF16):
+        for cols, pitch in ((64, 64), (64, 72), (60, 64), (63, 67), (128, 136), (8, 8), (16, 24)):
+            base = tensor(values(dtype, 9 * pitch, 63), dtype, [9, pitch])
+            bias = tensor(values(dtype, cols, 64), dtype, [cols])
+            scale = tensor(values(dtype, 9, 65), dtype, [9, 1])
+            v, gv = base.narrow(1, 0, cols), base.to(GPU).narrow(1, 0, cols)
+            assert_bitwise(gv.add(bias.to(GPU)), v.add(bias), f"bias {dtype} {cols}/{pitch}")
+            assert_bitwise(gv.mul(scale.to(GPU)), v.mul(scale), f"scale {dtype} {cols}/{pitch}")
+
+
+def test_uniform_operands_in_every_position():
+    """An operand broadcast from one element, in each position (ref: rocm_elementwise.rs:864-937)."""
+    for dtype in (DT.F32, DT.BF16, DT.I32):
+        x = tensor(values(dtype, 1031, 71), dtype, [1031])
+        one = tensor(values(dtype, 80, 72)[70:71], dtype, [1])
+        gx, gone = x.to(GPU), one.to(GPU)
+        assert_bitwise(gx.add(gone), x.add(one), f"{dtype} x + one")
+        assert_bitwise(gone.sub(gx), one.sub(x), f"{dtype} one - x")
+        assert_bitwise(gone.expand([1031]).mul(gone.expand([1031])), one.expand([1031]).mul(one.expand([1031])), "both")
+        cond = tensor(values(DT.Bool, 1031, 73), DT.Bool, [1031])
+        t = tensor(np.array([1], dtype=np.uint8), DT.Bool, [1])
+        assert_bitwise(h.where_(t.to(GPU), gx, gone), h.where_(t, x, one), f"{dtype} uniform cond")
+        assert_bitwise(h.where_(cond.to(GPU), gone, gx), h.where_(cond, one, x), f"{dtype} uniform x")
+
+
+def test_concurrent_callers_get_the_serial_bits():
+    """ref: rocm_elementwise.rs:939-957"""
+    x = tensor(values(DT.F32, 5000, 81), DT.F32, [5000]).to(GPU)
+    y = tensor(values(DT.F32, 5000, 82), DT.F32, [5000]).to(GPU)
+    want = bits(x.mul(y).add(x).silu())
+    errors = []
+
+    def work():
+        try:
+            for _ in range(20):
+                if not np.array_equal(bits(x.mul(y).add(x).silu()), want):
+                    errors.append("bits differ")
+        except Exception as e:  # noqa: BLE001
+            errors.append(repr(e))
+
+    threads = [threading.Thread(target=work) for _ in range(8)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors[:3]
+
+
+def test_the_judges_reject_wrong_results():
+    """A judge that cannot fail pins nothing (ref: rocm_elementwise.rs:238-267)."""
+    x = float_tensor(uniform(91, 512, -4.0, 4.0), DT.F32)
+    good = x.exp()
+    # exp computed in bf16 precision: far outside one f32 ulp.
+    coarse = x.to(DT.BF16).exp().to(DT.F32).to(GPU)
+    with pytest.raises(AssertionError):
+        check_within(coarse, good, extra=0.0, max_ulp=1, what="coarse")
+    with pytest.raises(AssertionError):
+        assert_bitwise(x.to(GPU).neg(), x.abs(), "neg is not abs")
+    nan = float_tensor([math.nan, 1.0], DT.F32)
+    with pytest.raises(AssertionError):
+        check_within(float_tensor([0.0, 1.0], DT.F32).to(GPU), nan, what="nan vs 0")

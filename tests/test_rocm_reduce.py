@@ -1,0 +1,399 @@
+"""Reductions, variance, arg reductions and softmax on the GPU against the CPU oracle, through the
+host layer and the C ABI. Modelled on the reference's tests/rocm_reduce.rs.
+
+Classes (ref: tests/rocm_reduce.rs:148-289), eps = 2^-53 because both sides accumulate in f64:
+  bitwise   integer/bool sums and products, all, any, max, min, arg reductions; float reductions
+            whose every partial result is exact; special values
+  sum       |gpu - cpu| <= 2 n eps sum|x| (/ n for a mean) + ulp_out
+  product   |gpu - cpu| <= 2 n eps |cpu| + ulp_out
+  variance  delta = 4 n eps v: |gpu - cpu| <= delta + ulp_out (std: min(delta/sqrt v, sqrt delta))
+  softmax   (2 n eps + 2 eps)|cpu| + ulp_out, rows sum to 1
+For well-conditioned inputs the allowances vanish next to ulp_out and the bound is one ulp of the
+output dtype."""
+import itertools
+import math
+
+import numpy as np
+import pytest
+
+from tests import oracle
+from tests.support import (DT, DTYPES, FLOATS, GPU, INTS, array, assert_bitwise, bits, check_within, from_f64, h,
+                           tensor, to_f64, ulp_of, values, words)
+
+pytestmark = pytest.mark.gpu
+h.register_cpu_backend(oracle.backend_address())
+EPS = 2.0 ** -53
+
+SHAPES = [[], [7], [4, 5], [3, 1, 4], [3, 0, 2], [2, 3, 2, 5], [2, 1, 3, 2, 3]]
+
+
+def prod(shape):
+    return int(np.prod(shape)) if shape else 1
+
+
+def cases(shape, make):
+    """`shape` in four layouts: contiguous, reversed strides, narrowed (offset and gaps), broadcast
+    (ref: tests/rocm_reduce.rs:44-88). make(n) gives a 1-D CPU tensor of n elements."""
+    n, rank, out = prod(shape), len(shape), []
+
+    def add(name, base, view):
+        cpu, gpu = view(base), view(base.to(GPU))
+        assert list(cpu.shape) == list(shape) and gpu.strides == cpu.strides, name
+        out.append((f"{name} {shape}", cpu, gpu))
+
+    add("contiguous", make(n), lambda t: t.reshape(shape))
+    if rank >= 2:
+        add("reversed strides", make(n), lambda t: t.reshape(shape[::-1]).permute(list(range(rank))[::-1]))
+    if rank >= 1:
+        wide = list(shape)
+        wide[-1] = 2 * shape[-1] + 1
+        add("narrowed", make(prod(wide)), lambda t: t.reshape(wide).narrow(rank - 1, 1, shape[-1]))
+        if shape[0] > 1:
+            one = [1] + list(shape[1:])
+            add("broadcast", make(n // shape[0]), lambda t: t.reshape(one).expand(shape))
+    return out
+
+
+def dim_sets(rank):
+    """Every subset of the dimensions, every other one spelled negatively."""
+    sets = []
+    for m in range(1 << rank):
+        sets.append([d if (m + d) % 2 == 0 else d - rank for d in range(rank) if m >> d & 1])
+    return sets
+
+
+def finite(dtype, n, scale, seed):
+    """+-m * 2^e, m in [1, 2), e in [-scale, scale], mixed signs (ref: tests/rocm_reduce.rs:114-128)."""
+    w = words(seed, n)
+    e = (w % np.uint64(2 * scale + 1)).astype(np.int64) - scale
+    m = 1.0 + (w >> np.uint64(11)).astype(np.float64) / float(1 << 53)
+    s = np.where((w & np.uint64(1 << 8)) != 0, -1.0, 1.0)
+    return tensor(from_f64(s * np.ldexp(m, e), dtype), dtype)
+
+
+def factors(dtype, n, seed):
+    w = words(seed, n)
+    m = 0.5 + 1.5 * ((w >> np.uint64(11)).astype(np.float64) / float(1 << 53))
+    return tensor(from_f64(np.where((w & np.uint64(1)) == 1, -m, m), dtype), dtype)
+
+
+def f64(t):
+    return to_f64(array(t).reshape(-1), t.dtype)
+
+
+def folded(x, out):
+    return 0 if out.num_elements() == 0 else x.num_elements() // out.num_elements()
+
+
+def test_integer_sums_truth_folds_extremes_and_arg_reductions_match_the_cpu():
+    for dtype in DTYPES:
+        floating = dtype in FLOATS
+        for s, shape in enumerate(SHAPES):
+            for name, cpu, gpu in cases(shape, lambda n: tensor(values(dtype, n, 11 + s), dtype)):
+                for dims in dim_sets(len(shape)):
+                    for keepdim in (False, True):
+                        what = f"{dtype} {name} dims {dims} keepdim {keepdim}"
+                        if not floating:
+                            assert_bitwise(gpu.sum_dim(dims, keepdim), cpu.sum_dim(dims, keepdim), "sum " + what)
+                            assert_bitwise(gpu.prod_dim(dims[0], keepdim), cpu.prod_dim(dims[0], keepdim),
+                                           "prod " + what) if len(dims) == 1 else None
+                        assert_bitwise(gpu.all_dim(dims, keepdim), cpu.all_dim(dims, keepdim), "all " + what)
+                        assert_bitwise(gpu.any_dim(dims, keepdim), cpu.any_dim(dims, keepdim), "any " + what)
+                if prod(shape) > 0:
+                    assert_bitwise(gpu.max(), cpu.max(), f"max {dtype} {name}")
+                    assert_bitwise(gpu.min(), cpu.min(), f"min {dtype} {name}")
+                    assert_bitwise(gpu.argmax(), cpu.argmax(), f"argmax {dtype} {name}")
+                    assert_bitwise(gpu.argmin(), cpu.argmin(), f"argmin {dtype} {name}")
+                for d in range(len(shape)):
+                    if shape[d] == 0:
+                        continue
+                    for keepdim in (False, True):
+                        gv, gi = gpu.max_dim(d, keepdim)
+                        cv, ci = cpu.max_dim(d - len(shape), keepdim)
+                        assert_bitwise(gv, cv, f"max_dim values {dtype} {name} {d}")
+                        assert_bitwise(gi, ci, f"max_dim indices {dtype} {name} {d}")
+                        assert_bitwise(gpu.argmin_dim(d, keepdim), cpu.argmin_dim(d, keepdim), f"argmin {dtype} {name} {d}")
+                        gv, gi = gpu.min_dim(d, keepdim)
+                        cv, ci = cpu.min_dim(d, keepdim)
+                        assert_bitwise(gv, cv, f"min_dim values {dtype} {name} {d}")
+                        assert_bitwise(gi, ci, f"min_dim indices {dtype} {name} {d}")
+
+
+def check_sum(gpu, cpu, abs_sum, n, mean, what):
+    div = max(n, 1) if mean else 1.0
+    return check_within(gpu, cpu, extra=2.0 * n * EPS * f64(abs_sum) / div, what=what)
+
+
+def test_float_sums_means_products_and_variances_stay_within_their_classes():
+    for dtype in FLOATS:
+        scale = 12 if dtype == DT.F16 else 30
+        for s, shape in enumerate(SHAPES):
+            for name, cpu, gpu in cases(shape, lambda n: finite(dtype, n, scale, 31 + s)):
+                wide = cpu.to(DT.F64)
+                for dims in dim_sets(len(shape)):
+                    what = f"{dtype} {name} dims {dims}"
+                    c = cpu.sum_dim(dims, False)
+                    n = folded(cpu, c)
+                    abs_sum = wide.abs().sum_dim(dims, False)
+                    check_sum(gpu.sum_dim(dims, False), c, abs_sum, n, False, "sum " + what)
+                    check_sum(gpu.mean_dim(dims, True), cpu.mean_dim(dims, True), abs_sum, n, True, "mean " + what)
+                    for correction in (0, 1):
+                        v = f64(wide.var_dim(dims, correction, False))
+                        with np.errstate(all="ignore"):
+                            delta = np.nan_to_num(4.0 * n * EPS * v, nan=0.0, posinf=0.0)
+                            sd = np.where(v > 0, np.minimum(delta / np.sqrt(np.where(v > 0, v, 1.0)), np.sqrt(delta)),
+                                          np.sqrt(delta))
+                        check_within(gpu.var_dim(dims, correction, False), cpu.var_dim(dims, correction, False),
+                                     extra=delta, what="var " + what)
+                        check_within(gpu.std_dim(dims, correction, True), cpu.std_dim(dims, correction, True),
+                                     extra=sd, what="std " + what)
+            for name, cpu, gpu in cases(shape, lambda n: factors(dtype, n, 41 + s)):
+                for d in range(len(shape)):
+                    c = cpu.prod_dim(d, False)
+                    check_within(gpu.prod_dim(d, False), c, extra=2.0 * shape[d] * EPS * np.abs(f64(c)),
+                                 what=f"prod {dtype} {name} {d}")
+                c = cpu.prod()
+                check_within(gpu.prod(), c, extra=2.0 * max(prod(shape), 1) * EPS * np.abs(f64(c)), what=f"prod {dtype} {name}")
+
+
+def test_exact_cases_and_special_values_match_the_cpu():
+    """ref: tests/rocm_reduce.rs:523-613"""
+    for dtype in FLOATS:
+        v = np.array([((i * 37) % 17) - 8.0 for i in range(256)])
+        x = tensor(from_f64(v, dtype), dtype, [8, 32])
+        g = x.to(GPU)
+        for d in (0, 1):
+            assert_bitwise(g.sum_dim(d, False), x.sum_dim(d, False), f"{dtype} sum {d}")
+            assert_bitwise(g.mean_dim(d, False), x.mean_dim(d, False), f"{dtype} mean {d}")
+            assert_bitwise(g.var_dim(d, 0, False), x.var_dim(d, 0, False), f"{dtype} var {d}")
+            assert_bitwise(g.std_dim(d, 1, False), x.std_dim(d, 1, False), f"{dtype} std {d}")
+        m = {DT.F16: [1401.0, 1401.0, 1400.0], DT.F32: [16777215.0, 16777215.0, 16777213.0]}.get(dtype, [1.0, 2.0, 2.0])
+        m = tensor(from_f64(np.array(m), dtype), dtype, [1, 3])
+        assert_bitwise(m.to(GPU).mean_dim(1, False), m.mean_dim(1, False), f"{dtype} mean of an unrepresentable sum")
+        if dtype == DT.F16:
+            assert to_f64(array(m.to(GPU).mean_dim(1, False)), dtype)[0] == 1401.0
+        if dtype == DT.F32:
+            assert array(m.to(GPU).mean_dim(1, False))[0] == 16777214.0
+        p = tensor(from_f64(np.array([2.0, -0.5, 4.0, 0.25, -1.0, 8.0]), dtype), dtype)
+        assert_bitwise(p.to(GPU).prod(), p.prod(), f"{dtype} prod")
+        w = tensor(from_f64(np.array([1.0, 3.0, 2.0, 2.0]), dtype), dtype, [2, 2])
+        for correction in (2, 3):
+            assert_bitwise(w.to(GPU).var_dim(1, correction, False), w.var_dim(1, correction, False),
+                           f"{dtype} var correction {correction}")
+        e = tensor(np.zeros(0, dtype=np.float64), DT.F64, [3, 0]).to(dtype)
+        eg = e.to(GPU)
+        assert_bitwise(eg.sum_dim(1, False), e.sum_dim(1, False), "empty sum")
+        assert_bitwise(eg.prod_dim(1, False), e.prod_dim(1, False), "empty prod")
+        assert_bitwise(eg.mean_dim(1, False), e.mean_dim(1, False), "empty mean")
+        assert_bitwise(eg.var_dim(1, 0, False), e.var_dim(1, 0, False), "empty var")
+        assert_bitwise(eg.all_dim(1, False), e.all_dim(1, False), "empty all")
+        assert_bitwise(eg.any_dim(1, False), e.any_dim(1, False), "empty any")
+        inf, nan = math.inf, math.nan
+        special = [[1.0, nan, 2.0, 3.0], [1.0, inf, 2.0, 3.0], [1.0, -inf, 2.0, 3.0], [inf, 1.0, -inf, 3.0],
+                   [0.0, inf, 2.0, 3.0]]
+        x = tensor(from_f64(np.array(special).reshape(-1), dtype), dtype, [5, 4])
+        g = x.to(GPU)
+        assert_bitwise(g.sum_dim(1, False), x.sum_dim(1, False), f"{dtype} sum of special values")
+        assert_bitwise(g.mean_dim(1, False), x.mean_dim(1, False), f"{dtype} mean of special values")
+        assert_bitwise(g.prod_dim(1, False), x.prod_dim(1, False), f"{dtype} prod of special values")
+        assert_bitwise(g.var_dim(1, 1, False), x.var_dim(1, 1, False), f"{dtype} var of special values")
+    with pytest.raises(h.HomuraError):
+        tensor(np.zeros(0, dtype=np.float32), DT.F32, [0]).to(GPU).max()
+
+
+def rows_of(t, dim):
+    a = to_f64(array(t), t.dtype)
+    if a.ndim == 0:
+        return a.reshape(1, 1)
+    return np.moveaxis(a, dim, -1).reshape(-1, a.shape[dim])
+
+
+def check_softmax(gpu, cpu, x, dim, log, what):
+    """ref: tests/rocm_reduce.rs:206-289"""
+    dtype = cpu.dtype
+    xr, cr = rows_of(x, dim), rows_of(cpu, dim)
+    n = xr.shape[1] if xr.size else 1
+    acc, e_exp = 2.0 * n * EPS, 2.0 * EPS
+    with np.errstate(all="ignore"):
+        mx = np.where(np.isnan(xr), -np.inf, xr).max(axis=1, keepdims=True) if xr.size else xr
+        s = np.exp(xr - mx).sum(axis=1, keepdims=True) if xr.size else xr
+        extra_rows = (acc + 2.0 * EPS * np.abs(np.log(s))) * np.ones_like(cr) if log else (acc + e_exp) * np.abs(cr)
+    extra_rows = np.nan_to_num(extra_rows, nan=0.0, posinf=0.0)
+    if x.shape:
+        moved = list(np.moveaxis(np.empty(x.shape), dim, -1).shape)
+        extra = np.moveaxis(extra_rows.reshape(moved), -1, dim).reshape(-1)
+    else:
+        extra = extra_rows.reshape(-1)
+    stats = check_within(gpu, cpu, extra=extra, what=what)
+    for r, gs in enumerate(rows_of(gpu, dim)):
+        if not np.all(np.isfinite(gs)):
+            continue
+        if log:
+            e = np.exp(gs)
+            total, slack = e.sum(), float((e * ulp_of(dtype, np.abs(gs))).sum())
+        else:
+            total, slack = gs.sum(), n * float(ulp_of(dtype, np.array(1.0)))
+        assert abs(total - 1.0) <= acc + n * e_exp + slack, f"{what}: row {r} sums to {total!r}"
+    return stats
+
+
+def test_softmax_and_log_softmax_stay_within_their_class():
+    for dtype in FLOATS:
+        for s, shape in enumerate(SHAPES):
+            if prod(shape) == 0:
+                continue
+            for name, cpu, gpu in cases(shape, lambda n: finite(dtype, n, 3, 51 + s)):
+                for dim in range(max(len(shape), 1)):
+                    for log in (False, True):
+                        c = cpu.log_softmax(dim) if log else cpu.softmax(dim)
+                        g = gpu.log_softmax(dim - len(shape) if shape else dim) if log else gpu.softmax(dim)
+                        check_softmax(g, c, cpu.to(DT.F64), dim, log, f"{dtype} {name} dim {dim} log {log}")
+        # Longer rows: every register plan and the streaming plan, ragged ends included.
+        for n in (17, 64, 100, 513, 2048, 2049, 5000, 16384, 16385, 40000, 70000):
+            x = finite(dtype, 3 * n, 2, 60 + n).reshape([3, n])
+            for log in (False, True):
+                c = x.log_softmax(1) if log else x.softmax(1)
+                g = x.to(GPU).log_softmax(1) if log else x.to(GPU).softmax(1)
+                d, m = check_softmax(g, c, x.to(DT.F64), 1, log, f"{dtype} rows of {n} log {log}")
+                assert m <= 1 or dtype == DT.F64  # f64 outputs carry the f64 summation-order error itself
+            # ... and the same rows strided (softmax along dim 0 of the transpose).
+            xt = x.transpose(0, 1)
+            check_softmax(xt.to(GPU).softmax(0), xt.softmax(0), xt.to(DT.F64), 0, False, f"{dtype} strided rows of {n}")
+
+
+def test_softmax_extreme_rows_match_the_cpu():
+    """ref: tests/rocm_reduce.rs:615-653; plus the KAT of ref: tests/m0_boundaries.rs:468-480."""
+    inf, nan = math.inf, math.nan
+    for dtype in FLOATS:
+        big = {DT.F16: 6e4, DT.F64: 1e300}.get(dtype, 3e38)
+        rows = [[-inf, -inf, -inf, -inf], [1.0, nan, 2.0, 3.0], [1.0, inf, 2.0, 3.0], [big, -big, big, 0.0],
+                [-big, -big, 1.0, -inf], [0.0, -0.0, 0.0, -0.0]]
+        x = tensor(from_f64(np.array(rows).reshape(-1), dtype), dtype, [6, 4])
+        g = x.to(GPU)
+        for log in (False, True):
+            gv, cv = (g.log_softmax(1), x.log_softmax(1)) if log else (g.softmax(1), x.softmax(1))
+            check_softmax(gv, cv, x.to(DT.F64), 1, log, f"{dtype} extreme rows log {log}")
+        # Wide rows of the same kinds, so that the register kernels see them too.
+        wide = np.full((5, 300), -inf)
+        wide[1, :] = np.linspace(-3, 3, 300)
+        wide[1, 17] = nan
+        wide[2, :] = np.linspace(-3, 3, 300)
+        wide[2, 250] = inf
+        wide[3, :] = np.where(np.arange(300) % 2 == 0, -inf, np.linspace(-5, 5, 300))
+        wide[4, 299] = 0.5
+        xw = tensor(from_f64(wide.reshape(-1), dtype), dtype, [5, 300])
+        for log in (False, True):
+            gv, cv = (xw.to(GPU).log_softmax(1), xw.log_softmax(1)) if log else (xw.to(GPU).softmax(1), xw.softmax(1))
+            check_softmax(gv, cv, xw.to(DT.F64), 1, log, f"{dtype} wide extreme rows log {log}")
+            out = to_f64(array(gv), dtype)
+            assert np.all(np.isnan(out[0])) and np.all(np.isnan(out[1])) and np.all(np.isnan(out[2]))
+            assert np.all(out[3, 0::2] == (-inf if log else 0.0))
+        one = tensor(from_f64(np.array([3.0, -inf, nan]), dtype), dtype, [3, 1])
+        assert_bitwise(one.to(GPU).softmax(1), one.softmax(1), "one-element rows")
+        assert_bitwise(one.to(GPU).log_softmax(1), one.log_softmax(1), "one-element rows")
+    kat = tensor(np.array([1.0, 2.0, 3.0], dtype=np.float32), DT.F32).to(GPU).softmax(0)
+    assert np.allclose(array(kat), [0.09003057, 0.24472848, 0.66524094], rtol=1e-6, atol=0)
+    zero_dim = tensor(np.array([5.0], dtype=np.float32), DT.F32, [])
+    assert array(zero_dim.to(GPU).softmax(0)) == 1.0 and array(zero_dim.to(GPU).log_softmax(0)) == 0.0
+
+
+# Shapes and reduced dims that reach every plan of this library, with the plan each must get:
+# (lanes per output, number of slices > 1?).
+PLAN_SHAPES = [
+    ([3000, 512], [1], 64, False),          # a wave per contiguous row
+    ([600, 8192], [1], 256, False),         # a workgroup per contiguous row
+    ([4, 100000], [1], 256, True),          # rows cut into slices
+    ([1 << 21], [0], 256, True),            # a full reduction
+    ([8, 1 << 20], [0], 4, False),          # columns, one slice
+    ([5000, 256], [0], 4, True),            # columns cut into row slices
+    ([6, 700, 96], [1], 4, True),           # columns under an outer kept dimension
+    ([5000, 20], [1], 1, False),            # short rows: a lane per output
+    ([9, 2, 3000], [0, 2], 256, True),      # two reduced dimensions: any layout, 256 lanes
+    ([70, 600, 70], [0, 2], 256, False),    # ... without slices
+    ([7, 9, 11], [0, 2], 64, False),        # ... a wave per output
+    ([100000, 3], [0], 256, True),          # narrow outputs: too few columns for the column kernel
+    ([5, 1], [1], 1, False),
+    ([(1 << 22) + 1000, 2], [1], 1, False),  # more outputs than one pass of the grid
+]
+
+
+def test_every_plan_folds_each_element_once():
+    """Integer sums of random words change with any missing or repeated element; max_dim over values
+    with many ties must return the first position across lanes and slices
+    (ref: tests/rocm_reduce.rs:676-738)."""
+    seen = set()
+    for k, (shape, dims, group, split) in enumerate(PLAN_SHAPES):
+        n = prod(shape)
+        x = tensor(values(DT.I32, n, 100 + k), DT.I32, shape)
+        g = x.to(GPU)
+        p_group, p_splits, p_chunk = h.reduce_plan(g, dims)
+        assert (p_group, p_splits > 1) == (group, split), f"{shape} {dims}: plan {(p_group, p_splits, p_chunk)}"
+        seen.add((p_group, p_splits > 1))
+        assert_bitwise(g.sum_dim(dims, False), x.sum_dim(dims, False), f"i32 sum {shape} {dims}")
+        f = tensor(values(DT.F32, n, 200 + k), DT.F32, shape)
+        few = tensor((values(DT.U8, n, 300 + k) % 3).astype(np.float32), DT.F32, shape)
+        fin = finite(DT.F32, n, 20, 400 + k).reshape(shape)
+        gf = fin.to(GPU)
+        c = fin.sum_dim(dims, False)
+        check_sum(gf.sum_dim(dims, False), c, fin.to(DT.F64).abs().sum_dim(dims, False), folded(fin, c), False,
+                  f"f32 sum {shape} {dims}")
+        v = f64(fin.to(DT.F64).var_dim(dims, 1, False))
+        check_within(gf.var_dim(dims, 1, False), fin.var_dim(dims, 1, False),
+                     extra=np.nan_to_num(4.0 * folded(fin, c) * EPS * v), what=f"f32 var {shape} {dims}")
+        assert_bitwise(f.to(GPU).max(), f.max(), f"f32 max with NaNs {shape}")
+        if len(dims) == 1:
+            for t in (few, f):
+                gv, gi = t.to(GPU).max_dim(dims[0], False)
+                cv, ci = t.max_dim(dims[0], False)
+                assert_bitwise(gv, cv, f"max_dim values {shape}")
+                assert_bitwise(gi, ci, f"max_dim indices {shape}")
+            assert_bitwise(few.to(GPU).argmin_dim(dims[0], True), few.argmin_dim(dims[0], True), f"argmin {shape}")
+        assert_bitwise(few.to(GPU).argmax(), few.argmax(), f"argmax {shape}")
+        assert_bitwise(x.to(DT.Bool).to(GPU).all_dim(dims, False), x.to(DT.Bool).all_dim(dims, False), f"all {shape}")
+    assert seen >= {(64, False), (256, False), (256, True), (4, False), (4, True), (1, False)}
+
+
+SOFTMAX_PLAN_SHAPES = [
+    ([700, 200], 1, DT.F32, 64, 4), ([64, 2048], 1, DT.F32, 64, 32), ([16, 4096], 1, DT.F32, 256, 16),
+    ([8, 32000], 1, DT.BF16, 1024, 32), ([8, 32768], 1, DT.F32, 1024, 32), ([3, 70000], 1, DT.F32, 256, 0),
+    ([2048, 9], 0, DT.F32, 64, 0), ([40, 8, 1000], 1, DT.F16, 64, 0),
+]
+
+
+def test_softmax_plans_cover_every_path():
+    """(lanes per row, elements a lane keeps in registers; 0 = streamed)."""
+    for shape, dim, dtype, group, cache in SOFTMAX_PLAN_SHAPES:
+        x = finite(dtype, prod(shape), 2, 500 + shape[0]).reshape(shape)
+        split, p_group, p_cache = h.softmax_plan(x.to(GPU), dim)
+        assert (split, p_group, p_cache) == (False, group, cache), f"{shape} dim {dim}: {(split, p_group, p_cache)}"
+        for log in (False, True):
+            c = x.log_softmax(dim) if log else x.softmax(dim)
+            g = x.to(GPU).log_softmax(dim) if log else x.to(GPU).softmax(dim)
+            check_softmax(g, c, x.to(DT.F64), dim, log, f"{dtype} {shape} dim {dim} log {log}")
+
+
+def test_results_repeat_from_run_to_run():
+    """ref: tests/rocm_reduce.rs:797-811"""
+    x = finite(DT.F32, 1 << 20, 30, 600).reshape([1024, 1024]).to(GPU)
+    for f in (lambda t: t.sum(), lambda t: t.sum_dim(0, False), lambda t: t.sum_dim(1, False), lambda t: t.var_dim(0, 1, False),
+              lambda t: t.softmax(1), lambda t: t.mean()):
+        first = bits(f(x))
+        for _ in range(3):
+            assert np.array_equal(bits(f(x)), first)
+
+
+def test_the_judges_reject_wrong_results():
+    """ref: tests/rocm_reduce.rs:817-893: a dropped element, a wrong divisor, swapped outputs."""
+    x = finite(DT.F32, 4096, 3, 700).reshape([4, 1024])
+    wide = x.to(DT.F64)
+    good = x.sum_dim(1, False)
+    dropped = x.narrow(1, 0, 1023).to(GPU).sum_dim(1, False)
+    with pytest.raises(AssertionError):
+        check_sum(dropped, good, wide.abs().sum_dim(1, False), 1024, False, "dropped element")
+    with pytest.raises(AssertionError):
+        check_within(x.to(GPU).var_dim(1, 0, False), x.var_dim(1, 1, False), what="wrong divisor")
+    gv, gi = x.to(GPU).max_dim(1, False)
+    with pytest.raises(AssertionError):
+        assert_bitwise(gv, x.min_dim(1, False)[0], "max is not min")
+    with pytest.raises(AssertionError):
+        check_softmax(x.to(GPU).log_softmax(1), x.softmax(1), wide, 1, False, "log_softmax is not softmax")
