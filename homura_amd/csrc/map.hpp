@@ -5,8 +5,9 @@
 // Two kernels, picked on the host from the operands' merged dimensions:
 //
 //  map_rows_kernel   every operand walks its innermost dimension with stride 1 or 0. A lane owns
-//                    V consecutive elements of a row, V = 16 bytes of the narrowest operand, so
-//                    every operand moves in 128-bit accesses (wider operands take several). The
+//                    V consecutive elements of a row, V = 16 bytes of the widest operand, so the
+//                    widest operands move in 128-bit accesses and narrower ones in 64/32/16-bit
+//                    accesses, each instruction of a wave covering one contiguous span. The
 //                    outer dimensions are resolved once per V elements with 32-bit multiply-shift
 //                    division; a contiguous tensor is the one-dimensional case with no division
 //                    at all. Stride-0 operands (bias rows, per-row scales, scalars) are read once
@@ -37,6 +38,12 @@ namespace hmr {
 constexpr int kBlock = 256;      // 4 waves of 64
 constexpr int kFastDims = 6;     // merged dimensions the 32-bit kernels take
 constexpr int kMaxOperands = 4;  // output + 3 inputs
+// The vector kernels mark their 128-bit accesses nontemporal (see load_tile). The hint has to be
+// fixed at compile time: a run-time choice between the two forms is merged by the compiler into
+// one plain access.
+constexpr bool kStreamLoads = true;
+constexpr bool kStreamStores = false;
+constexpr int64_t kStreamBytes = int64_t{32} << 20;
 
 struct Unused {};
 
@@ -97,6 +104,7 @@ struct RowsArgs {
     uint64_t cbits[NOPS];
     uint32_t const_mask;   // bit k: operand k is a constant
     uint32_t bcast_mask;   // bit k: operand k has inner stride 0
+    uint32_t stream;       // nonzero: nontemporal loads and stores (large, read-once operands)
     int64_t n;             // elements
     uint32_t inner;        // size of the innermost dimension
     int32_t nouter;        // outer dimensions (0 for contiguous)
@@ -120,13 +128,22 @@ struct AnyArgs {
 
 // ---- register tiles ---------------------------------------------------------------------------------
 
-template <class T, int V>
+// 128-bit words as a native vector type, which the nontemporal builtins accept.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// NT marks the access nontemporal ("streaming"). Measured on MI355X with an f32 add over
+// 3 x 256 MB: plain 5.77 TB/s; nontemporal loads 6.24 TB/s with cold buffers and 6.9-7.6 TB/s
+// when the output buffer is one that was written recently (a chain of ops, or a loop that
+// recycles its buffers: the memory-side cache absorbs the plain stores); nontemporal stores as
+// well: 6.6 TB/s in every case. Loads stream, stores stay plain.
+template <class T, int V, bool NT = false>
 __device__ __forceinline__ void load_tile(const char *p, T (&r)[V]) {
     constexpr int bytes = V * static_cast<int>(sizeof(T));
     if constexpr (bytes % 16 == 0) {
 #pragma unroll
         for (int i = 0; i < bytes / 16; ++i) {
-            uint4 w = reinterpret_cast<const uint4 *>(p)[i];
+            const u32x4 *q = reinterpret_cast<const u32x4 *>(p) + i;
+            u32x4 w = NT ? __builtin_nontemporal_load(q) : *q;
             __builtin_memcpy(reinterpret_cast<char *>(r) + 16 * i, &w, 16);
         }
     } else if constexpr (bytes == 8) {
@@ -144,15 +161,17 @@ __device__ __forceinline__ void load_tile(const char *p, T (&r)[V]) {
     }
 }
 
-template <class T, int V>
+template <class T, int V, bool NT = false>
 __device__ __forceinline__ void store_tile(char *p, const T (&r)[V]) {
     constexpr int bytes = V * static_cast<int>(sizeof(T));
     if constexpr (bytes % 16 == 0) {
 #pragma unroll
         for (int i = 0; i < bytes / 16; ++i) {
-            uint4 w;
+            u32x4 w;
             __builtin_memcpy(&w, reinterpret_cast<const char *>(r) + 16 * i, 16);
-            reinterpret_cast<uint4 *>(p)[i] = w;
+            u32x4 *q = reinterpret_cast<u32x4 *>(p) + i;
+            if constexpr (NT) __builtin_nontemporal_store(w, q);
+            else *q = w;
         }
     } else if constexpr (bytes == 8) {
         uint2 w;
@@ -200,8 +219,12 @@ struct MapTraits {
     static constexpr int cmax(int a, int b) { return b > a ? b : a; }
     static constexpr int narrow = cmin(cmin(cmin(so, s0), s1), s2);
     static constexpr int wide = cmax(cmax(cmax(so, s0), s1), s2);
-    // Elements per lane-tile: 16 bytes of the narrowest operand.
-    static constexpr int V = 16 / narrow;
+    // Elements per lane-tile: 16 bytes of the WIDEST operand, so that no operand needs more than
+    // one access per tile and every access instruction of a wave covers one contiguous span
+    // (narrower operands move 8, 4 or 2 bytes per lane). Measured on MI355X: letting a lane own
+    // 128 contiguous bytes (16 bytes of the narrowest operand) makes each 128-bit load touch 64
+    // different cache lines, which with streaming loads multiplies the traffic.
+    static constexpr int V = 16 / wide;
     // Tiles per lane per pass: aim at 64 bytes of the widest operand in flight.
     static constexpr int U = (V * wide >= 64) ? 1 : 64 / (V * wide);
 };
@@ -214,25 +237,125 @@ __device__ __forceinline__ typename F::Out apply(const F &f, typename F::In0 a, 
     else return f(a, b, c);
 }
 
-// Reads the tile of input K (operand K+1) at element offset `off`.
+// ---- map_rows_kernel ---------------------------------------------------------------------------------
+//
+// The pass of a workgroup over its U*256 tiles comes in two forms. When every one of those tiles is
+// whole (all but the last workgroup of a ragged contiguous tensor) the body is straight-line code:
+// every address is computed, every load of every tile is issued, and only then does arithmetic
+// start, so a lane has U loads per operand in flight. Operands that are not plain vectors - a
+// stride-0 operand or a kernel-argument constant - must not put a branch between those loads (the
+// compiler would wait for memory at every join), so they are loaded too, as the aligned 16-byte
+// (or narrower) chunk that holds their element, and the element is picked out and replicated
+// afterwards. A constant's chunk is read from the output's first bytes and ignored.
+// The ragged pass handles partial tiles with per-element accesses.
+
+// The bytes of one operand's tile as they sit in registers between the load and the arithmetic:
+// an SSA vector of 32-bit words (never an array in memory, which a variable pick index would pin
+// to scratch).
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+template <int BYTES>
+struct RawOf;
+template <>
+struct RawOf<16> {
+    using type = u32x4;
+};
+template <>
+struct RawOf<8> {
+    using type = u32x2;
+};
+template <>
+struct RawOf<4> {
+    using type = uint32_t;
+};
+template <>
+struct RawOf<2> {
+    using type = uint16_t;
+};
+template <>
+struct RawOf<1> {
+    using type = uint8_t;
+};
+
 template <class T, int V>
-__device__ __forceinline__ void read_input(T (&r)[V], const char *base, uint64_t cbits, bool is_const, bool bcast,
-                                           int64_t off, bool full, int valid) {
+struct Chunk {
+    static constexpr int bytes = V * static_cast<int>(sizeof(T));
+    static_assert(bytes == 16 || bytes == 8 || bytes == 4 || bytes == 2 || bytes == 1, "chunk size");
+    using Raw = typename RawOf<bytes>::type;
+};
+template <int V>
+struct Chunk<Unused, V> {
+    static constexpr int bytes = 0;
+    using Raw = Unused;
+};
+
+// Loads the chunk at `p` (dense) or the aligned chunk containing the element at `p` (splat);
+// `low` is the element's byte offset inside that chunk.
+template <class T, int V>
+__device__ __forceinline__ typename Chunk<T, V>::Raw load_chunk(const char *p, bool splat, int &low) {
+    using Raw = typename Chunk<T, V>::Raw;
+    constexpr int bytes = Chunk<T, V>::bytes;
+    // Pointer arithmetic only: an integer-to-pointer cast would lose the global address space.
+    low = static_cast<int>(reinterpret_cast<uintptr_t>(p) & static_cast<uintptr_t>(bytes - 1));
+    const Raw *q = reinterpret_cast<const Raw *>(splat ? p - low : p);
+    if constexpr (kStreamLoads) return __builtin_nontemporal_load(q);
+    else return *q;
+}
+
+// The 32-bit word `wi` of a chunk, chosen with selects.
+template <class Raw>
+__device__ __forceinline__ uint32_t chunk_word(Raw raw, int wi) {
+    if constexpr (std::is_same_v<Raw, u32x4>) {
+        uint32_t w = raw[0];
+        w = wi == 1 ? raw[1] : w;
+        w = wi == 2 ? raw[2] : w;
+        w = wi == 3 ? raw[3] : w;
+        return w;
+    } else if constexpr (std::is_same_v<Raw, u32x2>) {
+        return wi == 1 ? raw[1] : raw[0];
+    } else {
+        return static_cast<uint32_t>(raw);
+    }
+}
+
+// Turns a loaded chunk into the tile's V elements: as loaded (dense), or V copies of the element
+// at byte offset `low` (splat), or V copies of the constant.
+template <class T, int V>
+__device__ __forceinline__ void unpack_chunk(typename Chunk<T, V>::Raw raw, bool splat, int low, bool is_const,
+                                             uint64_t cbits, T (&r)[V]) {
     if constexpr (std::is_same_v<T, Unused>) {
         return;
     } else {
+        if (!splat) {
+            __builtin_memcpy(r, &raw, sizeof(raw));
+            return;
+        }
+        uint64_t bits = chunk_word(raw, low >> 2);
+        if constexpr (sizeof(T) == 8) bits |= static_cast<uint64_t>(chunk_word(raw, (low >> 2) + 1)) << 32;
+        if constexpr (sizeof(T) < 4) bits >>= (low & 3) * 8;
+        if (is_const) bits = cbits;
+        const T v = from_cbits<T>(bits);
+#pragma unroll
+        for (int i = 0; i < V; ++i) r[i] = v;
+    }
+}
+
+// Reads the tile of one input in the ragged pass.
+template <class T, int V>
+__device__ __forceinline__ void read_ragged(T (&r)[V], const char *base, uint64_t cbits, bool is_const, bool bcast,
+                                            int64_t off, int valid) {
+    if constexpr (std::is_same_v<T, Unused>) {
+        return;
+    } else {
+        const T *p = reinterpret_cast<const T *>(base + off * static_cast<int64_t>(sizeof(T)));
         if (is_const) {
             T v = from_cbits<T>(cbits);
 #pragma unroll
             for (int i = 0; i < V; ++i) r[i] = v;
         } else if (bcast) {
-            T v = *reinterpret_cast<const T *>(base + off * static_cast<int64_t>(sizeof(T)));
+            T v = *p;
 #pragma unroll
             for (int i = 0; i < V; ++i) r[i] = v;
-        } else if (full) {
-            load_tile<T, V>(base + off * static_cast<int64_t>(sizeof(T)), r);
         } else {
-            const T *p = reinterpret_cast<const T *>(base + off * static_cast<int64_t>(sizeof(T)));
 #pragma unroll
             for (int i = 0; i < V; ++i) {
                 if (i < valid) r[i] = p[i];
@@ -251,70 +374,96 @@ __global__ void __launch_bounds__(kBlock) map_rows_kernel(RowsArgs<F::N + 1> a) 
     using A = typename F::In0;
     using B = typename F::In1;
     using C = typename F::In2;
+    using Off = std::conditional_t<FLAT, int64_t, uint32_t>;
     const F f{};
     const int64_t tiles = (a.n + V - 1) / V;
+    const int64_t whole = a.n / V;  // tiles [0, whole) have all V elements
     const bool c0 = a.const_mask & 2u, c1 = a.const_mask & 4u, c2 = a.const_mask & 8u;
-    const bool b0 = a.bcast_mask & 2u, b1 = a.bcast_mask & 4u, b2 = a.bcast_mask & 8u;
-    for (int64_t t0 = static_cast<int64_t>(blockIdx.x) * (U * kBlock) + threadIdx.x; t0 < tiles;
-         t0 += static_cast<int64_t>(gridDim.x) * (U * kBlock)) {
-        A ra[U][V];
-        B rb[U][V];
-        C rc[U][V];
-        using Off = std::conditional_t<FLAT, int64_t, uint32_t>;
-        Off oo[U];
-        int valid[U];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            int64_t t = t0 + static_cast<int64_t>(u) * kBlock;
-            valid[u] = 0;
-            if (t < tiles) {
-                int64_t e = t * V;
-                int64_t rem = a.n - e;
-                valid[u] = rem >= V ? V : static_cast<int>(rem);
-                Off off[4];
-                if constexpr (FLAT) {
-                    off[0] = e;
-                    off[1] = b0 ? 0 : e;
-                    off[2] = b1 ? 0 : e;
-                    off[3] = b2 ? 0 : e;
-                } else {
-                    uint32_t e32 = static_cast<uint32_t>(e);
-                    uint32_t row = divide(e32, a.inner_div);
-                    uint32_t col = e32 - row * a.inner;
-                    off[0] = col;
-                    off[1] = b0 ? 0 : col;
-                    off[2] = b1 ? 0 : col;
-                    off[3] = b2 ? 0 : col;
-                    for (int d = 0; d < a.nouter; ++d) {
-                        uint32_t q = divide(row, a.div[d]);
-                        uint32_t idx = row - q * a.div[d].div;
-                        row = q;
-                        off[0] += idx * static_cast<uint32_t>(a.ostride[0][d]);
-                        if constexpr (N >= 1) off[1] += idx * static_cast<uint32_t>(a.ostride[1][d]);
-                        if constexpr (N >= 2) off[2] += idx * static_cast<uint32_t>(a.ostride[2][d]);
-                        if constexpr (N >= 3) off[3] += idx * static_cast<uint32_t>(a.ostride[3][d]);
-                    }
-                }
-                oo[u] = off[0];
-                bool full = valid[u] == V;
-                read_input<A, V>(ra[u], a.ptr[1], a.cbits[1], c0, b0, off[1], full, valid[u]);
-                if constexpr (N >= 2) read_input<B, V>(rb[u], a.ptr[2], a.cbits[2], c1, b1, off[2], full, valid[u]);
-                if constexpr (N >= 3) read_input<C, V>(rc[u], a.ptr[3], a.cbits[3], c2, b2, off[3], full, valid[u]);
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            if (valid[u] == 0) continue;
-            Out ro[V];
-#pragma unroll
-            for (int i = 0; i < V; ++i) ro[i] = apply(f, ra[u][i], rb[u][i], rc[u][i]);
-            char *po = a.ptr[0] + static_cast<int64_t>(oo[u]) * static_cast<int64_t>(sizeof(Out));
-            if (valid[u] == V) {
-                store_tile<Out, V>(po, ro);
+    // "splat": the operand contributes one element per tile (stride 0 inside the tile, or a constant).
+    const bool s0 = (a.bcast_mask | a.const_mask) & 2u, s1 = (a.bcast_mask | a.const_mask) & 4u,
+               s2 = (a.bcast_mask | a.const_mask) & 8u;
+    for (int64_t base = static_cast<int64_t>(blockIdx.x) * (U * kBlock); base < tiles;
+         base += static_cast<int64_t>(gridDim.x) * (U * kBlock)) {
+        const int64_t t0 = base + threadIdx.x;
+        // Element offsets of tile t in each operand.
+        auto offsets = [&](int64_t t, Off(&off)[4]) {
+            if constexpr (FLAT) {
+                const int64_t e = t * V;
+                off[0] = e;
+                off[1] = s0 ? 0 : e;
+                off[2] = s1 ? 0 : e;
+                off[3] = s2 ? 0 : e;
             } else {
+                const uint32_t e32 = static_cast<uint32_t>(t * V);
+                uint32_t row = divide(e32, a.inner_div);
+                const uint32_t col = e32 - row * a.inner;
+                off[0] = col;
+                off[1] = s0 ? 0 : col;
+                off[2] = s1 ? 0 : col;
+                off[3] = s2 ? 0 : col;
+                for (int d = 0; d < a.nouter; ++d) {
+                    const uint32_t q = divide(row, a.div[d]);
+                    const uint32_t idx = row - q * a.div[d].div;
+                    row = q;
+                    off[0] += idx * static_cast<uint32_t>(a.ostride[0][d]);
+                    if constexpr (N >= 1) off[1] += idx * static_cast<uint32_t>(a.ostride[1][d]);
+                    if constexpr (N >= 2) off[2] += idx * static_cast<uint32_t>(a.ostride[2][d]);
+                    if constexpr (N >= 3) off[3] += idx * static_cast<uint32_t>(a.ostride[3][d]);
+                }
+            }
+        };
+        if (base + U * kBlock <= whole) {
+            // Whole pass: addresses, then all loads, then arithmetic and stores.
+            typename Chunk<A, V>::Raw wa[U];
+            typename Chunk<B, V>::Raw wb[U];
+            typename Chunk<C, V>::Raw wc[U];
+            int la[U], lb[U], lc[U];
+            Off oo[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                Off off[4];
+                offsets(t0 + static_cast<int64_t>(u) * kBlock, off);
+                oo[u] = off[0];
+                wa[u] = load_chunk<A, V>(a.ptr[1] + static_cast<int64_t>(off[1]) * static_cast<int64_t>(sizeof(A)), s0, la[u]);
+                if constexpr (N >= 2) {
+                    wb[u] = load_chunk<B, V>(a.ptr[2] + static_cast<int64_t>(off[2]) * static_cast<int64_t>(sizeof(B)), s1, lb[u]);
+                }
+                if constexpr (N >= 3) {
+                    wc[u] = load_chunk<C, V>(a.ptr[3] + static_cast<int64_t>(off[3]) * static_cast<int64_t>(sizeof(C)), s2, lc[u]);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                A ra[V];
+                B rb[V];
+                C rc[V];
+                unpack_chunk<A, V>(wa[u], s0, la[u], c0, a.cbits[1], ra);
+                if constexpr (N >= 2) unpack_chunk<B, V>(wb[u], s1, lb[u], c1, a.cbits[2], rb);
+                if constexpr (N >= 3) unpack_chunk<C, V>(wc[u], s2, lc[u], c2, a.cbits[3], rc);
+                Out ro[V];
+#pragma unroll
+                for (int i = 0; i < V; ++i) ro[i] = apply(f, ra[i], rb[i], rc[i]);
+                store_tile<Out, V, kStreamStores>(a.ptr[0] + static_cast<int64_t>(oo[u]) * static_cast<int64_t>(sizeof(Out)), ro);
+            }
+        } else {
+            // Ragged pass (the last workgroup): tile by tile, partial tiles element by element.
+            for (int u = 0; u < U; ++u) {
+                const int64_t t = t0 + static_cast<int64_t>(u) * kBlock;
+                if (t >= tiles) break;
+                const int64_t rem = a.n - t * V;
+                const int valid = rem >= V ? V : static_cast<int>(rem);
+                Off off[4];
+                offsets(t, off);
+                A xa[V];
+                B xb[V];
+                C xc[V];
+                read_ragged<A, V>(xa, a.ptr[1], a.cbits[1], c0, s0, off[1], valid);
+                if constexpr (N >= 2) read_ragged<B, V>(xb, a.ptr[2], a.cbits[2], c1, s1, off[2], valid);
+                if constexpr (N >= 3) read_ragged<C, V>(xc, a.ptr[3], a.cbits[3], c2, s2, off[3], valid);
+                Out *po = reinterpret_cast<Out *>(a.ptr[0] + static_cast<int64_t>(off[0]) * static_cast<int64_t>(sizeof(Out)));
 #pragma unroll
                 for (int i = 0; i < V; ++i) {
-                    if (i < valid[u]) reinterpret_cast<Out *>(po)[i] = ro[i];
+                    if (i < valid) po[i] = apply(f, xa[i], xb[i], xc[i]);
                 }
             }
         }
@@ -445,13 +594,14 @@ void launch_map(const MapCall &c, hipStream_t stream) {
         a.bcast_mask = 0;
         const int last = c.ndim - 1;
         for (int k = 0; k < NOPS; ++k) {
-            a.ptr[k] = c.ptr[k];
+            a.ptr[k] = c.is_const[k] ? c.ptr[0] : c.ptr[k];  // a constant's (ignored) chunk is read from the output
             a.cbits[k] = c.cbits[k];
             if (c.is_const[k]) a.const_mask |= 1u << k;
             else if (c.ndim == 0 || c.stride[k][last] == 0) a.bcast_mask |= k == 0 ? 0u : 1u << k;
         }
         int64_t tiles = (c.n + T::V - 1) / T::V;
         unsigned grid = grid_for(tiles, int64_t{T::U} * kBlock);
+        a.stream = c.n * (T::so + T::s0 + T::s1 + T::s2) >= kStreamBytes ? 1u : 0u;
         if (variant == 0) {
             a.inner = static_cast<uint32_t>(c.n < (int64_t{1} << 31) ? c.n : 0);
             a.nouter = 0;

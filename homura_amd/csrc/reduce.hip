@@ -85,6 +85,8 @@ hmr_status plan_reduction(const hmr_tensor_desc *out, const hmr_tensor_desc &kep
     p.chunk = a.nred;
     p.rstride = 0;
     p.inner = 0;
+    p.across = 4;
+    a.stream = 0;
     if (a.nout == 0 || a.nred == 0) return HMR_OK;  // nothing to read: one lane per output writes the identity
 
     const bool base_aligned = reinterpret_cast<uintptr_t>(a.src) % 16 == 0;
@@ -96,6 +98,12 @@ hmr_status plan_reduction(const hmr_tensor_desc *out, const hmr_tensor_desc &kep
     };
     const bool red_contiguous = a.red.ndim == 1 && a.red.stride[0] == 1;
     const int vec = 16 / elem;
+    // Read-once sources far larger than an XCD's L2 stream past the caches. (A broadcast source,
+    // whose elements are visited repeatedly, is smaller than nout*nred and stays cached.)
+    bool dense = true;
+    for (int d = 0; d < a.kept.ndim; ++d) dense = dense && a.kept.stride[d] != 0;
+    for (int d = 0; d < a.red.ndim; ++d) dense = dense && a.red.stride[d] != 0;
+    a.stream = dense && a.nout * a.nred >= kStreamSourceBytes / elem ? 1u : 0u;
 
     // Rows: one contiguous run per output.
     if (red_contiguous && a.nred >= 256 && base_aligned && strides_aligned(a.kept, 0)) {
@@ -121,8 +129,10 @@ hmr_status plan_reduction(const hmr_tensor_desc *out, const hmr_tensor_desc &kep
             a.kept.stride[d - 1] = a.kept.stride[d];
         }
         a.kept.ndim -= 1;
-        int64_t tiles = ceil_div(p.inner, int64_t{kWave} * vec) * (a.nout / p.inner);
-        cut(p, ceil_div(8 * 256, tiles), 16);
+        // As many waves side by side as the run of outputs fills (wide spans read best).
+        p.across = p.inner > 2 * kWave * vec ? 4 : (p.inner > kWave * vec ? 2 : 1);
+        int64_t tiles = ceil_div(p.inner, int64_t{p.across} * kWave * vec) * (a.nout / p.inner);
+        cut(p, ceil_div(4 * 256, tiles), 32);
         return HMR_OK;
     }
     // Any layout.
@@ -138,13 +148,15 @@ int64_t means_bytes(const ReducePlan &p, bool var) {
     return (p.args.nout * 8 + 255) / 256 * 256;
 }
 
-int64_t partial_bytes(const ReducePlan &p) { return p.splits > 1 ? p.splits * p.args.nout * kPartialBytes : 0; }
+int64_t partial_bytes(const ReducePlan &p, bool var) {
+    return p.splits > 1 ? p.splits * p.args.nout * (var ? kVarPartialBytes : kPartialBytes) : 0;
+}
 
 namespace {
 
 // Checks the workspace and returns where the partials start.
 hmr_status take_workspace(const ReducePlan &p, bool var, void *workspace, int64_t bytes, void *&partials) {
-    int64_t need = means_bytes(p, var) + partial_bytes(p);
+    int64_t need = means_bytes(p, var) + partial_bytes(p, var);
     if (need > 0 && (workspace == nullptr || bytes < need)) {
         return fail(HMR_INVALID, "a reduction's workspace is too small");
     }
@@ -168,7 +180,7 @@ hmr_status hmr_reduce_workspace(const hmr_tensor_desc *kept, const hmr_tensor_de
     return guarded([&] {
         hmr::ReducePlan p;
         if (hmr_status s = hmr::plan_reduction(nullptr, *kept, *red, p)) return s;
-        *bytes = hmr::means_bytes(p, var != 0) + hmr::partial_bytes(p);
+        *bytes = hmr::means_bytes(p, var != 0) + hmr::partial_bytes(p, var != 0);
         return HMR_OK;
     });
 }
@@ -237,6 +249,10 @@ hmr_status hmr_var(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_tens
             double *means = static_cast<double *>(workspace);
             double divisor = static_cast<double>(p.args.nred) - correction;
             divisor = divisor > 0.0 ? divisor : 0.0;
+            if (hmr::launch_var_single_pass(kept->dtype, p, partials, hmr::element0(*out), divisor, take_sqrt != 0,
+                                            stream)) {
+                return true;
+            }
             if (!hmr::launch_mean_pass(kept->dtype, p, partials, means, stream)) return false;
             return hmr::launch_deviation_pass(kept->dtype, p, partials, means, hmr::element0(*out), divisor,
                                               take_sqrt != 0, stream);

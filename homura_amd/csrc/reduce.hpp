@@ -1,4 +1,4 @@
-// Reduction machinery for gfx950 (wave64): accumulator ops, wave/block combining and three kernels.
+// Reduction machinery for gfx950 (wave64): accumulator ops, wave/block combining and the kernels.
 //
 // What is computed follows homura's CPU reductions (ref: src/backend/cpu/reduce.rs:43-225): float
 // sums/products/means accumulate in f64, integer ones wrap in i64, max/min keep the first NaN and
@@ -11,13 +11,21 @@
 //                       or one 256-lane workgroup, per output row; 128-bit loads, four in flight
 //                       per lane; lanes combine with wave shuffles, waves through LDS.
 //   reduce_cols_kernel  outputs are contiguous in memory and the reduced dimension strides over
-//                       them ("dim=0"): a lane owns V adjacent columns (one 128-bit load per row),
-//                       the four waves of a workgroup take interleaved rows of a row slice and
-//                       combine through LDS; row slices are spread over blockIdx.y.
+//                       them ("dim=0"): a lane owns V adjacent columns (one 128-bit load per row)
+//                       and the workgroup spans up to 256 lanes * V contiguous columns, so each
+//                       row is read in spans of up to 4 KB; row slices are spread over blockIdx.y.
+//                       Narrow outputs use fewer waves across and let the others take interleaved
+//                       rows, combined through LDS.
+//   var_rows_kernel     variance of contiguous rows that fit in registers: the row is read once
+//                       and both CPU passes (mean, squared deviations) run on the registers.
 //   reduce_any_kernel   any other layout: G lanes per output walk the reduced index space with
 //                       div/mod; scalar loads.
 // When the reduced range is cut into slices (few outputs, long ranges), each slice leaves a
-// partial accumulator in the workspace and combine_kernel folds them in slice order.
+// partial accumulator in the workspace and a combine kernel folds them in slice order.
+//
+// An op has two faces. Inside a lane elements arrive in increasing position, one at a time, and
+// are folded into a cheap `Lane` state (lane_add). Lane states become `Acc` values (lane_done)
+// that `combine` folds across lanes, waves and slices in a fixed order.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -77,70 +85,88 @@ __device__ __forceinline__ typename Op::Acc wave_fold(const Op &op, typename Op:
 }
 
 // ---- accumulator ops --------------------------------------------------------------------------------
-// Acc lift(T x, int64 index, Ctx) turns the element at reduced position `index` into an
-// accumulator; combine(a, b) folds two (a's elements come from lower lanes/slices).
 
 struct NoCtx {};
 
-template <class T, bool PROD>
-struct FloatFold {
+// Ops whose lane state is the accumulator itself: lane_add(acc, x) = combine(acc, lift(x)).
+template <class Derived, class T, class A>
+struct SimpleFold {
     using In = T;
-    using Acc = double;
+    using Acc = A;
+    using Lane = A;
     using Ctx = NoCtx;
     __device__ __forceinline__ Ctx context(int64_t) const { return {}; }
-    __device__ __forceinline__ Acc init() const { return PROD ? 1.0 : 0.0; }
-    __device__ __forceinline__ Acc lift(T x, int64_t, Ctx) const { return Conv<T>::to_f64(x); }
-    __device__ __forceinline__ Acc combine(Acc a, Acc b) const { return PROD ? a * b : a + b; }
+    __device__ __forceinline__ Lane lane_init() const { return static_cast<const Derived *>(this)->init(); }
+    __device__ __forceinline__ void lane_add(Lane &l, T x, int64_t, Ctx) const {
+        const Derived *d = static_cast<const Derived *>(this);
+        l = d->combine(l, d->lift(x));
+    }
+    __device__ __forceinline__ Acc lane_done(const Lane &l) const { return l; }
 };
 
 template <class T, bool PROD>
-struct IntFold {
-    using In = T;
-    using Acc = int64_t;
-    using Ctx = NoCtx;
-    __device__ __forceinline__ Ctx context(int64_t) const { return {}; }
-    __device__ __forceinline__ Acc init() const { return PROD ? 1 : 0; }
-    __device__ __forceinline__ Acc lift(T x, int64_t, Ctx) const { return Conv<T>::to_i64(x); }
-    __device__ __forceinline__ Acc combine(Acc a, Acc b) const {
+struct FloatFold : SimpleFold<FloatFold<T, PROD>, T, double> {
+    __device__ __forceinline__ double init() const { return PROD ? 1.0 : 0.0; }
+    __device__ __forceinline__ double lift(T x) const { return Conv<T>::to_f64(x); }
+    __device__ __forceinline__ double combine(double a, double b) const { return PROD ? a * b : a + b; }
+};
+
+template <class T, bool PROD>
+struct IntFold : SimpleFold<IntFold<T, PROD>, T, int64_t> {
+    __device__ __forceinline__ int64_t init() const { return PROD ? 1 : 0; }
+    __device__ __forceinline__ int64_t lift(T x) const { return Conv<T>::to_i64(x); }
+    __device__ __forceinline__ int64_t combine(int64_t a, int64_t b) const {
         uint64_t x = static_cast<uint64_t>(a), y = static_cast<uint64_t>(b);
         return static_cast<int64_t>(PROD ? x * y : x + y);
     }
 };
 
 template <class T, bool ALL>
-struct TruthFold {
-    using In = T;
-    using Acc = uint32_t;
-    using Ctx = NoCtx;
-    __device__ __forceinline__ Ctx context(int64_t) const { return {}; }
-    __device__ __forceinline__ Acc init() const { return ALL ? 1u : 0u; }
-    __device__ __forceinline__ Acc lift(T x, int64_t, Ctx) const { return Conv<T>::to_bool(x) ? 1u : 0u; }
-    __device__ __forceinline__ Acc combine(Acc a, Acc b) const { return ALL ? (a & b) : (a | b); }
+struct TruthFold : SimpleFold<TruthFold<T, ALL>, T, uint32_t> {
+    __device__ __forceinline__ uint32_t init() const { return ALL ? 1u : 0u; }
+    __device__ __forceinline__ uint32_t lift(T x) const { return Conv<T>::to_bool(x) ? 1u : 0u; }
+    __device__ __forceinline__ uint32_t combine(uint32_t a, uint32_t b) const { return ALL ? (a & b) : (a | b); }
 };
 
-// The best element so far and its position in the reduced range (-1: none yet). The rule of
-// ref: src/backend/cpu/reduce.rs:75-86 for a sequential scan - the first NaN wins and sticks,
-// otherwise a strictly better value replaces - is the same as: NaN beats non-NaN, better value
-// beats worse, and among equals (or among NaNs) the lower position wins. That form is
-// associative and commutative, so lanes may combine in any order.
+// The best element so far and its position in the reduced range (-1: none yet).
 template <class T>
 struct Best {
     T v;
     int64_t i;
 };
 
+// ref: src/backend/cpu/reduce.rs:75-86. Inside a lane positions only grow, so the CPU's scan rule
+// applies as it stands: a NaN already held sticks; otherwise a NaN, or a strictly better value,
+// replaces. Across lanes the same outcome is: NaN beats non-NaN, better beats worse, and among
+// equals (or among NaNs) the lower position wins - associative and commutative.
 template <class T, bool MAX>
 struct ExtremeFold {
     using In = T;
     using Acc = Best<T>;
+    using Lane = Best<T>;
     using Ctx = NoCtx;
+    template <class U>
+    static __device__ __forceinline__ auto key(U x) {
+        if constexpr (std::is_same_v<U, f16_t>) return f16_widen(x);
+        else if constexpr (std::is_same_v<U, bf16_t>) return bf16_up(x);
+        else if constexpr (std::is_same_v<U, bool_t>) return static_cast<int>(x.v);
+        else return x;
+    }
     __device__ __forceinline__ Ctx context(int64_t) const { return {}; }
     __device__ __forceinline__ Acc init() const { return Acc{T{}, -1}; }
-    __device__ __forceinline__ Acc lift(T x, int64_t index, Ctx) const { return Acc{x, index}; }
+    __device__ __forceinline__ Lane lane_init() const { return Lane{T{}, -1}; }
+    __device__ __forceinline__ void lane_add(Lane &l, T x, int64_t index, Ctx) const {
+        auto a = key(l.v), b = key(x);
+        bool better = MAX ? (b > a) : (b < a);
+        bool take = l.i < 0 || (a == a && (better || b != b));
+        l.v = take ? x : l.v;
+        l.i = take ? index : l.i;
+    }
+    __device__ __forceinline__ Acc lane_done(const Lane &l) const { return l; }
     __device__ __forceinline__ Acc combine(Acc a, Acc b) const {
         if (b.i < 0) return a;
         if (a.i < 0) return b;
-        auto x = cmp_key(a.v), y = cmp_key(b.v);
+        auto x = key(a.v), y = key(b.v);
         bool xn = x != x, yn = y != y;
         bool a_wins;
         if (xn || yn) a_wins = (xn && yn) ? (a.i < b.i) : xn;
@@ -148,34 +174,71 @@ struct ExtremeFold {
         else a_wins = MAX ? (x > y) : (x < y);
         return a_wins ? a : b;
     }
-    template <class U>
-    static __device__ __forceinline__ auto cmp_key(U x) {
-        if constexpr (std::is_same_v<U, f16_t>) return f16_widen(x);
-        else if constexpr (std::is_same_v<U, bf16_t>) return bf16_up(x);
-        else if constexpr (std::is_same_v<U, bool_t>) return static_cast<int>(x.v);
-        else return x;
-    }
 };
 
-// Second pass of the variance: sum of squared deviations from the output's f64 mean.
+// Second pass of the two-pass variance: sum of squared deviations from the output's f64 mean.
 template <class T>
 struct DeviationFold {
     using In = T;
     using Acc = double;
+    using Lane = double;
     using Ctx = double;
     const double *means;
     __device__ __forceinline__ Ctx context(int64_t o) const { return means[o]; }
     __device__ __forceinline__ Acc init() const { return 0.0; }
-    __device__ __forceinline__ Acc lift(T x, int64_t, Ctx mean) const {
+    __device__ __forceinline__ Lane lane_init() const { return 0.0; }
+    __device__ __forceinline__ void lane_add(Lane &l, T x, int64_t, Ctx mean) const {
         double d = Conv<T>::to_f64(x) - mean;
-        return d * d;
+        l += d * d;
     }
+    __device__ __forceinline__ Acc lane_done(const Lane &l) const { return l; }
     __device__ __forceinline__ Acc combine(Acc a, Acc b) const { return a + b; }
+};
+
+// One-pass variance for layouts where a second pass would read the source from memory again
+// (column reductions). A lane keeps sums of (x - K) and (x - K)^2 about its first element K, which
+// is as stable as the two-pass form unless K lies many standard deviations from the mean; lanes,
+// waves and slices then merge (count, mean, M2) triples with Chan's update, all in f64. The
+// result differs from the CPU's two-pass f64 value by rounding only (a few f64 ulps), far below
+// one ulp of any output dtype.
+struct Moments {
+    double n, mean, m2;
+};
+
+template <class T>
+struct MomentsFold {
+    using In = T;
+    using Acc = Moments;
+    struct Lane {
+        double k, s1, s2, n;
+    };
+    using Ctx = NoCtx;
+    __device__ __forceinline__ Ctx context(int64_t) const { return {}; }
+    __device__ __forceinline__ Acc init() const { return Acc{0.0, 0.0, 0.0}; }
+    __device__ __forceinline__ Lane lane_init() const { return Lane{0.0, 0.0, 0.0, 0.0}; }
+    __device__ __forceinline__ void lane_add(Lane &l, T x, int64_t, Ctx) const {
+        double v = Conv<T>::to_f64(x);
+        l.k = l.n == 0.0 ? v : l.k;
+        double d = v - l.k;
+        l.s1 += d;
+        l.s2 += d * d;
+        l.n += 1.0;
+    }
+    __device__ __forceinline__ Acc lane_done(const Lane &l) const {
+        if (l.n == 0.0) return Acc{0.0, 0.0, 0.0};
+        return Acc{l.n, l.k + l.s1 / l.n, l.s2 - l.s1 * l.s1 / l.n};
+    }
+    __device__ __forceinline__ Acc combine(Acc a, Acc b) const {
+        if (b.n == 0.0) return a;
+        if (a.n == 0.0) return b;
+        double n = a.n + b.n;
+        double delta = b.mean - a.mean;
+        return Acc{n, a.mean + delta * (b.n / n), a.m2 + b.m2 + delta * delta * (a.n * b.n / n)};
+    }
 };
 
 // ---- sinks: what happens to a finished accumulator ------------------------------------------------
 
-// Rounds a float fold to the dtype (dividing by the count first for a mean).
 template <class T, bool MEAN>
 struct RoundSink {
     T *out;
@@ -204,7 +267,6 @@ struct ExtremeSink {
     }
 };
 
-// The f64 mean of each output, kept for the deviation pass.
 struct MeanSink {
     double *means;
     __device__ __forceinline__ void put(int64_t o, double a, int64_t count) const {
@@ -212,18 +274,20 @@ struct MeanSink {
     }
 };
 
+// ref: src/backend/cpu/reduce.rs:160-166: NaN for an empty reduction, else sq / max(0, n - correction).
 template <class T>
 struct VarSink {
     T *out;
     double divisor;
     bool take_sqrt;
-    __device__ __forceinline__ void put(int64_t o, double sq, int64_t count) const {
+    __device__ __forceinline__ void finish(int64_t o, double sq, int64_t count) const {
         double v = count == 0 ? __builtin_nan("") : sq / divisor;
         out[o] = Conv<T>::from_f64(take_sqrt ? sqrt(v) : v);
     }
+    __device__ __forceinline__ void put(int64_t o, double sq, int64_t count) const { finish(o, sq, count); }
+    __device__ __forceinline__ void put(int64_t o, Moments m, int64_t count) const { finish(o, m.m2, count); }
 };
 
-// Writes slice `split` of output o into the workspace instead of finishing it.
 template <class Acc>
 __device__ __forceinline__ void put_partial(void *partials, int64_t nout, int64_t split, int64_t o, Acc a) {
     static_cast<Acc *>(partials)[split * nout + o] = a;
@@ -240,7 +304,14 @@ struct ReduceArgs {
     int64_t splits;   // slices of the reduced range
     int64_t chunk;    // reduced elements per slice
     void *partials;   // workspace for splits > 1
+    uint32_t stream;  // nonzero: nontemporal loads (a source much larger than the caches, read once)
 };
+
+template <class T, int V>
+__device__ __forceinline__ void load_tile_rt(const char *p, T (&r)[V], bool nt) {
+    (void)nt;  // a run-time choice would be merged into one plain load; the hint is compile-time
+    load_tile<T, V, kStreamLoads>(p, r);
+}
 
 // ---- kernels -----------------------------------------------------------------------------------------
 
@@ -259,12 +330,13 @@ __global__ void __launch_bounds__(kBlock) reduce_any_kernel(ReduceArgs a, Op op,
     for (int64_t g = blockIdx.x; g < groups; g += gridDim.x) {
         const int64_t o = g * kPerBlock + threadIdx.x / G;
         const bool live = o < a.nout;
-        Acc acc = op.init();
+        typename Op::Lane state = op.lane_init();
         if (live) {
             const typename Op::Ctx ctx = op.context(o);
             const T *p = reinterpret_cast<const T *>(a.src) + a.kept.offset(o);
-            for (int64_t r = begin + lane; r < end; r += G) acc = op.combine(acc, op.lift(p[a.red.offset(r)], r, ctx));
+            for (int64_t r = begin + lane; r < end; r += G) op.lane_add(state, p[a.red.offset(r)], r, ctx);
         }
+        Acc acc = op.lane_done(state);
         if constexpr (G >= kWave) acc = wave_fold(op, acc);
         if constexpr (G == kBlock) {
             __syncthreads();  // lds reuse across iterations
@@ -281,15 +353,39 @@ __global__ void __launch_bounds__(kBlock) reduce_any_kernel(ReduceArgs a, Op op,
     }
 }
 
+// Folds the slices of each output in slice order. 64 adjacent outputs per workgroup; its four
+// waves take interleaved slices (coalesced 64-output reads, eight in flight) and meet in LDS.
 template <class Op, class Sink>
 __global__ void __launch_bounds__(kBlock) combine_kernel(ReduceArgs a, Op op, Sink sink) {
     using Acc = typename Op::Acc;
+    constexpr int kWaves = kBlock / kWave;
+    constexpr int U = 8;
+    __shared__ Acc lds[kWaves - 1][kWave];
     const Acc *partials = static_cast<const Acc *>(a.partials);
-    for (int64_t o = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; o < a.nout;
-         o += static_cast<int64_t>(gridDim.x) * kBlock) {
-        Acc acc = partials[o];
-        for (int64_t s = 1; s < a.splits; ++s) acc = op.combine(acc, partials[s * a.nout + o]);
-        sink.put(o, acc, a.nred);
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const int64_t groups = (a.nout + kWave - 1) / kWave;
+    for (int64_t g = blockIdx.x; g < groups; g += gridDim.x) {
+        const int64_t o = g * kWave + lane;
+        Acc acc = op.init();
+        if (o < a.nout) {
+            int64_t s = wave;
+            for (; s + (U - 1) * kWaves < a.splits; s += U * kWaves) {
+                Acc t[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) t[u] = partials[(s + u * kWaves) * a.nout + o];
+#pragma unroll
+                for (int u = 0; u < U; ++u) acc = op.combine(acc, t[u]);
+            }
+            for (; s < a.splits; s += kWaves) acc = op.combine(acc, partials[s * a.nout + o]);
+        }
+        __syncthreads();
+        if (wave > 0) lds[wave - 1][lane] = acc;
+        __syncthreads();
+        if (wave == 0 && o < a.nout) {
+#pragma unroll
+            for (int w = 0; w < kWaves - 1; ++w) acc = op.combine(acc, lds[w][lane]);
+            sink.put(o, acc, a.nred);
+        }
     }
 }
 
@@ -311,18 +407,19 @@ __global__ void __launch_bounds__(kBlock) combine_wave_kernel(ReduceArgs a, Op o
     }
 }
 
-// Contiguous rows. WAVES = 1: a wave per row, four rows per workgroup. WAVES = 4: a workgroup per
-// row (or per row slice when splits > 1). VEC: rows start 16-byte aligned, so 128-bit loads.
-template <class Op, class Sink, int WAVES, bool VEC>
+// Contiguous rows, each starting 16-byte aligned. WAVES = 1: a wave per row, four rows per
+// workgroup. WAVES = 4: a workgroup per row (or per row slice when splits > 1).
+template <class Op, class Sink, int WAVES>
 __global__ void __launch_bounds__(kBlock) reduce_rows_kernel(ReduceArgs a, Op op, Sink sink) {
     using T = typename Op::In;
     using Acc = typename Op::Acc;
-    constexpr int V = VEC ? 16 / static_cast<int>(sizeof(T)) : 1;
+    constexpr int V = 16 / static_cast<int>(sizeof(T));
     constexpr int G = WAVES * kWave;
     constexpr int kPerBlock = kBlock / G;
     constexpr int U = 4;  // loads in flight per lane
     __shared__ Acc lds[WAVES == 4 ? 4 : 1];
     const int lane = threadIdx.x % G;
+    const bool nt = a.stream != 0;
     const int64_t split = blockIdx.y;
     const int64_t begin = split * a.chunk;
     const int64_t end = begin + a.chunk < a.nred ? begin + a.chunk : a.nred;
@@ -330,7 +427,7 @@ __global__ void __launch_bounds__(kBlock) reduce_rows_kernel(ReduceArgs a, Op op
     for (int64_t g = blockIdx.x; g < groups; g += gridDim.x) {
         const int64_t o = g * kPerBlock + threadIdx.x / G;
         const bool live = o < a.nout;
-        Acc acc = op.init();
+        typename Op::Lane state = op.lane_init();
         if (live) {
             const typename Op::Ctx ctx = op.context(o);
             const T *p = reinterpret_cast<const T *>(a.src) + a.kept.offset(o);
@@ -341,26 +438,24 @@ __global__ void __launch_bounds__(kBlock) reduce_rows_kernel(ReduceArgs a, Op op
                 T r[U][V];
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
-                    load_tile<T, V>(reinterpret_cast<const char *>(p + begin + (k + u * G) * V), r[u]);
+                    load_tile_rt<T, V>(reinterpret_cast<const char *>(p + begin + (k + u * G) * V), r[u], nt);
                 }
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
 #pragma unroll
-                    for (int i = 0; i < V; ++i) {
-                        acc = op.combine(acc, op.lift(r[u][i], begin + (k + u * G) * V + i, ctx));
-                    }
+                    for (int i = 0; i < V; ++i) op.lane_add(state, r[u][i], begin + (k + u * G) * V + i, ctx);
                 }
             }
             for (; k < nvec; k += G) {
                 T r[V];
-                load_tile<T, V>(reinterpret_cast<const char *>(p + begin + k * V), r);
+                load_tile_rt<T, V>(reinterpret_cast<const char *>(p + begin + k * V), r, nt);
 #pragma unroll
-                for (int i = 0; i < V; ++i) acc = op.combine(acc, op.lift(r[i], begin + k * V + i, ctx));
+                for (int i = 0; i < V; ++i) op.lane_add(state, r[i], begin + k * V + i, ctx);
             }
             // Ragged end of the range (fewer than V elements).
-            for (int64_t r = begin + nvec * V + lane; r < end; r += G) acc = op.combine(acc, op.lift(p[r], r, ctx));
+            for (int64_t r = begin + nvec * V + lane; r < end; r += G) op.lane_add(state, p[r], r, ctx);
         }
-        acc = wave_fold(op, acc);
+        Acc acc = wave_fold(op, op.lane_done(state));
         if constexpr (WAVES == 4) {
             __syncthreads();
             if (threadIdx.x % kWave == 0) lds[threadIdx.x / kWave] = acc;
@@ -378,82 +473,163 @@ __global__ void __launch_bounds__(kBlock) reduce_rows_kernel(ReduceArgs a, Op op
 
 // Contiguous outputs ("columns"), one strided reduced dimension. `rstride` is that stride and
 // `inner` the length of the contiguous run of outputs (the innermost kept dimension); a.kept
-// holds the remaining, outer kept dimensions. VEC: every row of every column tile starts 16-byte
-// aligned.
-template <class Op, class Sink, bool VEC>
+// holds the remaining, outer kept dimensions. Every row of every tile starts 16-byte aligned.
+// `across` (1, 2 or 4) waves of the workgroup sit side by side on a span of across*64*V columns;
+// the other 4/across wave groups take interleaved rows of the slice.
+template <class Op, class Sink>
 __global__ void __launch_bounds__(kBlock)
-    reduce_cols_kernel(ReduceArgs a, int64_t rstride, int64_t inner, Op op, Sink sink) {
+    reduce_cols_kernel(ReduceArgs a, int64_t rstride, int64_t inner, int across, Op op, Sink sink) {
     using T = typename Op::In;
     using Acc = typename Op::Acc;
-    constexpr int V = VEC ? 16 / static_cast<int>(sizeof(T)) : 1;
+    constexpr int V = 16 / static_cast<int>(sizeof(T));
     constexpr int kWaves = kBlock / kWave;
     constexpr int U = 4;
     __shared__ Acc lds[kWaves - 1][kWave * V];
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const int cgroup = wave % across, rgroup = wave / across, rgroups = kWaves / across;
+    const bool nt = a.stream != 0;
     const int64_t split = blockIdx.y;
     const int64_t begin = split * a.chunk;
     const int64_t end = begin + a.chunk < a.nred ? begin + a.chunk : a.nred;
-    const int64_t tiles_inner = (inner + kWave * V - 1) / (kWave * V);
+    const int64_t span = static_cast<int64_t>(across) * kWave * V;
+    const int64_t tiles_inner = (inner + span - 1) / span;
     const int64_t tiles = tiles_inner * (a.nout / inner);
     for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
         const int64_t outer = tile / tiles_inner;
-        const int64_t col = (tile - outer * tiles_inner) * (kWave * V) + lane * V;  // within the run
-        const int64_t obase = outer * inner;                                       // first output of the run
+        const int64_t col = (tile - outer * tiles_inner) * span + (cgroup * kWave + lane) * V;  // within the run
+        const int64_t obase = outer * inner;                                                    // first output of the run
         const T *src = reinterpret_cast<const T *>(a.src) + a.kept.offset(outer);
         const int valid = inner - col >= V ? V : (inner > col ? static_cast<int>(inner - col) : 0);
-        Acc acc[V];
+        typename Op::Lane state[V];
         typename Op::Ctx ctx[V];
 #pragma unroll
         for (int i = 0; i < V; ++i) {
-            acc[i] = op.init();
+            state[i] = op.lane_init();
             ctx[i] = op.context(i < valid ? obase + col + i : 0);
         }
         if (valid == V) {
-            int64_t r = begin + wave;
-            for (; r + (U - 1) * kWaves < end; r += U * kWaves) {
+            int64_t r = begin + rgroup;
+            for (; r + (U - 1) * rgroups < end; r += U * rgroups) {
                 T t[U][V];
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
-                    load_tile<T, V>(reinterpret_cast<const char *>(src + (r + u * kWaves) * rstride + col), t[u]);
+                    load_tile_rt<T, V>(reinterpret_cast<const char *>(src + (r + u * rgroups) * rstride + col), t[u], nt);
                 }
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
 #pragma unroll
-                    for (int i = 0; i < V; ++i) acc[i] = op.combine(acc[i], op.lift(t[u][i], r + u * kWaves, ctx[i]));
+                    for (int i = 0; i < V; ++i) op.lane_add(state[i], t[u][i], r + u * rgroups, ctx[i]);
                 }
             }
-            for (; r < end; r += kWaves) {
+            for (; r < end; r += rgroups) {
                 T t[V];
-                load_tile<T, V>(reinterpret_cast<const char *>(src + r * rstride + col), t);
+                load_tile_rt<T, V>(reinterpret_cast<const char *>(src + r * rstride + col), t, nt);
 #pragma unroll
-                for (int i = 0; i < V; ++i) acc[i] = op.combine(acc[i], op.lift(t[i], r, ctx[i]));
+                for (int i = 0; i < V; ++i) op.lane_add(state[i], t[i], r, ctx[i]);
             }
         } else if (valid > 0) {
-            for (int64_t r = begin + wave; r < end; r += kWaves) {
+            for (int64_t r = begin + rgroup; r < end; r += rgroups) {
 #pragma unroll
                 for (int i = 0; i < V; ++i) {
-                    if (i < valid) acc[i] = op.combine(acc[i], op.lift(src[r * rstride + col + i], r, ctx[i]));
+                    if (i < valid) op.lane_add(state[i], src[r * rstride + col + i], r, ctx[i]);
                 }
             }
         }
-        // Waves 1..3 hand their accumulators to wave 0, which folds them in wave order.
-        __syncthreads();
-        if (wave > 0) {
+        Acc acc[V];
 #pragma unroll
-            for (int i = 0; i < V; ++i) lds[wave - 1][lane * V + i] = acc[i];
+        for (int i = 0; i < V; ++i) acc[i] = op.lane_done(state[i]);
+        if (rgroups > 1) {
+            // Row groups 1.. hand their accumulators to row group 0, which folds them in order.
+            __syncthreads();
+            if (rgroup > 0) {
+#pragma unroll
+                for (int i = 0; i < V; ++i) lds[wave - across][lane * V + i] = acc[i];
+            }
+            __syncthreads();
+            if (rgroup == 0) {
+                for (int g = 1; g < rgroups; ++g) {
+#pragma unroll
+                    for (int i = 0; i < V; ++i) acc[i] = op.combine(acc[i], lds[g * across + cgroup - across][lane * V + i]);
+                }
+            }
         }
-        __syncthreads();
-        if (wave == 0) {
+        if (rgroup == 0) {
 #pragma unroll
             for (int i = 0; i < V; ++i) {
-#pragma unroll
-                for (int w = 0; w < kWaves - 1; ++w) acc[i] = op.combine(acc[i], lds[w][lane * V + i]);
                 if (i < valid) {
                     if (a.splits > 1) put_partial(a.partials, a.nout, split, obase + col + i, acc[i]);
                     else sink.put(obase + col + i, acc[i], a.nred);
                 }
             }
         }
+    }
+}
+
+// Variance of contiguous, 16-byte aligned rows of at most G*C*V elements: the row is read once
+// into registers, then the CPU's two passes run on them (ref: src/backend/cpu/reduce.rs:150-166):
+// mean = sum / n in f64, then the sum of squared deviations from that mean.
+template <class T, int WAVES, int C>
+__global__ void __launch_bounds__(kBlock) var_rows_kernel(ReduceArgs a, VarSink<T> sink) {
+    constexpr int V = 16 / static_cast<int>(sizeof(T));
+    constexpr int G = WAVES * kWave;
+    constexpr int kPerBlock = kBlock / G;
+    __shared__ double lds[WAVES == 4 ? 4 : 1];
+    const int lane = threadIdx.x % G;
+    const bool nt = a.stream != 0;
+    const FloatFold<T, false> add{};
+    const int64_t groups = (a.nout + kPerBlock - 1) / kPerBlock;
+    const int64_t nvec = a.nred / V;
+    auto fold = [&](double v) {
+        v = wave_fold(add, v);
+        if constexpr (WAVES == 4) {
+            __syncthreads();
+            if (threadIdx.x % kWave == 0) lds[threadIdx.x / kWave] = v;
+            __syncthreads();
+            v = lds[0];
+#pragma unroll
+            for (int w = 1; w < 4; ++w) v += lds[w];
+        }
+        return v;
+    };
+    for (int64_t g = blockIdx.x; g < groups; g += gridDim.x) {
+        const int64_t o = g * kPerBlock + threadIdx.x / G;
+        const bool live = o < a.nout;
+        const T *p = reinterpret_cast<const T *>(a.src) + (live ? a.kept.offset(o) : 0);
+        T x[C][V];
+        bool have[C][V];
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const int64_t tile = static_cast<int64_t>(c) * G + lane;
+            if (live && tile < nvec) {
+                load_tile_rt<T, V>(reinterpret_cast<const char *>(p + tile * V), x[c], nt);
+#pragma unroll
+                for (int i = 0; i < V; ++i) have[c][i] = true;
+            } else {
+#pragma unroll
+                for (int i = 0; i < V; ++i) {
+                    have[c][i] = live && tile * V + i < a.nred;
+                    x[c][i] = have[c][i] ? p[tile * V + i] : T{};
+                }
+            }
+        }
+        double sum = 0.0;
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+#pragma unroll
+            for (int i = 0; i < V; ++i) sum += have[c][i] ? Conv<T>::to_f64(x[c][i]) : 0.0;
+        }
+        const double mean = fold(sum) / static_cast<double>(a.nred);
+        double sq = 0.0;
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+#pragma unroll
+            for (int i = 0; i < V; ++i) {
+                double d = Conv<T>::to_f64(x[c][i]) - mean;
+                sq += have[c][i] ? d * d : 0.0;
+            }
+        }
+        sq = fold(sq);
+        if (live && lane == 0) sink.finish(o, sq, a.nred);
     }
 }
 

@@ -18,6 +18,53 @@ bool launch_float_reduce(int op, int dtype, const ReducePlan &plan, void *partia
     });
 }
 
+// Rows plan, one slice, and a row that fits G lanes x 16 tiles of 16 bytes: registers.
+static int var_row_tiles(const ReducePlan &plan, int elem) {
+    if (plan.kind != ReduceKind::Rows || plan.splits != 1) return 0;
+    const int64_t vec = 16 / elem;
+    const int64_t per = (plan.args.nred + vec * plan.group - 1) / (vec * plan.group);
+    return per <= 4 ? 4 : (per <= 8 ? 8 : (per <= 16 ? 16 : 0));
+}
+
+bool var_is_single_pass(const ReducePlan &plan) {
+    return plan.kind == ReduceKind::Cols || (plan.kind == ReduceKind::Rows && plan.splits == 1);
+}
+
+bool launch_var_single_pass(int dtype, const ReducePlan &plan, void *partials, void *out, double divisor,
+                            bool take_sqrt, hipStream_t stream) {
+    if (plan.args.nred == 0) return false;
+    bool done = false;
+    with_float_type(dtype, [&](auto t) {
+        using T = typename decltype(t)::type;
+        VarSink<T> sink{static_cast<T *>(out), divisor, take_sqrt};
+        if (plan.kind == ReduceKind::Cols) {
+            launch_reduce(plan, partials, MomentsFold<T>{}, sink, stream);
+            done = true;
+            return;
+        }
+        const int tiles = var_row_tiles(plan, static_cast<int>(sizeof(T)));
+        if (tiles == 0) return;
+        ReduceArgs a = plan.args;
+        a.splits = 1;
+        a.chunk = a.nred;
+        const int64_t cap = 1 << 20;
+        auto run = [&](auto w, auto c) {
+            constexpr int W = decltype(w)::value, C = decltype(c)::value;
+            dim3 grid(capped((a.nout + (4 / W) - 1) / (4 / W), cap));
+            hipLaunchKernelGGL((var_rows_kernel<T, W, C>), grid, dim3(kBlock), 0, stream, a, sink);
+        };
+        auto with_tiles = [&](auto w) {
+            if (tiles == 4) run(w, IntTag<4>{});
+            else if (tiles == 8) run(w, IntTag<8>{});
+            else run(w, IntTag<16>{});
+        };
+        if (plan.group == kWave) with_tiles(IntTag<1>{});
+        else with_tiles(IntTag<4>{});
+        done = true;
+    });
+    return done;
+}
+
 bool launch_mean_pass(int dtype, const ReducePlan &plan, void *partials, double *means, hipStream_t stream) {
     return with_float_type(dtype, [&](auto t) {
         using T = typename decltype(t)::type;

@@ -16,12 +16,16 @@ struct ReducePlan {
     int64_t chunk = 0;    // reduced elements per slice
     int64_t rstride = 0;  // Cols: stride of the reduced dimension
     int64_t inner = 0;    // Cols: length of the contiguous run of outputs
+    int across = 4;       // Cols: waves side by side on a column span (1, 2 or 4)
     ReduceArgs args{};    // src, walks, counts (partials filled in at launch)
 };
 
-// Bytes one partial accumulator occupies in the workspace, whatever the op (the largest is a
-// value + position pair).
+// Bytes one partial accumulator occupies in the workspace, whatever the op: a value + position
+// pair at most, or for hmr_var a (count, mean, M2) triple.
 constexpr int64_t kPartialBytes = 16;
+constexpr int64_t kVarPartialBytes = 32;
+// A source at least this large is read with nontemporal loads (see load_tile in map.hpp).
+constexpr int64_t kStreamSourceBytes = int64_t{32} << 20;
 // Machine width the plans aim at: lanes of a full MI355X at 4 waves per SIMD.
 constexpr int64_t kTargetLanes = 256 * 4 * 4 * 64;
 
@@ -32,7 +36,7 @@ hmr_status plan_reduction(const hmr_tensor_desc *out, const hmr_tensor_desc &kep
 
 // Workspace: [f64 means for hmr_var when nout > 0][partials when splits > 1].
 int64_t means_bytes(const ReducePlan &p, bool var);
-int64_t partial_bytes(const ReducePlan &p);
+int64_t partial_bytes(const ReducePlan &p, bool var);
 
 inline unsigned capped(int64_t blocks, int64_t cap) {
     if (blocks < 1) blocks = 1;
@@ -43,7 +47,7 @@ inline unsigned capped(int64_t blocks, int64_t cap) {
 template <class Op, class Sink>
 void launch_reduce(const ReducePlan &plan, void *partials, Op op, Sink sink, hipStream_t stream) {
     using Acc = typename Op::Acc;
-    static_assert(sizeof(Acc) <= kPartialBytes, "partial slot too small");
+    static_assert(sizeof(Acc) <= (std::is_same_v<Acc, Moments> ? kVarPartialBytes : kPartialBytes), "partial slot too small");
     ReduceArgs a = plan.args;
     a.splits = plan.splits;
     a.chunk = plan.chunk;
@@ -54,19 +58,20 @@ void launch_reduce(const ReducePlan &plan, void *partials, Op op, Sink sink, hip
         case ReduceKind::Rows: {
             if (plan.group == kWave) {
                 dim3 grid(capped((a.nout + 3) / 4, cap), ysplits);
-                hipLaunchKernelGGL((reduce_rows_kernel<Op, Sink, 1, true>), grid, dim3(kBlock), 0, stream, a, op, sink);
+                hipLaunchKernelGGL((reduce_rows_kernel<Op, Sink, 1>), grid, dim3(kBlock), 0, stream, a, op, sink);
             } else {
                 dim3 grid(capped(a.nout, cap), ysplits);
-                hipLaunchKernelGGL((reduce_rows_kernel<Op, Sink, 4, true>), grid, dim3(kBlock), 0, stream, a, op, sink);
+                hipLaunchKernelGGL((reduce_rows_kernel<Op, Sink, 4>), grid, dim3(kBlock), 0, stream, a, op, sink);
             }
             break;
         }
         case ReduceKind::Cols: {
             constexpr int V = 16 / static_cast<int>(sizeof(typename Op::In));
-            int64_t tiles = (plan.inner + kWave * V - 1) / (kWave * V) * (a.nout / plan.inner);
+            int64_t span = int64_t{plan.across} * kWave * V;
+            int64_t tiles = (plan.inner + span - 1) / span * (a.nout / plan.inner);
             dim3 grid(capped(tiles, cap), ysplits);
-            hipLaunchKernelGGL((reduce_cols_kernel<Op, Sink, true>), grid, dim3(kBlock), 0, stream, a, plan.rstride,
-                               plan.inner, op, sink);
+            hipLaunchKernelGGL((reduce_cols_kernel<Op, Sink>), grid, dim3(kBlock), 0, stream, a, plan.rstride,
+                               plan.inner, plan.across, op, sink);
             break;
         }
         case ReduceKind::Any: {
@@ -89,7 +94,7 @@ void launch_reduce(const ReducePlan &plan, void *partials, Op op, Sink sink, hip
             hipLaunchKernelGGL((combine_wave_kernel<Op, Sink>), dim3(capped((a.nout + 3) / 4, cap)), dim3(kBlock), 0,
                                stream, a, op, sink);
         } else {
-            hipLaunchKernelGGL((combine_kernel<Op, Sink>), dim3(capped((a.nout + kBlock - 1) / kBlock, cap)),
+            hipLaunchKernelGGL((combine_kernel<Op, Sink>), dim3(capped((a.nout + kWave - 1) / kWave, cap)),
                                dim3(kBlock), 0, stream, a, op, sink);
         }
     }
@@ -102,6 +107,11 @@ bool launch_int_reduce(int op, int dtype, const ReducePlan &plan, void *partials
 bool launch_truth_reduce(int op, int dtype, const ReducePlan &plan, void *partials, void *out, hipStream_t stream);
 bool launch_extreme_reduce(bool is_max, int dtype, const ReducePlan &plan, void *partials, void *values,
                            void *indices, hipStream_t stream);
+// Variance in one launch where the plan allows it (rows that fit in registers; columns in one
+// pass over memory); false when the two-pass form below has to run.
+bool launch_var_single_pass(int dtype, const ReducePlan &plan, void *partials, void *out, double divisor,
+                            bool take_sqrt, hipStream_t stream);
+bool var_is_single_pass(const ReducePlan &plan);
 // The two passes of the variance: means (f64) then squared deviations.
 bool launch_mean_pass(int dtype, const ReducePlan &plan, void *partials, double *means, hipStream_t stream);
 bool launch_deviation_pass(int dtype, const ReducePlan &plan, void *partials, const double *means, void *out,

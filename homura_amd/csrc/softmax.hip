@@ -180,7 +180,7 @@ __global__ void __launch_bounds__(G > kBlock ? G : kBlock) softmax_regs_kernel(S
             const int64_t tile = static_cast<int64_t>(c) * G + lane;
             T raw[V];
             if (live && tile < nvec) {
-                load_tile<T, V>(reinterpret_cast<const char *>(src + tile * V), raw);
+                load_tile<T, V, kStreamLoads>(reinterpret_cast<const char *>(src + tile * V), raw);
 #pragma unroll
                 for (int i = 0; i < V; ++i) x[c][i] = M::load(raw[i]);
             } else {
@@ -228,7 +228,7 @@ __global__ void __launch_bounds__(G > kBlock ? G : kBlock) softmax_regs_kernel(S
                 else res[i] = M::soft(ex[c][i], scale);
             }
             if (live && tile < nvec) {
-                store_tile<T, V>(reinterpret_cast<char *>(out + tile * V), res);
+                store_tile<T, V, kStreamStores>(reinterpret_cast<char *>(out + tile * V), res);
             } else if (live) {
 #pragma unroll
                 for (int i = 0; i < V; ++i) {
