@@ -31,6 +31,10 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the bf16 + f32 -> f32 add kernel at configs[1], from rocprofv3 --pmc FETCH_SIZE
+# and --pmc WRITE_SIZE (two runs), each scaled by the reading of a plain copy of known size:
+# (196 638.1 x 1.99957 + 262 144.0 x 1.0) KiB; profiles/map_rows_add_bf16_f32_configs1_chain.md.
+ADD_KERNEL_TRAFFIC_BYTES = 671064064
 METRIC = "achieved HBM GB/s & % of MI355X peak per op; speedup vs host-CPU reference"
 
 
@@ -41,6 +45,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--ops", choices=["all", "none"], default="all")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--calibrate", type=int, default=0, metavar="K",
+                    help="first run K plain f32 copies of 67 108 864 elements (268 435 456 B read, the same written): "
+                         "the known-size kernel that rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this path has no cross-GPU step (every box has one GPU); got --gpus {args.gpus}",
@@ -92,6 +99,21 @@ def main():
     def chain():
         return x.add(bias).mul(scale).add(residual)
 
+    if args.calibrate:
+        from homura_amd import capi
+
+        ctx = capi.Context(0)
+        src, dst = ctx.malloc(4 * N), ctx.malloc(4 * N)
+        capi.check(capi.lib.hmr_memset(ctx.handle, src.ptr, 0x3C, 4 * N))
+        flat = lambda buf: capi.make_desc(buf.ptr, capi.F32, [N], [1])
+        d_dst, d_src = flat(dst), flat(src)
+        for _ in range(args.calibrate):
+            capi.check(capi.lib.hmr_copy(ctx.handle, ctypes.byref(d_dst), ctypes.byref(d_src)))
+        ctx.synchronize()
+        src.free()
+        dst.free()
+        ctx.close()
+
     chain_bytes = (4 * N + 2 * H) + (4 * N + 2 * B * S) + 10 * N  # BASELINE.md section 3, promotion fused
     ms_step = timed(chain, args.steps, args.warmup)
     value = chain_bytes / (ms_step * 1e-3) / 1e9
@@ -102,7 +124,7 @@ def main():
     add_bytes = 10 * N
     achieved = add_bytes / (ms_add * 1e-3) / 1e9
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": ADD_KERNEL_TRAFFIC_BYTES,
                 "kernel": "map_rows_kernel<FloatBinary<ADD, f32, bf16, f32>> (bf16 + f32 -> f32)",
                 "algorithmic_bytes_per_launch": add_bytes, "us_per_launch": round(ms_add * 1e3, 2)}
 
