@@ -1,0 +1,111 @@
+"""The C-ABI library as a link target (no GPU, no compute calls): it loads, exports every symbol that
+include/*.h declares and every one of the 77 functions homura's Rust crate declares in
+src/backend/rocm/ffi.rs, keeps everything else local, and reports the struct layouts and enum values the
+Rust side asserts (ref: src/backend/rocm/tests.rs:10-59, csrc/homura_rocm.h:592-610)."""
+import ctypes
+import os
+import re
+import subprocess
+
+import pytest
+
+from homura_amd import capi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+INCLUDE = os.path.join(ROOT, "include")
+
+# The `extern "C"` block of src/backend/rocm/ffi.rs, names only.
+RUST_FFI = """
+    hmr_abi_check hmr_adaptive_avg_pool2d hmr_adaptive_avg_pool2d_backward hmr_addr hmr_arg_reduce hmr_binary
+    hmr_binary_constant hmr_binary_scalar hmr_built_archs hmr_context_create hmr_context_destroy
+    hmr_context_synchronize hmr_copy hmr_copy_device hmr_copy_from_host hmr_copy_to_host hmr_device_count
+    hmr_device_properties_get hmr_exclusive_cumprod hmr_fill hmr_flip hmr_free hmr_fused hmr_gather hmr_gemm
+    hmr_gemm_fold hmr_gemm_path_name hmr_gemm_select hmr_gemm_workspace hmr_index_add hmr_index_add_workspace
+    hmr_index_check hmr_index_overwrite hmr_index_overwrite_workspace hmr_index_positions hmr_index_select
+    hmr_last_error hmr_malloc hmr_mask_coordinates hmr_mask_count hmr_mask_workspace hmr_max_pool2d
+    hmr_max_pool2d_backward hmr_max_pool2d_backward_workspace hmr_max_pool2d_check
+    hmr_max_pool2d_gather_backward hmr_mem_get_info hmr_memset hmr_random_int hmr_random_normal
+    hmr_random_uniform hmr_reduce hmr_reduce_workspace hmr_scatter_add hmr_scatter_add_workspace hmr_softmax
+    hmr_softmax_workspace hmr_test_current_device hmr_test_fail hmr_test_fail_after_probe hmr_test_fail_data
+    hmr_test_fail_properties hmr_test_fail_stream_create hmr_test_force_gemm_path hmr_test_index_value
+    hmr_test_live_streams hmr_test_pool_candidates hmr_test_reduce_plan hmr_test_set_current_device
+    hmr_test_softmax_plan hmr_test_wide_pool hmr_triangle hmr_unary hmr_unfold_backward hmr_var hmr_where
+    hmr_where_constant
+""".split()
+
+
+def declared_in_headers():
+    names = set()
+    for f in sorted(os.listdir(INCLUDE)):
+        text = open(os.path.join(INCLUDE, f)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        text = re.sub(r"//[^\n]*", "", text)
+        names.update(re.findall(r"\b(hmr_[a-z0-9_]+)\s*\(", text))
+    return names
+
+
+def exported():
+    out = subprocess.check_output(["nm", "-D", "--defined-only", capi.LIB_PATH], text=True)
+    return {line.split()[-1] for line in out.splitlines() if line.strip()}
+
+
+def test_rust_ffi_list_is_complete():
+    assert len(RUST_FFI) == 77 and len(set(RUST_FFI)) == 77
+
+
+def test_every_declared_symbol_is_exported():
+    declared = declared_in_headers()
+    assert len(declared) >= 78
+    have = exported()
+    assert not (declared - have), f"declared in include/*.h but not exported: {sorted(declared - have)}"
+    assert not (set(RUST_FFI) - have), f"needed by the Rust crate but not exported: {sorted(set(RUST_FFI) - have)}"
+    assert not (set(RUST_FFI) - declared), f"not declared in include/*.h: {sorted(set(RUST_FFI) - declared)}"
+
+
+def test_only_hmr_symbols_are_global():
+    """ref: build.rs:232-250 keeps only hmr_* global in the relocatable object."""
+    stray = {s for s in exported() if not s.startswith("hmr_")}
+    assert not stray, sorted(stray)
+
+
+def test_every_symbol_binds_through_ctypes():
+    lib = ctypes.CDLL(capi.LIB_PATH)
+    for name in sorted(declared_in_headers()):
+        assert getattr(lib, name) is not None
+    assert set(capi.PROTOTYPES) | set(capi.UNBUILT) >= set(RUST_FFI)
+
+
+def test_static_archive_is_built_beside_the_shared_library():
+    archive = os.path.join(os.path.dirname(capi.LIB_PATH), "libhomura_rocm.a")
+    assert os.path.exists(archive), "the Rust build links libhomura_rocm.a (ref: build.rs:60-70)"
+    out = subprocess.check_output(["nm", "--defined-only", "-g", archive], text=True, stderr=subprocess.DEVNULL)
+    have = {line.split()[-1] for line in out.splitlines() if len(line.split()) == 3}
+    assert set(RUST_FFI) <= have
+
+
+def test_abi_layout():
+    """What the_abi_matches_the_library asserts on the Rust side (ref: src/backend/rocm/tests.rs:10-59)."""
+    info = capi.hmr_abi_info()
+    capi.lib.hmr_abi_check(ctypes.byref(info))
+    D, P = capi.hmr_tensor_desc, capi.hmr_device_properties
+    assert info.abi_info_size == ctypes.sizeof(capi.hmr_abi_info)
+    assert (info.desc_size, info.desc_align) == (ctypes.sizeof(D), ctypes.alignment(D)) == (424, 8)
+    assert list(info.desc_offsets) == [D.data.offset, D.offset.offset, D.dtype.offset, D.ndim.offset, D.sizes.offset,
+                                       D.strides.offset] == [0, 8, 16, 20, 24, 224]
+    assert (info.properties_size, info.properties_align) == (ctypes.sizeof(P), ctypes.alignment(P))
+    assert list(info.properties_offsets) == [P.name.offset, P.arch.offset, P.multiprocessor_count.offset,
+                                             P.warp_size.offset, P.total_memory.offset]
+    assert list(info.status_values) == [0, 1, 2, 3, 4]
+    assert list(info.dtype_values) == list(range(10))
+    assert info.max_dims == 25
+    assert capi.lib.hmr_built_archs().decode() == "gfx950"
+
+
+def test_out_of_scope_entry_points_fail_loudly():
+    """Kernel families outside this library return HMR_INVALID with a message; they never pretend."""
+    lib = ctypes.CDLL(capi.LIB_PATH)
+    lib.hmr_last_error.restype = ctypes.c_char_p
+    lib.hmr_gemm_path_name.restype = ctypes.c_char_p
+    rc = lib.hmr_flip(None, None, None, 0)
+    assert rc == 2
+    assert lib.hmr_last_error() == b"hmr_flip: not built in this library"

@@ -1,0 +1,380 @@
+"""Pins the CPU oracle (no GPU): every known answer homura's own tests hold for this path, plus what
+the mathematics fixes (exact rational arithmetic, brute force, an independent libm), chosen so that a
+dropped term, a wrong sign or index, or a wrong rounding step fails at least one of them.
+
+ref: src/backend/cpu/num.rs:222-246 (erf table), src/dtype.rs:611-665 (element_cast,
+     half_casts_round_through_f32), tests/tensor_api.rs:686-701 (scalars stay f32 for half products),
+     tests/m0_boundaries.rs:122-154, 380-392, 468-480 (empty reductions, NaN/ties, softmax),
+     tests/rocm_reduce.rs:526-653 (exact sums, special values, extreme softmax rows),
+     src/backend/cpu/iter.rs:112-121 (iteration order).
+"""
+import math
+from fractions import Fraction
+
+import numpy as np
+import pytest
+
+from tests import oracle
+from tests.support import DT, FLOATS, NP, array, bits, from_f64, h, tensor, to_f64
+
+h.register_cpu_backend(oracle.backend_address())
+L = oracle.lib()
+INF = float("inf")
+NAN = float("nan")
+
+
+def f64t(values, shape=None):
+    a = np.asarray(values, dtype=np.float64)
+    return tensor(a, DT.F64, list(a.shape if shape is None else shape))
+
+
+def vals(t):
+    """Elements of a tensor as exact f64."""
+    return to_f64(array(t).reshape(-1), t.dtype)
+
+
+def ulps64(a, b):
+    if a == b:
+        return 0
+    ia, ib = (np.array([v], dtype=np.float64).view(np.int64)[0] for v in (a, b))
+    return abs(int(ia) - int(ib))
+
+
+def round_to(dtype, q):
+    """A rational rounded once to the dtype (halves through f32, as homura rounds them)."""
+    v = np.float64(float(q))  # Fraction -> nearest f64, correctly rounded
+    return float(to_f64(from_f64([v], dtype), dtype)[0])
+
+
+# ---- erf -----------------------------------------------------------------------------------------------
+
+ERF_TABLE = [(0.0, 0.0), (1e-10, 1.1283791670955126e-10), (0.5, 0.5204998778130465), (1.0, 0.8427007929497149),
+             (2.0, 0.9953222650189527), (2.4999, 0.9995928300996666), (2.5, 0.999593047982555),
+             (3.0, 0.9999779095030014), (4.0, 0.9999999845827421), (-1.5, -0.9661051464753108)]
+
+
+def test_erf_table():
+    for x, want in ERF_TABLE:
+        assert ulps64(L.orc_erf(x), want) <= 3, (x, L.orc_erf(x), want)
+    assert L.orc_erf(INF) == 1.0 and L.orc_erf(-INF) == -1.0
+    assert math.isnan(L.orc_erf(NAN))
+    assert L.orc_erf(7.0) == 1.0
+
+
+def test_erf_against_an_independent_libm():
+    """glibc's erf is a different algorithm (rational approximations); the series / continued fraction
+    must agree with it to a few ulp everywhere, be odd, and switch branches at 1.5 and 6 without a step."""
+    xs = np.concatenate([np.linspace(-6.5, 6.5, 5201), [1.4999999, 1.5, 1.5000001, 5.9999999, 6.0, 1e-300, -0.0]])
+    worst = 0
+    for x in xs:
+        got, want = L.orc_erf(float(x)), math.erf(float(x))
+        # The series multiplies by exp(-x*x), whose argument carries the rounding of x*x: a few ulp.
+        assert abs(got - want) <= 8 * math.ulp(want) + 1e-300, (x, got, want)
+        assert L.orc_erf(-float(x)) == -got
+        worst = max(worst, ulps64(got, want))
+    assert worst <= 8
+
+
+# ---- integer powers --------------------------------------------------------------------------------------
+
+def wrap(v, nbits):
+    v &= (1 << nbits) - 1
+    return v - (1 << nbits) if v >> (nbits - 1) else v
+
+
+def test_int_pow_brute_force():
+    for base in range(-128, 128):
+        for e in range(0, 12):
+            assert L.orc_int_pow_i8(base, e) == wrap(base ** e, 8), (base, e)
+    for base in (-7, -2, -1, 0, 1, 2, 3, 10, 46341, 2147483647):
+        for e in (0, 1, 2, 3, 5, 31, 32, 33, 63, 64):
+            assert L.orc_int_pow_i32(wrap(base, 32), e) == wrap(base ** e, 32), (base, e)
+            assert L.orc_int_pow_i64(base, e) == wrap(base ** e, 64), (base, e)
+    # Negative exponents (ref: src/backend/cpu/num.rs:162-187): 1 -> 1, -1 -> +-1, else 0.
+    for e in (-1, -2, -3, -64):
+        assert L.orc_int_pow_i64(1, e) == 1
+        assert L.orc_int_pow_i64(-1, e) == (1 if e % 2 == 0 else -1)
+        assert L.orc_int_pow_i64(2, e) == 0 and L.orc_int_pow_i64(0, e) == 0 and L.orc_int_pow_i64(-5, e) == 0
+
+
+# ---- conversions --------------------------------------------------------------------------------------------
+
+def cast(values, src, dst):
+    t = tensor(from_f64(values, src) if src != DT.F64 else np.asarray(values, dtype=np.float64), src, [len(values)])
+    return array(t.to(dst)).reshape(-1)
+
+
+def test_element_casts():
+    assert cast([-1.7], DT.F32, DT.I32)[0] == -1
+    assert tensor(np.array([300], dtype=np.int64), DT.I64, [1]).to(DT.U8).to_bytes() == bytes([44])
+    assert cast([300.0], DT.F32, DT.U8)[0] == 44
+    assert cast([-1.0], DT.F64, DT.U8)[0] == 255
+    assert cast([-129.9], DT.F32, DT.I8)[0] == 127
+    assert cast([-2.5], DT.F16, DT.U8)[0] == 254
+    assert cast([NAN], DT.F64, DT.I32)[0] == 0
+    assert cast([INF], DT.F64, DT.I64)[0] == np.iinfo(np.int64).max
+    assert cast([INF], DT.F64, DT.I32)[0] == -1
+    assert cast([1e30], DT.F32, DT.I16)[0] == -1
+    assert cast([0.1], DT.F64, DT.Bool)[0] == 1
+    assert tensor(np.array([1], dtype=np.uint8), DT.Bool, [1]).to(DT.F16).to_bytes() == (0x3C00).to_bytes(2, "little")
+    assert cast([2.5], DT.F16, DT.F32)[0] == 2.5
+
+
+def test_half_casts_round_through_f32():
+    p = lambda e: 2.0 ** e
+    assert cast([np.float32(1.0 + p(-8) + p(-21))], DT.F32, DT.BF16)[0] == 0x3F81
+    assert cast([1.0 + p(-8) + p(-21)], DT.F64, DT.BF16)[0] == 0x3F81
+    assert cast([1.0 + p(-8) + p(-40)], DT.F64, DT.BF16)[0] == 0x3F80
+    assert cast([1.0 + p(-11) + p(-40)], DT.F64, DT.F16)[0] == 0x3C00
+
+    def from_i64(v, dst):
+        return vals(tensor(np.array([v], dtype=np.int64), DT.I64, [1]).to(dst))[0]
+
+    assert from_i64((1 << 24) + 1, DT.BF16) == p(24)
+    assert from_i64((1 << 24) + (1 << 16) + 1, DT.BF16) == p(24)
+    assert from_i64((1 << 63) - 1, DT.BF16) == p(63)
+    assert from_i64(70000, DT.F16) == INF
+    assert math.isnan(vals(f64t([NAN]).to(DT.F16))[0])
+    neg_nan = np.array([0xFFF8000000000000], dtype=np.uint64).view(np.float64)
+    assert int(bits(tensor(neg_nan, DT.F64, [1]).to(DT.BF16))[0]) & 0x8000
+
+
+def test_every_f32_to_bf16_rounding_against_integer_arithmetic():
+    """Round-to-nearest-even on the bit pattern, restated with integers only, over a dense sample of
+    f32 patterns including every exponent, ties and the carry into the exponent."""
+    rng = np.random.default_rng(11)
+    pat = np.concatenate([rng.integers(0, 1 << 32, 200000, dtype=np.uint64).astype(np.uint32),
+                          (np.arange(0, 1 << 16, dtype=np.uint32) << 16) | np.uint32(0x8000),   # exact ties
+                          (np.arange(0, 1 << 16, dtype=np.uint32) << 16) | np.uint32(0x8001),
+                          (np.arange(0, 1 << 16, dtype=np.uint32) << 16) | np.uint32(0x7FFF)])
+    f = pat.view(np.float32)
+    got = array(tensor(f, DT.F32, [len(f)]).to(DT.BF16)).reshape(-1).astype(np.uint32)
+    p = pat.astype(np.uint64)
+    rounded = ((p + 0x7FFF + ((p >> 16) & 1)) >> 16) & 0xFFFF
+    nan = (p & 0x7FFFFFFF) > 0x7F800000
+    want = np.where(nan, ((p >> 16) | 0x0040) & 0xFFFF, rounded).astype(np.uint32)
+    np.testing.assert_array_equal(got, want)
+
+
+def test_f16_conversion_matches_numpy_ieee():
+    """numpy's float16 is IEEE binary16 with round-to-nearest-even: an independent implementation."""
+    rng = np.random.default_rng(12)
+    f = rng.integers(0, 1 << 32, 300000, dtype=np.uint64).astype(np.uint32).view(np.float32)
+    f = f[~np.isnan(f)]
+    got = array(tensor(f, DT.F32, [len(f)]).to(DT.F16)).reshape(-1)
+    with np.errstate(all="ignore"):
+        want = f.astype(np.float16).view(np.uint16)
+    np.testing.assert_array_equal(got, want)
+    allh = np.arange(0, 1 << 16, dtype=np.uint16)
+    wide = array(tensor(allh, DT.F16, [1 << 16]).to(DT.F32)).reshape(-1)
+    ref = allh.view(np.float16).astype(np.float32)
+    ok = (wide == ref) | (np.isnan(wide) & np.isnan(ref))
+    assert ok.all()
+
+
+# ---- elementwise ----------------------------------------------------------------------------------------------
+
+def test_half_products_keep_the_scalar_in_f32():
+    s = 1.0 / 3.0
+    for dtype, mul, add, sub in [(DT.F16, 2.333984375, 7.33203125, 6.66796875), (DT.BF16, 2.328125, 7.34375, 6.65625)]:
+        x = f64t([7.0]).to(dtype)
+        assert vals(x.mul(s))[0] == mul
+        assert vals(x.rdiv(s))[0] == 0.047607421875
+        assert vals(x.add(s))[0] == add
+        assert vals(x.sub(s))[0] == sub
+
+
+def test_ieee_arithmetic_is_correctly_rounded():
+    """+ - * / in f32 and the halves equal exact rational arithmetic rounded once to the dtype."""
+    rng = np.random.default_rng(13)
+    for dtype in (DT.F16, DT.BF16, DT.F32):
+        a64 = rng.normal(0, 3, 400)
+        b64 = rng.normal(0, 3, 400)
+        a, b = tensor(from_f64(a64, dtype), dtype, [400]), tensor(from_f64(b64, dtype), dtype, [400])
+        av, bv = vals(a), vals(b)
+        for name, fn in (("add", lambda x, y: x + y), ("sub", lambda x, y: x - y), ("mul", lambda x, y: x * y),
+                         ("div", lambda x, y: x / y)):
+            got = vals(getattr(a, name)(b))
+            for i in range(400):
+                exact = fn(Fraction(float(av[i])), Fraction(float(bv[i])))
+                if dtype == DT.F32:
+                    want = float(np.float32(float(exact)))  # may double-round through f64: check below
+                    # f64 -> f32 double rounding only matters within 2^-29 relative of an f32 tie; rule it out
+                    lo, hi = np.nextafter(np.float32(want), np.float32(-INF)), np.nextafter(np.float32(want), np.float32(INF))
+                    assert abs(exact - Fraction(want)) <= min(abs(exact - Fraction(float(lo))), abs(exact - Fraction(float(hi))))
+                else:
+                    # halves: computed in f32 then rounded to the half: two roundings, by definition of the reference
+                    want = float(to_f64(from_f64([np.float64(np.float32(float(exact)))], dtype), dtype)[0])
+                assert got[i] == want, (dtype, name, av[i], bv[i], got[i], want)
+
+
+def test_unary_formulas_against_python_math():
+    xs = np.array([-20.0, -3.0, -1.0, -0.5, -0.0, 0.0, 0.25, 1.0, 2.0, 10.0, 30.0])
+    x = f64t(xs)
+    want = {
+        "sigmoid": [1 / (1 + math.exp(-v)) for v in xs],
+        "silu": [v / (1 + math.exp(-v)) for v in xs],
+        "gelu": [0.5 * v * (1 + math.erf(v * math.sqrt(0.5))) for v in xs],
+        "gelu_tanh": [0.5 * v * (1 + math.tanh(math.sqrt(2 / math.pi) * (v + 0.044715 * v * v * v))) for v in xs],
+        "log_sigmoid": [min(v, 0.0) - math.log1p(math.exp(-abs(v))) for v in xs],
+        "tanh": [math.tanh(v) for v in xs],
+        "exp": [math.exp(v) for v in xs],
+        "relu": [max(v, 0.0) for v in xs],
+        "sign": [float(v > 0) - float(v < 0) for v in xs],
+    }
+    for name, w in want.items():
+        got = vals(getattr(x, name)())
+        for g, e, v in zip(got, w, xs):
+            assert abs(g - e) <= 8 * math.ulp(e) + 1e-300, (name, v, g, e)
+    # Special values (ref: src/backend/cpu/mod.rs:362-403).
+    s = f64t([NAN, -0.0, INF, -INF])
+    assert np.array_equal(vals(s.sign()), [0.0, 0.0, 1.0, -1.0])
+    r = vals(s.relu())
+    assert math.isnan(r[0]) and r[1] == 0 and r[2] == INF and r[3] == 0
+    assert np.array_equal(array(s.logical_not()).reshape(-1), [0, 1, 0, 0])
+
+
+def test_iteration_order_of_a_transposed_view():
+    x = tensor(np.arange(6, dtype=np.int64), DT.I64, [3, 2]).transpose(0, 1)      # shape [2,3], strides [1,2]
+    assert array(x.contiguous()).reshape(-1).tolist() == [0, 2, 4, 1, 3, 5]
+    e = tensor(np.arange(3, dtype=np.int64), DT.I64, [3]).narrow(0, 1, 1).expand([3])
+    assert array(e.contiguous()).reshape(-1).tolist() == [1, 1, 1]
+
+
+# ---- reductions ---------------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", FLOATS)
+def test_exact_sums_means_variances(dtype):
+    v = np.array([((i * 37) % 17) - 8.0 for i in range(256)]).reshape(8, 32)
+    x = f64t(v).to(dtype)
+    for d in (0, 1):
+        n = v.shape[d]
+        lines = np.moveaxis(v, d, -1).reshape(-1, n)
+        sums = [sum(Fraction(int(e)) for e in line) for line in lines]
+        means = [s / n for s in sums]
+        var0 = [sum((Fraction(int(e)) - m) ** 2 for e in line) / n for line, m in zip(lines, means)]
+        var1 = [sum((Fraction(int(e)) - m) ** 2 for e in line) / (n - 1) for line, m in zip(lines, means)]
+        assert vals(x.sum_dim(d, False)).tolist() == [round_to(dtype, s) for s in sums]
+        assert vals(x.mean_dim(d, False)).tolist() == [round_to(dtype, m) for m in means]
+        assert vals(x.var_dim(d, 0, False)).tolist() == [round_to(dtype, q) for q in var0]
+        got = vals(x.std_dim(d, 1, False))
+        for g, q in zip(got, var1):
+            want = float(to_f64(from_f64([math.sqrt(float(q))], dtype), dtype)[0])
+            assert g == want
+    # The mean divides the f64 sum, not its rounding to the dtype.
+    m = {DT.F16: [1401.0, 1401.0, 1400.0], DT.F32: [16777215.0, 16777215.0, 16777213.0]}.get(dtype, [1.0, 2.0, 2.0])
+    got = vals(f64t([m]).to(dtype).mean_dim(1, False))[0]
+    assert got == round_to(dtype, Fraction(int(sum(m))) / 3)
+    if dtype == DT.F16:
+        assert got == 1401.0
+    if dtype == DT.F32:
+        assert got == 16777214.0
+    assert vals(f64t([2.0, -0.5, 4.0, 0.25, -1.0, 8.0]).to(dtype).prod())[0] == 8.0
+    # Too few elements for the correction: x / 0.
+    w = f64t([[1.0, 3.0], [2.0, 2.0]]).to(dtype)
+    for c in (2, 3):
+        r = vals(w.var_dim(1, c, False))
+        assert r[0] == INF and math.isnan(r[1])
+
+
+@pytest.mark.parametrize("dtype", FLOATS)
+def test_empty_and_special_reductions(dtype):
+    e = tensor(np.zeros(0, dtype=NP[dtype]), dtype, [3, 0])
+    assert vals(e.sum_dim(1, False)).tolist() == [0.0] * 3
+    assert vals(e.prod_dim(1, False)).tolist() == [1.0] * 3
+    assert np.isnan(vals(e.mean_dim(1, False))).all()
+    assert np.isnan(vals(e.var_dim(1, 0, False))).all()
+    assert array(e.all_dim(1, False)).reshape(-1).tolist() == [1, 1, 1]
+    assert array(e.any_dim(1, False)).reshape(-1).tolist() == [0, 0, 0]
+    with pytest.raises(Exception):
+        e.max()
+    with pytest.raises(Exception):
+        e.min_dim(1, False)
+    with pytest.raises(Exception):
+        e.argmax()
+    rows = [[1.0, NAN, 2.0, 3.0], [1.0, INF, 2.0, 3.0], [1.0, -INF, 2.0, 3.0], [INF, 1.0, -INF, 3.0], [0.0, INF, 2.0, 3.0]]
+    x = f64t(rows).to(dtype)
+    s = vals(x.sum_dim(1, False))
+    assert math.isnan(s[0]) and s[1] == INF and s[2] == -INF and math.isnan(s[3]) and s[4] == INF
+    p = vals(x.prod_dim(1, False))
+    assert math.isnan(p[0]) and p[1] == INF and p[2] == -INF and p[3] == -INF and math.isnan(p[4])
+    assert np.isnan(vals(x.var_dim(1, 1, False))).all()
+
+
+def test_nan_ties_and_integer_reductions():
+    x = f64t([[1.0, NAN, NAN], [4.0, 4.0, 2.0]])
+    assert array(x.argmax_dim(1, False)).reshape(-1).tolist() == [1, 0]
+    assert array(x.argmin_dim(1, False)).reshape(-1).tolist() == [1, 2]
+    assert math.isnan(vals(x.max())[0])
+    z = f64t([[0.0, -0.0], [-0.0, 0.0]])
+    assert array(z.argmax_dim(1, False)).reshape(-1).tolist() == [0, 0]      # +0 / -0 tie: the first
+    assert bits(z.max_dim(1, False)[0]).tolist() == [0, 1 << 63]
+    u = tensor(np.array([0, 2], dtype=np.uint8), DT.U8, [2])
+    assert u.any().dtype == DT.U8 and array(u.any()).item() == 1 and array(u.all()).item() == 0
+    b = tensor(np.array([1, 0, 1], dtype=np.uint8), DT.Bool, [3])
+    assert b.prod().dtype == DT.I64 and array(b.prod()).item() == 0
+    big = tensor(np.array([2**63 - 1, 1], dtype=np.int64), DT.I64, [2])
+    assert array(big.sum()).item() == -2**63
+
+
+def test_sum_is_a_sequential_f64_fold():
+    """Order matters in floating point: 1e16 + 1 + 1 + ... folded left to right in f64 loses every 1,
+    while any pairwise or compensated order would not; the oracle must reproduce the sequential result."""
+    v = np.array([1e16] + [1.0] * 64)
+    assert vals(f64t(v).sum())[0] == 1e16
+    assert vals(f64t(v[::-1].copy()).sum())[0] == 1e16 + 64
+    # f32 input accumulates in f64, not f32: 2^24 + 1 + 1 ... is exact in f64.
+    w = f64t([16777216.0] + [1.0] * 3).to(DT.F32)
+    assert vals(w.sum())[0] == float(np.float32(16777219.0))
+
+
+# ---- softmax ----------------------------------------------------------------------------------------------------------
+
+def test_softmax_known_answers():
+    x = f64t([[10000.0, 10001.0, 10002.0], [NAN, 1.0, 2.0]])
+    p = vals(x.softmax(-1).to(DT.F32))
+    assert abs(p[0] - 0.09003057) < 1e-6 and abs(p[1] - 0.24472848) < 1e-6 and abs(p[2] - 0.66524094) < 1e-6
+    assert np.isnan(p[3:]).all()
+    y = f64t([0.0, -INF])
+    assert vals(y.softmax(0)).tolist() == [1.0, 0.0]
+    assert vals(y.log_softmax(0)).tolist() == [0.0, -INF]
+    t = f64t(3.0, [])
+    assert vals(t.softmax(0))[0] == 1.0 and vals(t.log_softmax(-1))[0] == 0.0
+
+
+@pytest.mark.parametrize("dtype", FLOATS)
+def test_softmax_extreme_rows(dtype):
+    big = {DT.F16: 6e4, DT.BF16: 3e38, DT.F32: 3e38, DT.F64: 1e300}[dtype]
+    rows = [[-INF, -INF, -INF, -INF], [1.0, NAN, 2.0, 3.0], [1.0, INF, 2.0, 3.0], [big, -big, big, 0.0],
+            [-big, -big, 1.0, -INF], [0.0, -0.0, 0.0, -0.0]]
+    x = f64t(rows).to(dtype)
+    s = vals(x.softmax(1)).reshape(6, 4)
+    l = vals(x.log_softmax(1)).reshape(6, 4)
+    assert np.isnan(s[:3]).all() and np.isnan(l[:3]).all()
+    assert s[3].tolist() == [0.5, 0.0, 0.5, 0.0]
+    assert l[3][1] <= -big and l[3][0] == round_to(dtype, Fraction(math.log(0.5)))
+    assert s[4].tolist() == [0.0, 0.0, 1.0, 0.0] and l[4][2] == 0.0 and l[4][3] == -INF
+    assert s[5].tolist() == [0.25] * 4
+    one = f64t([[3.0], [-INF], [NAN]]).to(dtype)
+    o = vals(one.softmax(1))
+    assert o[0] == 1.0 and math.isnan(o[1]) and math.isnan(o[2])
+
+
+def test_softmax_against_exact_arithmetic():
+    """exp(x - max) from libm, then the sum and the quotient in exact rational arithmetic: the oracle's
+    sequential f64 sum of 257 terms may differ from that by a few ulp (far below one dropped term, 1/257),
+    and each row must sum to one."""
+    rng = np.random.default_rng(21)
+    x = rng.normal(0, 3, (16, 257))
+    got = vals(f64t(x).softmax(-1)).reshape(16, 257)
+    glog = vals(f64t(x).log_softmax(-1)).reshape(16, 257)
+    for r in range(16):
+        m = max(x[r])
+        e = [Fraction(math.exp(v - m)) for v in x[r]]
+        tot = sum(e)
+        for c in range(257):
+            want = float(e[c] / tot)
+            assert abs(got[r, c] - want) <= 16 * math.ulp(want)
+            wl = (x[r, c] - m) - math.log(float(tot))
+            assert abs(glog[r, c] - wl) <= 16 * math.ulp(wl)
+        assert abs(sum(Fraction(float(g)) for g in got[r]) - 1) < Fraction(1, 10**13)

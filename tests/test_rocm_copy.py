@@ -1,0 +1,80 @@
+"""hmr_copy / hmr_fill on the GPU against the CPU oracle, byte for byte, NaN payloads included
+(ref: tests/rocm_copy.rs:12-130, src/dtype.rs:186-277, csrc/elem.hpp:276-287)."""
+import numpy as np
+import pytest
+
+from tests import oracle
+from tests.support import DT, DTYPES, GPU, NP, array, assert_same, h, large_layouts, layouts, tensor, words
+
+pytestmark = pytest.mark.gpu
+h.register_cpu_backend(oracle.backend_address())
+
+
+def test_every_conversion_matches_the_cpu_in_every_layout():
+    for k, src in enumerate(DTYPES):
+        for pair in layouts(src, 10 + k):
+            assert_same(pair.gpu.contiguous(), pair.cpu.contiguous(), f"{src} {pair.name} copied")
+            for dst in DTYPES:
+                what = f"{src} -> {dst}, {pair.name}"
+                gpu, cpu = pair.gpu.to(dst), pair.cpu.to(dst)
+                assert_same(gpu, cpu, what)
+                if dst != src:
+                    assert gpu.is_contiguous(), what
+
+
+def test_nan_payloads_convert_like_the_cpu():
+    n = 1 << 16
+    r, r32, r16, rb16 = (words(99 + k, n) for k in range(4))
+    f64s = ((r & np.uint64(0x800FFFFFFFFFFFFF)) | np.uint64(0x7FF0000000000001)).view(np.float64)
+    f32s = ((r32.astype(np.uint32) & np.uint32(0x807FFFFF)) | np.uint32(0x7F800001)).view(np.float32)
+    f16s = (r16.astype(np.uint16) & np.uint16(0x83FF)) | np.uint16(0x7C01)
+    bf16s = (rb16.astype(np.uint16) & np.uint16(0x807F)) | np.uint16(0x7F81)
+    for arr, dtype in ((f64s, DT.F64), (f32s, DT.F32), (f16s, DT.F16), (bf16s, DT.BF16)):
+        cpu = tensor(arr, dtype, [n])
+        gpu = cpu.to(GPU)
+        for dst in DTYPES:
+            assert_same(gpu.to(dst), cpu.to(dst), f"NaNs {dtype} -> {dst}")
+
+
+def test_conversions_of_large_tensors_take_several_grid_rounds():
+    for src, dst in ((DT.F32, DT.BF16), (DT.F64, DT.F16), (DT.I64, DT.F32), (DT.U8, DT.U8), (DT.BF16, DT.F32)):
+        for pair in large_layouts(src, 7):
+            assert_same(pair.gpu.to(dst), pair.cpu.to(dst), f"{src} -> {dst}, {pair.name}")
+
+
+def test_conversion_counterexamples():
+    def f(v, dtype):
+        return array(tensor(np.array([v], dtype=np.float32), DT.F32, [1], GPU).to(dtype)).item()
+
+    assert f(300.0, DT.U8) == 44
+    assert f(-129.9, DT.I8) == 127
+    assert f(np.inf, DT.I32) == -1
+    assert f(np.inf, DT.I64) == np.iinfo(np.int64).max
+    assert f(1e30, DT.I16) == -1
+    assert f(np.nan, DT.I32) == 0
+    assert array(tensor(np.array([0xC100], dtype=np.uint16), DT.F16, [1], GPU).to(DT.U8)).item() == 254   # -2.5
+
+    def g(v, dtype):
+        return array(tensor(np.array([v], dtype=np.float64), DT.F64, [1], GPU).to(dtype)).item()
+
+    p = lambda e: 2.0 ** e
+    assert array(tensor(np.array([1.0 + p(-8) + p(-21)]), DT.F64, [1], GPU).to(DT.F32).to(DT.BF16)).item() == 0x3F81
+    assert g(1.0 + p(-8) + p(-40), DT.BF16) == 0x3F80
+    assert g(1.0 + p(-11) + p(-40), DT.F16) == 0x3C00
+    i = tensor(np.array([(1 << 24) + (1 << 16) + 1], dtype=np.int64), DT.I64, [1], GPU)
+    assert array(i.to(DT.BF16)).item() == 0x4B80                                                       # 2^24
+    b = tensor(np.array([0.0, -0.0, 0.1, np.nan, -3.0]), DT.F64, [5], GPU).to(DT.Bool)
+    assert array(b).tolist() == [0, 0, 1, 1, 1]
+    assert array(b.to(DT.U8)).tolist() == [0, 0, 1, 1, 1]
+
+
+def test_fill_writes_every_dtype_and_layout():
+    for dtype, v in ((DT.Bool, True), (DT.U8, 200), (DT.I8, -3), (DT.I16, -30000), (DT.I32, 1 << 30), (DT.I64, -(1 << 40)),
+                     (DT.F16, 1.5), (DT.BF16, -2.5), (DT.F32, 3.25), (DT.F64, 1e-300)):
+        for shape in ([], [1], [7], [1031], [3, 257], [0, 4]):
+            gpu, cpu = h.full(shape, v, dtype, GPU), h.full(shape, v, dtype, "cpu")
+            assert_same(gpu, cpu, f"full {dtype} {shape}")
+            n = int(np.prod(shape)) if shape else 1
+            if n:
+                want = array(cpu).reshape(-1)
+                assert (want == want[0]).all() and want.dtype == NP[dtype]
