@@ -127,13 +127,41 @@ HMR_HD float bf16_widen(bf16_t h) {
 
 // f32 -> bf16, nearest even; NaN keeps the top 7 payload bits and turns quiet.
 HMR_HD bf16_t bf16_round(float f) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    // gfx950 converts in hardware (v_cvt_pk_bf16_f32) with the same bits for every f32 pattern, NaNs
+    // included. Written as the instruction itself: the compiler's own lowering of a float -> __bf16
+    // cast pairs neighbouring conversions into vector operations that this build (packed FP32
+    // instructions off) cannot always select.
+    uint32_t packed;
+    asm("v_cvt_pk_bf16_f32 %0, %1, 0" : "=v"(packed) : "v"(f));
+    return bf16_t{static_cast<uint16_t>(packed)};
+#endif
     uint32_t x = bits_as<uint32_t>(f);
     if ((x & 0x7FFFFFFFu) > 0x7F800000u) return bf16_t{static_cast<uint16_t>((x >> 16) | 0x0040u)};
     return bf16_t{static_cast<uint16_t>((x + 0x7FFFu + ((x >> 16) & 1u)) >> 16)};
 }
 
+// Two f32 values rounded to bf16 and packed (lo in bits 0-15): one instruction on the device.
+HMR_HD uint32_t bf16_round_pair(float lo, float hi) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    uint32_t packed;
+    asm("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(packed) : "v"(lo), "v"(hi));
+    return packed;
+#else
+    return static_cast<uint32_t>(bf16_round(lo).bits) | (static_cast<uint32_t>(bf16_round(hi).bits) << 16);
+#endif
+}
+
 // f16 -> f32, exact, by integer arithmetic. NaN: quiet, payload at the top of the mantissa.
 HMR_HD float f16_widen(f16_t h) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    // v_cvt_f32_f16: same bits for all 65 536 patterns. As the instruction itself, so that the compiler
+    // cannot fold the conversion into a mixed-precision multiply-add (x * s became fma(x, s, +0), which
+    // turns -0 into +0).
+    float f;
+    asm("v_cvt_f32_f16 %0, %1" : "=v"(f) : "v"(static_cast<uint32_t>(h.bits)));
+    return f;
+#endif
     uint32_t sign = static_cast<uint32_t>(h.bits & 0x8000u) << 16;
     uint32_t exp = (h.bits >> 10) & 0x1Fu;
     uint32_t man = h.bits & 0x3FFu;
@@ -155,6 +183,11 @@ HMR_HD float f16_widen(f16_t h) {
 
 // f32 -> f16, nearest even; NaN keeps the top 10 payload bits and turns quiet.
 HMR_HD f16_t f16_round(float f) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    uint32_t hw;  // v_cvt_f16_f32: same bits for every f32 pattern
+    asm("v_cvt_f16_f32 %0, %1" : "=v"(hw) : "v"(f));
+    return f16_t{static_cast<uint16_t>(hw)};
+#endif
     uint32_t x = bits_as<uint32_t>(f);
     uint32_t sign = (x >> 16) & 0x8000u;
     uint32_t a = x & 0x7FFFFFFFu;

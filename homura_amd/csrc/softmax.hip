@@ -34,14 +34,14 @@ namespace {
 
 // ---- exp in the evaluation type ------------------------------------------------------------------
 
-// exp(t) for t <= 0 (or NaN) in f64. |relative error| < 2^-45.
+// exp(t) for t <= 0 (or NaN) in f64, without a branch. |relative error| < 2^-45.
 __device__ __forceinline__ double exp_neg_f64(double t) {
-    if (!(t >= -708.0)) return t != t ? t : 0.0;  // underflow region (and -inf) -> 0; NaN stays NaN
     const double kLog2e = 1.4426950408889634074;
     const double kLn2Hi = 6.93147180369123816490e-01;
     const double kLn2Lo = 1.90821492927058770002e-10;
-    double n = rint(t * kLog2e);
-    double r = fma(-n, kLn2Hi, t);
+    const double tc = t < -708.0 ? -708.0 : t;  // the underflow region (and -inf) is answered below; NaN passes
+    double n = rint(tc * kLog2e);
+    double r = fma(-n, kLn2Hi, tc);
     r = fma(-n, kLn2Lo, r);  // |r| <= 0.3466
     // Taylor to degree 11: remainder < 0.3466^12 / 12! < 2^-47.
     double p = 1.0 / 39916800.0;
@@ -56,26 +56,64 @@ __device__ __forceinline__ double exp_neg_f64(double t) {
     p = fma(p, r, 0.5);
     p = fma(p, r, 1.0);
     p = fma(p, r, 1.0);
-    // Scale by 2^n, n in [-1022, 0]: add to the exponent field.
-    int64_t bits = __double_as_longlong(p) + (static_cast<int64_t>(n) << 52);
-    return __longlong_as_double(bits);
+    // Scale by 2^n, n in [-1022, 0]: add to the exponent field (of a NaN: n is 0).
+    int64_t bits = __double_as_longlong(p) + (static_cast<int64_t>(static_cast<int32_t>(n)) << 52);
+    return t < -708.0 ? 0.0 : __longlong_as_double(bits);
 }
 
 template <class T>
 struct SoftmaxMath;
 
-// Halves: values travel as f32.
+constexpr float kLog2eF = 1.44269504088896340736f;
+
+// Halves: values travel as f32. Anything whose relative error stays near 2^-17 lands within one ulp
+// of an 8- or 11-bit result, so the exponentials come from the hardware's 2^x (v_exp_f32, 1 ulp):
+//   for the sum   2^((x - max) log2 e)              (results below 2^-126 may flush: they are
+//                                                    below 2^-126 of a sum that is at least 1)
+//   for the output 2^((x - max) log2 e - log2 sum)  through exp2f, which keeps subnormal results.
+// The output form is evaluated per element in the last phase instead of keeping every exponential
+// in registers, which lets a lane hold 128 packed elements of its row.
 template <class T>
 struct HalfMath {
     using X = float;  // a row element in registers
     using E = float;  // exp(x - max), and the per-row scale
+    static constexpr bool kKeep = false;
+    static constexpr uint32_t kNegInfPair = std::is_same_v<T, bf16_t> ? 0xFF80FF80u : 0xFC00FC00u;
     static __device__ __forceinline__ X load(T v) { return Comp<T>::up(v); }
-    static __device__ __forceinline__ E ex(X x, X mx) { return expf(x - mx); }
+    static __device__ __forceinline__ void unpack(const u32x4 &r, X (&x)[8]) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if constexpr (std::is_same_v<T, bf16_t>) {
+                x[2 * j] = __uint_as_float(r[j] << 16);
+                x[2 * j + 1] = __uint_as_float(r[j] & 0xFFFF0000u);
+            } else {
+                x[2 * j] = f16_widen(f16_t{static_cast<uint16_t>(r[j] & 0xFFFFu)});
+                x[2 * j + 1] = f16_widen(f16_t{static_cast<uint16_t>(r[j] >> 16)});
+            }
+        }
+    }
+    // Results in the evaluation type -> a packed chunk of the row.
+    static __device__ __forceinline__ u32x4 pack(const float (&y)[8]) {
+        u32x4 r;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if constexpr (std::is_same_v<T, bf16_t>) {
+                r[j] = bf16_round_pair(y[2 * j], y[2 * j + 1]);
+            } else {
+                r[j] = static_cast<uint32_t>(f16_round(y[2 * j]).bits) | (static_cast<uint32_t>(f16_round(y[2 * j + 1]).bits) << 16);
+            }
+        }
+        return r;
+    }
+    static __device__ __forceinline__ E ex(X x, X mx) { return __builtin_amdgcn_exp2f((x - mx) * kLog2eF); }
     static __device__ __forceinline__ double wide(E e) { return static_cast<double>(e); }
-    static __device__ __forceinline__ E inv(double sum) { return static_cast<float>(sum); }  // keeps the sum; see soft()
+    static __device__ __forceinline__ E scale(double sum) { return __builtin_log2f(static_cast<float>(sum)); }
     static __device__ __forceinline__ E lg(double sum) { return static_cast<float>(log(sum)); }
-    static __device__ __forceinline__ T soft(E e, E sum) { return Comp<T>::down(e / sum); }
-    static __device__ __forceinline__ T logsoft(X x, X mx, E log_sum) { return Comp<T>::down(x - mx - log_sum); }
+    static __device__ __forceinline__ float soft(X x, X mx, E, E log2_sum) {
+        return __builtin_exp2f((x - mx) * kLog2eF - log2_sum);
+    }
+    static __device__ __forceinline__ float logsoft(X x, X mx, E log_sum) { return x - mx - log_sum; }
+    static __device__ __forceinline__ T down(float y) { return Comp<T>::down(y); }
 };
 template <>
 struct SoftmaxMath<f16_t> : HalfMath<f16_t> {};
@@ -86,14 +124,23 @@ template <>
 struct SoftmaxMath<float> {
     using X = float;
     using E = double;
+    static constexpr bool kKeep = true;  // the f64 exponentials stay in registers for the last phase
     static __device__ __forceinline__ X load(float v) { return v; }
+    static __device__ __forceinline__ void unpack(const u32x4 &r, X (&x)[4]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) x[i] = __uint_as_float(r[i]);
+    }
     static __device__ __forceinline__ E ex(X x, X mx) { return exp_neg_f64(static_cast<double>(x) - static_cast<double>(mx)); }
     static __device__ __forceinline__ double wide(E e) { return e; }
-    static __device__ __forceinline__ E inv(double sum) { return 1.0 / sum; }
+    static __device__ __forceinline__ E scale(double sum) { return 1.0 / sum; }
     static __device__ __forceinline__ E lg(double sum) { return log(sum); }
-    static __device__ __forceinline__ float soft(E e, E inv_sum) { return static_cast<float>(e * inv_sum); }
+    static __device__ __forceinline__ float soft(X, X, E e, E inv_sum) { return static_cast<float>(e * inv_sum); }
     static __device__ __forceinline__ float logsoft(X x, X mx, E log_sum) {
         return static_cast<float>(static_cast<double>(x) - static_cast<double>(mx) - log_sum);
+    }
+    static __device__ __forceinline__ float down(float y) { return y; }
+    static __device__ __forceinline__ u32x4 pack(const float (&y)[4]) {
+        return u32x4{__float_as_uint(y[0]), __float_as_uint(y[1]), __float_as_uint(y[2]), __float_as_uint(y[3])};
     }
 };
 
@@ -101,14 +148,48 @@ template <>
 struct SoftmaxMath<double> {
     using X = double;
     using E = double;
+    static constexpr bool kKeep = true;
     static __device__ __forceinline__ X load(double v) { return v; }
+    static __device__ __forceinline__ void unpack(const u32x4 &r, X (&x)[2]) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            x[i] = __longlong_as_double(static_cast<int64_t>(static_cast<uint64_t>(r[2 * i]) |
+                                                             (static_cast<uint64_t>(r[2 * i + 1]) << 32)));
+        }
+    }
     static __device__ __forceinline__ E ex(X x, X mx) { return exp(x - mx); }
     static __device__ __forceinline__ double wide(E e) { return e; }
-    static __device__ __forceinline__ E inv(double sum) { return sum; }
+    static __device__ __forceinline__ E scale(double sum) { return sum; }
     static __device__ __forceinline__ E lg(double sum) { return log(sum); }
-    static __device__ __forceinline__ double soft(E e, E sum) { return e / sum; }
+    static __device__ __forceinline__ double soft(X, X, E e, E sum) { return e / sum; }
     static __device__ __forceinline__ double logsoft(X x, X mx, E log_sum) { return x - mx - log_sum; }
+    static __device__ __forceinline__ double down(double y) { return y; }
+    static __device__ __forceinline__ u32x4 pack(const double (&y)[2]) {
+        u32x4 r;
+        __builtin_memcpy(&r, y, 16);
+        return r;
+    }
 };
+
+// A 16-byte chunk whose every element is -inf: what pads a row past its end. -inf neither raises the
+// max nor adds to the sum (exp(-inf - max) is exactly 0; when the max itself is -inf the row's own
+// elements already make everything NaN, as on the CPU).
+template <class T>
+__device__ __forceinline__ u32x4 neg_inf_chunk() {
+    if constexpr (std::is_same_v<T, float>) {
+        return u32x4{0xFF800000u, 0xFF800000u, 0xFF800000u, 0xFF800000u};
+    } else if constexpr (std::is_same_v<T, double>) {
+        return u32x4{0u, 0xFFF00000u, 0u, 0xFFF00000u};
+    } else {
+        constexpr uint32_t w = SoftmaxMath<T>::kNegInfPair;
+        return u32x4{w, w, w, w};
+    }
+}
+
+// Makes the compiler treat a chunk as newly produced. Each phase unpacks the row's chunks again; without
+// this the unpacked values of one phase are kept alive for the next and the packed row costs more
+// registers than an unpacked one.
+__device__ __forceinline__ void forget(u32x4 &r) { asm volatile("" : "+v"(r)); }
 
 // ---- combining across the lanes of a row ---------------------------------------------------------
 
@@ -151,10 +232,17 @@ struct SoftmaxArgs {
     int64_t so, si;
 };
 
-// Contiguous rows held in registers. G lanes per row, each with up to C tiles of V elements:
-// tile c of lane l covers elements (c*G + l)*V .. +V, so every load of the group is one
-// contiguous, coalesced span.
-template <class T, int G, int C, bool LOG>
+// Contiguous rows held in registers, as loaded (16-byte chunks). G lanes per row, each with C
+// chunks of V elements: chunk c of lane l covers elements (c*G + l)*V .. +V, so every load of the
+// group is one contiguous, coalesced span. Rows are whole chunks (n is a multiple of V).
+//
+// All C loads of a lane are issued back to back and unconditionally (a chunk past the row's end
+// re-reads the row's last chunk and is then replaced by -inf): a branch between loads would make
+// each wait for the one before.
+//
+// WALK = false: the rows form one dimension (row r starts r * stride elements in), which is what a
+// contiguous tensor gives; WALK = true: up to 25 row dimensions, decoded per row.
+template <class T, int G, int C, bool LOG, bool WALK>
 __global__ void __launch_bounds__(G > kBlock ? G : kBlock) softmax_regs_kernel(SoftmaxArgs a) {
     using M = SoftmaxMath<T>;
     using X = typename M::X;
@@ -163,79 +251,107 @@ __global__ void __launch_bounds__(G > kBlock ? G : kBlock) softmax_regs_kernel(S
     constexpr int V = 16 / static_cast<int>(sizeof(T));
     constexpr int kThreads = G > kBlock ? G : kBlock;
     constexpr int kRowsPerBlock = kThreads / G;
+    constexpr bool kKeep = M::kKeep && !LOG;
     __shared__ double lds[G > kWave ? G / kWave : 1];
     const int lane = threadIdx.x % G;
     const int64_t groups = (a.nrows + kRowsPerBlock - 1) / kRowsPerBlock;
-    const int64_t nvec = a.n / V;  // whole tiles in a row; the rest (< V elements) is the ragged end
+    const int nvec = static_cast<int>(a.n / V);  // chunks in a row (>= 1)
     for (int64_t g = blockIdx.x; g < groups; g += gridDim.x) {
         const int64_t row = g * kRowsPerBlock + threadIdx.x / G;
         const bool live = row < a.nrows;
-        const T *src = reinterpret_cast<const T *>(a.src) + (live ? a.src_rows.offset(row) : 0);
-        T *out = reinterpret_cast<T *>(a.out) + (live ? a.out_rows.offset(row) : 0);
-        X x[C][V];
-        const X ninf = -__builtin_huge_valf();
+        const int64_t r = live ? row : a.nrows - 1;  // idle lanes of the last group redo the last row, without storing
+        const T *src = reinterpret_cast<const T *>(a.src) + (WALK ? a.src_rows.offset(r) : r * a.src_rows.stride[0]);
+        T *out = reinterpret_cast<T *>(a.out) + (WALK ? a.out_rows.offset(r) : r * a.out_rows.stride[0]);
         // Phase 0: one pass over memory.
+        u32x4 raw[C];
 #pragma unroll
         for (int c = 0; c < C; ++c) {
-            const int64_t tile = static_cast<int64_t>(c) * G + lane;
-            T raw[V];
-            if (live && tile < nvec) {
-                load_tile<T, V, kStreamLoads>(reinterpret_cast<const char *>(src + tile * V), raw);
+            // A uniform row pointer plus a 32-bit byte offset per lane: one address register per chunk.
+            const uint32_t tile = static_cast<uint32_t>(c * G + lane);
+            const uint32_t t = tile < static_cast<uint32_t>(nvec) ? tile : static_cast<uint32_t>(nvec - 1);
+            const u32x4 *q = reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(src) + t * 16u);
+            if constexpr (kStreamLoads) raw[c] = __builtin_nontemporal_load(q);
+            else raw[c] = *q;
+        }
+        __builtin_amdgcn_sched_barrier(0);  // every load is out before anything waits for one
 #pragma unroll
-                for (int i = 0; i < V; ++i) x[c][i] = M::load(raw[i]);
-            } else {
-#pragma unroll
-                for (int i = 0; i < V; ++i) {
-                    const int64_t e = tile * V + i;
-                    // Past the row: -inf neither raises the max nor adds to the sum.
-                    x[c][i] = (live && e < a.n) ? M::load(src[e]) : ninf;
-                }
-            }
+        for (int c = 0; c < C; ++c) {
+            if (c * G + lane >= nvec) raw[c] = neg_inf_chunk<T>();
         }
         // Phase 1: max. A NaN never replaces (v > m is false), as on the CPU.
-        X mx = ninf;
+        X mx = -__builtin_huge_valf();
 #pragma unroll
         for (int c = 0; c < C; ++c) {
+            X x[V];
+            M::unpack(raw[c], x);
 #pragma unroll
-            for (int i = 0; i < V; ++i) mx = x[c][i] > mx ? x[c][i] : mx;
+            for (int i = 0; i < V; ++i) mx = x[i] > mx ? x[i] : mx;
         }
         mx = row_fold<G>(MaxFold{}, mx, reinterpret_cast<X *>(lds));
-        // Phase 2: exponentials and their f64 sum. Padding past the row must add exactly 0 even
-        // when the row's max is -inf (where a real -inf entry yields NaN).
+        // Phase 2: exponentials and their f64 sum.
         double sum = 0.0;
-        E ex[LOG ? 1 : C][LOG ? 1 : V];
+        E ex[kKeep ? C : 1][kKeep ? V : 1];
 #pragma unroll
         for (int c = 0; c < C; ++c) {
+            X x[V];
+            forget(raw[c]);
+            M::unpack(raw[c], x);
+            E e[V];
+            if constexpr (std::is_same_v<E, double>) {
+                // An f64 exponential is some thirty instructions. When no lane of the wave holds an
+                // element of this chunk within 708 of the max (a masked span of attention scores, the
+                // padding past the row), every exponential of the chunk is exactly 0: skip them all.
+                bool some = false;
 #pragma unroll
-            for (int i = 0; i < V; ++i) {
-                const int64_t e = (static_cast<int64_t>(c) * G + lane) * V + i;
-                E v = M::ex(x[c][i], mx);
-                if (!(e < a.n)) v = E(0);
-                sum += M::wide(v);
-                if constexpr (!LOG) ex[c][i] = v;
+                for (int i = 0; i < V; ++i) some |= !(static_cast<double>(x[i]) - static_cast<double>(mx) < -708.0);
+                if (__builtin_amdgcn_ballot_w64(some) != 0) {
+#pragma unroll
+                    for (int i = 0; i < V; ++i) e[i] = M::ex(x[i], mx);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < V; ++i) e[i] = 0.0;
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < V; ++i) e[i] = M::ex(x[i], mx);
             }
+            if constexpr (std::is_same_v<E, float>) {
+                // Eight f32 terms pairwise (relative error ~2^-22), then one f64 addition per chunk.
+                float part = ((e[0] + e[1]) + (e[2] + e[3])) + ((e[4] + e[5]) + (e[6] + e[7]));
+                sum += static_cast<double>(part);
+            } else {
+#pragma unroll
+                for (int i = 0; i < V; ++i) sum += M::wide(e[i]);
+            }
+            if constexpr (kKeep) {
+#pragma unroll
+                for (int i = 0; i < V; ++i) ex[c][i] = e[i];
+            }
+            // One chunk at a time: interleaving the chunks' independent chains would multiply the live
+            // temporaries.
+            __builtin_amdgcn_sched_barrier(0);
         }
         sum = row_fold<G>(SumOp{}, sum, lds);
         // Phase 3: write once.
-        const E scale = LOG ? M::lg(sum) : M::inv(sum);
+        const E scale = LOG ? M::lg(sum) : M::scale(sum);
 #pragma unroll
         for (int c = 0; c < C; ++c) {
-            const int64_t tile = static_cast<int64_t>(c) * G + lane;
-            T res[V];
+            const int tile = c * G + lane;
+            X x[V];
+            forget(raw[c]);
+            M::unpack(raw[c], x);
+            decltype(M::logsoft(x[0], mx, scale)) res[V];
 #pragma unroll
             for (int i = 0; i < V; ++i) {
-                if constexpr (LOG) res[i] = M::logsoft(x[c][i], mx, scale);
-                else res[i] = M::soft(ex[c][i], scale);
+                if constexpr (LOG) res[i] = M::logsoft(x[i], mx, scale);
+                else res[i] = M::soft(x[i], mx, kKeep ? ex[kKeep ? c : 0][kKeep ? i : 0] : E(0), scale);
             }
             if (live && tile < nvec) {
-                store_tile<T, V, kStreamStores>(reinterpret_cast<char *>(out + tile * V), res);
-            } else if (live) {
-#pragma unroll
-                for (int i = 0; i < V; ++i) {
-                    const int64_t e = tile * V + i;
-                    if (e < a.n) out[e] = res[i];
-                }
+                u32x4 *q = reinterpret_cast<u32x4 *>(reinterpret_cast<char *>(out) + static_cast<uint32_t>(tile) * 16u);
+                if constexpr (kStreamStores) __builtin_nontemporal_store(M::pack(res), q);
+                else *q = M::pack(res);
             }
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
 }
@@ -266,10 +382,11 @@ __global__ void __launch_bounds__(kBlock) softmax_stream_kernel(SoftmaxArgs a) {
         double sum = 0.0;
         for (int64_t k = lane; k < n; k += G) sum += M::wide(M::ex(M::load(src[k * a.si]), mx));
         sum = row_fold<G>(SumOp{}, sum, lds);
-        const E scale = LOG ? M::lg(sum) : M::inv(sum);
+        const E scale = LOG ? M::lg(sum) : M::scale(sum);
         for (int64_t k = lane; k < n; k += G) {
             X v = M::load(src[k * a.si]);
-            out[k * a.so] = LOG ? M::logsoft(v, mx, scale) : M::soft(M::ex(v, mx), scale);
+            if constexpr (LOG) out[k * a.so] = M::down(M::logsoft(v, mx, scale));
+            else out[k * a.so] = M::down(M::soft(v, mx, M::kKeep ? M::ex(v, mx) : E(0), scale));
         }
     }
 }
@@ -315,7 +432,9 @@ int64_t walk_pair(const hmr_tensor_desc &out_rows, const hmr_tensor_desc &src_ro
     return count;
 }
 
-constexpr int kMaxTiles = 8;  // 128-bit tiles a lane keeps (8 x 16 B of the row)
+// 128-bit chunks of the row a lane keeps: 8 (32 f32 or 16 f64 values, plus their f64 exponentials),
+// or 16 packed chunks (128 values) of a 16-bit type, whose exponentials are not kept.
+constexpr int max_tiles(int elem) { return elem == 2 ? 16 : 8; }
 
 // The plan depends on the source only (sizes, strides, alignment), so that the size query, which
 // does not see the output, agrees with the launch; the launch falls back to streaming by itself
@@ -328,13 +447,13 @@ SoftmaxPlan plan_softmax(const hmr_tensor_desc &src_rows, int64_t n, int64_t si,
                    reinterpret_cast<uintptr_t>(static_cast<char *>(src_rows.data) + src_rows.offset * elem) % 16 == 0;
     for (int d = 0; aligned && d < ws.ndim; ++d) aligned = (ws.stride[d] * elem) % 16 == 0;
     const int64_t tiles = (n + vec - 1) / vec;  // 128-bit tiles in a row
-    if (aligned && n >= 16) {
+    if (aligned && n >= 16 && n % vec == 0) {
         for (int g : {kWave, kBlock, 1024}) {
             int64_t per = (tiles + g - 1) / g;
-            if (per <= kMaxTiles) {
+            if (per <= max_tiles(elem)) {
                 p.regs = true;
                 p.group = g;
-                p.tiles = per <= 1 ? 1 : (per <= 2 ? 2 : (per <= 4 ? 4 : 8));
+                p.tiles = per <= 1 ? 1 : (per <= 2 ? 2 : (per <= 4 ? 4 : (per <= 8 ? 8 : 16)));
                 return p;
             }
         }
@@ -356,14 +475,21 @@ void launch_softmax(const SoftmaxPlan &p, const SoftmaxArgs &a, bool out_ok, hip
         auto run = [&](auto g, auto c) {
             constexpr int G = decltype(g)::value, C = decltype(c)::value;
             constexpr int kThreads = G > kBlock ? G : kBlock;
-            hipLaunchKernelGGL((softmax_regs_kernel<T, G, C, LOG>), blocks(kThreads / G), dim3(kThreads), 0, stream, a);
+            if (a.src_rows.ndim <= 1) {
+                hipLaunchKernelGGL((softmax_regs_kernel<T, G, C, LOG, false>), blocks(kThreads / G), dim3(kThreads), 0, stream, a);
+            } else {
+                hipLaunchKernelGGL((softmax_regs_kernel<T, G, C, LOG, true>), blocks(kThreads / G), dim3(kThreads), 0, stream, a);
+            }
         };
         auto with_tiles = [&](auto g) {
             switch (p.tiles) {
                 case 1: run(g, IntTag<1>{}); break;
                 case 2: run(g, IntTag<2>{}); break;
                 case 4: run(g, IntTag<4>{}); break;
-                default: run(g, IntTag<8>{}); break;
+                case 8: run(g, IntTag<8>{}); break;
+                default:
+                    if constexpr (sizeof(T) == 2) run(g, IntTag<16>{});
+                    break;
             }
         };
         if (p.group == kWave) with_tiles(IntTag<kWave>{});
