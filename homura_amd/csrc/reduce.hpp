@@ -73,13 +73,22 @@ __device__ __forceinline__ A shfl_xor_any(A v, int mask) {
 
 // Folds the accumulators of the 64 lanes of a wave; every lane ends with the result. The fold is
 // a fixed butterfly, so the association order is the same in every run.
+template <class Op, class = void>
+struct IsCommutative : std::false_type {};
+template <class Op>
+struct IsCommutative<Op, std::enable_if_t<Op::kCommutative>> : std::true_type {};
+
 template <class Op>
 __device__ __forceinline__ typename Op::Acc wave_fold(const Op &op, typename Op::Acc a) {
 #pragma unroll
     for (int mask = 1; mask < kWave; mask <<= 1) {
         typename Op::Acc b = shfl_xor_any(a, mask);
-        // Lower lane first keeps the operand order identical on both partners.
-        a = (threadIdx.x & mask) ? op.combine(b, a) : op.combine(a, b);
+        if constexpr (IsCommutative<Op>::value) {
+            a = op.combine(a, b);  // combine(a, b) and combine(b, a) have the same bits: both partners agree
+        } else {
+            // Lower lane first keeps the operand order identical on both partners.
+            a = (threadIdx.x & mask) ? op.combine(b, a) : op.combine(a, b);
+        }
     }
     return a;
 }

@@ -34,31 +34,40 @@ namespace {
 
 // ---- exp in the evaluation type ------------------------------------------------------------------
 
-// exp(t) for t <= 0 (or NaN) in f64, without a branch. |relative error| < 2^-45.
-__device__ __forceinline__ double exp_neg_f64(double t) {
+// exp(t) for t <= 0 (or NaN) in f64, without a branch. |relative error| < 2^-36: an f32 result
+// computed from it differs from the correctly rounded one only within 2^-12 ulp of a rounding boundary.
+// Below -708 (where exp underflows; -inf included) the arithmetic runs on meaningless values, which the
+// final select replaces by 0; a NaN propagates through every step.
+//
+// The Horner steps are written as the instruction itself with the coefficient in a scalar register pair:
+// left to the compiler each step becomes a register copy of the coefficient plus a two-address v_fmac_f64.
+__device__ __forceinline__ double horner_step(double p, double r, double coefficient) {
+    double out;
+    asm("v_fma_f64 %0, %1, %2, %3" : "=v"(out) : "v"(p), "v"(r), "s"(coefficient));
+    return out;
+}
+
+// `dead`: the caller does not want this lane's value (it gets 0).
+__device__ __forceinline__ double exp_neg_f64(double t, bool dead = false) {
     const double kLog2e = 1.4426950408889634074;
     const double kLn2Hi = 6.93147180369123816490e-01;
     const double kLn2Lo = 1.90821492927058770002e-10;
-    const double tc = t < -708.0 ? -708.0 : t;  // the underflow region (and -inf) is answered below; NaN passes
-    double n = rint(tc * kLog2e);
-    double r = fma(-n, kLn2Hi, tc);
+    double n = rint(t * kLog2e);
+    double r = fma(-n, kLn2Hi, t);
     r = fma(-n, kLn2Lo, r);  // |r| <= 0.3466
-    // Taylor to degree 11: remainder < 0.3466^12 / 12! < 2^-47.
-    double p = 1.0 / 39916800.0;
-    p = fma(p, r, 1.0 / 3628800.0);
-    p = fma(p, r, 1.0 / 362880.0);
-    p = fma(p, r, 1.0 / 40320.0);
-    p = fma(p, r, 1.0 / 5040.0);
-    p = fma(p, r, 1.0 / 720.0);
-    p = fma(p, r, 1.0 / 120.0);
-    p = fma(p, r, 1.0 / 24.0);
-    p = fma(p, r, 1.0 / 6.0);
+    // Taylor to degree 9: remainder < 0.3466^10 / 10! < 2^-37.
+    double p = horner_step(1.0 / 362880.0, r, 1.0 / 40320.0);
+    p = horner_step(p, r, 1.0 / 5040.0);
+    p = horner_step(p, r, 1.0 / 720.0);
+    p = horner_step(p, r, 1.0 / 120.0);
+    p = horner_step(p, r, 1.0 / 24.0);
+    p = horner_step(p, r, 1.0 / 6.0);
     p = fma(p, r, 0.5);
     p = fma(p, r, 1.0);
     p = fma(p, r, 1.0);
-    // Scale by 2^n, n in [-1022, 0]: add to the exponent field (of a NaN: n is 0).
-    int64_t bits = __double_as_longlong(p) + (static_cast<int64_t>(static_cast<int32_t>(n)) << 52);
-    return t < -708.0 ? 0.0 : __longlong_as_double(bits);
+    // Scale by 2^n, n in [-1022, 0].
+    p = ldexp(p, static_cast<int>(n));
+    return (t < -708.0 || dead) ? 0.0 : p;
 }
 
 template <class T>
@@ -70,7 +79,8 @@ constexpr float kLog2eF = 1.44269504088896340736f;
 // of an 8- or 11-bit result, so the exponentials come from the hardware's 2^x (v_exp_f32, 1 ulp):
 //   for the sum   2^((x - max) log2 e)              (results below 2^-126 may flush: they are
 //                                                    below 2^-126 of a sum that is at least 1)
-//   for the output 2^((x - max) log2 e - log2 sum)  through exp2f, which keeps subnormal results.
+//   for the output 2^((x - max) log2 e - log2 sum)  evaluated as ldexp(2^(.. + 64), -64), which keeps
+//                                                    subnormal results (v_exp_f32 alone flushes them).
 // The output form is evaluated per element in the last phase instead of keeping every exponential
 // in registers, which lets a lane hold 128 packed elements of its row.
 template <class T>
@@ -78,7 +88,6 @@ struct HalfMath {
     using X = float;  // a row element in registers
     using E = float;  // exp(x - max), and the per-row scale
     static constexpr bool kKeep = false;
-    static constexpr uint32_t kNegInfPair = std::is_same_v<T, bf16_t> ? 0xFF80FF80u : 0xFC00FC00u;
     static __device__ __forceinline__ X load(T v) { return Comp<T>::up(v); }
     static __device__ __forceinline__ void unpack(const u32x4 &r, X (&x)[8]) {
 #pragma unroll
@@ -107,10 +116,10 @@ struct HalfMath {
     }
     static __device__ __forceinline__ E ex(X x, X mx) { return __builtin_amdgcn_exp2f((x - mx) * kLog2eF); }
     static __device__ __forceinline__ double wide(E e) { return static_cast<double>(e); }
-    static __device__ __forceinline__ E scale(double sum) { return __builtin_log2f(static_cast<float>(sum)); }
+    static __device__ __forceinline__ E scale(double sum) { return 64.0f - __builtin_log2f(static_cast<float>(sum)); }
     static __device__ __forceinline__ E lg(double sum) { return static_cast<float>(log(sum)); }
-    static __device__ __forceinline__ float soft(X x, X mx, E, E log2_sum) {
-        return __builtin_exp2f((x - mx) * kLog2eF - log2_sum);
+    static __device__ __forceinline__ float soft(X x, X mx, E, E bias) {  // bias = 64 - log2 sum
+        return __builtin_ldexpf(__builtin_amdgcn_exp2f(__builtin_fmaf(x - mx, kLog2eF, bias)), -64);
     }
     static __device__ __forceinline__ float logsoft(X x, X mx, E log_sum) { return x - mx - log_sum; }
     static __device__ __forceinline__ T down(float y) { return Comp<T>::down(y); }
@@ -130,7 +139,9 @@ struct SoftmaxMath<float> {
 #pragma unroll
         for (int i = 0; i < 4; ++i) x[i] = __uint_as_float(r[i]);
     }
-    static __device__ __forceinline__ E ex(X x, X mx) { return exp_neg_f64(static_cast<double>(x) - static_cast<double>(mx)); }
+    static __device__ __forceinline__ E ex(X x, X mx, bool dead = false) {
+        return exp_neg_f64(static_cast<double>(x) - static_cast<double>(mx), dead);
+    }
     static __device__ __forceinline__ double wide(E e) { return e; }
     static __device__ __forceinline__ E scale(double sum) { return 1.0 / sum; }
     static __device__ __forceinline__ E lg(double sum) { return log(sum); }
@@ -157,7 +168,7 @@ struct SoftmaxMath<double> {
                                                              (static_cast<uint64_t>(r[2 * i + 1]) << 32)));
         }
     }
-    static __device__ __forceinline__ E ex(X x, X mx) { return exp(x - mx); }
+    static __device__ __forceinline__ E ex(X x, X mx, bool dead = false) { return dead ? 0.0 : exp(x - mx); }
     static __device__ __forceinline__ double wide(E e) { return e; }
     static __device__ __forceinline__ E scale(double sum) { return sum; }
     static __device__ __forceinline__ E lg(double sum) { return log(sum); }
@@ -171,19 +182,16 @@ struct SoftmaxMath<double> {
     }
 };
 
-// A 16-byte chunk whose every element is -inf: what pads a row past its end. -inf neither raises the
-// max nor adds to the sum (exp(-inf - max) is exactly 0; when the max itself is -inf the row's own
-// elements already make everything NaN, as on the CPU).
-template <class T>
-__device__ __forceinline__ u32x4 neg_inf_chunk() {
-    if constexpr (std::is_same_v<T, float>) {
-        return u32x4{0xFF800000u, 0xFF800000u, 0xFF800000u, 0xFF800000u};
-    } else if constexpr (std::is_same_v<T, double>) {
-        return u32x4{0u, 0xFFF00000u, 0u, 0xFFF00000u};
-    } else {
-        constexpr uint32_t w = SoftmaxMath<T>::kNegInfPair;
-        return u32x4{w, w, w, w};
-    }
+// max(m, a, b) in one instruction. How a NaN operand is treated does not matter to softmax: a row
+// holding a NaN comes out all NaN whatever its max is taken to be.
+__device__ __forceinline__ float max3(float m, float a, float b) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(m), "v"(a), "v"(b));
+    return r;
+}
+__device__ __forceinline__ double max3(double m, double a, double b) {
+    m = a > m ? a : m;
+    return b > m ? b : m;
 }
 
 // Makes the compiler treat a chunk as newly produced. Each phase unpacks the row's chunks again; without
@@ -194,30 +202,35 @@ __device__ __forceinline__ void forget(u32x4 &r) { asm volatile("" : "+v"(r)); }
 // ---- combining across the lanes of a row ---------------------------------------------------------
 
 struct MaxOp {
+    static constexpr bool kCommutative = true;
     using Acc = double;
     __device__ __forceinline__ Acc combine(Acc a, Acc b) const { return b > a ? b : a; }
 };
 struct MaxOpF {
+    static constexpr bool kCommutative = true;
     using Acc = float;
     __device__ __forceinline__ Acc combine(Acc a, Acc b) const { return b > a ? b : a; }
 };
 struct SumOp {
+    static constexpr bool kCommutative = true;  // IEEE addition is
     using Acc = double;
     __device__ __forceinline__ Acc combine(Acc a, Acc b) const { return a + b; }
 };
 
-// Folds `v` over the G lanes that share a row (G = 64: one wave; else the whole workgroup).
+// Folds `v` over the G lanes that share a row: one wave, or G / 64 neighbouring waves of the workgroup
+// that meet in LDS (`lds` has one slot per wave of the workgroup).
 template <int G, class Op>
 __device__ __forceinline__ typename Op::Acc row_fold(const Op &op, typename Op::Acc v, typename Op::Acc *lds) {
     v = wave_fold(op, v);
     if constexpr (G > kWave) {
         constexpr int kWaves = G / kWave;
+        const int first = static_cast<int>(threadIdx.x) / G * kWaves;
         __syncthreads();
         if (threadIdx.x % kWave == 0) lds[threadIdx.x / kWave] = v;
         __syncthreads();
-        v = lds[0];
+        v = lds[first];
 #pragma unroll
-        for (int w = 1; w < kWaves; ++w) v = op.combine(v, lds[w]);
+        for (int w = 1; w < kWaves; ++w) v = op.combine(v, lds[first + w]);
     }
     return v;
 }
@@ -236,9 +249,9 @@ struct SoftmaxArgs {
 // chunks of V elements: chunk c of lane l covers elements (c*G + l)*V .. +V, so every load of the
 // group is one contiguous, coalesced span. Rows are whole chunks (n is a multiple of V).
 //
-// All C loads of a lane are issued back to back and unconditionally (a chunk past the row's end
-// re-reads the row's last chunk and is then replaced by -inf): a branch between loads would make
-// each wait for the one before.
+// All C loads of a lane are issued back to back and unconditionally: a branch between loads would
+// make each wait for the one before. A chunk past the row's end re-reads the row's last chunk, which
+// cannot change the max, and is left out of the sum and of the stores.
 //
 // WALK = false: the rows form one dimension (row r starts r * stride elements in), which is what a
 // contiguous tensor gives; WALK = true: up to 25 row dimensions, decoded per row.
@@ -252,7 +265,7 @@ __global__ void __launch_bounds__(G > kBlock ? G : kBlock) softmax_regs_kernel(S
     constexpr int kThreads = G > kBlock ? G : kBlock;
     constexpr int kRowsPerBlock = kThreads / G;
     constexpr bool kKeep = M::kKeep && !LOG;
-    __shared__ double lds[G > kWave ? G / kWave : 1];
+    __shared__ double lds[kThreads / kWave];
     const int lane = threadIdx.x % G;
     const int64_t groups = (a.nrows + kRowsPerBlock - 1) / kRowsPerBlock;
     const int nvec = static_cast<int>(a.n / V);  // chunks in a row (>= 1)
@@ -274,58 +287,51 @@ __global__ void __launch_bounds__(G > kBlock ? G : kBlock) softmax_regs_kernel(S
             else raw[c] = *q;
         }
         __builtin_amdgcn_sched_barrier(0);  // every load is out before anything waits for one
-#pragma unroll
-        for (int c = 0; c < C; ++c) {
-            if (c * G + lane >= nvec) raw[c] = neg_inf_chunk<T>();
-        }
-        // Phase 1: max. A NaN never replaces (v > m is false), as on the CPU.
+        // Phase 1: max.
         X mx = -__builtin_huge_valf();
 #pragma unroll
         for (int c = 0; c < C; ++c) {
             X x[V];
             M::unpack(raw[c], x);
 #pragma unroll
-            for (int i = 0; i < V; ++i) mx = x[i] > mx ? x[i] : mx;
+            for (int i = 0; i < V; i += 2) mx = max3(mx, x[i], x[i + 1]);
         }
         mx = row_fold<G>(MaxFold{}, mx, reinterpret_cast<X *>(lds));
         // Phase 2: exponentials and their f64 sum.
         double sum = 0.0;
-        E ex[kKeep ? C : 1][kKeep ? V : 1];
+        E ex[kKeep ? C : 1][kKeep ? V : 1];  // chunk c is defined where did[c]
+        bool did[C];
 #pragma unroll
         for (int c = 0; c < C; ++c) {
             X x[V];
             forget(raw[c]);
             M::unpack(raw[c], x);
-            E e[V];
+            const bool inside = c * G + lane < nvec;
             if constexpr (std::is_same_v<E, double>) {
-                // An f64 exponential is some thirty instructions. When no lane of the wave holds an
-                // element of this chunk within 708 of the max (a masked span of attention scores, the
-                // padding past the row), every exponential of the chunk is exactly 0: skip them all.
+                // An f64 exponential is some twenty-five instructions. When no lane of the wave holds an
+                // element of this chunk within 708 of the max (a masked span of attention scores, a
+                // chunk past the row's end), every exponential of the chunk is exactly 0: skip them all.
                 bool some = false;
 #pragma unroll
                 for (int i = 0; i < V; ++i) some |= !(static_cast<double>(x[i]) - static_cast<double>(mx) < -708.0);
-                if (__builtin_amdgcn_ballot_w64(some) != 0) {
+                did[c] = __builtin_amdgcn_ballot_w64(some && inside) != 0;
+                if (did[c]) {
 #pragma unroll
-                    for (int i = 0; i < V; ++i) e[i] = M::ex(x[i], mx);
-                } else {
-#pragma unroll
-                    for (int i = 0; i < V; ++i) e[i] = 0.0;
+                    for (int i = 0; i < V; ++i) {
+                        const double v = M::ex(x[i], mx, !inside);
+                        sum += v;
+                        if constexpr (kKeep) ex[c][i] = v;
+                    }
                 }
             } else {
-#pragma unroll
-                for (int i = 0; i < V; ++i) e[i] = M::ex(x[i], mx);
-            }
-            if constexpr (std::is_same_v<E, float>) {
                 // Eight f32 terms pairwise (relative error ~2^-22), then one f64 addition per chunk.
-                float part = ((e[0] + e[1]) + (e[2] + e[3])) + ((e[4] + e[5]) + (e[6] + e[7]));
-                sum += static_cast<double>(part);
-            } else {
+                if (inside) {
+                    E e[V];
 #pragma unroll
-                for (int i = 0; i < V; ++i) sum += M::wide(e[i]);
-            }
-            if constexpr (kKeep) {
-#pragma unroll
-                for (int i = 0; i < V; ++i) ex[c][i] = e[i];
+                    for (int i = 0; i < V; ++i) e[i] = M::ex(x[i], mx);
+                    float part = ((e[0] + e[1]) + (e[2] + e[3])) + ((e[4] + e[5]) + (e[6] + e[7]));
+                    sum += static_cast<double>(part);
+                }
             }
             // One chunk at a time: interleaving the chunks' independent chains would multiply the live
             // temporaries.
@@ -343,8 +349,15 @@ __global__ void __launch_bounds__(G > kBlock ? G : kBlock) softmax_regs_kernel(S
             decltype(M::logsoft(x[0], mx, scale)) res[V];
 #pragma unroll
             for (int i = 0; i < V; ++i) {
-                if constexpr (LOG) res[i] = M::logsoft(x[i], mx, scale);
-                else res[i] = M::soft(x[i], mx, kKeep ? ex[kKeep ? c : 0][kKeep ? i : 0] : E(0), scale);
+                if constexpr (LOG) {
+                    res[i] = M::logsoft(x[i], mx, scale);
+                } else if constexpr (kKeep) {
+                    // A skipped chunk holds exact zeros: 0 * scale, which is 0 unless the row's sum is NaN.
+                    res[i] = M::soft(x[i], mx, E(0), scale);
+                    if (did[c]) res[i] = M::soft(x[i], mx, ex[c][i], scale);
+                } else {
+                    res[i] = M::soft(x[i], mx, E(0), scale);
+                }
             }
             if (live && tile < nvec) {
                 u32x4 *q = reinterpret_cast<u32x4 *>(reinterpret_cast<char *>(out) + static_cast<uint32_t>(tile) * 16u);
@@ -364,7 +377,7 @@ __global__ void __launch_bounds__(kBlock) softmax_stream_kernel(SoftmaxArgs a) {
     using E = typename M::E;
     using MaxFold = std::conditional_t<std::is_same_v<X, float>, MaxOpF, MaxOp>;
     constexpr int kRowsPerBlock = kBlock / G;
-    __shared__ double lds[G > kWave ? G / kWave : 1];
+    __shared__ double lds[kBlock / kWave];
     const int lane = threadIdx.x % G;
     const int64_t groups = (a.nrows + kRowsPerBlock - 1) / kRowsPerBlock;
     for (int64_t g = blockIdx.x; g < groups; g += gridDim.x) {
@@ -448,9 +461,21 @@ SoftmaxPlan plan_softmax(const hmr_tensor_desc &src_rows, int64_t n, int64_t si,
     for (int d = 0; aligned && d < ws.ndim; ++d) aligned = (ws.stride[d] * elem) % 16 == 0;
     const int64_t tiles = (n + vec - 1) / vec;  // 128-bit tiles in a row
     if (aligned && n >= 16 && n % vec == 0) {
-        for (int g : {kWave, kBlock, 1024}) {
+        // Lanes per row and chunks per lane, first fit. 16-bit rows stay packed (4 registers per chunk);
+        // wider rows also keep their f64 exponentials (8 more registers per f32 chunk), so they spread over
+        // two waves before a lane takes more than four chunks: more resident waves hide the row loads.
+        struct Step {
+            int group, tiles;
+        };
+        static const Step half_steps[] = {{kWave, 16}, {kBlock, 16}, {1024, 16}};
+        static const Step wide_steps[] = {{kWave, 4}, {128, 4}, {kBlock, 8}, {1024, 8}};
+        const Step *steps = elem == 2 ? half_steps : wide_steps;
+        const int nsteps = elem == 2 ? 3 : 4;
+        for (int k = 0; k < nsteps; ++k) {
+            const int g = steps[k].group;
+            const int64_t lim = steps[k].tiles;
             int64_t per = (tiles + g - 1) / g;
-            if (per <= max_tiles(elem)) {
+            if (per <= lim && per <= max_tiles(elem)) {
                 p.regs = true;
                 p.group = g;
                 p.tiles = per <= 1 ? 1 : (per <= 2 ? 2 : (per <= 4 ? 4 : (per <= 8 ? 8 : 16)));
@@ -493,6 +518,7 @@ void launch_softmax(const SoftmaxPlan &p, const SoftmaxArgs &a, bool out_ok, hip
             }
         };
         if (p.group == kWave) with_tiles(IntTag<kWave>{});
+        else if (p.group == 128) with_tiles(IntTag<128>{});
         else if (p.group == kBlock) with_tiles(IntTag<kBlock>{});
         else with_tiles(IntTag<1024>{});
         return;

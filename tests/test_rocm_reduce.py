@@ -354,7 +354,7 @@ def test_every_plan_folds_each_element_once():
 
 
 SOFTMAX_PLAN_SHAPES = [
-    ([700, 200], 1, DT.F32, 64, 4), ([64, 2048], 1, DT.F32, 64, 32), ([16, 4096], 1, DT.F32, 256, 16),
+    ([700, 200], 1, DT.F32, 64, 4), ([64, 1024], 1, DT.F32, 64, 16), ([64, 2048], 1, DT.F32, 128, 16), ([16, 4096], 1, DT.F32, 256, 16),
     ([8, 32000], 1, DT.BF16, 256, 128), ([4, 100000], 1, DT.BF16, 1024, 128), ([5, 8192], 1, DT.F16, 64, 128),
     ([8, 32768], 1, DT.F32, 1024, 32), ([3, 70000], 1, DT.F32, 256, 0),
     ([2048, 9], 0, DT.F32, 64, 0), ([40, 8, 1000], 1, DT.F16, 64, 0),
