@@ -5,7 +5,9 @@
 
 #include <hip/hip_runtime.h>
 
+#include <cstdint>
 #include <exception>
+#include <mutex>
 #include <new>
 #include <string>
 
@@ -16,6 +18,12 @@ struct hmr_context {
     int device;
     hipStream_t stream;
     int compute_units;  // multiProcessorCount of the device (256 on MI355X), for grid sizing
+    // Result tables of the 16-bit unary operations (one 128 KiB table per operation and dtype, every
+    // input pattern -> its output pattern). The block is allocated at the first use and lives as long
+    // as the context; a table is filled, on `stream`, by the first call that needs it.
+    std::mutex table_lock;
+    void *tables = nullptr;
+    uint64_t tables_filled = 0;  // bit per table
 };
 
 namespace hmr {

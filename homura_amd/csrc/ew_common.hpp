@@ -10,14 +10,22 @@ namespace hmr {
 // Runs an elementwise entry point: prepares the call from `descs` (nullptr = constant), returns
 // early for empty tensors, and launches through `pick`, which returns false when there is no
 // kernel for the dtypes/op.
-template <class Pick>
+// `before(call)` runs after the checks and before the launch bracket; it may fail the call.
+template <class Pick, class Before>
 hmr_status run_map(hmr_context_t ctx, const char *what, int count, const hmr_tensor_desc *const *descs,
-                   const uint64_t *bits, Pick pick) {
+                   const uint64_t *bits, Pick pick, Before before) {
     MapCall call;
     if (hmr_status s = prepare_map(call, count, descs, bits)) return s;
     if (call.n == 0) return HMR_OK;
     call.compute_units = ctx->compute_units;
+    if (hmr_status s = before(call)) return s;
     return launch_on(ctx, what, [&](hipStream_t stream) { return pick(call, stream); });
+}
+
+template <class Pick>
+hmr_status run_map(hmr_context_t ctx, const char *what, int count, const hmr_tensor_desc *const *descs,
+                   const uint64_t *bits, Pick pick) {
+    return run_map(ctx, what, count, descs, bits, pick, [](const MapCall &) { return HMR_OK; });
 }
 
 }  // namespace hmr

@@ -1,8 +1,33 @@
 // hmr_unary (ref: csrc/homura_rocm.h:202, csrc/elementwise.hip:996-1007).
 #include "ew_common.hpp"
+#include "map_table.hpp"
 
 namespace hmr {
 namespace {
+
+// 16-bit operations that go through a result table when the tensor is large: everything that costs
+// more than a handful of instructions per element.
+constexpr int kFirstTableOp = HMR_UNARY_EXP, kLastTableOp = HMR_UNARY_GELU_TANH;
+constexpr int kTableOps = kLastTableOp - kFirstTableOp + 1;
+constexpr int kTableSlots = 2 * kTableOps;  // f16, bf16
+
+bool is_table_op(int op, int dtype) {
+    return (dtype == HMR_F16 || dtype == HMR_BF16) && op >= kFirstTableOp && op <= kLastTableOp;
+}
+int table_slot(int op, int dtype) { return (dtype == HMR_BF16 ? kTableOps : 0) + (op - kFirstTableOp); }
+
+// Allocates the context's block of tables at the first use.
+hmr_status ensure_tables(hmr_context_t ctx) {
+    std::lock_guard<std::mutex> lock(ctx->table_lock);
+    if (ctx->tables != nullptr) return HMR_OK;
+    DeviceGuard guard;
+    if (hmr_status s = guard.enter(ctx->device)) return s;
+    void *p = nullptr;
+    HMR_HIP(hipMalloc(&p, kTableSlots * kTableBytes));
+    ctx->tables = p;
+    ctx->tables_filled = 0;
+    return HMR_OK;
+}
 
 using FloatOps = std::integer_sequence<int, HMR_UNARY_NEG, HMR_UNARY_ABS, HMR_UNARY_SIGN, HMR_UNARY_RELU,
                                        HMR_UNARY_EXP, HMR_UNARY_LOG, HMR_UNARY_SQRT, HMR_UNARY_RSQRT,
@@ -11,7 +36,7 @@ using FloatOps = std::integer_sequence<int, HMR_UNARY_NEG, HMR_UNARY_ABS, HMR_UN
                                        HMR_UNARY_GELU, HMR_UNARY_GELU_TANH>;
 using IntOps = std::integer_sequence<int, HMR_UNARY_NEG, HMR_UNARY_ABS, HMR_UNARY_SIGN, HMR_UNARY_RELU>;
 
-bool pick_unary(int op, int out_dtype, int dtype, const MapCall &call, hipStream_t stream) {
+bool pick_unary(hmr_context_t ctx, int op, int out_dtype, int dtype, const MapCall &call, hipStream_t stream) {
     if (op == HMR_UNARY_LOGICAL_NOT) {
         if (out_dtype != HMR_BOOL) return false;
         return with_any_type(dtype, [&](auto t) {
@@ -34,7 +59,27 @@ bool pick_unary(int op, int out_dtype, int dtype, const MapCall &call, hipStream
     }
     with_float_type(dtype, [&](auto t) {
         using T = typename decltype(t)::type;
-        done = with_code(op, FloatOps{}, [&](auto o) { launch_map<UnaryFloat<decltype(o)::value, T>>(call, stream); });
+        done = with_code(op, FloatOps{}, [&](auto o) {
+            using F = UnaryFloat<decltype(o)::value, T>;
+            if constexpr (sizeof(T) == 2 && decltype(o)::value >= kFirstTableOp && decltype(o)::value <= kLastTableOp) {
+                if (ctx->tables != nullptr && table_applies<F>(call)) {
+                    const int slot = table_slot(op, dtype);
+                    uint16_t *table = reinterpret_cast<uint16_t *>(static_cast<char *>(ctx->tables) + slot * kTableBytes);
+                    {
+                        // The fill is queued, under the lock, on the context's one stream: ahead of every
+                        // lookup of this table that any thread queues afterwards.
+                        std::lock_guard<std::mutex> lock(ctx->table_lock);
+                        if (!(ctx->tables_filled >> slot & 1u)) {
+                            launch_table_fill<F>(table, stream);
+                            ctx->tables_filled |= uint64_t{1} << slot;
+                        }
+                    }
+                    launch_table<F>(call, table, stream);
+                    return;
+                }
+            }
+            launch_map<F>(call, stream);
+        });
     });
     return done;
 }
@@ -46,8 +91,16 @@ extern "C" hmr_status hmr_unary(hmr_context_t ctx, int32_t op, const hmr_tensor_
                                 const hmr_tensor_desc *src) {
     return hmr::guarded([&] {
         const hmr_tensor_desc *descs[2] = {out, src};
-        return hmr::run_map(ctx, "unary", 2, descs, nullptr, [&](const hmr::MapCall &call, hipStream_t stream) {
-            return hmr::pick_unary(op, out->dtype, src->dtype, call, stream);
-        });
+        return hmr::run_map(
+            ctx, "unary", 2, descs, nullptr,
+            [&](const hmr::MapCall &call, hipStream_t stream) {
+                return hmr::pick_unary(ctx, op, out->dtype, src->dtype, call, stream);
+            },
+            [&](const hmr::MapCall &call) {
+                if (out->dtype == src->dtype && hmr::is_table_op(op, src->dtype) && call.n >= hmr::kTableMinElements) {
+                    return hmr::ensure_tables(ctx);
+                }
+                return HMR_OK;
+            });
     });
 }

@@ -570,10 +570,10 @@ int pick_variant(const MapCall &c) {
     return 2;
 }
 
+// The variant a call takes with -1 (one huge contiguous dimension) resolved to 0 or 3.
 template <class F>
-void launch_map(const MapCall &c, hipStream_t stream) {
+int resolve_variant(const MapCall &c) {
     using T = MapTraits<F>;
-    constexpr int NOPS = F::N + 1;
     int variant = pick_variant<F>(c);
     if (variant == -1) {
         // One huge contiguous dimension (>= 2^31 elements): the FLAT rows kernel indexes in 64 bits.
@@ -587,38 +587,55 @@ void launch_map(const MapCall &c, hipStream_t stream) {
         }
         variant = ok ? 0 : 3;
     }
-    if (variant <= 1) {
-        RowsArgs<NOPS> a{};
-        a.n = c.n;
-        a.const_mask = 0;
-        a.bcast_mask = 0;
-        const int last = c.ndim - 1;
-        for (int k = 0; k < NOPS; ++k) {
-            a.ptr[k] = c.is_const[k] ? c.ptr[0] : c.ptr[k];  // a constant's (ignored) chunk is read from the output
-            a.cbits[k] = c.cbits[k];
-            if (c.is_const[k]) a.const_mask |= 1u << k;
-            else if (c.ndim == 0 || c.stride[k][last] == 0) a.bcast_mask |= k == 0 ? 0u : 1u << k;
+    return variant;
+}
+
+// Kernel arguments of the rows kernel for a call of variant 0 (flat) or 1 (outer dimensions).
+template <class F>
+RowsArgs<F::N + 1> rows_args(const MapCall &c, int variant) {
+    using T = MapTraits<F>;
+    constexpr int NOPS = F::N + 1;
+    RowsArgs<NOPS> a{};
+    a.n = c.n;
+    a.const_mask = 0;
+    a.bcast_mask = 0;
+    const int last = c.ndim - 1;
+    for (int k = 0; k < NOPS; ++k) {
+        a.ptr[k] = c.is_const[k] ? c.ptr[0] : c.ptr[k];  // a constant's (ignored) chunk is read from the output
+        a.cbits[k] = c.cbits[k];
+        if (c.is_const[k]) a.const_mask |= 1u << k;
+        else if (c.ndim == 0 || c.stride[k][last] == 0) a.bcast_mask |= k == 0 ? 0u : 1u << k;
+    }
+    a.stream = c.n * (T::so + T::s0 + T::s1 + T::s2) >= kStreamBytes ? 1u : 0u;
+    if (variant == 0) {
+        a.inner = static_cast<uint32_t>(c.n < (int64_t{1} << 31) ? c.n : 0);
+        a.nouter = 0;
+    } else {
+        a.inner = static_cast<uint32_t>(c.size[last]);
+        a.inner_div = make_fastdiv(a.inner);
+        a.nouter = last;
+        for (int d = 0; d < last; ++d) {
+            int src = last - 1 - d;  // innermost outer dimension first
+            a.div[d] = make_fastdiv(static_cast<uint32_t>(c.size[src]));
+            for (int k = 0; k < NOPS; ++k) {
+                a.ostride[k][d] = c.is_const[k] ? 0 : static_cast<int32_t>(c.stride[k][src]);
+            }
         }
+    }
+    return a;
+}
+
+template <class F>
+void launch_map(const MapCall &c, hipStream_t stream) {
+    using T = MapTraits<F>;
+    constexpr int NOPS = F::N + 1;
+    const int variant = resolve_variant<F>(c);
+    if (variant <= 1) {
+        RowsArgs<NOPS> a = rows_args<F>(c, variant);
         int64_t tiles = (c.n + T::V - 1) / T::V;
         unsigned grid = grid_for(tiles, int64_t{T::U} * kBlock);
-        a.stream = c.n * (T::so + T::s0 + T::s1 + T::s2) >= kStreamBytes ? 1u : 0u;
-        if (variant == 0) {
-            a.inner = static_cast<uint32_t>(c.n < (int64_t{1} << 31) ? c.n : 0);
-            a.nouter = 0;
-            hipLaunchKernelGGL((map_rows_kernel<F, true>), dim3(grid), dim3(kBlock), 0, stream, a);
-        } else {
-            a.inner = static_cast<uint32_t>(c.size[last]);
-            a.inner_div = make_fastdiv(a.inner);
-            a.nouter = last;
-            for (int d = 0; d < last; ++d) {
-                int src = last - 1 - d;  // innermost outer dimension first
-                a.div[d] = make_fastdiv(static_cast<uint32_t>(c.size[src]));
-                for (int k = 0; k < NOPS; ++k) {
-                    a.ostride[k][d] = c.is_const[k] ? 0 : static_cast<int32_t>(c.stride[k][src]);
-                }
-            }
-            hipLaunchKernelGGL((map_rows_kernel<F, false>), dim3(grid), dim3(kBlock), 0, stream, a);
-        }
+        if (variant == 0) hipLaunchKernelGGL((map_rows_kernel<F, true>), dim3(grid), dim3(kBlock), 0, stream, a);
+        else hipLaunchKernelGGL((map_rows_kernel<F, false>), dim3(grid), dim3(kBlock), 0, stream, a);
         return;
     }
     unsigned grid = grid_for(c.n, kBlock);

@@ -251,6 +251,7 @@ hmr_status hmr_context_destroy(hmr_context_t ctx) {
         std::unique_ptr<hmr_context> owned(ctx);
         hipError_t e = hmr::StreamHolder::drop(owned->stream);
         if (e != hipSuccess) return hmr::hip_fail(e, "hipStreamDestroy(ctx->stream)");
+        if (owned->tables != nullptr) HMR_HIP(hipFree(owned->tables));  // waits for the device
         return HMR_OK;
     });
 }

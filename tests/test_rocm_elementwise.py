@@ -126,6 +126,47 @@ def test_half_unary_ops_over_every_input(name, dtype):
     print(f"exhaustive {name} {dtype}: {differ} of 65536 differ, max {worst} ulp")
 
 
+TABLE_OPS = ["exp", "log", "sqrt", "rsqrt", "reciprocal", "sin", "cos", "erf", "tanh", "sigmoid", "log_sigmoid", "silu",
+             "gelu", "gelu_tanh"]
+
+
+@pytest.mark.parametrize("dtype", [DT.BF16, DT.F16], ids=["bf16", "f16"])
+def test_large_half_tensors_take_the_table_and_get_the_direct_kernels_bits(dtype):
+    """From 2^20 elements on, 16-bit unary operations are looked up in a table of all 65 536 results. Every
+    pattern, in a contiguous tensor with a ragged end, in rows of a wider buffer, through a permuted view
+    and in place (out == src through the C ABI): the same bits as the direct kernel on the patterns alone."""
+    import ctypes
+
+    from homura_amd import capi
+
+    patterns = np.arange(65536, dtype=np.uint16)
+    reps = 17
+    flat = np.concatenate([np.tile(patterns, reps), patterns[:5]])                     # 1 114 117 elements
+    small = tensor(patterns, dtype).to(GPU)
+    g_flat = tensor(flat, dtype).to(GPU)
+    heads = tensor(np.tile(patterns, 32), dtype, [4, 128, 32, 128]).to(GPU).permute([0, 2, 1, 3])   # 2^21, strided rows
+    wide = tensor(np.tile(patterns, 20), dtype, [2048, 640]).to(GPU).narrow(1, 128, 512)            # rows of a wider buffer
+    for name in TABLE_OPS:
+        direct = array(getattr(small, name)()).reshape(-1)
+        got = array(getattr(g_flat, name)()).reshape(-1)
+        np.testing.assert_array_equal(got, direct[flat], err_msg=f"{name} {dtype} contiguous")
+        got = array(getattr(heads, name)())
+        want = direct[array(heads)]
+        np.testing.assert_array_equal(got, want, err_msg=f"{name} {dtype} permuted heads")
+        got = array(getattr(wide, name)())
+        np.testing.assert_array_equal(got, direct[array(wide)], err_msg=f"{name} {dtype} rows of a wider buffer")
+    # In place, straight through the C ABI.
+    ctx = capi.Context(0)
+    buf = ctx.upload(flat)
+    code = capi.BF16 if dtype == DT.BF16 else capi.F16
+    d = capi.make_desc(buf.ptr, code, [flat.size], [1])
+    capi.check(capi.lib.hmr_unary(ctx.handle, capi.UNARY["gelu"], ctypes.byref(d), ctypes.byref(d)))
+    ctx.synchronize()
+    np.testing.assert_array_equal(buf.download(np.uint16, flat.size), array(small.gelu()).reshape(-1)[flat])
+    buf.free()
+    ctx.close()
+
+
 BINARY_FLOAT = ["add", "sub", "mul", "div", "maximum", "minimum"]
 BINARY_INT = ["add", "sub", "mul", "maximum", "minimum", "pow", "bitwise_and"]
 BINARY_BOOL = ["add", "mul", "maximum", "minimum", "bitwise_and"]
