@@ -132,7 +132,13 @@ hmr_status plan_reduction(const hmr_tensor_desc *out, const hmr_tensor_desc &kep
         // As many waves side by side as the run of outputs fills (wide spans read best).
         p.across = p.inner > 2 * kWave * vec ? 4 : (p.inner > kWave * vec ? 2 : 1);
         int64_t tiles = ceil_div(p.inner, int64_t{p.across} * kWave * vec) * (a.nout / p.inner);
-        cut(p, ceil_div(4 * 256, tiles), 32);
+        if (elem >= 4 && p.across == 4 && tiles < 256 && a.nred >= 4096) {
+            // Few tiles of long columns: 1024-lane workgroups, one per compute unit.
+            p.group = 1024 / kWave;
+            cut(p, ceil_div(256, tiles), 128);
+        } else {
+            cut(p, ceil_div(4 * 256, tiles), 32);
+        }
         return HMR_OK;
     }
     // Any layout.

@@ -57,6 +57,11 @@ struct Walk {
     }
 };
 
+// Makes the compiler treat a chunk as newly produced. Kernels that keep a row in registers unpack its chunks again in each phase; without
+// this the unpacked values of one phase are kept alive for the next and the packed row costs more
+// registers than an unpacked one.
+__device__ __forceinline__ void forget(u32x4 &r) { asm volatile("" : "+v"(r)); }
+
 // ---- moving accumulators between lanes ------------------------------------------------------------
 
 template <class A>
@@ -115,6 +120,7 @@ struct SimpleFold {
 
 template <class T, bool PROD>
 struct FloatFold : SimpleFold<FloatFold<T, PROD>, T, double> {
+    static constexpr bool kCommutative = true;  // IEEE + and * are
     __device__ __forceinline__ double init() const { return PROD ? 1.0 : 0.0; }
     __device__ __forceinline__ double lift(T x) const { return Conv<T>::to_f64(x); }
     __device__ __forceinline__ double combine(double a, double b) const { return PROD ? a * b : a + b; }
@@ -122,6 +128,7 @@ struct FloatFold : SimpleFold<FloatFold<T, PROD>, T, double> {
 
 template <class T, bool PROD>
 struct IntFold : SimpleFold<IntFold<T, PROD>, T, int64_t> {
+    static constexpr bool kCommutative = true;
     __device__ __forceinline__ int64_t init() const { return PROD ? 1 : 0; }
     __device__ __forceinline__ int64_t lift(T x) const { return Conv<T>::to_i64(x); }
     __device__ __forceinline__ int64_t combine(int64_t a, int64_t b) const {
@@ -132,6 +139,7 @@ struct IntFold : SimpleFold<IntFold<T, PROD>, T, int64_t> {
 
 template <class T, bool ALL>
 struct TruthFold : SimpleFold<TruthFold<T, ALL>, T, uint32_t> {
+    static constexpr bool kCommutative = true;
     __device__ __forceinline__ uint32_t init() const { return ALL ? 1u : 0u; }
     __device__ __forceinline__ uint32_t lift(T x) const { return Conv<T>::to_bool(x) ? 1u : 0u; }
     __device__ __forceinline__ uint32_t combine(uint32_t a, uint32_t b) const { return ALL ? (a & b) : (a | b); }
@@ -150,6 +158,7 @@ struct Best {
 // equals (or among NaNs) the lower position wins - associative and commutative.
 template <class T, bool MAX>
 struct ExtremeFold {
+    static constexpr bool kCommutative = true;  // combine picks the same element whichever side it is on
     using In = T;
     using Acc = Best<T>;
     using Lane = Best<T>;
@@ -167,6 +176,9 @@ struct ExtremeFold {
     __device__ __forceinline__ void lane_add(Lane &l, T x, int64_t index, Ctx) const {
         auto a = key(l.v), b = key(x);
         bool better = MAX ? (b > a) : (b < a);
+        // Once a few elements are in, a new best is rare: when no lane of the wave can have one (not
+        // better, not a NaN, not the lane's first element) the update below is skipped as a whole.
+        if (__builtin_amdgcn_ballot_w64(better || b != b || l.i < 0) == 0) return;
         bool take = l.i < 0 || (a == a && (better || b != b));
         l.v = take ? x : l.v;
         l.i = take ? index : l.i;
@@ -188,6 +200,7 @@ struct ExtremeFold {
 // Second pass of the two-pass variance: sum of squared deviations from the output's f64 mean.
 template <class T>
 struct DeviationFold {
+    static constexpr bool kCommutative = true;
     using In = T;
     using Acc = double;
     using Lane = double;
@@ -362,57 +375,51 @@ __global__ void __launch_bounds__(kBlock) reduce_any_kernel(ReduceArgs a, Op op,
     }
 }
 
-// Folds the slices of each output in slice order. 64 adjacent outputs per workgroup; its four
-// waves take interleaved slices (coalesced 64-output reads, eight in flight) and meet in LDS.
-template <class Op, class Sink>
+// Folds the slices of each output, in an order fixed by the sizes alone. A workgroup takes OUTS
+// adjacent outputs (64, 16, 4 or 1: the fewer outputs there are, the fewer each workgroup takes, so
+// that the grid still covers the GPU); its 256 lanes are 256/OUTS slice lanes per output. A lane folds
+// every (256/OUTS)-th slice, eight loads in flight; the slice lanes of an output that share a wave meet
+// by shuffles, the four waves through LDS.
+template <class Op, class Sink, int OUTS>
 __global__ void __launch_bounds__(kBlock) combine_kernel(ReduceArgs a, Op op, Sink sink) {
     using Acc = typename Op::Acc;
     constexpr int kWaves = kBlock / kWave;
+    constexpr int L = kBlock / OUTS;  // slice lanes per output
     constexpr int U = 8;
     __shared__ Acc lds[kWaves - 1][kWave];
     const Acc *partials = static_cast<const Acc *>(a.partials);
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-    const int64_t groups = (a.nout + kWave - 1) / kWave;
+    const int ol = threadIdx.x % OUTS, sl = threadIdx.x / OUTS;
+    const int64_t groups = (a.nout + OUTS - 1) / OUTS;
     for (int64_t g = blockIdx.x; g < groups; g += gridDim.x) {
-        const int64_t o = g * kWave + lane;
+        const int64_t o = g * OUTS + ol;
         Acc acc = op.init();
         if (o < a.nout) {
-            int64_t s = wave;
-            for (; s + (U - 1) * kWaves < a.splits; s += U * kWaves) {
+            int64_t s = sl;
+            for (; s + (U - 1) * L < a.splits; s += U * L) {
                 Acc t[U];
 #pragma unroll
-                for (int u = 0; u < U; ++u) t[u] = partials[(s + u * kWaves) * a.nout + o];
+                for (int u = 0; u < U; ++u) t[u] = partials[(s + u * L) * a.nout + o];
 #pragma unroll
                 for (int u = 0; u < U; ++u) acc = op.combine(acc, t[u]);
             }
-            for (; s < a.splits; s += kWaves) acc = op.combine(acc, partials[s * a.nout + o]);
+            for (; s < a.splits; s += L) acc = op.combine(acc, partials[s * a.nout + o]);
+        }
+        // Slice lanes of one output inside a wave sit OUTS lanes apart.
+#pragma unroll
+        for (int mask = OUTS; mask < kWave; mask <<= 1) {
+            Acc other = shfl_xor_any(acc, mask);
+            if constexpr (IsCommutative<Op>::value) acc = op.combine(acc, other);
+            else acc = (lane & mask) ? op.combine(other, acc) : op.combine(acc, other);
         }
         __syncthreads();
         if (wave > 0) lds[wave - 1][lane] = acc;
         __syncthreads();
-        if (wave == 0 && o < a.nout) {
+        if (wave == 0 && lane < OUTS && o < a.nout) {
 #pragma unroll
             for (int w = 0; w < kWaves - 1; ++w) acc = op.combine(acc, lds[w][lane]);
             sink.put(o, acc, a.nred);
         }
-    }
-}
-
-// The same with a wave per output, for few outputs cut into many slices (a full reduction).
-template <class Op, class Sink>
-__global__ void __launch_bounds__(kBlock) combine_wave_kernel(ReduceArgs a, Op op, Sink sink) {
-    using Acc = typename Op::Acc;
-    const Acc *partials = static_cast<const Acc *>(a.partials);
-    const int lane = threadIdx.x % kWave;
-    const int64_t groups = (a.nout + 3) / 4;
-    for (int64_t g = blockIdx.x; g < groups; g += gridDim.x) {
-        const int64_t o = g * 4 + threadIdx.x / kWave;
-        Acc acc = op.init();
-        if (o < a.nout) {
-            for (int64_t s = lane; s < a.splits; s += kWave) acc = op.combine(acc, partials[s * a.nout + o]);
-        }
-        acc = wave_fold(op, acc);
-        if (o < a.nout && lane == 0) sink.put(o, acc, a.nred);
     }
 }
 
@@ -485,15 +492,20 @@ __global__ void __launch_bounds__(kBlock) reduce_rows_kernel(ReduceArgs a, Op op
 // holds the remaining, outer kept dimensions. Every row of every tile starts 16-byte aligned.
 // `across` (1, 2 or 4) waves of the workgroup sit side by side on a span of across*64*V columns;
 // the other 4/across wave groups take interleaved rows of the slice.
-template <class Op, class Sink>
-__global__ void __launch_bounds__(kBlock)
+//
+// BLOCK = 256, or 1024 with across = 4: sixteen waves, four row groups on one 4 KB-wide span. The big
+// workgroup is for few column tiles and long columns: the same number of waves per compute unit reads
+// the same spans, but a slice is four times as long, so four times fewer partial results are staged.
+template <class Op, class Sink, int BLOCK>
+__global__ void __launch_bounds__(BLOCK)
     reduce_cols_kernel(ReduceArgs a, int64_t rstride, int64_t inner, int across, Op op, Sink sink) {
     using T = typename Op::In;
     using Acc = typename Op::Acc;
     constexpr int V = 16 / static_cast<int>(sizeof(T));
-    constexpr int kWaves = kBlock / kWave;
+    constexpr int kWaves = BLOCK / kWave;
     constexpr int U = 4;
-    __shared__ Acc lds[kWaves - 1][kWave * V];
+    constexpr int kMinAcross = BLOCK == kBlock ? 1 : 4;
+    __shared__ Acc lds[kWaves - kMinAcross][kWave * V];
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
     const int cgroup = wave % across, rgroup = wave / across, rgroups = kWaves / across;
     const bool nt = a.stream != 0;
@@ -574,9 +586,11 @@ __global__ void __launch_bounds__(kBlock)
     }
 }
 
-// Variance of contiguous, 16-byte aligned rows of at most G*C*V elements: the row is read once
-// into registers, then the CPU's two passes run on them (ref: src/backend/cpu/reduce.rs:150-166):
-// mean = sum / n in f64, then the sum of squared deviations from that mean.
+// Variance of contiguous, 16-byte aligned rows of G*C*V elements at most, a multiple of V: the row
+// is read once into registers (C 16-byte chunks per lane, all loads issued back to back and
+// unconditionally - a chunk past the row's end re-reads the last chunk and is left out of the sums),
+// then the CPU's two passes run on them (ref: src/backend/cpu/reduce.rs:150-166): mean = sum / n in
+// f64, then the sum of squared deviations from that mean.
 template <class T, int WAVES, int C>
 __global__ void __launch_bounds__(kBlock) var_rows_kernel(ReduceArgs a, VarSink<T> sink) {
     constexpr int V = 16 / static_cast<int>(sizeof(T));
@@ -584,10 +598,9 @@ __global__ void __launch_bounds__(kBlock) var_rows_kernel(ReduceArgs a, VarSink<
     constexpr int kPerBlock = kBlock / G;
     __shared__ double lds[WAVES == 4 ? 4 : 1];
     const int lane = threadIdx.x % G;
-    const bool nt = a.stream != 0;
     const FloatFold<T, false> add{};
     const int64_t groups = (a.nout + kPerBlock - 1) / kPerBlock;
-    const int64_t nvec = a.nred / V;
+    const int nvec = static_cast<int>(a.nred / V);
     auto fold = [&](double v) {
         v = wave_fold(add, v);
         if constexpr (WAVES == 4) {
@@ -603,39 +616,42 @@ __global__ void __launch_bounds__(kBlock) var_rows_kernel(ReduceArgs a, VarSink<
     for (int64_t g = blockIdx.x; g < groups; g += gridDim.x) {
         const int64_t o = g * kPerBlock + threadIdx.x / G;
         const bool live = o < a.nout;
-        const T *p = reinterpret_cast<const T *>(a.src) + (live ? a.kept.offset(o) : 0);
-        T x[C][V];
-        bool have[C][V];
+        const char *p = a.src + a.kept.offset(live ? o : a.nout - 1) * static_cast<int64_t>(sizeof(T));
+        u32x4 raw[C];
 #pragma unroll
         for (int c = 0; c < C; ++c) {
-            const int64_t tile = static_cast<int64_t>(c) * G + lane;
-            if (live && tile < nvec) {
-                load_tile_rt<T, V>(reinterpret_cast<const char *>(p + tile * V), x[c], nt);
-#pragma unroll
-                for (int i = 0; i < V; ++i) have[c][i] = true;
-            } else {
-#pragma unroll
-                for (int i = 0; i < V; ++i) {
-                    have[c][i] = live && tile * V + i < a.nred;
-                    x[c][i] = have[c][i] ? p[tile * V + i] : T{};
-                }
-            }
+            const uint32_t tile = static_cast<uint32_t>(c * G + lane);
+            const uint32_t t = tile < static_cast<uint32_t>(nvec) ? tile : static_cast<uint32_t>(nvec - 1);
+            const u32x4 *q = reinterpret_cast<const u32x4 *>(p + t * 16u);
+            if constexpr (kStreamLoads) raw[c] = __builtin_nontemporal_load(q);
+            else raw[c] = *q;
         }
+        __builtin_amdgcn_sched_barrier(0);  // every load is out before anything waits for one
         double sum = 0.0;
 #pragma unroll
         for (int c = 0; c < C; ++c) {
+            T x[V];
+            __builtin_memcpy(x, &raw[c], 16);
+            double part = 0.0;
 #pragma unroll
-            for (int i = 0; i < V; ++i) sum += have[c][i] ? Conv<T>::to_f64(x[c][i]) : 0.0;
+            for (int i = 0; i < V; ++i) part += Conv<T>::to_f64(x[i]);
+            // Lane-local order: chunk by chunk, left to right inside a chunk.
+            sum += c * G + lane < nvec ? part : 0.0;
         }
         const double mean = fold(sum) / static_cast<double>(a.nred);
         double sq = 0.0;
 #pragma unroll
         for (int c = 0; c < C; ++c) {
+            T x[V];
+            forget(raw[c]);  // convert again rather than keep every f64 value of the first pass
+            __builtin_memcpy(x, &raw[c], 16);
+            double part = 0.0;
 #pragma unroll
             for (int i = 0; i < V; ++i) {
-                double d = Conv<T>::to_f64(x[c][i]) - mean;
-                sq += have[c][i] ? d * d : 0.0;
+                const double d = Conv<T>::to_f64(x[i]) - mean;
+                part += d * d;
             }
+            sq += c * G + lane < nvec ? part : 0.0;
         }
         sq = fold(sq);
         if (live && lane == 0) sink.finish(o, sq, a.nred);

@@ -22,6 +22,7 @@ bool launch_float_reduce(int op, int dtype, const ReducePlan &plan, void *partia
 static int var_row_tiles(const ReducePlan &plan, int elem) {
     if (plan.kind != ReduceKind::Rows || plan.splits != 1) return 0;
     const int64_t vec = 16 / elem;
+    if (plan.args.nred % vec != 0) return 0;  // the register kernel takes whole 16-byte chunks
     const int64_t per = (plan.args.nred + vec * plan.group - 1) / (vec * plan.group);
     return per <= 4 ? 4 : (per <= 8 ? 8 : (per <= 16 ? 16 : 0));
 }

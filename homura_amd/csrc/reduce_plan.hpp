@@ -1,6 +1,7 @@
 // Host-side planning of a reduction and the typed launch of its kernels.
 #pragma once
 
+#include "dispatch.hpp"
 #include "reduce.hpp"
 
 namespace hmr {
@@ -70,8 +71,16 @@ void launch_reduce(const ReducePlan &plan, void *partials, Op op, Sink sink, hip
             int64_t span = int64_t{plan.across} * kWave * V;
             int64_t tiles = (plan.inner + span - 1) / span * (a.nout / plan.inner);
             dim3 grid(capped(tiles, cap), ysplits);
-            hipLaunchKernelGGL((reduce_cols_kernel<Op, Sink>), grid, dim3(kBlock), 0, stream, a, plan.rstride,
-                               plan.inner, plan.across, op, sink);
+            if (plan.group == 1024 / kWave) {
+                // Planned for 4- and 8-byte elements only (wider tiles would not fit LDS).
+                if constexpr (sizeof(typename Op::In) >= 4) {
+                    hipLaunchKernelGGL((reduce_cols_kernel<Op, Sink, 1024>), grid, dim3(1024), 0, stream, a,
+                                       plan.rstride, plan.inner, plan.across, op, sink);
+                }
+            } else {
+                hipLaunchKernelGGL((reduce_cols_kernel<Op, Sink, kBlock>), grid, dim3(kBlock), 0, stream, a,
+                                   plan.rstride, plan.inner, plan.across, op, sink);
+            }
             break;
         }
         case ReduceKind::Any: {
@@ -89,14 +98,16 @@ void launch_reduce(const ReducePlan &plan, void *partials, Op op, Sink sink, hip
         }
     }
     if (plan.splits > 1) {
-        // Few outputs with many slices: a wave per output; otherwise a lane per output.
-        if (a.nout < 4096 && plan.splits >= 32) {
-            hipLaunchKernelGGL((combine_wave_kernel<Op, Sink>), dim3(capped((a.nout + 3) / 4, cap)), dim3(kBlock), 0,
-                               stream, a, op, sink);
-        } else {
-            hipLaunchKernelGGL((combine_kernel<Op, Sink>), dim3(capped((a.nout + kWave - 1) / kWave, cap)),
+        // Outputs per workgroup: as many as still leave a workgroup per compute unit.
+        auto run = [&](auto outs) {
+            constexpr int OUTS = decltype(outs)::value;
+            hipLaunchKernelGGL((combine_kernel<Op, Sink, OUTS>), dim3(capped((a.nout + OUTS - 1) / OUTS, cap)),
                                dim3(kBlock), 0, stream, a, op, sink);
-        }
+        };
+        if (a.nout >= 64 * 256) run(IntTag<64>{});
+        else if (a.nout >= 16 * 256) run(IntTag<16>{});
+        else if (a.nout >= 4 * 64) run(IntTag<4>{});
+        else run(IntTag<1>{});
     }
 }
 

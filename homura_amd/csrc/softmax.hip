@@ -194,11 +194,6 @@ __device__ __forceinline__ double max3(double m, double a, double b) {
     return b > m ? b : m;
 }
 
-// Makes the compiler treat a chunk as newly produced. Each phase unpacks the row's chunks again; without
-// this the unpacked values of one phase are kept alive for the next and the packed row costs more
-// registers than an unpacked one.
-__device__ __forceinline__ void forget(u32x4 &r) { asm volatile("" : "+v"(r)); }
-
 // ---- combining across the lanes of a row ---------------------------------------------------------
 
 struct MaxOp {

@@ -306,6 +306,7 @@ PLAN_SHAPES = [
     ([1 << 21], [0], 256, True),            # a full reduction
     ([8, 1 << 20], [0], 4, False),          # columns, one slice
     ([5000, 256], [0], 4, True),            # columns cut into row slices
+    ([8192, 2048], [0], 16, True),          # long columns in few tiles: 1024-lane workgroups, four row groups
     ([6, 700, 96], [1], 4, True),           # columns under an outer kept dimension
     ([5000, 20], [1], 1, False),            # short rows: a lane per output
     ([9, 2, 3000], [0, 2], 256, True),      # two reduced dimensions: any layout, 256 lanes
@@ -350,7 +351,7 @@ def test_every_plan_folds_each_element_once():
             assert_bitwise(few.to(GPU).argmin_dim(dims[0], True), few.argmin_dim(dims[0], True), f"argmin {shape}")
         assert_bitwise(few.to(GPU).argmax(), few.argmax(), f"argmax {shape}")
         assert_bitwise(x.to(DT.Bool).to(GPU).all_dim(dims, False), x.to(DT.Bool).all_dim(dims, False), f"all {shape}")
-    assert seen >= {(64, False), (256, False), (256, True), (4, False), (4, True), (1, False)}
+    assert seen >= {(64, False), (256, False), (256, True), (4, False), (4, True), (16, True), (1, False)}
 
 
 SOFTMAX_PLAN_SHAPES = [
