@@ -12,7 +12,8 @@ The same JSON line carries
   cpu_baseline  the CPU oracle (a port of homura's single-threaded CPU backend) timed on one host
                 core on the same workload;
   ops           achieved GB/s and fraction of the 8 TB/s HBM peak for every op of every BASELINE
-                config (--ops none to skip), algorithmic bytes as in BASELINE.md section 3.
+                config (--ops none to skip; cfg = index into BASELINE.json's configs), algorithmic bytes as in
+                BASELINE.md section 3.
 
 usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--ops all|none]
 """
@@ -172,7 +173,7 @@ def main():
 
 
 def per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP, x, bias, scale, residual, t2):
-    """[{cfg, op, bytes, us, gbs, frac}] for the ops of BASELINE configs 1-5."""
+    """[{cfg, op, bytes, us, gbs, frac}] for the ops of BASELINE.json configs[0..4] (cfg = index)."""
     rows = []
 
     def add(cfg, op, nbytes, fns, iters=20):
@@ -185,77 +186,84 @@ def per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP
             fns[k[0] % len(fns)]()
             k[0] += 1
 
+        # The host work between two ops (generating the next inputs) lets the GPU fall back to idle clocks:
+        # run the op untimed for about 30 ms first, then time `iters` launches.
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < 0.03:
+            for _ in range(10):
+                call()
+            h.synchronize(GPU)
         ms = timed(call, iters, 3)
         gbs = nbytes / (ms * 1e-3) / 1e9
         rows.append({"cfg": cfg, "op": op, "bytes": nbytes, "us": round(ms * 1e3, 2), "gbs": round(gbs, 1),
                      "frac": round(gbs / HBM_PEAK_GBS, 4)})
 
     N = x.num_elements()
-    # cfg 1: f32 add [4096, 4096], four disjoint buffer sets (805 MB in rotation).
+    # configs[0]: f32 add [4096, 4096], four disjoint buffer sets (805 MB in rotation).
     n1 = 4096 * 4096
     sets = []
     for i in range(4):
         a = tensor(uniform(0x5EED0100 + 2 * i, n1, -1.0, 1.0).astype(np.float32), DT.F32, [4096, 4096], GPU)
         b = tensor(uniform(0x5EED0101 + 2 * i, n1, -1.0, 1.0).astype(np.float32), DT.F32, [4096, 4096], GPU)
         sets.append((a, b))
-    add(1, "add f32 [4096,4096] (HBM-resident, rotating buffers)", 12 * n1, [lambda a=a, b=b: a.add(b) for a, b in sets], 40)
+    add(0, "add f32 [4096,4096] (HBM-resident, rotating buffers)", 12 * n1, [lambda a=a, b=b: a.add(b) for a, b in sets], 40)
     a0, b0 = sets[0]
-    add(1, "add f32 [4096,4096] (same buffers, Infinity-Cache-resident)", 12 * n1, lambda: a0.add(b0), 40)
+    add(0, "add f32 [4096,4096] (same buffers, Infinity-Cache-resident)", 12 * n1, lambda: a0.add(b0), 40)
     del sets
-    # cfg 2: the three steps.
+    # configs[1]: the three steps.
     t1 = x.add(bias)
-    add(2, "x_bf16 + bias_bf16[4096] (inner broadcast)", 4 * N + 2 * 4096, lambda: x.add(bias))
-    add(2, "t_bf16 * scale_bf16[8,2048,1] (row broadcast)", 4 * N + 2 * 8 * 2048, lambda: t1.mul(scale))
-    add(2, "t_bf16 + residual_f32 -> f32 (promotion fused)", 10 * N, lambda: t2.add(residual))
+    add(1, "x_bf16 + bias_bf16[4096] (inner broadcast)", 4 * N + 2 * 4096, lambda: x.add(bias))
+    add(1, "t_bf16 * scale_bf16[8,2048,1] (row broadcast)", 4 * N + 2 * 8 * 2048, lambda: t1.mul(scale))
+    add(1, "t_bf16 + residual_f32 -> f32 (promotion fused)", 10 * N, lambda: t2.add(residual))
     h.set_fused_promotion(False)
-    add(2, "t_bf16 + residual_f32 -> f32 (reference style: cast kernel + add, 2 launches)", 18 * N,
+    add(1, "t_bf16 + residual_f32 -> f32 (reference style: cast kernel + add, 2 launches)", 18 * N,
         lambda: t2.add(residual))
     h.set_fused_promotion(True)
     del t1
-    # cfg 3: reductions of f32 [16384, 4096] and of its bf16 copy.
+    # configs[2]: reductions of f32 [16384, 4096] and of its bf16 copy.
     R, C = 16384, 4096
     xf = residual.reshape([R, C])
-    add(3, "sum dim=-1 f32", 4 * N + 4 * R, lambda: xf.sum_dim(-1, False))
-    add(3, "mean dim=-1 f32", 4 * N + 4 * R, lambda: xf.mean_dim(-1, False))
-    add(3, "amax dim=-1 f32 (max_dim: values + i64 indices)", 4 * N + 12 * R, lambda: xf.max_dim(-1, False))
-    add(3, "var(unbiased) dim=-1 f32", 4 * N + 4 * R, lambda: xf.var_dim(-1, 1, False))
-    add(3, "sum dim=0 f32", 4 * N + 4 * C, lambda: xf.sum_dim(0, False))
-    add(3, "mean dim=0 f32", 4 * N + 4 * C, lambda: xf.mean_dim(0, False))
-    add(3, "amax dim=0 f32 (max_dim: values + i64 indices)", 4 * N + 12 * C, lambda: xf.max_dim(0, False))
-    add(3, "var(unbiased) dim=0 f32", 4 * N + 4 * C, lambda: xf.var_dim(0, 1, False))
-    add(3, "sum over all elements f32", 4 * N + 4, lambda: xf.sum())
+    add(2, "sum dim=-1 f32", 4 * N + 4 * R, lambda: xf.sum_dim(-1, False))
+    add(2, "mean dim=-1 f32", 4 * N + 4 * R, lambda: xf.mean_dim(-1, False))
+    add(2, "amax dim=-1 f32 (max_dim: values + i64 indices)", 4 * N + 12 * R, lambda: xf.max_dim(-1, False))
+    add(2, "var(unbiased) dim=-1 f32", 4 * N + 4 * R, lambda: xf.var_dim(-1, 1, False))
+    add(2, "sum dim=0 f32", 4 * N + 4 * C, lambda: xf.sum_dim(0, False))
+    add(2, "mean dim=0 f32", 4 * N + 4 * C, lambda: xf.mean_dim(0, False))
+    add(2, "amax dim=0 f32 (max_dim: values + i64 indices)", 4 * N + 12 * C, lambda: xf.max_dim(0, False))
+    add(2, "var(unbiased) dim=0 f32", 4 * N + 4 * C, lambda: xf.var_dim(0, 1, False))
+    add(2, "sum over all elements f32", 4 * N + 4, lambda: xf.sum())
     xb = xf.to(DT.BF16)
-    add(3, "sum dim=-1 bf16", 2 * N + 2 * R, lambda: xb.sum_dim(-1, False))
+    add(2, "sum dim=-1 bf16", 2 * N + 2 * R, lambda: xb.sum_dim(-1, False))
     del xb
-    # cfg 4: permuted bf16 unary; int64 ops.
+    # configs[3]: permuted bf16 unary; int64 ops.
     p = tensor(from_f64(normal(0x5EED0400, N, 0.0, 2.0), DT.BF16), DT.BF16, [8, 2048, 32, 128], GPU).permute([0, 2, 1, 3])
-    add(4, "silu bf16 [8,2048,32,128].permute(0,2,1,3) -> contiguous", 4 * N, lambda: p.silu())
-    add(4, "gelu(erf) bf16, same view", 4 * N, lambda: p.gelu())
+    add(3, "silu bf16 [8,2048,32,128].permute(0,2,1,3) -> contiguous", 4 * N, lambda: p.silu())
+    add(3, "gelu(erf) bf16, same view", 4 * N, lambda: p.gelu())
     del p
     w1 = words(0x5EED0401, N)
     w2 = words(0x5EED0402, N)
     ia = tensor(((w1 % np.uint64(2001)).astype(np.int64) - 1000), DT.I64, [8, 2048, 4096], GPU)
     ib = tensor(((w2 % np.uint64(2001)).astype(np.int64) - 1000), DT.I64, [8, 2048, 4096], GPU)
     del w1, w2
-    add(4, "bitwise_and i64", 24 * N, lambda: ia.bitwise_and(ib))
-    add(4, "greater i64 -> bool", 17 * N, lambda: ia.greater(ib))
+    add(3, "bitwise_and i64", 24 * N, lambda: ia.bitwise_and(ib))
+    add(3, "greater i64 -> bool", 17 * N, lambda: ia.greater(ib))
     mask = ia.greater(ib)
-    add(4, "where(mask, a, b) i64", 25 * N, lambda: h.where_(mask, ia, ib))
+    add(3, "where(mask, a, b) i64", 25 * N, lambda: h.where_(mask, ia, ib))
     del ia, ib, mask
-    # cfg 5a: bf16 logits [4096, 32000].
+    # configs[4] case 1: bf16 logits [4096, 32000].
     n5a = 4096 * 32000
     logits = tensor(from_f64(normal(0x5EED0500, n5a, 0.0, 3.0), DT.BF16), DT.BF16, [4096, 32000], GPU)
-    add(5, "softmax bf16 [4096,32000]", 4 * n5a, lambda: logits.softmax(-1))
-    add(5, "log_softmax bf16 [4096,32000]", 4 * n5a, lambda: logits.log_softmax(-1))
+    add(4, "softmax bf16 [4096,32000]", 4 * n5a, lambda: logits.softmax(-1))
+    add(4, "log_softmax bf16 [4096,32000]", 4 * n5a, lambda: logits.log_softmax(-1))
     del logits
-    # cfg 5b: causal f32 scores [32, 2048, 2048].
+    # configs[4] case 2: causal f32 scores [32, 2048, 2048].
     n5b = 32 * 2048 * 2048
     s = normal(0x5EED0501, n5b).astype(np.float32).reshape(32, 2048, 2048)
     s[:, np.triu_indices(2048, 1)[0], np.triu_indices(2048, 1)[1]] = -np.inf
     scores = tensor(s, DT.F32, [32, 2048, 2048], GPU)
     del s
-    add(5, "softmax f32 [32,2048,2048] causal", 8 * n5b, lambda: scores.softmax(-1))
-    add(5, "log_softmax f32 [32,2048,2048] causal", 8 * n5b, lambda: scores.log_softmax(-1))
+    add(4, "softmax f32 [32,2048,2048] causal", 8 * n5b, lambda: scores.softmax(-1))
+    add(4, "log_softmax f32 [32,2048,2048] causal", 8 * n5b, lambda: scores.log_softmax(-1))
     return rows
 
 
