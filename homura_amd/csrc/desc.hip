@@ -6,7 +6,7 @@
 
 namespace hmr {
 
-hmr_status check_desc(const hmr_tensor_desc &d, int64_t &n) {
+hmr_status check_desc(const hmr_tensor_desc &d, int64_t &n, bool negative_strides) {
     if (d.dtype < HMR_BOOL || d.dtype > HMR_F64) return fail(HMR_INVALID, "invalid dtype " + std::to_string(d.dtype));
     if (d.ndim < 0 || d.ndim > HMR_MAX_DIMS) {
         return fail(HMR_INVALID, "invalid number of dimensions " + std::to_string(d.ndim));
@@ -14,13 +14,14 @@ hmr_status check_desc(const hmr_tensor_desc &d, int64_t &n) {
     n = 1;
     for (int k = 0; k < d.ndim; ++k) {
         if (d.sizes[k] < 0) return fail(HMR_INVALID, "negative size");
-        if (d.strides[k] < 0) return fail(HMR_INVALID, "negative stride");
+        if (d.strides[k] < 0 && !negative_strides) return fail(HMR_INVALID, "negative stride");
         n *= d.sizes[k];
     }
     return HMR_OK;
 }
 
-hmr_status prepare_map(MapCall &c, int count, const hmr_tensor_desc *const *descs, const uint64_t *bits) {
+hmr_status prepare_map(MapCall &c, int count, const hmr_tensor_desc *const *descs, const uint64_t *bits,
+                       bool negative_inputs) {
     const hmr_tensor_desc &out = *descs[0];
     c.nops = count;
     if (hmr_status s = check_desc(out, c.n)) return s;
@@ -33,7 +34,7 @@ hmr_status prepare_map(MapCall &c, int count, const hmr_tensor_desc *const *desc
         const hmr_tensor_desc &d = *descs[k];
         if (k > 0) {
             int64_t m = 0;
-            if (hmr_status s = check_desc(d, m)) return s;
+            if (hmr_status s = check_desc(d, m, negative_inputs)) return s;
             bool same = d.ndim == out.ndim;
             for (int j = 0; same && j < out.ndim; ++j) same = d.sizes[j] == out.sizes[j];
             if (!same) return fail(HMR_INVALID, "kernel operands have different sizes");

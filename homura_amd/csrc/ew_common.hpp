@@ -13,9 +13,9 @@ namespace hmr {
 // `before(call)` runs after the checks and before the launch bracket; it may fail the call.
 template <class Pick, class Before>
 hmr_status run_map(hmr_context_t ctx, const char *what, int count, const hmr_tensor_desc *const *descs,
-                   const uint64_t *bits, Pick pick, Before before) {
+                   const uint64_t *bits, Pick pick, Before before, bool negative_inputs = false) {
     MapCall call;
-    if (hmr_status s = prepare_map(call, count, descs, bits)) return s;
+    if (hmr_status s = prepare_map(call, count, descs, bits, negative_inputs)) return s;
     if (call.n == 0) return HMR_OK;
     call.compute_units = ctx->compute_units;
     if (hmr_status s = before(call)) return s;

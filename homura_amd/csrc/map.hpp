@@ -66,12 +66,13 @@ struct MapCall {
 
 // Validates one description (ref: csrc/kernel.hpp:62-78): dtype and rank in range, no negative
 // size or stride. Leaves the element count in n.
-hmr_status check_desc(const hmr_tensor_desc &d, int64_t &n);
+hmr_status check_desc(const hmr_tensor_desc &d, int64_t &n, bool negative_strides = false);
 
 // Builds the call for `descs[0..count)` (descs[k] == nullptr marks a constant with bits[k]):
 // checks that all have the output's sizes, then drops size-1 dimensions and joins neighbours
 // that are contiguous with each other in every operand.
-hmr_status prepare_map(MapCall &call, int count, const hmr_tensor_desc *const *descs, const uint64_t *bits);
+hmr_status prepare_map(MapCall &call, int count, const hmr_tensor_desc *const *descs, const uint64_t *bits,
+                       bool negative_inputs = false);
 
 // ---- device-side argument blocks ------------------------------------------------------------------
 
@@ -237,6 +238,14 @@ __device__ __forceinline__ typename F::Out apply(const F &f, typename F::In0 a, 
     else return f(a, b, c);
 }
 
+// A functor that carries a run-time parameter (a coefficient in its computation type) takes it from
+// the 64 bits that travel in the output's otherwise unused constant slot.
+template <class F>
+__device__ __forceinline__ F make_functor(uint64_t param) {
+    if constexpr (std::is_constructible_v<F, uint64_t>) return F{param};
+    else return F{};
+}
+
 // ---- map_rows_kernel ---------------------------------------------------------------------------------
 //
 // The pass of a workgroup over its U*256 tiles comes in two forms. When every one of those tiles is
@@ -375,7 +384,7 @@ __global__ void __launch_bounds__(kBlock) map_rows_kernel(RowsArgs<F::N + 1> a) 
     using B = typename F::In1;
     using C = typename F::In2;
     using Off = std::conditional_t<FLAT, int64_t, uint32_t>;
-    const F f{};
+    const F f = make_functor<F>(a.cbits[0]);
     const int64_t tiles = (a.n + V - 1) / V;
     const int64_t whole = a.n / V;  // tiles [0, whole) have all V elements
     const bool c0 = a.const_mask & 2u, c1 = a.const_mask & 4u, c2 = a.const_mask & 8u;
@@ -484,9 +493,10 @@ template <class F, class Idx>
 __global__ void __launch_bounds__(kBlock) map_any_kernel(AnyArgs<F::N + 1, Idx> a) {
     constexpr int N = F::N;
     using Out = typename F::Out;
-    const F f{};
+    const F f = make_functor<F>(a.cbits[0]);
     const bool c0 = a.const_mask & 2u, c1 = a.const_mask & 4u, c2 = a.const_mask & 8u;
-    using Off = std::conditional_t<std::is_same_v<Idx, uint32_t>, uint32_t, int64_t>;
+    // Signed: an input's strides may be negative (hmr_flip); every partial sum fits 31 bits then.
+    using Off = std::conditional_t<std::is_same_v<Idx, uint32_t>, int32_t, int64_t>;
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; i < a.n;
          i += static_cast<int64_t>(gridDim.x) * kBlock) {
         Off off[4] = {0, 0, 0, 0};
@@ -497,7 +507,7 @@ __global__ void __launch_bounds__(kBlock) map_any_kernel(AnyArgs<F::N + 1, Idx> 
                 uint32_t idx = rest - q * a.div[d].div;
                 rest = q;
 #pragma unroll
-                for (int k = 0; k <= N; ++k) off[k] += idx * static_cast<uint32_t>(a.stride[k][d]);
+                for (int k = 0; k <= N; ++k) off[k] += static_cast<int32_t>(idx) * a.stride[k][d];
             }
         } else {
             int64_t rest = i;
@@ -533,8 +543,11 @@ inline bool fits_32(const MapCall &c) {
     if (c.n >= (int64_t{1} << 31)) return false;
     for (int k = 0; k < c.nops; ++k) {
         if (c.is_const[k]) continue;
-        __int128 reach = 0;
-        for (int d = 0; d < c.ndim; ++d) reach += static_cast<__int128>(c.size[d] - 1) * c.stride[k][d];
+        __int128 reach = 0;  // largest magnitude any partial sum of index * stride can take
+        for (int d = 0; d < c.ndim; ++d) {
+            const __int128 span = static_cast<__int128>(c.size[d] - 1) * c.stride[k][d];
+            reach += span < 0 ? -span : span;
+        }
         if (reach >= (int64_t{1} << 31)) return false;
     }
     return true;
@@ -545,6 +558,12 @@ template <class F>
 int pick_variant(const MapCall &c) {
     using T = MapTraits<F>;
     constexpr int sizes[4] = {T::so, T::s0, T::s1, T::s2};
+    // A reversed dimension (negative input stride, hmr_flip only) goes through the general kernels.
+    for (int k = 1; k < c.nops; ++k) {
+        for (int d = 0; d < c.ndim && !c.is_const[k]; ++d) {
+            if (c.stride[k][d] < 0) return c.ndim <= kFastDims && fits_32(c) ? 2 : 3;
+        }
+    }
     if (c.ndim > kFastDims || !fits_32(c)) return c.ndim <= 1 && c.n < (int64_t{1} << 62) ? -1 : 3;
     if (c.ndim == 0) return 0;
     const int last = c.ndim - 1;

@@ -346,6 +346,36 @@ struct ScalarBinary {
     }
 };
 
+// ---- the optimizers' fused steps (ref: src/backend/cpu/mod.rs:509-569) -------------------------------
+//
+// One rounding to the dtype; the multiply-adds are fused exactly where the CPU's mul_add is. The
+// coefficient arrives in the computation type (the bits of a C value).
+template <int OP, class T, bool SMALL>
+struct FusedStep {
+    static constexpr int N = OP <= HMR_FUSED_LERP ? 2 : 3;
+    using Out = T;
+    using In0 = T;
+    using In1 = T;
+    using In2 = std::conditional_t<N == 3, T, Unused>;
+    using C = typename Comp<T>::C;
+    C coefficient;
+    __device__ __forceinline__ explicit FusedStep(uint64_t bits) { __builtin_memcpy(&coefficient, &bits, sizeof(C)); }
+    static __device__ __forceinline__ C fused(C a, C b, C c) {
+        if constexpr (std::is_same_v<C, float>) return __builtin_fmaf(a, b, c);
+        else return __builtin_fma(a, b, c);
+    }
+    __device__ __forceinline__ T operator()(T a, T b) const {
+        const C x = Comp<T>::up(a), y = Comp<T>::up(b);
+        if constexpr (OP == HMR_FUSED_SCALED_ADD) return Comp<T>::down(fused(y, coefficient, x));
+        else return Comp<T>::down(fused(coefficient, y - x, SMALL ? x : y));
+    }
+    __device__ __forceinline__ T operator()(T a, T b, T c) const {
+        const C x = Comp<T>::up(a), y = Comp<T>::up(b), z = Comp<T>::up(c);
+        if constexpr (OP == HMR_FUSED_ADDCMUL) return Comp<T>::down(fused(coefficient * y, z, x));
+        else return Comp<T>::down(x + coefficient * y / z);
+    }
+};
+
 // ---- where --------------------------------------------------------------------------------------------
 
 template <class W>

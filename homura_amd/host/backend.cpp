@@ -1,5 +1,6 @@
 // Storage, the device dispatch of every kernel, and the ROCm host side that turns tensors into
 // hmr_tensor_desc's and calls the C ABI. See homura.hpp for the map to the reference's files.
+#include <cmath>
 #include <cstdlib>
 #include <cstring>
 #include <map>
@@ -509,6 +510,112 @@ void softmax(const TensorData &out, const TensorData &src, size_t dim, bool log)
     exec(out, [&](hmr_context_t ctx) {
         expect(hmr_softmax(ctx, &o, &s, n, so, si, log, ws ? ws->ptr() : nullptr, bytes));
     });
+}
+
+// ref: src/backend/rocm/elementwise.rs:155-215: the coefficient travels in the computation type.
+void fused(const Fused &op, const TensorData &out, const TensorData &a, const TensorData &b, const TensorData *c) {
+    check_shape(out, a);
+    check_shape(out, b);
+    if (c) check_shape(out, *c);
+    if (on_cpu(out)) {
+        hcb_tensor o = cpu_desc(out), x = cpu_desc(a), y = cpu_desc(b), z{};
+        if (c) z = cpu_desc(*c);
+        cpu_check(cpu_backend("fused").fused(static_cast<int32_t>(op.kind), op.scalar, &o, &x, &y, c ? &z : nullptr));
+        return;
+    }
+    if (!is_floating_point(out.dtype)) throw Error(std::string("expected a floating point dtype, got ") + name_of(out.dtype));
+    // As `C::of` and `T::down(..).up()` of the reference, for C = f32 (F16, BF16, F32) or f64.
+    const bool wide = out.dtype == DType::F64;
+    auto of = [&](double v) { return wide ? v : static_cast<double>(static_cast<float>(v)); };
+    double coefficient = 0.0;
+    bool small = false;
+    switch (op.kind) {
+        case Fused::ScaledAdd:
+            coefficient = round_through(op.scalar, out.dtype);  // alpha rounded to the dtype first
+            break;
+        case Fused::Lerp: {
+            double w = of(op.scalar);
+            small = std::fabs(w) < 0.5;
+            coefficient = small ? w : of(w - 1.0);
+            break;
+        }
+        default: coefficient = of(op.scalar); break;
+    }
+    std::vector<hmr_tensor_desc> ds;
+    std::vector<const TensorData *> ops = {&out, &a, &b};
+    if (c) ops.push_back(c);
+    if (!descs("fused", ops, ds)) return;
+    exec(out, [&](hmr_context_t ctx) {
+        expect(hmr_fused(ctx, static_cast<int32_t>(op.kind), &ds[0], &ds[1], &ds[2], c ? &ds[3] : nullptr, coefficient,
+                         small ? 1 : 0));
+    });
+}
+
+// ref: src/backend/rocm/elementwise.rs:323-346: batch dimensions merged, the two matrix dimensions kept.
+void triangle(const TensorData &out, const TensorData &src, int64_t diagonal, bool upper) {
+    const Layout &ls = src.layout, &lo = out.layout;
+    const size_t nd = ls.shape.size();
+    if (nd < 2 || ls.shape != lo.shape) throw Error("triangle: operands must have the same shape of two or more dimensions");
+    if (on_cpu(out)) {
+        hcb_tensor o = cpu_desc(out), s = cpu_desc(src);
+        cpu_check(cpu_backend("triangle").triangle(&o, &s, diagonal, upper));
+        return;
+    }
+    if (ls.num_elements() == 0) return;
+    Shape batch(ls.shape.begin(), ls.shape.end() - 2);
+    Strides bo(lo.strides.begin(), lo.strides.end() - 2), bs(ls.strides.begin(), ls.strides.end() - 2);
+    auto merged = merge_dims(batch, {&bo, &bs});
+    std::vector<MergedDim> dims = merged ? *merged : std::vector<MergedDim>{};
+    for (size_t d = nd - 2; d < nd; ++d) dims.push_back(MergedDim{ls.shape[d], {lo.strides[d], ls.strides[d]}});
+    hmr_tensor_desc o = desc_with_dims("triangle", out, lo.offset, dims, 0);
+    hmr_tensor_desc s = desc_with_dims("triangle", src, ls.offset, dims, 1);
+    exec(out, [&](hmr_context_t ctx) { expect(hmr_triangle(ctx, &o, &s, diagonal, upper ? 1 : 0)); });
+}
+
+// ref: src/backend/rocm/elementwise.rs:348-386: the source is read through negative strides from the
+// last element of each reversed dimension.
+void flip(const TensorData &out, const TensorData &src, const std::vector<bool> &mask) {
+    const Layout &l = src.layout;
+    if (!out.layout.is_contiguous() || out.layout.shape != l.shape) throw Error("flip writes a contiguous tensor of the source's shape");
+    if (on_cpu(out)) {
+        hcb_tensor o = cpu_desc(out), s = cpu_desc(src);
+        std::vector<uint8_t> m(mask.begin(), mask.end());
+        cpu_check(cpu_backend("flip").flip(&o, &s, m.data()));
+        return;
+    }
+    if (l.num_elements() == 0) return;
+    int64_t src_offset = l.offset;
+    std::vector<MergedDim> dims;
+    Strides out_strides = contiguous_strides(l.shape);
+    for (size_t d = 0; d < l.shape.size(); ++d) {
+        const int64_t size = l.shape[d];
+        if (size == 1) continue;
+        int64_t st = l.strides[d];
+        if (mask[d]) {
+            src_offset += (size - 1) * st;
+            st = -st;
+        }
+        const int64_t pair[2] = {out_strides[d], st};
+        // Neighbours merge when they are contiguous with each other in both operands, which with signed
+        // strides also requires both to be reversed or neither.
+        if (!dims.empty()) {
+            MergedDim &outer = dims.back();
+            bool joins = true;
+            for (int k = 0; k < 2; ++k) {
+                int64_t prod = 0;
+                joins = joins && !__builtin_mul_overflow(pair[k], size, &prod) && prod == outer.strides[k];
+            }
+            if (joins) {
+                outer.size *= size;
+                outer.strides = {pair[0], pair[1]};
+                continue;
+            }
+        }
+        dims.push_back(MergedDim{size, {pair[0], pair[1]}});
+    }
+    hmr_tensor_desc o = desc_with_dims("flip", out, out.layout.offset, dims, 0);
+    hmr_tensor_desc s = desc_with_dims("flip", src, src_offset, dims, 1);
+    exec(out, [&](hmr_context_t ctx) { expect(hmr_flip(ctx, &o, &s)); });
 }
 
 void upload(const TensorData &dst, const TensorData &src) {

@@ -200,6 +200,16 @@ uint64_t scalar_bits(Scalar value, DType dtype) {
     }
 }
 
+double round_through(double value, DType dtype) {
+    const float narrow = static_cast<float>(value);
+    switch (dtype) {
+        case DType::F16: return hmr::Conv<hmr::f16_t>::to_f64(hmr::f16_round(narrow));
+        case DType::BF16: return hmr::Conv<hmr::bf16_t>::to_f64(hmr::bf16_round(narrow));
+        case DType::F32: return static_cast<double>(narrow);
+        default: return value;
+    }
+}
+
 // ---- shapes (ref: src/shape.rs) --------------------------------------------------------------------------
 
 std::string shape_str(const Shape &s) {

@@ -72,6 +72,13 @@ typedef struct hcb_backend {
                       int32_t dim, int32_t is_max);
     /* ref: src/backend/cpu/misc.rs:15-51 */
     int (*softmax)(const hcb_tensor *out, const hcb_tensor *src, int32_t dim, int32_t log);
+    /* ref: src/backend/cpu/mod.rs:509-569; kind 0 ScaledAdd(alpha), 1 Lerp(weight), 2 Addcmul(value),
+     * 3 Addcdiv(value), with the caller's f64 scalar; c is NULL for kinds 0 and 1 */
+    int (*fused)(int32_t kind, double scalar, const hcb_tensor *out, const hcb_tensor *a,
+                 const hcb_tensor *b, const hcb_tensor *c);
+    /* ref: src/backend/cpu/misc.rs:347-411; flip's mask has src->ndim entries (1 = reversed) */
+    int (*triangle)(const hcb_tensor *out, const hcb_tensor *src, int64_t diagonal, int32_t upper);
+    int (*flip)(const hcb_tensor *out, const hcb_tensor *src, const uint8_t *mask);
 } hcb_backend;
 
 #ifdef __cplusplus

@@ -78,6 +78,9 @@ class ResultType {
 // `value` converted to `dtype` as the CPU's fill converts it, little-endian in the low bytes
 // (ref: src/backend/rocm/copy.rs:253-270).
 uint64_t scalar_bits(Scalar value, DType dtype);
+// `value` taken to a floating point dtype's computation type (f32, or f64 for F64), rounded to the dtype,
+// and read back.
+double round_through(double value, DType dtype);
 
 // ---- shapes -------------------------------------------------------------------------------------------
 
@@ -291,6 +294,14 @@ class Tensor {
     // ref: src/ops/composite.rs:10-27
     Tensor softmax(int64_t dim) const;
     Tensor log_softmax(int64_t dim) const;
+    // ref: src/ops/shape_ops.rs:182-263
+    Tensor triu(int64_t diagonal) const;
+    Tensor tril(int64_t diagonal) const;
+    Tensor flip(const std::vector<int64_t> &dims) const;
+    // ref: src/ops/composite.rs:450-508 (compositions of the ops above, as the reference's are)
+    Tensor addcmul(const Tensor &tensor1, const Tensor &tensor2, Scalar value) const;
+    Tensor addcdiv(const Tensor &tensor1, const Tensor &tensor2, Scalar value) const;
+    Tensor lerp(const Tensor &end, const Operand &weight) const;
 
   private:
     TensorData d_;
@@ -305,8 +316,44 @@ struct ValuesAndIndices {
 Tensor binary_op(BinaryOp op, const Operand &lhs, const Operand &rhs);
 // torch.where (ref: src/ops/binary.rs:152-176).
 Tensor where_(const Tensor &condition, const Operand &x, const Operand &y);
+// The optimizers' single-rounding steps (ref: src/optim/mod.rs:569-616): new tensors from tensors of one
+// shape, floating point dtype and device. A finite scalar beyond the range of the type it is converted
+// to (the dtype for alpha, the computation type otherwise) is an error.
+namespace optim {
+Tensor scaled_add(const Tensor &a, const Tensor &b, double alpha);                // a + alpha * b
+Tensor lerp(const Tensor &a, const Tensor &b, double weight);                     // lerp(a, b, weight)
+Tensor addcmul(const Tensor &a, const Tensor &b, const Tensor &c, double value);  // a + value * b * c
+Tensor addcdiv(const Tensor &a, const Tensor &b, const Tensor &c, double value);  // a + value * b / c
+
+// One parameter's update, as the loop bodies of Sgd::step (ref: src/optim/sgd.rs:152-191) and of Adam's
+// and AdamW's (ref: src/optim/adam.rs:123-171) compute it. Tensors here are values, so where the reference
+// updates the parameter and its state in place these return the new parameter and replace the state's
+// tensors; the bits are the same. Every coefficient is checked before anything is computed.
+struct SgdOptions {
+    double lr = 0.0, momentum = 0.0, dampening = 0.0, weight_decay = 0.0;
+    bool nesterov = false, maximize = false;
+};
+struct AdamOptions {
+    double lr = 1e-3, beta1 = 0.9, beta2 = 0.999, eps = 1e-8, weight_decay = 0.0;
+    bool amsgrad = false, maximize = false;
+};
+struct AdamState {
+    double step;  // counted in f32 like the reference's default-dtype step tensor
+    Tensor exp_avg, exp_avg_sq;
+    std::optional<Tensor> max_exp_avg_sq;
+};
+Tensor sgd_step(const Tensor &p, const Tensor &grad, std::optional<Tensor> &momentum_buffer, const SgdOptions &o);
+Tensor adam_step(const Tensor &p, const Tensor &grad, std::optional<AdamState> &state, const AdamOptions &o,
+                 bool decoupled_weight_decay);
+}  // namespace optim
 
 // ---- backend dispatch (ref: src/backend/mod.rs:298-534) ---------------------------------------------
+
+// The optimizers' fused steps (ref: src/backend/cpu/mod.rs:509-530).
+struct Fused {
+    enum Kind { ScaledAdd = 0, Lerp = 1, Addcmul = 2, Addcdiv = 3 } kind;
+    double scalar;  // alpha, weight or value
+};
 
 namespace backend {
 struct Branch {
@@ -327,6 +374,9 @@ void var(const TensorData &out, const TensorData &src, const std::vector<bool> &
 void arg_reduce(const TensorData *values, const TensorData &indices, const TensorData &src, size_t dim,
                 bool is_max);
 void softmax(const TensorData &out, const TensorData &src, size_t dim, bool log);
+void fused(const Fused &op, const TensorData &out, const TensorData &a, const TensorData &b, const TensorData *c);
+void triangle(const TensorData &out, const TensorData &src, int64_t diagonal, bool upper);
+void flip(const TensorData &out, const TensorData &src, const std::vector<bool> &mask);
 // Host <-> device and device <-> host transfers of contiguous data of one dtype.
 void upload(const TensorData &dst, const TensorData &src);
 void download(const TensorData &dst, const TensorData &src);

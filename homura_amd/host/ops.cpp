@@ -1,5 +1,6 @@
 // The ops front end: argument checks, type promotion, broadcasting, output allocation and the
 // call into the backend. See homura.hpp for the map to the reference's files.
+#include <cmath>
 #include <cstring>
 
 #include "homura.hpp"
@@ -199,6 +200,29 @@ Tensor softmax_op(const Tensor &x, int64_t dim, bool log) {
     size_t d = normalize_dim(dim, src.layout.shape.size());
     TensorData out = uninit_data(src.layout.shape, src.dtype, src.device());
     backend::softmax(out, src, d, log);
+    return Tensor(out);
+}
+
+// ref: src/ops/shape_ops.rs:181-196
+Tensor triangle_op(const Tensor &x, int64_t diagonal, bool upper) {
+    const TensorData &src = x.data();
+    if (src.layout.shape.size() < 2) {
+        throw Error(std::string(upper ? "triu" : "tril") + ": input tensor must have at least 2 dimensions");
+    }
+    TensorData out = uninit_data(src.layout.shape, src.dtype, src.device());
+    backend::triangle(out, src, diagonal, upper);
+    return Tensor(out);
+}
+
+// ref: src/optim/mod.rs:602-640
+Tensor fused_op(Fused op, const Tensor &a, const Tensor &b, const Tensor *c) {
+    DType dtype = a.dtype();
+    DType converted = op.kind == Fused::ScaledAdd || dtype == DType::F64 ? dtype : DType::F32;
+    if (!Scalar::of_float(op.scalar).checked_to(converted)) {
+        throw Error(std::string("value cannot be converted to type ") + name_of(converted) + " without overflow");
+    }
+    TensorData out = uninit_data(a.shape(), dtype, a.device());
+    backend::fused(op, out, a.data(), b.data(), c ? &c->data() : nullptr);
     return Tensor(out);
 }
 
@@ -449,5 +473,146 @@ Tensor Tensor::any_dim(const std::vector<int64_t> &dims, bool keepdim) const {
 
 Tensor Tensor::softmax(int64_t dim) const { return softmax_op(*this, dim, false); }
 Tensor Tensor::log_softmax(int64_t dim) const { return softmax_op(*this, dim, true); }
+
+// ---- triangles and flips (ref: src/ops/shape_ops.rs:181-263) ---------------------------------------------
+
+Tensor Tensor::triu(int64_t diagonal) const { return triangle_op(*this, diagonal, true); }
+Tensor Tensor::tril(int64_t diagonal) const { return triangle_op(*this, diagonal, false); }
+
+Tensor Tensor::flip(const std::vector<int64_t> &dims) const {
+    const size_t nd = d_.layout.shape.size();
+    std::vector<bool> mask = dims.empty() ? std::vector<bool>(nd, false) : dims_mask(dims, nd);
+    TensorData out = uninit_data(d_.layout.shape, d_.dtype, d_.device());
+    backend::flip(out, d_, mask);
+    return Tensor(out);
+}
+
+// ---- compositions (ref: src/ops/composite.rs:448-508) ----------------------------------------------------
+
+Tensor Tensor::addcmul(const Tensor &tensor1, const Tensor &tensor2, Scalar value) const {
+    return add(tensor1.mul(value).mul(tensor2));
+}
+
+Tensor Tensor::addcdiv(const Tensor &tensor1, const Tensor &tensor2, Scalar value) const {
+    if (!is_floating_point(tensor1.dtype()) && !is_floating_point(tensor2.dtype())) {
+        throw Error("Integer division with addcdiv is no longer supported. Use self.add(tensor1.div(tensor2).mul(value)) "
+                    "instead.");
+    }
+    return add(tensor1.mul(value).div(tensor2));
+}
+
+Tensor Tensor::lerp(const Tensor &end, const Operand &weight) const {
+    Tensor diff = end.sub(*this);
+    if (std::holds_alternative<Scalar>(weight)) {
+        Scalar w = std::get<Scalar>(weight);
+        double wf = w.to_f64();
+        if (std::fabs(wf) < 0.5) return add(diff.mul(w));
+        return end.sub(diff.mul(Scalar::of_float(1.0 - wf)));
+    }
+    const Tensor &w = std::get<Tensor>(weight);
+    Tensor low = add(w.mul(diff));
+    Tensor high = end.sub(diff.mul(w.neg().add(Scalar::of_float(1.0))));
+    return where_(w.abs().less(Scalar::of_float(0.5)), low, high);
+}
+
+// ---- the optimizers' steps (ref: src/optim/mod.rs:569-616) -----------------------------------------------
+
+namespace optim {
+Tensor scaled_add(const Tensor &a, const Tensor &b, double alpha) { return fused_op(Fused{Fused::ScaledAdd, alpha}, a, b, nullptr); }
+Tensor lerp(const Tensor &a, const Tensor &b, double weight) { return fused_op(Fused{Fused::Lerp, weight}, a, b, nullptr); }
+Tensor addcmul(const Tensor &a, const Tensor &b, const Tensor &c, double value) {
+    return fused_op(Fused{Fused::Addcmul, value}, a, b, &c);
+}
+Tensor addcdiv(const Tensor &a, const Tensor &b, const Tensor &c, double value) {
+    return fused_op(Fused{Fused::Addcdiv, value}, a, b, &c);
+}
+
+namespace {
+DType computation(DType dtype) { return dtype == DType::F16 || dtype == DType::BF16 ? DType::F32 : dtype; }
+
+// ref: src/optim/mod.rs:618-640
+void check_coefficient(double value, DType dtype) {
+    if (!Scalar::of_float(value).checked_to(dtype)) {
+        throw Error(std::string("value cannot be converted to type ") + name_of(dtype) + " without overflow");
+    }
+}
+
+void check_like(const Tensor &p, const Tensor &t, const char *what) {
+    if (t.shape() != p.shape() || t.dtype() != p.dtype() || t.device() != p.device()) {
+        throw Error(std::string(what) + " must have the parameter's shape, dtype and device");
+    }
+}
+}  // namespace
+
+Tensor sgd_step(const Tensor &p, const Tensor &grad_in, std::optional<Tensor> &momentum_buffer, const SgdOptions &o) {
+    check_like(p, grad_in, "the gradient");
+    if (o.nesterov && (o.momentum <= 0.0 || o.dampening != 0.0)) {
+        throw Error("Nesterov momentum requires a momentum and zero dampening");
+    }
+    // ref: src/optim/sgd.rs:257-263, 275-299: every alpha of the step, in the parameter's dtype.
+    check_coefficient(-o.lr, p.dtype());
+    if (o.weight_decay != 0.0) check_coefficient(o.weight_decay, p.dtype());
+    if (o.momentum != 0.0) {
+        if (momentum_buffer) {
+            check_like(p, *momentum_buffer, "the momentum buffer");
+            check_coefficient(1.0 - o.dampening, p.dtype());
+        }
+        if (o.nesterov) check_coefficient(o.momentum, p.dtype());
+    }
+    Tensor grad = o.maximize ? grad_in.neg() : grad_in;
+    if (o.weight_decay != 0.0) grad = scaled_add(grad, p, o.weight_decay);
+    if (o.momentum != 0.0) {
+        if (!momentum_buffer) {
+            // A copy of its own: the gradient may be the caller's tensor.
+            momentum_buffer = grad.mul(Scalar::of_int(1));
+        } else {
+            Tensor scaled = momentum_buffer->mul(Scalar::of_float(o.momentum));
+            momentum_buffer = scaled_add(scaled, grad, 1.0 - o.dampening);
+        }
+        grad = o.nesterov ? scaled_add(grad, *momentum_buffer, o.momentum) : *momentum_buffer;
+    }
+    return scaled_add(p, grad, -o.lr);
+}
+
+Tensor adam_step(const Tensor &p_in, const Tensor &grad_in, std::optional<AdamState> &state, const AdamOptions &o,
+                 bool decoupled_weight_decay) {
+    check_like(p_in, grad_in, "the gradient");
+    const DType dtype = p_in.dtype();
+    const double next = static_cast<double>(static_cast<float>((state ? state->step : 0.0) + 1.0));
+    auto step_size = [&](double step) { return o.lr / (1.0 - std::pow(o.beta1, step)); };
+    // ref: src/optim/adam.rs:291-304
+    check_coefficient(-step_size(next), computation(dtype));
+    if (o.weight_decay != 0.0 && !decoupled_weight_decay) check_coefficient(o.weight_decay, dtype);
+    if (state) {
+        check_like(p_in, state->exp_avg, "exp_avg");
+        check_like(p_in, state->exp_avg_sq, "exp_avg_sq");
+        if (o.amsgrad) {
+            if (!state->max_exp_avg_sq) throw Error("the state has no max_exp_avg_sq, but amsgrad is set");
+            check_like(p_in, *state->max_exp_avg_sq, "max_exp_avg_sq");
+        }
+    } else {
+        Tensor zeros = Tensor::full(p_in.shape(), Scalar::of_int(0), dtype, p_in.device());
+        state = AdamState{0.0, zeros, zeros, o.amsgrad ? std::optional<Tensor>(zeros) : std::nullopt};
+    }
+    Tensor p = p_in;
+    Tensor grad = o.maximize ? grad_in.neg() : grad_in;
+    state->step = next;
+    if (o.weight_decay != 0.0) {
+        if (decoupled_weight_decay) p = p.mul(Scalar::of_float(1.0 - o.lr * o.weight_decay));
+        else grad = scaled_add(grad, p, o.weight_decay);
+    }
+    state->exp_avg = lerp(state->exp_avg, grad, 1.0 - o.beta1);
+    state->exp_avg_sq = addcmul(state->exp_avg_sq.mul(Scalar::of_float(o.beta2)), grad, grad, 1.0 - o.beta2);
+    const double bias_correction2 = 1.0 - std::pow(o.beta2, next);
+    const double bias_correction2_sqrt = std::pow(bias_correction2, 0.5);
+    const Tensor *second = &state->exp_avg_sq;
+    if (o.amsgrad && state->max_exp_avg_sq) {
+        state->max_exp_avg_sq = state->max_exp_avg_sq->maximum(state->exp_avg_sq);
+        second = &*state->max_exp_avg_sq;
+    }
+    Tensor denom = second->sqrt().div(Scalar::of_float(bias_correction2_sqrt)).add(Scalar::of_float(o.eps));
+    return addcdiv(p, state->exp_avg, denom, -step_size(next));
+}
+}  // namespace optim
 
 }  // namespace homura

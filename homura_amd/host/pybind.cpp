@@ -82,6 +82,38 @@ PYBIND11_MODULE(_host, m) {
     m.def("full", [](const Shape &shape, const py::handle &v, DType d, const std::string &dev) {
         return Tensor::full(shape, std::get<Scalar>(to_operand(v)), d, parse_device(dev));
     });
+    // The optimizers' single-rounding steps (ref: src/optim/mod.rs:569-592).
+    m.def("scaled_add", &optim::scaled_add);
+    m.def("lerp_step", &optim::lerp);
+    m.def("addcmul_step", &optim::addcmul);
+    m.def("addcdiv_step", &optim::addcdiv);
+    // One parameter's optimizer update; the state goes in and comes out as tensors (None before the first step).
+    m.def("sgd_step",
+          [](const Tensor &p, const Tensor &grad, std::optional<Tensor> buffer, double lr, double momentum, double dampening,
+             double weight_decay, bool nesterov, bool maximize) {
+              optim::SgdOptions o{lr, momentum, dampening, weight_decay, nesterov, maximize};
+              Tensor out = optim::sgd_step(p, grad, buffer, o);
+              return py::make_tuple(out, buffer);
+          },
+          py::arg("p"), py::arg("grad"), py::arg("momentum_buffer"), py::arg("lr"), py::arg("momentum") = 0.0,
+          py::arg("dampening") = 0.0, py::arg("weight_decay") = 0.0, py::arg("nesterov") = false,
+          py::arg("maximize") = false);
+    m.def("adam_step",
+          [](const Tensor &p, const Tensor &grad, const py::object &state, double lr, double beta1, double beta2, double eps,
+             double weight_decay, bool amsgrad, bool maximize, bool decoupled) {
+              std::optional<optim::AdamState> st;
+              if (!state.is_none()) {
+                  py::tuple t = state.cast<py::tuple>();
+                  st = optim::AdamState{t[0].cast<double>(), t[1].cast<Tensor>(), t[2].cast<Tensor>(),
+                                        t[3].is_none() ? std::nullopt : std::optional<Tensor>(t[3].cast<Tensor>())};
+              }
+              optim::AdamOptions o{lr, beta1, beta2, eps, weight_decay, amsgrad, maximize};
+              Tensor out = optim::adam_step(p, grad, st, o, decoupled);
+              return py::make_tuple(out, py::make_tuple(st->step, st->exp_avg, st->exp_avg_sq, st->max_exp_avg_sq));
+          },
+          py::arg("p"), py::arg("grad"), py::arg("state"), py::arg("lr"), py::arg("beta1") = 0.9, py::arg("beta2") = 0.999,
+          py::arg("eps") = 1e-8, py::arg("weight_decay") = 0.0, py::arg("amsgrad") = false, py::arg("maximize") = false,
+          py::arg("decoupled_weight_decay") = false);
     m.def("reduce_plan", [](const Tensor &t, const std::vector<int64_t> &dims) {
         auto p = rocm_reduce_plan(t, dims);
         return py::make_tuple(p.group, p.splits, p.chunk);
@@ -201,4 +233,14 @@ PYBIND11_MODULE(_host, m) {
     T.def("any_dim", [](const Tensor &t, const py::handle &d, bool k) { return t.any_dim(to_dims(d), k); });
     T.def("softmax", &Tensor::softmax);
     T.def("log_softmax", &Tensor::log_softmax);
+    T.def("triu", &Tensor::triu, py::arg("diagonal") = 0);
+    T.def("tril", &Tensor::tril, py::arg("diagonal") = 0);
+    T.def("flip", &Tensor::flip);
+    T.def("addcmul", [](const Tensor &t, const Tensor &t1, const Tensor &t2, const py::handle &value) {
+        return t.addcmul(t1, t2, std::get<Scalar>(to_operand(value)));
+    });
+    T.def("addcdiv", [](const Tensor &t, const Tensor &t1, const Tensor &t2, const py::handle &value) {
+        return t.addcdiv(t1, t2, std::get<Scalar>(to_operand(value)));
+    });
+    T.def("lerp", [](const Tensor &t, const Tensor &end, const py::handle &weight) { return t.lerp(end, to_operand(weight)); });
 }

@@ -199,6 +199,32 @@ hmr_status hmr_where_constant(hmr_context_t ctx, const hmr_tensor_desc *out,
                               const hmr_tensor_desc *cond, const hmr_tensor_desc *x,
                               uint64_t x_bits, const hmr_tensor_desc *y, uint64_t y_bits);
 
+/* ---- fused optimiser steps, triangle, flip ------------------- ref: csrc/homura_rocm.h:195-263 */
+#define HMR_FUSED_SCALED_ADD 0
+#define HMR_FUSED_LERP 1
+#define HMR_FUSED_ADDCMUL 2
+#define HMR_FUSED_ADDCDIV 3
+
+/* ref :221-230  cpu::fused (src/backend/cpu/mod.rs:509-569): floating point operands of one dtype,
+ * one rounding to it; `c` is NULL for SCALED_ADD and LERP. `coefficient` is already in the
+ * computation type (f32 for F16/BF16/F32): alpha rounded to the dtype first, the Lerp coefficient
+ * (weight, or weight - 1 when `small` is 0), or value.
+ *   SCALED_ADD fma(b, coefficient, a)          LERP    fma(coefficient, b - a, small ? a : b)
+ *   ADDCMUL    fma(coefficient * b, c, a)      ADDCDIV a + coefficient * b / c */
+hmr_status hmr_fused(hmr_context_t ctx, int32_t op, const hmr_tensor_desc *out,
+                     const hmr_tensor_desc *a, const hmr_tensor_desc *b,
+                     const hmr_tensor_desc *c, double coefficient, int32_t small);
+
+/* ref :257-260  cpu::triangle (src/backend/cpu/misc.rs:347-381): out = src where the column minus
+ * the row index (the last two dimensions, ndim >= 2) is at least (upper) or at most `diagonal`,
+ * else 0. Any dtype, one for both. */
+hmr_status hmr_triangle(hmr_context_t ctx, const hmr_tensor_desc *out,
+                        const hmr_tensor_desc *src, int64_t diagonal, int32_t upper);
+
+/* ref :262-263  cpu::flip (src/backend/cpu/misc.rs:384-411): out = src for one dtype, where src's
+ * strides may be negative (reversed dimensions, offset at the last element of each). */
+hmr_status hmr_flip(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_tensor_desc *src);
+
 /* ---- reductions --------------------------------------------- ref: csrc/homura_rocm.h:297-346 */
 /*
  * `kept`: the kept dimensions with the SOURCE's strides, data, offset, dtype; `red`: the reduced

@@ -18,25 +18,10 @@
 extern "C" {
 #endif
 
-/* ref :195-199 */
-#define HMR_FUSED_SCALED_ADD 0
-#define HMR_FUSED_LERP 1
-#define HMR_FUSED_ADDCMUL 2
-#define HMR_FUSED_ADDCDIV 3
-
-/* ref :227 */
-hmr_status hmr_fused(hmr_context_t ctx, int32_t op, const hmr_tensor_desc *out,
-                     const hmr_tensor_desc *a, const hmr_tensor_desc *b,
-                     const hmr_tensor_desc *c, double coefficient, int32_t small);
 /* ref :242 */
 hmr_status hmr_addr(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_tensor_desc *v1,
                     const hmr_tensor_desc *v2, const hmr_tensor_desc *input, double alpha,
                     double beta, int64_t alpha_int, int64_t beta_int);
-/* ref :259 */
-hmr_status hmr_triangle(hmr_context_t ctx, const hmr_tensor_desc *out,
-                        const hmr_tensor_desc *src, int64_t diagonal, int32_t upper);
-/* ref :263 */
-hmr_status hmr_flip(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_tensor_desc *src);
 
 /* ref :276-295 */
 #define HMR_RANDOM_INT_TILE 256

@@ -606,6 +606,108 @@ void where_constant(const hcb_tensor &out, const hcb_tensor &cond, const hcb_ten
     where_(out, cond, x ? *x : cx.view, y ? *y : cy.view);
 }
 
+// ---- the optimizers' fused steps (ref: src/backend/cpu/mod.rs:509-569) -------------------------
+//
+// `kind`: 0 ScaledAdd(alpha), 1 Lerp(weight), 2 Addcmul(value), 3 Addcdiv(value); `c` only for 2
+// and 3. Each element is computed in the computation type and rounded to the dtype once; mul_add
+// is a true fused multiply-add (std::fma).
+void fused(int kind, double scalar, const hcb_tensor &out, const hcb_tensor &a, const hcb_tensor &b,
+           const hcb_tensor *c) {
+    dispatch_float(out.dtype, [&](auto t) {
+        using T = typename decltype(t)::type;
+        using C = typename Fl<T>::C;
+        auto mul_add = [](C x, C y, C z) { return static_cast<C>(std::fma(x, y, z)); };
+        switch (kind) {
+            case 0: {
+                const C alpha = Fl<T>::up(Fl<T>::down(of<C>(scalar)));  // alpha rounded to the dtype first
+                map2<T, T, T>(out, a, b, [=](T x, T y) { return Fl<T>::down(mul_add(Fl<T>::up(y), alpha, Fl<T>::up(x))); });
+                break;
+            }
+            case 1: {
+                const C weight = of<C>(scalar);
+                const bool small = std::fabs(weight) < of<C>(0.5);
+                const C coeff = small ? weight : weight - of<C>(1.0);
+                map2<T, T, T>(out, a, b, [=](T x, T y) {
+                    const C xc = Fl<T>::up(x), yc = Fl<T>::up(y);
+                    return Fl<T>::down(mul_add(coeff, yc - xc, small ? xc : yc));
+                });
+                break;
+            }
+            case 2: {
+                if (!c) panic("addcmul has three operands");
+                const C value = of<C>(scalar);
+                map3<T, T, T, T>(out, a, b, *c, [=](T x, T y, T z) {
+                    return Fl<T>::down(mul_add(value * Fl<T>::up(y), Fl<T>::up(z), Fl<T>::up(x)));
+                });
+                break;
+            }
+            case 3: {
+                if (!c) panic("addcdiv has three operands");
+                const C value = of<C>(scalar);
+                map3<T, T, T, T>(out, a, b, *c, [=](T x, T y, T z) {
+                    return Fl<T>::down(Fl<T>::up(x) + value * Fl<T>::up(y) / Fl<T>::up(z));
+                });
+                break;
+            }
+            default: panic("unknown fused step");
+        }
+    });
+}
+
+// ---- triangle, flip (ref: src/backend/cpu/misc.rs:347-411) ---------------------------------------
+
+void triangle(const hcb_tensor &out, const hcb_tensor &src, int64_t diagonal, bool upper) {
+    check_shape(out, src);
+    const int nd = src.ndim;
+    if (nd < 2) panic("triangle needs two dimensions");
+    if (num_elements(src) == 0) return;
+    const int64_t rows = src.shape[nd - 2], cols = src.shape[nd - 1];
+    dispatch_all(src.dtype, [&](auto t) {
+        using T = typename decltype(t)::type;
+        T *po = base<T>(out);
+        const T *ps = base<T>(src);
+        const int64_t *const st[2] = {out.strides, src.strides};
+        Plan<2> batches(nd - 2, src.shape, st);
+        const int64_t b[2] = {out.offset, src.offset};
+        const int64_t ro = out.strides[nd - 2], co = out.strides[nd - 1];
+        const int64_t rs = src.strides[nd - 2], cs = src.strides[nd - 1];
+        batches.for_each(b, [&](const int64_t(&o)[2]) {
+            for (int64_t r = 0; r < rows; ++r) {
+                for (int64_t c = 0; c < cols; ++c) {
+                    const int64_t d = c - r;
+                    const bool keep = upper ? d >= diagonal : d <= diagonal;
+                    po[o[0] + r * ro + c * co] = keep ? ps[o[1] + r * rs + c * cs] : T{};
+                }
+            }
+        });
+    });
+}
+
+// `out` is contiguous; `mask[d]` reverses dimension d.
+void flip(const hcb_tensor &out, const hcb_tensor &src, const uint8_t *mask) {
+    check_shape(out, src);
+    const int64_t n = num_elements(src);
+    const int nd = src.ndim;
+    dispatch_all(src.dtype, [&](auto t) {
+        using T = typename decltype(t)::type;
+        T *po = base<T>(out);
+        const T *ps = base<T>(src);
+        std::vector<int64_t> idx(static_cast<size_t>(nd), 0);
+        for (int64_t linear = 0; linear < n; ++linear) {
+            int64_t off = src.offset;
+            for (int d = 0; d < nd; ++d) {
+                const int64_t i = mask[d] ? src.shape[d] - 1 - idx[d] : idx[d];
+                off += i * src.strides[d];
+            }
+            po[out.offset + linear] = ps[off];
+            for (int d = nd - 1; d >= 0; --d) {
+                if (++idx[d] < src.shape[d]) break;
+                idx[d] = 0;
+            }
+        }
+    });
+}
+
 // ---- reductions (ref: src/backend/cpu/reduce.rs:10-225) ----------------------------------------
 
 struct Split {
@@ -925,6 +1027,17 @@ int orc_softmax(const hcb_tensor *out, const hcb_tensor *src, int32_t dim, int32
     return orc::guarded([&] { orc::softmax(*out, *src, dim, log != 0); });
 }
 
+int orc_fused(int32_t kind, double scalar, const hcb_tensor *out, const hcb_tensor *a, const hcb_tensor *b,
+              const hcb_tensor *c) {
+    return orc::guarded([&] { orc::fused(kind, scalar, *out, *a, *b, c); });
+}
+int orc_triangle(const hcb_tensor *out, const hcb_tensor *src, int64_t diagonal, int32_t upper) {
+    return orc::guarded([&] { orc::triangle(*out, *src, diagonal, upper != 0); });
+}
+int orc_flip(const hcb_tensor *out, const hcb_tensor *src, const uint8_t *mask) {
+    return orc::guarded([&] { orc::flip(*out, *src, mask); });
+}
+
 // erf in f64, for the known-answer table of ref: src/backend/cpu/num.rs:225-248.
 double orc_erf(double x) { return orc::erf64(x); }
 
@@ -939,6 +1052,7 @@ const hcb_backend *orc_backend(void) {
         "homura CPU oracle", orc_last_error, orc_copy,  orc_fill,           orc_unary,
         orc_binary,          orc_binary_constant,       orc_binary_scalar,  orc_where,
         orc_where_constant,  orc_reduce,     orc_var,   orc_arg_reduce,     orc_softmax,
+        orc_fused,           orc_triangle,   orc_flip,
     };
     return &table;
 }

@@ -378,3 +378,71 @@ def test_softmax_against_exact_arithmetic():
             wl = (x[r, c] - m) - math.log(float(tot))
             assert abs(glog[r, c] - wl) <= 16 * math.ulp(wl)
         assert abs(sum(Fraction(float(g)) for g in got[r]) - 1) < Fraction(1, 10**13)
+
+
+# ---- fused optimizer steps: exact rational arithmetic with the roundings where the reference has them ------
+
+def round_to(frac, dtype):
+    """`frac` (a Fraction) rounded to nearest-even in F32 or F64, as a Fraction; finite normal results only."""
+    if frac == 0:
+        return Fraction(0)
+    p = 24 if dtype == DT.F32 else 53
+    sign, mag = (-1 if frac < 0 else 1), abs(frac)
+    e = mag.numerator.bit_length() - mag.denominator.bit_length()
+    if Fraction(2) ** e > mag:
+        e -= 1
+    scaled = mag / Fraction(2) ** (e - p + 1)  # in [2^(p-1), 2^p)
+    q, r = divmod(scaled.numerator, scaled.denominator)
+    twice = 2 * r
+    if twice > scaled.denominator or (twice == scaled.denominator and q % 2 == 1):
+        q += 1
+    return sign * q * Fraction(2) ** (e - p + 1)
+
+
+@pytest.mark.parametrize("dtype", [DT.F32, DT.F64])
+def test_fused_steps_round_once_where_the_reference_does(dtype):
+    """ref: src/backend/cpu/mod.rs:540-567. ScaledAdd = R(a + alpha*b); Lerp = R(w*R(b-a) + a) or
+    R((w-1)*R(b-a) + b); Addcmul = R(R(v*b)*c + a); Addcdiv = R(a + R(R(v*b)/c)), R = one rounding to the
+    computation type. A product rounded before its sum (no FMA), or an FMA where the reference has none,
+    differs from these on some of the 300 samples."""
+    rng = np.random.default_rng(17)
+    n = 300
+    npdt = NP[dtype]
+    a, b, c = ((rng.standard_normal(n) * 2.0 ** rng.integers(-3, 4, n)).astype(npdt) for _ in range(3))
+    c = np.where(np.abs(c) < 0.01, npdt(0.5), c).astype(npdt)
+    R = lambda f: round_to(f, dtype)
+    F = lambda arr: [Fraction(float(v)) for v in arr]
+    fa, fb, fc = F(a), F(b), F(c)
+    ta, tb, tc = (tensor(v, dtype) for v in (a, b, c))
+
+    def check(got, want, what):
+        got = [Fraction(float(v)) for v in array(got)]
+        bad = [i for i in range(n) if got[i] != want[i]]
+        assert not bad, f"{what}: element {bad[0]}: {float(got[bad[0]])!r} != {float(want[bad[0]])!r} ({len(bad)} differ)"
+
+    differs_without_fma = 0
+    for v in (0.1, -0.3, 0.7, 1.0 / 3.0):
+        s = Fraction(float(npdt(v)))  # the coefficient in the computation type
+        check(h.scaled_add(ta, tb, v), [R(x + s * y) for x, y in zip(fa, fb)], f"scaled_add {v}")
+        differs_without_fma += sum(R(x + s * y) != R(x + R(s * y)) for x, y in zip(fa, fb))
+        if abs(v) < 0.5:
+            want = [R(s * R(y - x) + x) for x, y in zip(fa, fb)]
+        else:
+            w1 = R(s - 1)
+            want = [R(w1 * R(y - x) + y) for x, y in zip(fa, fb)]
+        check(h.lerp_step(ta, tb, v), want, f"lerp {v}")
+        check(h.addcmul_step(ta, tb, tc, v), [R(R(s * y) * z + x) for x, y, z in zip(fa, fb, fc)], f"addcmul {v}")
+        check(h.addcdiv_step(ta, tb, tc, v), [R(x + R(R(s * y) / z)) for x, y, z in zip(fa, fb, fc)], f"addcdiv {v}")
+    assert differs_without_fma > 20  # the samples do tell an FMA from a rounded product
+
+
+def test_scaled_add_rounds_alpha_to_the_dtype_first():
+    """ref: src/backend/cpu/mod.rs:543: alpha = down(of(alpha)).up(); the other steps keep their coefficient in
+    the computation type (f32 for BF16)."""
+    bf = lambda *v: tensor(from_f64(np.array(v, dtype=np.float64), DT.BF16), DT.BF16)
+    # 0.1 in BF16 is 0.10009765625; a + that, rounded to BF16's 8 bits.
+    assert list(vals(h.scaled_add(bf(1.0, 2.0, -3.0), bf(1.0, 1.0, 1.0), 0.1))) == [1.1015625, 2.09375, -2.90625]
+    # 1 + 2^-9 is an f32 but rounds to 1 in BF16. As an f32 value: 512 * (1 + 2^-9) * 1 + 1.5 = 514.5, which is
+    # 516 in BF16 (spacing 4); as a BF16 alpha: 512 + 1.5 = 513.5, which is 512.
+    assert list(vals(h.addcmul_step(bf(1.5), bf(512.0), bf(1.0), 1.0 + 2.0 ** -9))) == [516.0]
+    assert list(vals(h.scaled_add(bf(1.5), bf(512.0), 1.0 + 2.0 ** -9))) == [512.0]
