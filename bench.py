@@ -264,6 +264,30 @@ def per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP
     del s
     add(4, "softmax f32 [32,2048,2048] causal", 8 * n5b, lambda: scores.softmax(-1))
     add(4, "log_softmax f32 [32,2048,2048] causal", 8 * n5b, lambda: scores.log_softmax(-1))
+    # The callers next to the path (cfg null: not a BASELINE config): the optimizers' single-rounding steps on
+    # 67 108 864 parameters, a whole SGD / Adam update (bytes = the sum over its kernels), triangles of the causal
+    # scores and flips.
+    del scores
+    for dt, name, size in ((DT.F32, "f32", 4), (DT.BF16, "bf16", 2)):
+        prm = x.to(dt) if dt != DT.BF16 else x
+        grd = residual.to(dt) if dt != DT.F32 else residual
+        third = prm.mul(0.5).add(1.5)
+        add(None, f"scaled_add {name} (p + alpha * g)", 3 * size * N, lambda: h.scaled_add(prm, grd, -0.01))
+        add(None, f"lerp step {name}", 3 * size * N, lambda: h.lerp_step(prm, grd, 0.1))
+        add(None, f"addcmul step {name}", 4 * size * N, lambda: h.addcmul_step(prm, grd, third, 0.001))
+        add(None, f"addcdiv step {name}", 4 * size * N, lambda: h.addcdiv_step(prm, grd, third, -0.01))
+        buf = grd.mul(0.5)
+        add(None, f"sgd step {name}, momentum 0.9 (3 kernels: mul, 2 scaled_add)", 8 * size * N,
+            lambda: h.sgd_step(prm, grd, buf, lr=0.01, momentum=0.9))
+        state = h.adam_step(prm, grd, None, lr=1e-3)[1]
+        add(None, f"adam step {name} (7 kernels: lerp, mul, addcmul, sqrt, div, add, addcdiv)", 19 * size * N,
+            lambda: h.adam_step(prm, grd, state, lr=1e-3))
+        del prm, grd, third, buf, state
+    sq = residual.reshape([16, 2048, 2048])
+    add(None, "triu(1) f32 [16,2048,2048] (reads the kept half)", 6 * N, lambda: sq.triu(1))
+    add(None, "tril(0) f32 [16,2048,2048] (reads the kept half)", 6 * N, lambda: sq.tril(0))
+    add(None, "flip f32 [8,2048,4096] dims [1] (rows reversed)", 8 * N, lambda: residual.flip([1]))
+    add(None, "flip f32 [8,2048,4096] dims [2] (elements of a row reversed)", 8 * N, lambda: residual.flip([2]))
     return rows
 
 

@@ -14,6 +14,45 @@ uint64_t scalar_bits_of(double s) {
     return bits;
 }
 
+// ---- fill of a contiguous, 16-byte aligned destination -------------------------------------------------
+//
+// Nothing is read: a thread stores kFillTiles tiles of 16 bytes, a workgroup's width apart; the first
+// workgroup also writes the elements after the last whole tile. Other destinations go through the
+// map kernels with the value as a constant operand.
+constexpr int kFillTiles = 4;
+
+template <class W>
+__global__ void __launch_bounds__(kBlock) fill_kernel(char *out, int64_t n_tiles, int64_t n, W value) {
+    constexpr int V = 16 / static_cast<int>(sizeof(W));
+    W r[V];
+#pragma unroll
+    for (int i = 0; i < V; ++i) r[i] = value;
+    const int64_t first = static_cast<int64_t>(blockIdx.x) * (kFillTiles * kBlock) + threadIdx.x;
+#pragma unroll
+    for (int u = 0; u < kFillTiles; ++u) {
+        const int64_t t = first + static_cast<int64_t>(u) * kBlock;
+        if (t < n_tiles) store_tile<W, V, false>(out + t * 16, r);
+    }
+    const int64_t done = n_tiles * V;
+    if (blockIdx.x == 0 && done + threadIdx.x < n) reinterpret_cast<W *>(out)[done + threadIdx.x] = value;
+}
+
+template <class W>
+bool launch_fill(const MapCall &c, uint64_t bits, hipStream_t stream) {
+    constexpr int V = 16 / static_cast<int>(sizeof(W));
+    const bool flat = c.ndim == 0 || (c.ndim == 1 && c.stride[0][0] == 1);
+    if (!flat || reinterpret_cast<uintptr_t>(c.ptr[0]) % 16 != 0) return false;
+    const int64_t n_tiles = c.n / V;
+    const int64_t per_block = int64_t{kFillTiles} * kBlock;
+    const int64_t blocks = n_tiles / per_block + 1;  // at least one, for the elements after the last tile
+    if (blocks > (int64_t{1} << 22)) return false;
+    W value;
+    __builtin_memcpy(&value, &bits, sizeof(W));
+    hipLaunchKernelGGL((fill_kernel<W>), dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream, c.ptr[0], n_tiles, c.n,
+                       value);
+    return true;
+}
+
 }  // namespace
 }  // namespace hmr
 
@@ -73,7 +112,8 @@ hmr_status hmr_fill(hmr_context_t ctx, const hmr_tensor_desc *dst, uint64_t bits
         const uint64_t cbits[2] = {0, bits};
         return hmr::run_map(ctx, "fill", 2, descs, cbits, [&](const hmr::MapCall &call, hipStream_t stream) {
             return hmr::with_word(hmr::dtype_size(dst->dtype), [&](auto w) {
-                hmr::launch_map<hmr::Move<typename decltype(w)::type>>(call, stream);
+                using W = typename decltype(w)::type;
+                if (!hmr::launch_fill<W>(call, bits, stream)) hmr::launch_map<hmr::Move<W>>(call, stream);
             });
         });
     });

@@ -78,3 +78,42 @@ def test_fill_writes_every_dtype_and_layout():
             if n:
                 want = array(cpu).reshape(-1)
                 assert (want == want[0]).all() and want.dtype == NP[dtype]
+
+
+def test_fill_writes_exactly_its_span_at_every_offset_and_length():
+    """hmr_fill through the C ABI into the middle of a buffer: every alignment of the first element, every tail
+    after the last 16-byte tile, a span of several workgroups, a strided destination; the elements on both
+    sides keep their guard pattern."""
+    from ctypes import byref
+
+    from homura_amd import capi
+    L = capi.lib
+    ctx = capi.Context(0)
+    try:
+        for code, npdt, value, guard in ((capi.U8, np.uint8, 0xA5, 0x11), (capi.I16, np.int16, -1234, 0x1111),
+                                         (capi.F32, np.float32, 3.25, 7.0), (capi.I64, np.int64, -(1 << 40), 5)):
+            total = 70000
+            bits = int(np.array([value], dtype=npdt).view({1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}[
+                np.dtype(npdt).itemsize])[0])
+            spans = [(o, n) for o in range(0, 18) for n in (0, 1, 2, 3, 15, 16, 17, 33, 1023, 1031, 5000)] + [(3, 69000), (16, 65536)]
+            clean = np.full(total, guard, dtype=npdt)
+            buf = ctx.upload(clean)
+            for offset, n in spans:
+                capi.check(L.hmr_copy_from_host(ctx.handle, buf.ptr, clean.ctypes.data, clean.nbytes))
+                d = capi.make_desc(buf.ptr, code, [n], [1], offset)
+                capi.check(L.hmr_fill(ctx.handle, byref(d), bits))
+                ctx.synchronize()
+                got = buf.download(npdt, total)
+                want = np.full(total, guard, dtype=npdt)
+                want[offset:offset + n] = value
+                assert np.array_equal(got, want), f"{npdt.__name__} offset {offset} length {n}"
+            capi.check(L.hmr_copy_from_host(ctx.handle, buf.ptr, clean.ctypes.data, clean.nbytes))
+            d = capi.make_desc(buf.ptr, code, [100, 30], [600, 2], 8)
+            capi.check(L.hmr_fill(ctx.handle, byref(d), bits))
+            ctx.synchronize()
+            want = np.full(total, guard, dtype=npdt)
+            want[8:8 + 100 * 600].reshape(100, 600)[:, 0:60:2] = value
+            assert np.array_equal(buf.download(npdt, total), want), f"{npdt.__name__} strided"
+            buf.free()
+    finally:
+        ctx.close()
