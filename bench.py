@@ -283,6 +283,11 @@ def per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP
         add(None, f"adam step {name} (7 kernels: lerp, mul, addcmul, sqrt, div, add, addcdiv)", 19 * size * N,
             lambda: h.adam_step(prm, grd, state, lr=1e-3))
         del prm, grd, third, buf, state
+    mat = residual.reshape([8192, 8192])
+    v1, v2 = residual.narrow(0, 0, 1).narrow(1, 0, 2).reshape([8192]), residual.narrow(0, 1, 1).narrow(1, 0, 2).reshape([8192])
+    add(None, "addr f32 [8192,8192] (beta 0.5, alpha -1.5: one kernel)", 8 * N + 8 * 8192, lambda: mat.addr(v1, v2, 0.5, -1.5))
+    add(None, "addr f32 [8192,8192] without input (beta 0)", 4 * N + 8 * 8192, lambda: mat.addr(v1, v2, 0, -1.5))
+    del mat, v1, v2
     sq = residual.reshape([16, 2048, 2048])
     add(None, "triu(1) f32 [16,2048,2048] (reads the kept half)", 6 * N, lambda: sq.triu(1))
     add(None, "tril(0) f32 [16,2048,2048] (reads the kept half)", 6 * N, lambda: sq.tril(0))

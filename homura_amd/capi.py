@@ -78,6 +78,7 @@ PROTOTYPES = {
     "hmr_where": (c_int32, [CTX, DESC_P, DESC_P, DESC_P, DESC_P]),
     "hmr_where_constant": (c_int32, [CTX, DESC_P, DESC_P, DESC_P, c_uint64, DESC_P, c_uint64]),
     "hmr_fused": (c_int32, [CTX, c_int32, DESC_P, DESC_P, DESC_P, DESC_P, c_double, c_int32]),
+    "hmr_addr": (c_int32, [CTX, DESC_P, DESC_P, DESC_P, DESC_P, c_double, c_double, c_int64, c_int64]),
     "hmr_triangle": (c_int32, [CTX, DESC_P, DESC_P, c_int64, c_int32]),
     "hmr_flip": (c_int32, [CTX, DESC_P, DESC_P]),
     "hmr_reduce_workspace": (c_int32, [DESC_P, DESC_P, c_int32, POINTER(c_int64)]),
@@ -104,7 +105,7 @@ PROTOTYPES = {
 
 # Exported stubs of other kernel families (include/homura_rocm_unbuilt.h); bound without prototypes.
 UNBUILT = [
-    "hmr_addr", "hmr_random_uniform", "hmr_random_normal",
+    "hmr_random_uniform", "hmr_random_normal",
     "hmr_random_int", "hmr_exclusive_cumprod", "hmr_index_check", "hmr_index_select", "hmr_gather",
     "hmr_index_positions", "hmr_index_overwrite_workspace", "hmr_index_overwrite", "hmr_index_add_workspace",
     "hmr_index_add", "hmr_scatter_add_workspace", "hmr_scatter_add", "hmr_max_pool2d_backward_workspace",

@@ -1,4 +1,4 @@
-// hmr_fused, hmr_triangle, hmr_flip
+// hmr_fused, hmr_addr, hmr_triangle, hmr_flip
 // (ref: csrc/homura_rocm.h:195-263; csrc/elementwise.hip:334-371, 554-575, 1048-1175).
 #include "ew_common.hpp"
 
@@ -253,6 +253,51 @@ hmr_status hmr_fused(hmr_context_t ctx, int32_t op, const hmr_tensor_desc *out, 
                     default: hmr::launch_map<hmr::FusedStep<HMR_FUSED_ADDCDIV, T, false>>(call, stream); break;
                 }
             });
+        });
+    });
+}
+
+hmr_status hmr_addr(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_tensor_desc *v1, const hmr_tensor_desc *v2,
+                    const hmr_tensor_desc *input, double alpha, double beta, int64_t alpha_int, int64_t beta_int) {
+    return hmr::guarded([&] {
+        const bool is_float = out->dtype >= HMR_F16 && out->dtype <= HMR_F64;
+        const bool is_bool = out->dtype == HMR_BOOL;
+        // The coefficients as the kernels take them: bits of the computation type, i64, or 0 / 1.
+        uint64_t cbits[4] = {0, 0, 0, 0};
+        bool reads = false;
+        if (is_float) {
+            hmr::with_float_type(out->dtype, [&](auto t) {
+                using T = typename decltype(t)::type;
+                cbits[0] = hmr::coefficient_bits<T>(alpha);
+                cbits[1] = hmr::coefficient_bits<T>(beta);
+            });
+            reads = beta != 0.0;  // a NaN beta reads the input, as the CPU's `beta != 0` does
+        } else {
+            cbits[0] = is_bool ? static_cast<uint64_t>(alpha_int != 0) : static_cast<uint64_t>(alpha_int);
+            cbits[1] = is_bool ? static_cast<uint64_t>(beta_int != 0) : static_cast<uint64_t>(beta_int);
+            reads = beta_int != 0;
+        }
+        if (out->ndim != 2) return hmr::fail(HMR_INVALID, "addr: the output must have two dimensions");
+        if (reads && input == nullptr) return hmr::fail(HMR_INVALID, "addr: beta isn't zero but there is no input");
+        const hmr_tensor_desc *descs[4] = {out, v1, v2, reads ? input : nullptr};
+        return hmr::run_map(ctx, "addr", reads ? 4 : 3, descs, cbits, [&](const hmr::MapCall &call, hipStream_t stream) {
+            if (v1->dtype != out->dtype || v2->dtype != out->dtype || (reads && input->dtype != out->dtype)) return false;
+            if (is_bool) {
+                if (reads) hmr::launch_map<hmr::AddrBool<true>>(call, stream);
+                else hmr::launch_map<hmr::AddrBool<false>>(call, stream);
+                return true;
+            }
+            auto launch = [&](auto t) {
+                using T = typename decltype(t)::type;
+                if constexpr (hmr::Conv<T>::kind == hmr::Kind::Float) {
+                    if (reads) hmr::launch_map<hmr::AddrFloat<T, true>>(call, stream);
+                    else hmr::launch_map<hmr::AddrFloat<T, false>>(call, stream);
+                } else {
+                    if (reads) hmr::launch_map<hmr::AddrInt<T, true>>(call, stream);
+                    else hmr::launch_map<hmr::AddrInt<T, false>>(call, stream);
+                }
+            };
+            return hmr::with_int_type(out->dtype, launch) || hmr::with_float_type(out->dtype, launch);
         });
     });
 }

@@ -238,11 +238,12 @@ __device__ __forceinline__ typename F::Out apply(const F &f, typename F::In0 a, 
     else return f(a, b, c);
 }
 
-// A functor that carries a run-time parameter (a coefficient in its computation type) takes it from
-// the 64 bits that travel in the output's otherwise unused constant slot.
+// A functor that carries run-time parameters (coefficients in its computation type) takes them from
+// the 64-bit constant slots of operands that aren't constants: the output's, then the first input's.
 template <class F>
-__device__ __forceinline__ F make_functor(uint64_t param) {
-    if constexpr (std::is_constructible_v<F, uint64_t>) return F{param};
+__device__ __forceinline__ F make_functor(const uint64_t *slots) {
+    if constexpr (std::is_constructible_v<F, uint64_t, uint64_t>) return F{slots[0], slots[1]};
+    else if constexpr (std::is_constructible_v<F, uint64_t>) return F{slots[0]};
     else return F{};
 }
 
@@ -384,7 +385,7 @@ __global__ void __launch_bounds__(kBlock) map_rows_kernel(RowsArgs<F::N + 1> a) 
     using B = typename F::In1;
     using C = typename F::In2;
     using Off = std::conditional_t<FLAT, int64_t, uint32_t>;
-    const F f = make_functor<F>(a.cbits[0]);
+    const F f = make_functor<F>(a.cbits);
     const int64_t tiles = (a.n + V - 1) / V;
     const int64_t whole = a.n / V;  // tiles [0, whole) have all V elements
     const bool c0 = a.const_mask & 2u, c1 = a.const_mask & 4u, c2 = a.const_mask & 8u;
@@ -493,7 +494,7 @@ template <class F, class Idx>
 __global__ void __launch_bounds__(kBlock) map_any_kernel(AnyArgs<F::N + 1, Idx> a) {
     constexpr int N = F::N;
     using Out = typename F::Out;
-    const F f = make_functor<F>(a.cbits[0]);
+    const F f = make_functor<F>(a.cbits);
     const bool c0 = a.const_mask & 2u, c1 = a.const_mask & 4u, c2 = a.const_mask & 8u;
     // Signed: an input's strides may be negative (hmr_flip); every partial sum fits 31 bits then.
     using Off = std::conditional_t<std::is_same_v<Idx, uint32_t>, int32_t, int64_t>;

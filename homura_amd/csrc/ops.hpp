@@ -376,6 +376,79 @@ struct FusedStep {
     }
 };
 
+// ---- addr (ref: src/backend/cpu/linalg.rs:238-360) -----------------------------------------------------
+//
+// out = f(v1[i], v2[j], input[i][j]) with every step rounded to the dtype; READS = false leaves the
+// input out (beta is zero). alpha and beta arrive as bits of the computation type (floats) or as i64.
+template <class T, bool READS>
+struct AddrFloat {
+    static constexpr int N = READS ? 3 : 2;
+    using Out = T;
+    using In0 = T;
+    using In1 = T;
+    using In2 = std::conditional_t<READS, T, Unused>;
+    using C = typename Comp<T>::C;
+    C alpha, beta;
+    __device__ __forceinline__ AddrFloat(uint64_t a, uint64_t b) {
+        __builtin_memcpy(&alpha, &a, sizeof(C));
+        __builtin_memcpy(&beta, &b, sizeof(C));
+    }
+    __device__ __forceinline__ T product(T x, T y) const {
+        const T a = alpha == C(1) ? x : Comp<T>::down(Comp<T>::up(x) * alpha);
+        return Comp<T>::down(Comp<T>::up(a) * Comp<T>::up(y));
+    }
+    __device__ __forceinline__ T operator()(T x, T y) const { return product(x, y); }
+    __device__ __forceinline__ T operator()(T x, T y, T c) const {
+        const T p = product(x, y);
+        const T scaled = beta == C(1) ? c : Comp<T>::down(Comp<T>::up(c) * beta);
+        return Comp<T>::down(Comp<T>::up(scaled) + Comp<T>::up(p));
+    }
+};
+
+// Wrapping arithmetic in the element's width, which has the values of the CPU's wrapping i64
+// arithmetic truncated once.
+template <class T, bool READS>
+struct AddrInt {
+    static constexpr int N = READS ? 3 : 2;
+    using Out = T;
+    using In0 = T;
+    using In1 = T;
+    using In2 = std::conditional_t<READS, T, Unused>;
+    // At least 32 bits, so that no product is promoted to a signed int that could overflow.
+    using U = std::conditional_t<(sizeof(T) < 4), uint32_t, std::make_unsigned_t<T>>;
+    U alpha, beta;
+    __device__ __forceinline__ AddrInt(uint64_t a, uint64_t b) : alpha(static_cast<U>(a)), beta(static_cast<U>(b)) {}
+    __device__ __forceinline__ U product(T x, T y) const {
+        return static_cast<U>(static_cast<U>(static_cast<U>(x) * static_cast<U>(y)) * alpha);
+    }
+    __device__ __forceinline__ T operator()(T x, T y) const { return static_cast<T>(product(x, y)); }
+    __device__ __forceinline__ T operator()(T x, T y, T c) const {
+        U p = product(x, y);
+        // Keeps the sum of products of bytes away from the compiler's dot-product matcher, which (ROCm 7.2,
+        // gfx950) turns c * beta + (x * y) * alpha of 8-bit operands into v_dot4_u32_u8 of {x, c} and
+        // {alpha, beta} plus y: the value of x * alpha + c * beta + y.
+        if constexpr (sizeof(T) < 4) asm volatile("" : "+v"(p));
+        return static_cast<T>(static_cast<U>(static_cast<U>(static_cast<U>(c) * beta) + p));
+    }
+};
+
+template <bool READS>
+struct AddrBool {
+    static constexpr int N = READS ? 3 : 2;
+    using Out = bool_t;
+    using In0 = bool_t;
+    using In1 = bool_t;
+    using In2 = std::conditional_t<READS, bool_t, Unused>;
+    bool alpha;
+    __device__ __forceinline__ AddrBool(uint64_t a, uint64_t) : alpha(a != 0) {}
+    __device__ __forceinline__ bool_t operator()(bool_t x, bool_t y) const {
+        return bool_t{static_cast<uint8_t>(x.v != 0 && alpha && y.v != 0)};
+    }
+    __device__ __forceinline__ bool_t operator()(bool_t x, bool_t y, bool_t c) const {
+        return bool_t{static_cast<uint8_t>(c.v != 0 || (x.v != 0 && alpha && y.v != 0))};
+    }
+};
+
 // ---- where --------------------------------------------------------------------------------------------
 
 template <class W>

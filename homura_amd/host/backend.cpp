@@ -618,6 +618,32 @@ void flip(const TensorData &out, const TensorData &src, const std::vector<bool> 
     exec(out, [&](hmr_context_t ctx) { expect(hmr_flip(ctx, &o, &s)); });
 }
 
+// ref: src/backend/rocm/elementwise.rs:218-264: all four operands described with the output's two
+// dimensions, v1 broadcast along the columns and v2 along the rows.
+void addr(const TensorData &out, const TensorData &v1, const TensorData &v2, const TensorData &input, Scalar alpha,
+          Scalar beta) {
+    const Layout &lo = out.layout, &l1 = v1.layout, &l2 = v2.layout, &lc = input.layout;
+    if (l1.shape.size() != 1 || l2.shape.size() != 1 || lo.shape != Shape{l1.shape[0], l2.shape[0]} || lc.shape != lo.shape) {
+        throw Error("addr: the operands must be [n, m], [n], [m] and a view of [n, m]");
+    }
+    if (on_cpu(out)) {
+        hcb_tensor o = cpu_desc(out), a = cpu_desc(v1), b = cpu_desc(v2), c = cpu_desc(input);
+        cpu_check(cpu_backend("addr").addr(&o, &a, &b, &c, cpu_scalar(alpha), cpu_scalar(beta)));
+        return;
+    }
+    if (lo.num_elements() == 0) return;
+    const bool reads = beta.to_f64() != 0.0;
+    std::vector<MergedDim> dims = {MergedDim{lo.shape[0], {lo.strides[0], l1.strides[0], 0, lc.strides[0]}},
+                                   MergedDim{lo.shape[1], {lo.strides[1], 0, l2.strides[0], lc.strides[1]}}};
+    hmr_tensor_desc d_out = desc_with_dims("addr", out, lo.offset, dims, 0), d1 = desc_with_dims("addr", v1, l1.offset, dims, 1),
+                    d2 = desc_with_dims("addr", v2, l2.offset, dims, 2), d_in = desc_with_dims("addr", input, lc.offset, dims, 3);
+    const bool floating = is_floating_point(out.dtype);
+    exec(out, [&](hmr_context_t ctx) {
+        expect(hmr_addr(ctx, &d_out, &d1, &d2, reads ? &d_in : nullptr, floating ? alpha.to_f64() : 0.0,
+                        floating ? beta.to_f64() : 0.0, floating ? 0 : alpha.to_i64(), floating ? 0 : beta.to_i64()));
+    });
+}
+
 void upload(const TensorData &dst, const TensorData &src) {
     if (!src.layout.is_contiguous() || !dst.layout.is_contiguous() || !on_cpu(src) || on_cpu(dst)) {
         throw Error("internal error: upload needs a contiguous CPU source and a contiguous ROCm destination");

@@ -79,6 +79,10 @@ typedef struct hcb_backend {
     /* ref: src/backend/cpu/misc.rs:347-411; flip's mask has src->ndim entries (1 = reversed) */
     int (*triangle)(const hcb_tensor *out, const hcb_tensor *src, int64_t diagonal, int32_t upper);
     int (*flip)(const hcb_tensor *out, const hcb_tensor *src, const uint8_t *mask);
+    /* ref: src/backend/cpu/linalg.rs:224-388; out is [n, m], v1 [n], v2 [m], input a view of [n, m]
+     * that is read only when beta isn't zero; alpha and beta are values of the dtype */
+    int (*addr)(const hcb_tensor *out, const hcb_tensor *v1, const hcb_tensor *v2,
+                const hcb_tensor *input, hcb_scalar alpha, hcb_scalar beta);
 } hcb_backend;
 
 #ifdef __cplusplus

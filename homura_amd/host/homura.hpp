@@ -302,6 +302,8 @@ class Tensor {
     Tensor addcmul(const Tensor &tensor1, const Tensor &tensor2, Scalar value) const;
     Tensor addcdiv(const Tensor &tensor1, const Tensor &tensor2, Scalar value) const;
     Tensor lerp(const Tensor &end, const Operand &weight) const;
+    // beta * self + alpha * outer(vec1, vec2), one kernel (ref: src/ops/composite.rs:346-384).
+    Tensor addr(const Tensor &vec1, const Tensor &vec2, Scalar beta, Scalar alpha) const;
 
   private:
     TensorData d_;
@@ -377,6 +379,10 @@ void softmax(const TensorData &out, const TensorData &src, size_t dim, bool log)
 void fused(const Fused &op, const TensorData &out, const TensorData &a, const TensorData &b, const TensorData *c);
 void triangle(const TensorData &out, const TensorData &src, int64_t diagonal, bool upper);
 void flip(const TensorData &out, const TensorData &src, const std::vector<bool> &mask);
+// out [n, m] = beta * input + alpha * outer(v1 [n], v2 [m]); input is a view of [n, m], alpha and beta
+// values of the dtype (ref: src/backend/mod.rs:562-587).
+void addr(const TensorData &out, const TensorData &v1, const TensorData &v2, const TensorData &input, Scalar alpha,
+          Scalar beta);
 // Host <-> device and device <-> host transfers of contiguous data of one dtype.
 void upload(const TensorData &dst, const TensorData &src);
 void download(const TensorData &dst, const TensorData &src);

@@ -515,6 +515,51 @@ Tensor Tensor::lerp(const Tensor &end, const Operand &weight) const {
     return where_(w.abs().less(Scalar::of_float(0.5)), low, high);
 }
 
+// ---- addr (ref: src/ops/composite.rs:29-114, 210-249, 346-384) --------------------------------------------
+
+namespace {
+// ref: src/ops/composite.rs:38-65, rule Strict.
+Scalar addr_coefficient(Scalar s, DType dtype, const char *name) {
+    if (s.kind == Scalar::K::Bool && dtype != DType::Bool) {
+        throw Error(std::string("Boolean ") + name + " only supported for Boolean results");
+    }
+    if (s.kind == Scalar::K::Float && !is_floating_point(dtype)) {
+        throw Error(std::string("For integral input tensors, argument ") + name + " must not be a floating point number");
+    }
+    auto fits = s.checked_to(dtype);
+    if (!fits) throw Error(std::string(name) + "=" + s.str() + " cannot be converted to " + name_of(dtype) + " without overflow");
+    return *fits;
+}
+
+void check_dims(const Tensor &t, size_t n, const char *what) {
+    if (t.num_dims() != n) {
+        throw Error(std::string(what) + " must be a " + std::to_string(n) + "-D tensor, got " + std::to_string(t.num_dims()) +
+                    "-D tensor");
+    }
+}
+}  // namespace
+
+Tensor Tensor::addr(const Tensor &vec1, const Tensor &vec2, Scalar beta, Scalar alpha) const {
+    check_dims(vec1, 1, "vec1");
+    check_dims(vec2, 1, "vec2");
+    common_device({&d_, &vec1.data(), &vec2.data()});
+    // `self` takes full part in the promotion even when it is zero-dimensional.
+    const DType dtype = promote_types(promote_types(d_.dtype, vec1.dtype()), vec2.dtype());
+    const Tensor input = to(dtype), v1 = vec1.to(dtype), v2 = vec2.to(dtype);
+    const Shape shape{v1.shape()[0], v2.shape()[0]};
+    const TensorData c = input.data().expand_to(shape);  // fails for an input that doesn't broadcast
+    beta = addr_coefficient(beta, dtype, "beta");
+    alpha = addr_coefficient(alpha, dtype, "alpha");
+    if (is_floating_point(dtype)) {
+        // Rounded to the dtype whatever kind of scalar they are (ref: src/ops/composite.rs:99-114).
+        beta = Scalar::of_float(round_through(beta.to_f64(), dtype));
+        alpha = Scalar::of_float(round_through(alpha.to_f64(), dtype));
+    }
+    TensorData out = uninit_data(shape, dtype, v1.device());
+    backend::addr(out, v1.data(), v2.data(), c, alpha, beta);
+    return Tensor(out);
+}
+
 // ---- the optimizers' steps (ref: src/optim/mod.rs:569-616) -----------------------------------------------
 
 namespace optim {

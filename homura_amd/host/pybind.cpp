@@ -242,5 +242,8 @@ PYBIND11_MODULE(_host, m) {
     T.def("addcdiv", [](const Tensor &t, const Tensor &t1, const Tensor &t2, const py::handle &value) {
         return t.addcdiv(t1, t2, std::get<Scalar>(to_operand(value)));
     });
+    T.def("addr", [](const Tensor &t, const Tensor &v1, const Tensor &v2, const py::handle &beta, const py::handle &alpha) {
+        return t.addr(v1, v2, std::get<Scalar>(to_operand(beta)), std::get<Scalar>(to_operand(alpha)));
+    }, py::arg("vec1"), py::arg("vec2"), py::arg("beta") = 1, py::arg("alpha") = 1);
     T.def("lerp", [](const Tensor &t, const Tensor &end, const py::handle &weight) { return t.lerp(end, to_operand(weight)); });
 }

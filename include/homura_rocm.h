@@ -17,7 +17,7 @@
  *  - enumerations travel as int32_t.
  *
  * Entry points of the reference that belong to other kernel families (gemm, indexing, pooling,
- * random, fused optimiser steps ...) are declared in homura_rocm_unbuilt.h and exported as
+ * random, scans ...) are declared in homura_rocm_unbuilt.h and exported as
  * stubs that fail with HMR_INVALID, so that the reference crate still links.
  */
 #ifndef HOMURA_ROCM_H
@@ -199,7 +199,7 @@ hmr_status hmr_where_constant(hmr_context_t ctx, const hmr_tensor_desc *out,
                               const hmr_tensor_desc *cond, const hmr_tensor_desc *x,
                               uint64_t x_bits, const hmr_tensor_desc *y, uint64_t y_bits);
 
-/* ---- fused optimiser steps, triangle, flip ------------------- ref: csrc/homura_rocm.h:195-263 */
+/* ---- fused optimiser steps, addr, triangle, flip ------------- ref: csrc/homura_rocm.h:195-263 */
 #define HMR_FUSED_SCALED_ADD 0
 #define HMR_FUSED_LERP 1
 #define HMR_FUSED_ADDCMUL 2
@@ -214,6 +214,19 @@ hmr_status hmr_where_constant(hmr_context_t ctx, const hmr_tensor_desc *out,
 hmr_status hmr_fused(hmr_context_t ctx, int32_t op, const hmr_tensor_desc *out,
                      const hmr_tensor_desc *a, const hmr_tensor_desc *b,
                      const hmr_tensor_desc *c, double coefficient, int32_t small);
+
+/* ref :232-244  cpu::addr (src/backend/cpu/linalg.rs:224-388): out[i][j] = beta * input[i][j] +
+ * alpha * v1[i] * v2[j] for every dtype. All four descriptions have the output's two dimensions
+ * [n, m]: v1 with stride 0 along the columns, v2 along the rows, the input broadcast as needed;
+ * `input` may be NULL when beta is zero (it isn't read then).
+ *   floats (coefficients already rounded to the dtype, in `alpha` and `beta`): a = alpha * v1[i]
+ *     (skipped for alpha == 1), p = a * v2[j], out = p or (beta == 1 ? c : beta * c) + p, each step
+ *     in the computation type and rounded to the dtype;
+ *   integers (`alpha_int`, `beta_int`): wrapping, alpha * (v1[i] * v2[j]) + beta * c;
+ *   Bool (`alpha_int`, `beta_int` 0 or 1): (v1[i] and alpha and v2[j]) or (beta and c). */
+hmr_status hmr_addr(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_tensor_desc *v1,
+                    const hmr_tensor_desc *v2, const hmr_tensor_desc *input, double alpha,
+                    double beta, int64_t alpha_int, int64_t beta_int);
 
 /* ref :257-260  cpu::triangle (src/backend/cpu/misc.rs:347-381): out = src where the column minus
  * the row index (the last two dimensions, ndim >= 2) is at least (upper) or at most `diagonal`,

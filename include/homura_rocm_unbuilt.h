@@ -18,11 +18,6 @@
 extern "C" {
 #endif
 
-/* ref :242 */
-hmr_status hmr_addr(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_tensor_desc *v1,
-                    const hmr_tensor_desc *v2, const hmr_tensor_desc *input, double alpha,
-                    double beta, int64_t alpha_int, int64_t beta_int);
-
 /* ref :276-295 */
 #define HMR_RANDOM_INT_TILE 256
 hmr_status hmr_random_uniform(hmr_context_t ctx, const hmr_tensor_desc *out, uint64_t seed,

@@ -708,6 +708,78 @@ void flip(const hcb_tensor &out, const hcb_tensor &src, const uint8_t *mask) {
     });
 }
 
+// ---- addr (ref: src/backend/cpu/linalg.rs:224-388) ----------------------------------------------
+//
+// out[i][j] = beta * input[i][j] + alpha * v1[i] * v2[j] for out [n, m], v1 [n], v2 [m] and an input
+// viewed as [n, m] (read only when beta isn't zero), every step rounded to the dtype:
+//   floats  a = alpha * v1[i] (skipped for alpha == 1), p = a * v2[j], c = beta * input (skipped for
+//           beta == 1), out = c + p; alpha and beta in the computation type;
+//   ints    wrapping i64: p = v1[i] * v2[j], times alpha unless 1, plus input (times beta unless 1);
+//   bools   (input if beta) or (v1[i] and alpha and v2[j]).
+template <class T, class Row, class Write>
+void outer(const hcb_tensor &out, const hcb_tensor &v1, const hcb_tensor &v2, const hcb_tensor *input, Row row,
+           Write write) {
+    const int64_t n = v1.shape[0], m = v2.shape[0];
+    if (out.ndim != 2 || out.shape[0] != n || out.shape[1] != m) panic("addr: the output isn't [n, m]");
+    if (n == 0 || m == 0) return;
+    if (input && (input->ndim != 2 || input->shape[0] != n || input->shape[1] != m)) panic("addr: the input isn't [n, m]");
+    T *po = base<T>(out);
+    const T *p1 = base<T>(v1), *p2 = base<T>(v2), *pc = input ? base<T>(*input) : nullptr;
+    for (int64_t i = 0; i < n; ++i) {
+        const T a = row(p1[v1.offset + i * v1.strides[0]]);
+        for (int64_t j = 0; j < m; ++j) {
+            const T y = p2[v2.offset + j * v2.strides[0]];
+            const T *c = pc ? &pc[input->offset + i * input->strides[0] + j * input->strides[1]] : nullptr;
+            po[out.offset + i * out.strides[0] + j * out.strides[1]] = write(a, y, c);
+        }
+    }
+}
+
+void addr(const hcb_tensor &out, const hcb_tensor &v1, const hcb_tensor &v2, const hcb_tensor &input, hcb_scalar alpha_s,
+          hcb_scalar beta_s) {
+    const int dtype = v1.dtype;
+    auto f64_of = [](hcb_scalar s) { return s.kind == HCB_SCALAR_FLOAT ? s.f : static_cast<double>(s.i); };
+    auto i64_of = [](hcb_scalar s) { return s.kind == HCB_SCALAR_FLOAT ? El<int64_t>::from_f64(s.f) : s.i; };
+    auto bool_of = [](hcb_scalar s) { return s.kind == HCB_SCALAR_FLOAT ? s.f != 0.0 : s.i != 0; };
+    if (is_float(dtype)) {
+        dispatch_float(dtype, [&](auto t) {
+            using T = typename decltype(t)::type;
+            using C = typename Fl<T>::C;
+            const C alpha = of<C>(f64_of(alpha_s)), beta = of<C>(f64_of(beta_s));
+            outer<T>(
+                out, v1, v2, beta != C(0) ? &input : nullptr,
+                [=](T x) { return alpha == C(1) ? x : Fl<T>::down(Fl<T>::up(x) * alpha); },
+                [=](T a, T y, const T *c) {
+                    const T p = Fl<T>::down(Fl<T>::up(a) * Fl<T>::up(y));
+                    if (!c) return p;
+                    const T scaled = beta == C(1) ? *c : Fl<T>::down(Fl<T>::up(*c) * beta);
+                    return Fl<T>::down(Fl<T>::up(scaled) + Fl<T>::up(p));
+                });
+        });
+    } else if (is_integral(dtype)) {
+        dispatch_int(dtype, [&](auto t) {
+            using T = typename decltype(t)::type;
+            const int64_t alpha = i64_of(alpha_s), beta = i64_of(beta_s);
+            outer<T>(
+                out, v1, v2, beta != 0 ? &input : nullptr, [](T x) { return x; },
+                [=](T a, T y, const T *c) {
+                    int64_t p = wmul<int64_t>(El<T>::to_i64(a), El<T>::to_i64(y));
+                    if (alpha != 1) p = wmul<int64_t>(p, alpha);
+                    if (!c) return El<T>::from_i64(p);
+                    const int64_t ci = El<T>::to_i64(*c);
+                    return El<T>::from_i64(wadd<int64_t>(beta == 1 ? ci : wmul<int64_t>(ci, beta), p));
+                });
+        });
+    } else {
+        const bool alpha = bool_of(alpha_s), beta = bool_of(beta_s);
+        outer<boolean>(
+            out, v1, v2, beta ? &input : nullptr, [=](boolean x) { return boolean{static_cast<uint8_t>(x.v && alpha)}; },
+            [](boolean a, boolean y, const boolean *c) {
+                return boolean{static_cast<uint8_t>((c && c->v) || (a.v && y.v))};
+            });
+    }
+}
+
 // ---- reductions (ref: src/backend/cpu/reduce.rs:10-225) ----------------------------------------
 
 struct Split {
@@ -1037,6 +1109,10 @@ int orc_triangle(const hcb_tensor *out, const hcb_tensor *src, int64_t diagonal,
 int orc_flip(const hcb_tensor *out, const hcb_tensor *src, const uint8_t *mask) {
     return orc::guarded([&] { orc::flip(*out, *src, mask); });
 }
+int orc_addr(const hcb_tensor *out, const hcb_tensor *v1, const hcb_tensor *v2, const hcb_tensor *input, hcb_scalar alpha,
+             hcb_scalar beta) {
+    return orc::guarded([&] { orc::addr(*out, *v1, *v2, *input, alpha, beta); });
+}
 
 // erf in f64, for the known-answer table of ref: src/backend/cpu/num.rs:225-248.
 double orc_erf(double x) { return orc::erf64(x); }
@@ -1052,7 +1128,7 @@ const hcb_backend *orc_backend(void) {
         "homura CPU oracle", orc_last_error, orc_copy,  orc_fill,           orc_unary,
         orc_binary,          orc_binary_constant,       orc_binary_scalar,  orc_where,
         orc_where_constant,  orc_reduce,     orc_var,   orc_arg_reduce,     orc_softmax,
-        orc_fused,           orc_triangle,   orc_flip,
+        orc_fused,           orc_triangle,   orc_flip,  orc_addr,
     };
     return &table;
 }

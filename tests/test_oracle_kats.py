@@ -446,3 +446,96 @@ def test_scaled_add_rounds_alpha_to_the_dtype_first():
     # 516 in BF16 (spacing 4); as a BF16 alpha: 512 + 1.5 = 513.5, which is 512.
     assert list(vals(h.addcmul_step(bf(1.5), bf(512.0), bf(1.0), 1.0 + 2.0 ** -9))) == [516.0]
     assert list(vals(h.scaled_add(bf(1.5), bf(512.0), 1.0 + 2.0 ** -9))) == [512.0]
+
+
+# ---- addr: one kernel with the bits of the composition of pinned elementwise ops ------------------------------
+
+def addr_values(dtype, n, seed):
+    """Special values first, then random ones (ref: tests/gemm_writeback.rs:266-299)."""
+    rng = np.random.default_rng(seed)
+    if dtype == DT.Bool:
+        return tensor((rng.standard_normal(n) > 0).astype(np.uint8), DT.Bool)
+    if dtype not in FLOATS:
+        special = np.array([0, 1, -1, 2 ** 63 - 1, -2 ** 63, 255, -128], dtype=np.int64)
+        v = np.concatenate([special, (rng.standard_normal(n) * 1e6).astype(np.int64)])[:n]
+        return tensor(v, DT.I64).to(dtype)
+    special = np.array([NAN, -NAN, INF, -INF, 0.0, -0.0, 1e-40, -5.96e-8, 65504.0, 3.0e38, -1.0e300])
+    v = np.concatenate([special, rng.standard_normal(n) * 8.0])[:n]
+    return tensor(v, DT.F64).to(dtype)
+
+
+def addr_composite(inp, v1, v2, beta, alpha, dtype):
+    """ref: tests/gemm_writeback.rs:250-264: alpha scales vec1 (floats) or the outer product (integers, bools),
+    then beta * input is added unless beta is zero; a coefficient of one is skipped."""
+    scale = lambda t, s: t if float(s) == 1.0 else t.mul(s)
+    outer = lambda a, b: a.unsqueeze(1).mul(b.unsqueeze(0))
+    product = outer(scale(v1, alpha), v2) if dtype in FLOATS else scale(outer(v1, v2), alpha)
+    if float(beta) == 0.0:
+        return product
+    return scale(inp, beta).add(product)
+
+
+def addr_cases(dtype, device="cpu", n=13, m=12):
+    """(what, input, v1, v2, beta, alpha) over coefficients of the dtype and input layouts
+    (ref: tests/gemm_writeback.rs:301-375)."""
+    if dtype == DT.Bool:
+        coefficients = [False, True]
+    elif dtype in FLOATS:
+        raw = [0.0, 1.0, -1.0, 0.5, 2.0, -1.5, 0.1, 1e-30, INF, NAN]
+        coefficients = [float(v) for v in vals(tensor(np.array(raw), DT.F64).to(dtype))]  # rounded to the dtype first
+    else:
+        coefficients = [0, 1, -1, 2, 3, 127]
+    v1 = addr_values(dtype, 2 * n, 1).to(device).reshape([n, 2]).select(1, 1)  # every other element
+    v2 = addr_values(dtype, m, 2).to(device)
+    full = addr_values(dtype, n * m, 3).to(device)
+    inputs = [full.reshape([n, m]), full.reshape([m, n]).transpose(0, 1), full.narrow(0, 0, m),
+              full.narrow(0, 0, n).reshape([n, 1]), full.narrow(0, 0, 1), full.narrow(0, 0, 1).reshape([])]
+    for k, inp in enumerate(inputs):
+        for alpha in coefficients:
+            for beta in coefficients:
+                yield f"{dtype} input {k} alpha {alpha} beta {beta}", inp, v1, v2, beta, alpha
+
+
+@pytest.mark.parametrize("dtype", [DT.F16, DT.BF16, DT.F32, DT.F64, DT.U8, DT.I8, DT.I16, DT.I32, DT.I64, DT.Bool])
+def test_addr_gives_the_composites_bits(dtype):
+    checked = 0
+    for what, inp, v1, v2, beta, alpha in addr_cases(dtype):
+        got, want = inp.addr(v1, v2, beta, alpha), addr_composite(inp, v1, v2, beta, alpha, dtype)
+        assert got.shape == [13, 12] and got.dtype == dtype, what
+        g, w = bits(got), bits(want)
+        if dtype in FLOATS:
+            nan = {DT.F16: lambda b: (b & 0x7FFF) > 0x7C00, DT.BF16: lambda b: (b & 0x7FFF) > 0x7F80,
+                   DT.F32: lambda b: (b & 0x7FFFFFFF) > 0x7F800000,
+                   DT.F64: lambda b: (b & np.uint64(0x7FFFFFFFFFFFFFFF)) > np.uint64(0x7FF0000000000000)}[dtype]
+            same = (g == w) | (nan(g) & nan(w))
+        else:
+            same = g == w
+        assert same.all(), f"{what}: element {np.nonzero(~same)[0][0]}"
+        checked += 1
+    assert checked >= (4 * 6 if dtype == DT.Bool else 100)
+
+
+def test_addr_known_answers_and_coefficient_rules():
+    """ref: tests/m0_followup.rs:150-222, tests/m0_m1_readiness.rs:66."""
+    m = h.full([1, 1], 1, DT.I32, "cpu")
+    v = h.full([1], 1, DT.I32, "cpu")
+    assert array(m.addr(v, v, 2, 3)).tolist() == [[5]]
+    b = tensor(np.array([1], dtype=np.uint8), DT.Bool)
+    assert array(b.unsqueeze(0).addr(b, b, True, 2)).tolist() == [[1]]
+    with pytest.raises(Exception, match="Boolean alpha only supported for Boolean results"):
+        m.addr(v, v, 1, True)
+    for beta, alpha in ((1.0, 1), (1, 2.0), (0.5, 0.5)):
+        with pytest.raises(Exception, match="must not be a floating point number"):
+            m.addr(v, v, beta, alpha)
+    hh = h.full([1, 1], 1.0, DT.F16, "cpu")
+    with pytest.raises(Exception, match="alpha=100000 cannot be converted to f16 without overflow"):
+        hh.addr(hh.flatten(0, -1), hh.flatten(0, -1), 1, 1e5)
+    with pytest.raises(Exception, match="vec1 must be a 1-D tensor, got 2-D tensor"):
+        hh.addr(hh, hh.flatten(0, -1), 1, 1)
+    # All three inputs take part in the promotion, a zero-dimensional self included.
+    out = h.full([], 1.5, DT.F64, "cpu").addr(h.full([2], 2, DT.I32, "cpu"), h.full([3], 3.0, DT.F16, "cpu"), 1, 1)
+    assert out.dtype == DT.F64 and array(out).tolist() == [[7.5] * 3] * 2
+    # A zero or tiny alpha never meets the other factor's infinity: alpha scales vec1 first.
+    big, two = tensor(np.array([3.0e38], dtype=np.float32), DT.F32), tensor(np.array([2.0], dtype=np.float32), DT.F32)
+    got = array(h.full([1, 1], 0.0, DT.F32, "cpu").addr(big, two, 1, 1e-30))
+    assert got.tolist() == [[np.float32(1e-30) * np.float32(3.0e38) * np.float32(2.0)]] and np.isfinite(got).all()

@@ -1,6 +1,7 @@
-"""hmr_fused, hmr_triangle and hmr_flip on the GPU against the CPU oracle, through the host layer and through
-the C ABI directly. All three are bit-exact: a fused step is IEEE arithmetic with the FMAs where the CPU has them
-(ref: src/backend/cpu/mod.rs:509-569), the other two move bits. Modelled on ref: src/backend/rocm/tests.rs:886-935
+"""hmr_fused, hmr_addr, hmr_triangle and hmr_flip on the GPU against the CPU oracle, through the host layer and
+through the C ABI directly. All four are bit-exact: a fused step is IEEE arithmetic with the FMAs where the CPU has
+them (ref: src/backend/cpu/mod.rs:509-569), addr rounds every step to the dtype (ref: src/backend/cpu/linalg.rs:
+224-388, tests/gemm_writeback.rs:301-375), the other two move bits. Modelled on ref: src/backend/rocm/tests.rs:886-935
 (fused_steps_match_the_cpu) and tests/rocm_elementwise.rs:674-718 (triangles_are_bitwise, flips_are_bitwise)."""
 from ctypes import byref
 
@@ -69,6 +70,27 @@ def test_fused_steps_on_every_layout_and_on_large_tensors():
         for p in large_layouts(dtype, 61):
             for name, f in STEPS.items():
                 assert_bitwise(f(p.gpu, p.gpu, p.gpu, 0.6), f(p.cpu, p.cpu, p.cpu, 0.6), f"{dtype} {name} {p.name}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_addr_matches_the_cpu(dtype):
+    from tests.test_oracle_kats import addr_cases
+    checked = 0
+    for (what, inp, v1, v2, beta, alpha), (_, ginp, g1, g2, _, _) in zip(addr_cases(dtype), addr_cases(dtype, GPU)):
+        assert_bitwise(ginp.addr(g1, g2, beta, alpha), inp.addr(v1, v2, beta, alpha), what)
+        checked += 1
+    assert checked >= 24
+
+
+def test_addr_of_sizes_that_vectorise_and_of_sizes_that_do_not():
+    for dtype, beta, alpha in ((DT.BF16, 0.5, -1.5), (DT.F32, 1, 0.1), (DT.F64, 0, 2.0), (DT.I16, 3, -1), (DT.U8, 1, 2),
+                               (DT.Bool, True, True)):
+        for n, m in ((1031, 257), (64, 4096), (1, 1), (3, 0), (2048, 2048)):
+            v1 = tensor(values(dtype, n, 71), dtype)
+            v2 = tensor(values(dtype, m, 72), dtype)
+            for inp in (tensor(values(dtype, n * m, 73), dtype).reshape([n, m]), tensor(values(dtype, m, 74), dtype)):
+                got = inp.to(GPU).addr(v1.to(GPU), v2.to(GPU), beta, alpha)
+                assert_bitwise(got, inp.addr(v1, v2, beta, alpha), f"{dtype} [{n}, {m}] input {inp.shape}")
 
 
 def test_triangles_are_bitwise():
@@ -188,6 +210,44 @@ def test_fused_through_the_c_abi_in_place_and_its_errors(ctx):
     # No elements: nothing to do, whatever the pointers are.
     E = desc(None, capi.F32, [0, 4])
     capi.check(L.hmr_fused(ctx.handle, 3, byref(E), byref(E), byref(E), byref(E), 1.0, 0))
+
+
+def test_addr_through_the_c_abi_and_its_errors(ctx):
+    n, m = 300, 200
+    rng = np.random.default_rng(9)
+    v1, v2 = rng.standard_normal(n).astype(np.float32), rng.standard_normal(m).astype(np.float32)
+    c = rng.standard_normal((n, m)).astype(np.float32)
+    d1, d2, dc = ctx.upload(v1), ctx.upload(v2), ctx.upload(c)
+    O = desc(dc, capi.F32, [n, m])
+    V1, V2 = desc(d1, capi.F32, [n, m], [1, 0]), desc(d2, capi.F32, [n, m], [0, 1])
+    alpha, beta = np.float32(0.75), np.float32(-2.0)
+    # In place over the input: every step rounded to f32.
+    capi.check(L.hmr_addr(ctx.handle, byref(O), byref(V1), byref(V2), byref(O), float(alpha), float(beta), 0, 0))
+    ctx.synchronize()
+    want = (c * beta) + (v1 * alpha)[:, None] * v2[None, :]
+    np.testing.assert_array_equal(dc.download(np.float32, n * m).reshape(n, m), want)
+    # beta == 0: the input isn't read and may be missing.
+    capi.check(L.hmr_addr(ctx.handle, byref(O), byref(V1), byref(V2), None, 1.0, 0.0, 0, 0))
+    ctx.synchronize()
+    np.testing.assert_array_equal(dc.download(np.float32, n * m).reshape(n, m), v1[:, None] * v2[None, :])
+    assert L.hmr_addr(ctx.handle, byref(O), byref(V1), byref(V2), None, 1.0, 1.0, 0, 0) == capi.HMR_INVALID
+    assert last_error() == "addr: beta isn't zero but there is no input"
+    flat = desc(dc, capi.F32, [n * m])
+    assert L.hmr_addr(ctx.handle, byref(flat), byref(flat), byref(flat), None, 1.0, 0.0, 0, 0) == capi.HMR_INVALID
+    assert last_error() == "addr: the output must have two dimensions"
+    H = desc(d1, capi.F16, [n, m], [1, 0])
+    assert L.hmr_addr(ctx.handle, byref(O), byref(H), byref(V2), None, 1.0, 0.0, 0, 0) == capi.HMR_INVALID
+    assert last_error() == "addr: unsupported dtype"
+    # Integers wrap in the element's width.
+    a8, b8 = np.arange(-100, 100, dtype=np.int8), np.arange(-60, 68, dtype=np.int8)
+    c8 = np.full((200, 128), 7, dtype=np.int8)
+    da, db, dcc = ctx.upload(a8), ctx.upload(b8), ctx.upload(c8)
+    O8 = desc(dcc, capi.I8, [200, 128])
+    capi.check(L.hmr_addr(ctx.handle, byref(O8), byref(desc(da, capi.I8, [200, 128], [1, 0])),
+                          byref(desc(db, capi.I8, [200, 128], [0, 1])), byref(O8), 0.0, 0.0, -3, 5))
+    ctx.synchronize()
+    want8 = (c8.astype(np.int64) * 5 + a8.astype(np.int64)[:, None] * b8.astype(np.int64)[None, :] * -3).astype(np.int8)
+    np.testing.assert_array_equal(dcc.download(np.int8, 200 * 128).reshape(200, 128), want8)
 
 
 def test_triangle_and_flip_through_the_c_abi_and_their_errors(ctx):
