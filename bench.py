@@ -288,6 +288,12 @@ def per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP
     add(None, "addr f32 [8192,8192] (beta 0.5, alpha -1.5: one kernel)", 8 * N + 8 * 8192, lambda: mat.addr(v1, v2, 0.5, -1.5))
     add(None, "addr f32 [8192,8192] without input (beta 0)", 4 * N + 8 * 8192, lambda: mat.addr(v1, v2, 0, -1.5))
     del mat, v1, v2
+    xf = residual.reshape([16384, 4096])
+    add(None, "exclusive_cumprod f32 [16384,4096] dim=0 (a thread per column, sequential)", 8 * N,
+        lambda: h.exclusive_cumprod(xf, 0, False), 5)
+    add(None, "exclusive_cumprod f32 [16384,4096] dim=1 (a thread per row, sequential)", 8 * N,
+        lambda: h.exclusive_cumprod(xf, 1, True), 5)
+    del xf
     sq = residual.reshape([16, 2048, 2048])
     add(None, "triu(1) f32 [16,2048,2048] (reads the kept half)", 6 * N, lambda: sq.triu(1))
     add(None, "tril(0) f32 [16,2048,2048] (reads the kept half)", 6 * N, lambda: sq.tril(0))

@@ -512,6 +512,22 @@ void softmax(const TensorData &out, const TensorData &src, size_t dim, bool log)
     });
 }
 
+// ref: src/backend/rocm/reduce.rs:304-319
+void exclusive_cumprod(const TensorData &out, const TensorData &src, size_t dim, bool reverse) {
+    if (!out.layout.is_contiguous() || out.dtype != src.dtype) throw Error("exclusive_cumprod writes a contiguous tensor of the source's dtype");
+    if (on_cpu(out)) {
+        check_shape(out, src);
+        hcb_tensor o = cpu_desc(out), s = cpu_desc(src);
+        cpu_check(cpu_backend("exclusive_cumprod").exclusive_cumprod(&o, &s, static_cast<int32_t>(dim), reverse));
+        return;
+    }
+    if (!is_floating_point(src.dtype)) throw Error(std::string("expected a floating point dtype, got ") + name_of(src.dtype));
+    hmr_tensor_desc o, s;
+    int64_t n, so, si;
+    if (!lines("exclusive_cumprod", out, src, dim, o, s, n, so, si)) return;
+    exec(out, [&](hmr_context_t ctx) { expect(hmr_exclusive_cumprod(ctx, &o, &s, n, so, si, reverse ? 1 : 0)); });
+}
+
 // ref: src/backend/rocm/elementwise.rs:155-215: the coefficient travels in the computation type.
 void fused(const Fused &op, const TensorData &out, const TensorData &a, const TensorData &b, const TensorData *c) {
     check_shape(out, a);

@@ -83,6 +83,9 @@ typedef struct hcb_backend {
      * that is read only when beta isn't zero; alpha and beta are values of the dtype */
     int (*addr)(const hcb_tensor *out, const hcb_tensor *v1, const hcb_tensor *v2,
                 const hcb_tensor *input, hcb_scalar alpha, hcb_scalar beta);
+    /* ref: src/backend/cpu/reduce.rs:281-324; floating point operands of one shape and dtype */
+    int (*exclusive_cumprod)(const hcb_tensor *out, const hcb_tensor *src, int32_t dim,
+                             int32_t reverse);
 } hcb_backend;
 
 #ifdef __cplusplus

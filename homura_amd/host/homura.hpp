@@ -318,6 +318,10 @@ struct ValuesAndIndices {
 Tensor binary_op(BinaryOp op, const Operand &lhs, const Operand &rhs);
 // torch.where (ref: src/ops/binary.rs:152-176).
 Tensor where_(const Tensor &condition, const Operand &x, const Operand &y);
+// For each element of the floating point `x`, the product of the elements before it along `dim` (after it
+// when `reverse`), multiplied in order: what the gradient of `prod` uses for inputs with zeros
+// (ref: src/ops/reduce.rs:158-170).
+Tensor exclusive_cumprod(const Tensor &x, size_t dim, bool reverse);
 // The optimizers' single-rounding steps (ref: src/optim/mod.rs:569-616): new tensors from tensors of one
 // shape, floating point dtype and device. A finite scalar beyond the range of the type it is converted
 // to (the dtype for alpha, the computation type otherwise) is an error.
@@ -376,6 +380,7 @@ void var(const TensorData &out, const TensorData &src, const std::vector<bool> &
 void arg_reduce(const TensorData *values, const TensorData &indices, const TensorData &src, size_t dim,
                 bool is_max);
 void softmax(const TensorData &out, const TensorData &src, size_t dim, bool log);
+void exclusive_cumprod(const TensorData &out, const TensorData &src, size_t dim, bool reverse);
 void fused(const Fused &op, const TensorData &out, const TensorData &a, const TensorData &b, const TensorData *c);
 void triangle(const TensorData &out, const TensorData &src, int64_t diagonal, bool upper);
 void flip(const TensorData &out, const TensorData &src, const std::vector<bool> &mask);

@@ -474,6 +474,16 @@ Tensor Tensor::any_dim(const std::vector<int64_t> &dims, bool keepdim) const {
 Tensor Tensor::softmax(int64_t dim) const { return softmax_op(*this, dim, false); }
 Tensor Tensor::log_softmax(int64_t dim) const { return softmax_op(*this, dim, true); }
 
+// ref: src/ops/reduce.rs:158-170
+Tensor exclusive_cumprod(const Tensor &x, size_t dim, bool reverse) {
+    const TensorData &src = x.data();
+    if (!is_floating_point(src.dtype)) throw Error(std::string("expected a floating point dtype, got ") + name_of(src.dtype));
+    if (dim >= src.layout.shape.size()) throw Error("exclusive_cumprod: dimension out of range");
+    TensorData out = uninit_data(src.layout.shape, src.dtype, src.device());
+    backend::exclusive_cumprod(out, src, dim, reverse);
+    return Tensor(out);
+}
+
 // ---- triangles and flips (ref: src/ops/shape_ops.rs:181-263) ---------------------------------------------
 
 Tensor Tensor::triu(int64_t diagonal) const { return triangle_op(*this, diagonal, true); }

@@ -114,6 +114,7 @@ PYBIND11_MODULE(_host, m) {
           py::arg("p"), py::arg("grad"), py::arg("state"), py::arg("lr"), py::arg("beta1") = 0.9, py::arg("beta2") = 0.999,
           py::arg("eps") = 1e-8, py::arg("weight_decay") = 0.0, py::arg("amsgrad") = false, py::arg("maximize") = false,
           py::arg("decoupled_weight_decay") = false);
+    m.def("exclusive_cumprod", &exclusive_cumprod, py::arg("x"), py::arg("dim"), py::arg("reverse") = false);
     m.def("reduce_plan", [](const Tensor &t, const std::vector<int64_t> &dims) {
         auto p = rocm_reduce_plan(t, dims);
         return py::make_tuple(p.group, p.splits, p.chunk);

@@ -288,6 +288,14 @@ hmr_status hmr_softmax(hmr_context_t ctx, const hmr_tensor_desc *out_rows,
                        int64_t src_stride, int32_t log, void *workspace,
                        int64_t workspace_bytes);
 
+/* ref :348-351  cpu::exclusive_cumprod (src/backend/cpu/reduce.rs:281-324) along lines of n
+ * elements, described as for hmr_softmax: out[k] = the product of the line's elements before k
+ * (after k when `reverse`), 1 for the first (last), accumulated in order in f32 (F16, BF16) or
+ * f64 (F32, F64) and rounded to the dtype as it is written. Floating point dtypes, one for both. */
+hmr_status hmr_exclusive_cumprod(hmr_context_t ctx, const hmr_tensor_desc *out_lines,
+                                 const hmr_tensor_desc *src_lines, int64_t n, int64_t out_stride,
+                                 int64_t src_stride, int32_t reverse);
+
 /* ---- build facts and ABI self-description ------------------- ref: csrc/homura_rocm.h:589-610 */
 /* ';'-separated offload architectures compiled in ("gfx950"). */
 const char *hmr_built_archs(void);

@@ -28,11 +28,6 @@ hmr_status hmr_random_int(hmr_context_t ctx, const hmr_tensor_desc *out, uint64_
                           uint64_t offset, uint64_t blocks, int64_t low, uint64_t range,
                           uint64_t threshold, void *workspace);
 
-/* ref :349 */
-hmr_status hmr_exclusive_cumprod(hmr_context_t ctx, const hmr_tensor_desc *out_lines,
-                                 const hmr_tensor_desc *src_lines, int64_t n, int64_t out_stride,
-                                 int64_t src_stride, int32_t reverse);
-
 /* ref :361-426 (indexing) */
 hmr_status hmr_index_check(hmr_context_t ctx, const hmr_tensor_desc *index, int64_t low,
                            int64_t high, int32_t has_exempt, int64_t exempt, uint64_t *slot);

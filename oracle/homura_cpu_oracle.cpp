@@ -1035,6 +1035,62 @@ void softmax(const hcb_tensor &out, const hcb_tensor &src, int dim, bool log) {
     });
 }
 
+// ---- exclusive cumulative product (ref: src/backend/cpu/reduce.rs:227-324) -----------------------
+//
+// For each element, the product of the elements before it along `dim` (after it when `reverse`):
+// accumulated one element at a time in the accumulation type of the dtype (f32 for F16 and BF16,
+// f64 for F32 and F64), each output rounded from the accumulator, which itself is never rounded.
+template <class T>
+struct Accumulate {
+    using A = float;
+    static A widen(T x) { return Fl<T>::up(x); }
+    static T narrow(A acc) { return Fl<T>::down(acc); }
+};
+template <>
+struct Accumulate<float> {
+    using A = double;
+    static A widen(float x) { return static_cast<double>(x); }
+    static float narrow(A acc) { return static_cast<float>(acc); }
+};
+template <>
+struct Accumulate<double> {
+    using A = double;
+    static A widen(double x) { return x; }
+    static double narrow(A acc) { return acc; }
+};
+
+void exclusive_cumprod(const hcb_tensor &out, const hcb_tensor &src, int dim, bool reverse) {
+    check_shape(out, src);
+    if (out.dtype != src.dtype) panic("exclusive_cumprod: the operands have different dtypes");
+    if (num_elements(src) == 0) return;
+    if (dim < 0 || dim >= src.ndim) panic("exclusive_cumprod: dimension out of range");
+    const int64_t n = src.shape[dim], si = src.strides[dim], so = out.strides[dim];
+    std::vector<int64_t> kshape, ks_strides, ko_strides;
+    for (int i = 0; i < src.ndim; ++i) {
+        if (i == dim) continue;
+        kshape.push_back(src.shape[i]);
+        ks_strides.push_back(src.strides[i]);
+        ko_strides.push_back(out.strides[i]);
+    }
+    dispatch_float(src.dtype, [&](auto t) {
+        using T = typename decltype(t)::type;
+        using Acc = Accumulate<T>;
+        const T *ps = base<T>(src);
+        T *po = base<T>(out);
+        const int64_t *const st[2] = {ko_strides.data(), ks_strides.data()};
+        Plan<2> lines(static_cast<int>(kshape.size()), kshape.data(), st);
+        const int64_t b[2] = {out.offset, src.offset};
+        lines.for_each(b, [&](const int64_t(&o)[2]) {
+            typename Acc::A acc = 1;
+            for (int64_t k = 0; k < n; ++k) {
+                const int64_t at = reverse ? n - 1 - k : k;
+                po[o[0] + at * so] = Acc::narrow(acc);
+                acc = acc * Acc::widen(ps[o[1] + at * si]);
+            }
+        });
+    });
+}
+
 template <class F>
 int guarded(F f) {
     try {
@@ -1109,6 +1165,9 @@ int orc_triangle(const hcb_tensor *out, const hcb_tensor *src, int64_t diagonal,
 int orc_flip(const hcb_tensor *out, const hcb_tensor *src, const uint8_t *mask) {
     return orc::guarded([&] { orc::flip(*out, *src, mask); });
 }
+int orc_exclusive_cumprod(const hcb_tensor *out, const hcb_tensor *src, int32_t dim, int32_t reverse) {
+    return orc::guarded([&] { orc::exclusive_cumprod(*out, *src, dim, reverse != 0); });
+}
 int orc_addr(const hcb_tensor *out, const hcb_tensor *v1, const hcb_tensor *v2, const hcb_tensor *input, hcb_scalar alpha,
              hcb_scalar beta) {
     return orc::guarded([&] { orc::addr(*out, *v1, *v2, *input, alpha, beta); });
@@ -1128,7 +1187,7 @@ const hcb_backend *orc_backend(void) {
         "homura CPU oracle", orc_last_error, orc_copy,  orc_fill,           orc_unary,
         orc_binary,          orc_binary_constant,       orc_binary_scalar,  orc_where,
         orc_where_constant,  orc_reduce,     orc_var,   orc_arg_reduce,     orc_softmax,
-        orc_fused,           orc_triangle,   orc_flip,  orc_addr,
+        orc_fused,           orc_triangle,   orc_flip,  orc_addr,           orc_exclusive_cumprod,
     };
     return &table;
 }

@@ -150,6 +150,18 @@ def values(dtype, n, seed):
     return out
 
 
+def mixed_floats(dtype, n, seed):
+    """A mix of magnitudes, signs, zeros and values that overflow or vanish in F16
+    (ref: src/backend/rocm/tests.rs:809-830)."""
+    s, out = seed, np.empty(n, dtype=np.float64)
+    for i in range(n):
+        s = (s * 6364136223846793005 + 1442695040888963407) & ((1 << 64) - 1)
+        u = (s >> 11) / float(1 << 53)
+        e = ((s >> 3) % 40) - 20
+        out[i] = {0: 0.0, 1: -0.0, 2: 7e4, 3: 1e-7}.get(i % 17, (u * 2.0 - 1.0) * 2.0 ** e)
+    return tensor(from_f64(out, dtype), dtype)
+
+
 def normal(seed, n, mean=0.0, std=1.0):
     """Box-Muller in f64 from SplitMix64 words (the bench and config inputs)."""
     w = words(seed, 2 * ((n + 1) // 2))

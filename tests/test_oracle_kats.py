@@ -382,7 +382,7 @@ def test_softmax_against_exact_arithmetic():
 
 # ---- fused optimizer steps: exact rational arithmetic with the roundings where the reference has them ------
 
-def round_to(frac, dtype):
+def nearest_even(frac, dtype):
     """`frac` (a Fraction) rounded to nearest-even in F32 or F64, as a Fraction; finite normal results only."""
     if frac == 0:
         return Fraction(0)
@@ -410,7 +410,7 @@ def test_fused_steps_round_once_where_the_reference_does(dtype):
     npdt = NP[dtype]
     a, b, c = ((rng.standard_normal(n) * 2.0 ** rng.integers(-3, 4, n)).astype(npdt) for _ in range(3))
     c = np.where(np.abs(c) < 0.01, npdt(0.5), c).astype(npdt)
-    R = lambda f: round_to(f, dtype)
+    R = lambda f: nearest_even(f, dtype)
     F = lambda arr: [Fraction(float(v)) for v in arr]
     fa, fb, fc = F(a), F(b), F(c)
     ta, tb, tc = (tensor(v, dtype) for v in (a, b, c))

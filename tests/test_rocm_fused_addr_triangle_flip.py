@@ -11,7 +11,7 @@ import pytest
 from homura_amd import capi
 from tests import oracle
 from tests.support import (DT, DTYPES, FLOATS, GPU, NP, array, assert_bitwise, bits, from_f64, h, large_layouts, layouts,
-                           tensor, values)
+                           mixed_floats, tensor, values)
 
 pytestmark = pytest.mark.gpu
 h.register_cpu_backend(oracle.backend_address())
@@ -20,18 +20,6 @@ L = capi.lib
 COEFFICIENTS = [0.1, -0.3, 0.49999, 0.5, 0.9, 1.0 + 1e-4, -1.7, 1.0 / 3.0, 1e-30]
 STEPS = {"scaled_add": lambda a, b, c, v: h.scaled_add(a, b, v), "lerp": lambda a, b, c, v: h.lerp_step(a, b, v),
          "addcmul": lambda a, b, c, v: h.addcmul_step(a, b, c, v), "addcdiv": lambda a, b, c, v: h.addcdiv_step(a, b, c, v)}
-
-
-def mixed_floats(dtype, n, seed):
-    """A mix of magnitudes, signs, zeros and values that overflow or vanish in F16
-    (ref: src/backend/rocm/tests.rs:809-830)."""
-    s, out = seed, np.empty(n, dtype=np.float64)
-    for i in range(n):
-        s = (s * 6364136223846793005 + 1442695040888963407) & ((1 << 64) - 1)
-        u = (s >> 11) / float(1 << 53)
-        e = ((s >> 3) % 40) - 20
-        out[i] = {0: 0.0, 1: -0.0, 2: 7e4, 3: 1e-7}.get(i % 17, (u * 2.0 - 1.0) * 2.0 ** e)
-    return tensor(from_f64(out, dtype), dtype)
 
 
 @pytest.mark.parametrize("dtype", FLOATS)

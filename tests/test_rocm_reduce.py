@@ -399,3 +399,75 @@ def test_the_judges_reject_wrong_results():
         assert_bitwise(gv, x.min_dim(1, False)[0], "max is not min")
     with pytest.raises(AssertionError):
         check_softmax(x.to(GPU).log_softmax(1), x.softmax(1), wide, 1, False, "log_softmax is not softmax")
+
+
+# ---- exclusive cumulative product ---------------------------------------------------------------------------------
+
+
+def test_exclusive_cumprod_matches_the_cpu():
+    """The same bits on every float dtype, layout, dimension and direction: each line is multiplied in the CPU's
+    order (ref: src/backend/rocm/tests.rs:1025-1056)."""
+    from tests.support import mixed_floats
+    for dtype in FLOATS:
+        base = mixed_floats(dtype, 2 * 3 * 50, 7).mul(3.0)
+        views = [lambda t: t.reshape([6, 50]), lambda t: t.reshape([50, 6]).transpose(0, 1),
+                 lambda t: t.reshape([2, 3, 50]).narrow(2, 1, 40), lambda t: t.narrow(0, 0, 1)]
+        g = base.to(GPU)
+        for view in views:
+            x, xg = view(base), view(g)
+            for dim in range(len(x.shape)):
+                for reverse in (False, True):
+                    assert_bitwise(h.exclusive_cumprod(xg, dim, reverse), h.exclusive_cumprod(x, dim, reverse),
+                                   f"{dtype} {x.shape} dim {dim} reverse {reverse}")
+
+
+@pytest.mark.parametrize("dtype", FLOATS)
+def test_exclusive_cumprod_of_lines_that_vectorise_and_of_many_lines(dtype):
+    """Contiguous lines of whole 16-byte tiles (read by tile, also backwards), lines across a large tensor (one thread
+    each, several grid rounds), values near one so that long products stay finite, zeros and infinities on the way."""
+    rng = np.random.default_rng(31)
+    for shape, dim in (([300, 64], 1), ([300, 64], 0), ([3, 5, 128], 2), ([70000, 24], 1), ([40, 70000], 0), ([1, 4096], 1)):
+        v = 1.0 + rng.standard_normal(int(np.prod(shape))) * 0.05
+        v[rng.integers(0, v.size, 20)] = 0.0
+        v[rng.integers(0, v.size, 5)] = np.inf
+        v[rng.integers(0, v.size, 5)] = -2.5
+        x = tensor(from_f64(v, dtype), dtype).reshape(shape)
+        xg = x.to(GPU)
+        for reverse in (False, True):
+            assert_bitwise(h.exclusive_cumprod(xg, dim, reverse), h.exclusive_cumprod(x, dim, reverse),
+                           f"{dtype} {shape} dim {dim} reverse {reverse}")
+    with pytest.raises(Exception, match="expected a floating point dtype, got i32"):
+        h.exclusive_cumprod(h.full([4], 1, DT.I32, GPU), 0, False)
+
+
+def test_exclusive_cumprod_through_the_c_abi_in_place_and_its_errors():
+    from ctypes import byref
+
+    from homura_amd import capi
+    L = capi.lib
+    ctx = capi.Context(0)
+    try:
+        rows, n = 50, 37
+        x = (1.0 + np.random.default_rng(3).standard_normal((rows, n)) * 0.3).astype(np.float32)
+        dx = ctx.upload(x)
+        lines = capi.make_desc(dx.ptr, capi.F32, [rows], [n], 0)
+        # Over its own input: every element is read before its position is written.
+        capi.check(L.hmr_exclusive_cumprod(ctx.handle, byref(lines), byref(lines), n, 1, 1, 0))
+        ctx.synchronize()
+        want = np.empty_like(x)
+        for r in range(rows):
+            acc = np.float64(1.0)
+            for k in range(n):
+                want[r, k] = np.float32(acc)
+                acc = acc * np.float64(x[r, k])
+        np.testing.assert_array_equal(dx.download(np.float32, rows * n).reshape(rows, n), want)
+        assert L.hmr_exclusive_cumprod(ctx.handle, byref(lines), byref(lines), -1, 1, 1, 0) == capi.HMR_INVALID
+        assert L.hmr_last_error().decode() == "invalid row length or stride"
+        ints = capi.make_desc(dx.ptr, capi.I32, [rows], [n], 0)
+        assert L.hmr_exclusive_cumprod(ctx.handle, byref(ints), byref(ints), n, 1, 1, 0) == capi.HMR_INVALID
+        assert L.hmr_last_error().decode() == "exclusive_cumprod: unsupported dtype"
+        other = capi.make_desc(dx.ptr, capi.F32, [rows - 1], [n], 0)
+        assert L.hmr_exclusive_cumprod(ctx.handle, byref(lines), byref(other), n, 1, 1, 0) == capi.HMR_INVALID
+        capi.check(L.hmr_exclusive_cumprod(ctx.handle, byref(lines), byref(lines), 0, 1, 1, 1))  # nothing to do
+    finally:
+        ctx.close()
