@@ -294,6 +294,13 @@ def per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP
     add(None, "exclusive_cumprod f32 [16384,4096] dim=1 (a thread per row, sequential)", 8 * N,
         lambda: h.exclusive_cumprod(xf, 1, True), 5)
     del xf
+    shape = [8, 2048, 4096]
+    add(None, "rand f32 [8,2048,4096] (Philox on the device, write only)", 4 * N, lambda: h.rand(shape, DT.F32, GPU))
+    add(None, "rand bf16 [8,2048,4096]", 2 * N, lambda: h.rand(shape, DT.BF16, GPU))
+    add(None, "randn f32 [8,2048,4096] (Box-Muller in f64)", 4 * N, lambda: h.randn(shape, DT.F32, GPU), 10)
+    add(None, "randint [0, 1024) i64 [8,2048,4096] (no rejection)", 8 * N, lambda: h.randint(0, 1024, shape, DT.I64, GPU), 10)
+    add(None, "randint [-5, 6) i64 [8,2048,4096] (rejection: count, scan, write + a read-back)", 8 * N,
+        lambda: h.randint(-5, 6, shape, DT.I64, GPU), 5)
     sq = residual.reshape([16, 2048, 2048])
     add(None, "triu(1) f32 [16,2048,2048] (reads the kept half)", 6 * N, lambda: sq.triu(1))
     add(None, "tril(0) f32 [16,2048,2048] (reads the kept half)", 6 * N, lambda: sq.tril(0))

@@ -1,0 +1,329 @@
+// hmr_random_uniform, hmr_random_normal, hmr_random_int
+// (ref: csrc/homura_rocm.h:265-295, csrc/random.hip; the generator is src/ops/random.rs:29-266).
+//
+// Philox4x32-10 evaluated on the device: block n is the counter [n, n >> 32, 0, 0] under the key
+// [seed, seed >> 32]. The caller reserves a call's blocks (from `offset` on) exactly as the CPU
+// does, so uniform samples and integers are the CPU's bit for bit; normal samples go through the
+// device's f64 log, cos and sin. A thread owns one block: 4 (2 for F64) uniform samples, 2 normal
+// samples or 2 integer words, so a wave writes one contiguous span. The kernels only write: they
+// are bound by the stores (uniform, integers) or by the f64 transcendentals (normal).
+#include <cmath>
+
+#include "ew_common.hpp"
+
+namespace hmr {
+namespace {
+
+struct Word4 {
+    uint32_t v[4];
+};
+
+__device__ __forceinline__ Word4 philox_block(uint64_t n, uint64_t seed) {
+    constexpr uint32_t M0 = 0xD2511F53u, M1 = 0xCD9E8D57u, W0 = 0x9E3779B9u, W1 = 0xBB67AE85u;
+    uint32_t c0 = static_cast<uint32_t>(n), c1 = static_cast<uint32_t>(n >> 32), c2 = 0, c3 = 0;
+    uint32_t k0 = static_cast<uint32_t>(seed), k1 = static_cast<uint32_t>(seed >> 32);
+#pragma unroll
+    for (int round = 0; round < 10; ++round) {
+        if (round > 0) {
+            k0 += W0;
+            k1 += W1;
+        }
+        const uint32_t h0 = __umulhi(M0, c0), l0 = M0 * c0;
+        const uint32_t h1 = __umulhi(M1, c2), l1 = M1 * c2;
+        const uint32_t n0 = h1 ^ c1 ^ k0, n2 = h0 ^ c3 ^ k1;
+        c0 = n0, c1 = l1, c2 = n2, c3 = l0;
+    }
+    return Word4{{c0, c1, c2, c3}};
+}
+
+// A uniform f64 in [0, 1) from 53 random bits / from the top BITS bits of x (exact in f64).
+__device__ __forceinline__ double unit_f64(uint32_t hi, uint32_t lo) {
+    const uint64_t bits = (static_cast<uint64_t>(hi) << 21) ^ (static_cast<uint64_t>(lo) >> 11);
+    return static_cast<double>(bits) * (1.0 / 9007199254740992.0);
+}
+
+template <class T>
+struct Digits;
+template <>
+struct Digits<f16_t> {
+    static constexpr int value = 11;
+};
+template <>
+struct Digits<bf16_t> {
+    static constexpr int value = 8;
+};
+template <>
+struct Digits<float> {
+    static constexpr int value = 24;
+};
+
+// Stores the first `count` of a thread's PER elements at out + first: one vector store when the
+// span is whole and aligned, single elements otherwise (the tail, or an output at an odd offset).
+template <class T, int PER>
+__device__ __forceinline__ void store_span(T *out, int64_t first, int64_t n, const T (&v)[PER]) {
+    T *p = out + first;
+    if (first + PER <= n && reinterpret_cast<uintptr_t>(p) % (PER * sizeof(T)) == 0) {
+        store_tile<T, PER, false>(reinterpret_cast<char *>(p), v);
+    } else {
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            if (first + j < n) p[j] = v[j];
+        }
+    }
+}
+
+template <class T>
+__global__ void __launch_bounds__(kBlock) uniform_kernel(T *out, int64_t n, int64_t blocks, uint64_t seed, uint64_t offset,
+                                                         double from, double to) {
+    constexpr int PER = std::is_same_v<T, double> ? 2 : 4;  // F64 takes two words per value
+    const T low = Conv<T>::from_f64(from);
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; i < blocks;
+         i += static_cast<int64_t>(gridDim.x) * kBlock) {
+        const Word4 b = philox_block(offset + static_cast<uint64_t>(i), seed);
+        T v[PER];
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            double u;
+            if constexpr (PER == 2) {
+                u = unit_f64(b.v[2 * j], b.v[2 * j + 1]);
+            } else {
+                constexpr int bits = Digits<T>::value;
+                u = static_cast<double>(b.v[j] >> (32 - bits)) * (1.0 / static_cast<double>(uint64_t{1} << bits));
+            }
+            const double x = from + u * (to - from);
+            T r = Conv<T>::from_f64(x);
+            // Rounding can reach the excluded upper bound, which maps to the lower one.
+            if (from < to && Conv<T>::to_f64(r) >= to) r = low;
+            v[j] = r;
+        }
+        store_span<T, PER>(out, i * PER, n, v);
+    }
+}
+
+template <class T>
+__global__ void __launch_bounds__(kBlock) normal_kernel(T *out, int64_t n, int64_t blocks, uint64_t seed, uint64_t offset,
+                                                        double mean, double std) {
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; i < blocks;
+         i += static_cast<int64_t>(gridDim.x) * kBlock) {
+        const Word4 b = philox_block(offset + static_cast<uint64_t>(i), seed);
+        // Box-Muller in f64: each block gives two normals, the cosine first.
+        const double u1 = 1.0 - unit_f64(b.v[0], b.v[1]), u2 = unit_f64(b.v[2], b.v[3]);
+        const double r = sqrt(-2.0 * log(u1));
+        const double theta = 2.0 * 3.14159265358979323846 * u2;
+        const T v[2] = {Conv<T>::from_f64(mean + std * r * cos(theta)), Conv<T>::from_f64(mean + std * r * sin(theta))};
+        store_span<T, 2>(out, 2 * i, n, v);
+    }
+}
+
+// ---- integers: rejection sampling on 64-bit words -------------------------------------------------
+//
+// The words of a batch in order are [w0 w1] then [w2 w3] of each block; those >= threshold become
+// low + word % range and fill `out` in that order. With threshold 0 nothing is rejected and word j
+// is element j. Otherwise the batch is compacted in three launches over tiles of
+// HMR_RANDOM_INT_TILE blocks (one workgroup each): count the accepted words per tile, scan the
+// counts (one workgroup), write each tile's accepted words from its offset on. The workspace holds
+// the counts (tiles words), the offsets (tiles words) and the batch's total (one word).
+static_assert(HMR_RANDOM_INT_TILE == kBlock, "a tile is one workgroup's blocks");
+
+__device__ __forceinline__ void int_words(const Word4 &b, uint64_t (&w)[2]) {
+    w[0] = (static_cast<uint64_t>(b.v[0]) << 32) | b.v[1];
+    w[1] = (static_cast<uint64_t>(b.v[2]) << 32) | b.v[3];
+}
+
+__global__ void __launch_bounds__(kBlock) int_all_kernel(int64_t *out, int64_t n, int64_t blocks, uint64_t seed,
+                                                         uint64_t offset, int64_t low, uint64_t range) {
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; i < blocks;
+         i += static_cast<int64_t>(gridDim.x) * kBlock) {
+        uint64_t w[2];
+        int_words(philox_block(offset + static_cast<uint64_t>(i), seed), w);
+        const int64_t v[2] = {static_cast<int64_t>(static_cast<uint64_t>(low) + w[0] % range),
+                              static_cast<int64_t>(static_cast<uint64_t>(low) + w[1] % range)};
+        store_span<int64_t, 2>(out, 2 * i, n, v);
+    }
+}
+
+// The accepted words of this thread's block (0..2) and, in every thread, the exclusive count of
+// accepted words in the threads before it in the workgroup; `total` is the workgroup's count.
+__device__ __forceinline__ uint32_t rank_in_tile(uint32_t mine, uint32_t &total) {
+    __shared__ uint32_t wave_sum[kBlock / 64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    uint32_t inclusive = mine;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const uint32_t up = static_cast<uint32_t>(__shfl_up(static_cast<int>(inclusive), d, 64));
+        if (lane >= d) inclusive += up;
+    }
+    if (lane == 63) wave_sum[wave] = inclusive;
+    __syncthreads();
+    uint32_t before = 0;
+    total = 0;
+#pragma unroll
+    for (int k = 0; k < kBlock / 64; ++k) {
+        if (k < wave) before += wave_sum[k];
+        total += wave_sum[k];
+    }
+    __syncthreads();  // wave_sum may be written again by the caller's next use
+    return before + inclusive - mine;
+}
+
+__global__ void __launch_bounds__(kBlock) int_count_kernel(uint64_t *counts, int64_t blocks, uint64_t seed, uint64_t offset,
+                                                           uint64_t threshold) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    uint32_t mine = 0;
+    if (i < blocks) {
+        uint64_t w[2];
+        int_words(philox_block(offset + static_cast<uint64_t>(i), seed), w);
+        mine = (w[0] >= threshold ? 1u : 0u) + (w[1] >= threshold ? 1u : 0u);
+    }
+    uint32_t total;
+    rank_in_tile(mine, total);
+    if (threadIdx.x == 0) counts[blockIdx.x] = total;
+}
+
+// One workgroup: offsets[t] = the sum of counts[0..t), total = the sum of all.
+constexpr int kScanThreads = 1024;
+__global__ void __launch_bounds__(kScanThreads) int_scan_kernel(const uint64_t *counts, uint64_t *offsets, uint64_t *total,
+                                                                int64_t tiles) {
+    __shared__ uint64_t part[kScanThreads];
+    const int64_t per = (tiles + kScanThreads - 1) / kScanThreads;
+    const int64_t first = per * threadIdx.x, last = first + per < tiles ? first + per : tiles;
+    uint64_t sum = 0;
+    for (int64_t t = first; t < last; ++t) sum += counts[t];
+    part[threadIdx.x] = sum;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint64_t running = 0;
+        for (int k = 0; k < kScanThreads; ++k) {
+            const uint64_t s = part[k];
+            part[k] = running;
+            running += s;
+        }
+        *total = running;
+    }
+    __syncthreads();
+    uint64_t running = part[threadIdx.x];
+    for (int64_t t = first; t < last; ++t) {
+        offsets[t] = running;
+        running += counts[t];
+    }
+}
+
+__global__ void __launch_bounds__(kBlock) int_write_kernel(int64_t *out, int64_t n, const uint64_t *offsets, int64_t blocks,
+                                                           uint64_t seed, uint64_t offset, int64_t low, uint64_t range,
+                                                           uint64_t threshold) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    uint64_t w[2] = {0, 0};
+    bool take[2] = {false, false};
+    if (i < blocks) {
+        int_words(philox_block(offset + static_cast<uint64_t>(i), seed), w);
+        take[0] = w[0] >= threshold;
+        take[1] = w[1] >= threshold;
+    }
+    uint32_t total;
+    uint64_t at = offsets[blockIdx.x] + rank_in_tile((take[0] ? 1u : 0u) + (take[1] ? 1u : 0u), total);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        if (!take[j]) continue;
+        if (at < static_cast<uint64_t>(n)) out[at] = static_cast<int64_t>(static_cast<uint64_t>(low) + w[j] % range);
+        ++at;
+    }
+}
+
+inline unsigned grid_of(int64_t threads) {
+    const int64_t want = (threads + kBlock - 1) / kBlock;
+    const int64_t cap = int64_t{1} << 22;
+    return static_cast<unsigned>(want < 1 ? 1 : (want < cap ? want : cap));
+}
+
+// The flat contiguous output of a sampling call: its element count and first element.
+hmr_status flat_output(const hmr_tensor_desc &out, int64_t &n, char *&first) {
+    if (hmr_status s = check_desc(out, n)) return s;
+    int64_t expect = 1;
+    for (int d = out.ndim - 1; d >= 0; --d) {
+        if (out.sizes[d] != 1 && out.strides[d] != expect) return fail(HMR_INVALID, "random sampling writes a contiguous tensor");
+        expect *= out.sizes[d];
+    }
+    first = static_cast<char *>(out.data) + out.offset * dtype_size(out.dtype);
+    return HMR_OK;
+}
+
+}  // namespace
+}  // namespace hmr
+
+extern "C" {
+
+hmr_status hmr_random_uniform(hmr_context_t ctx, const hmr_tensor_desc *out, uint64_t seed, uint64_t offset, double from,
+                              double to) {
+    return hmr::guarded([&] {
+        int64_t n = 0;
+        char *first = nullptr;
+        if (hmr_status s = hmr::flat_output(*out, n, first)) return s;
+        if (n == 0) return HMR_OK;
+        return hmr::launch_on(ctx, "random_uniform", [&](hipStream_t stream) {
+            return hmr::with_float_type(out->dtype, [&](auto t) {
+                using T = typename decltype(t)::type;
+                const int64_t per = std::is_same_v<T, double> ? 2 : 4;
+                const int64_t blocks = (n + per - 1) / per;
+                hipLaunchKernelGGL((hmr::uniform_kernel<T>), dim3(hmr::grid_of(blocks)), dim3(hmr::kBlock), 0, stream,
+                                   reinterpret_cast<T *>(first), n, blocks, seed, offset, from, to);
+            });
+        });
+    });
+}
+
+hmr_status hmr_random_normal(hmr_context_t ctx, const hmr_tensor_desc *out, uint64_t seed, uint64_t offset, double mean,
+                             double std) {
+    return hmr::guarded([&] {
+        int64_t n = 0;
+        char *first = nullptr;
+        if (hmr_status s = hmr::flat_output(*out, n, first)) return s;
+        if (n == 0) return HMR_OK;
+        return hmr::launch_on(ctx, "random_normal", [&](hipStream_t stream) {
+            return hmr::with_float_type(out->dtype, [&](auto t) {
+                using T = typename decltype(t)::type;
+                const int64_t blocks = (n + 1) / 2;
+                hipLaunchKernelGGL((hmr::normal_kernel<T>), dim3(hmr::grid_of(blocks)), dim3(hmr::kBlock), 0, stream,
+                                   reinterpret_cast<T *>(first), n, blocks, seed, offset, mean, std);
+            });
+        });
+    });
+}
+
+hmr_status hmr_random_int(hmr_context_t ctx, const hmr_tensor_desc *out, uint64_t seed, uint64_t offset, uint64_t blocks,
+                          int64_t low, uint64_t range, uint64_t threshold, void *workspace) {
+    return hmr::guarded([&] {
+        int64_t n = 0;
+        char *first = nullptr;
+        if (hmr_status s = hmr::flat_output(*out, n, first)) return s;
+        if (out->dtype != HMR_I64) return hmr::fail(HMR_INVALID, "random_int: unsupported dtype");
+        if (range == 0) return hmr::fail(HMR_INVALID, "random_int: the range is empty");
+        if (blocks > (uint64_t{1} << 62)) return hmr::fail(HMR_INVALID, "random_int: too many blocks");
+        if (threshold != 0 && workspace == nullptr) return hmr::fail(HMR_INVALID, "random_int: a workspace is needed to reject words");
+        const int64_t nblocks = static_cast<int64_t>(blocks);
+        const int64_t tiles = (nblocks + HMR_RANDOM_INT_TILE - 1) / HMR_RANDOM_INT_TILE;
+        if (threshold != 0 && tiles > (int64_t{1} << 31) - 1) return hmr::fail(HMR_INVALID, "random_int: too many blocks in one batch");
+        if (blocks == 0 && threshold == 0) return HMR_OK;
+        return hmr::launch_on(ctx, "random_int", [&](hipStream_t stream) {
+            int64_t *po = reinterpret_cast<int64_t *>(first);
+            if (threshold == 0) {
+                if (n == 0) return true;
+                hipLaunchKernelGGL(hmr::int_all_kernel, dim3(hmr::grid_of(nblocks)), dim3(hmr::kBlock), 0, stream, po, n, nblocks,
+                                   seed, offset, low, range);
+                return true;
+            }
+            uint64_t *counts = static_cast<uint64_t *>(workspace), *offsets = counts + tiles, *total = counts + 2 * tiles;
+            if (tiles > 0) {
+                hipLaunchKernelGGL(hmr::int_count_kernel, dim3(static_cast<unsigned>(tiles)), dim3(hmr::kBlock), 0, stream, counts,
+                                   nblocks, seed, offset, threshold);
+            }
+            hipLaunchKernelGGL(hmr::int_scan_kernel, dim3(1), dim3(hmr::kScanThreads), 0, stream, counts, offsets, total, tiles);
+            if (tiles > 0 && n > 0) {
+                hipLaunchKernelGGL(hmr::int_write_kernel, dim3(static_cast<unsigned>(tiles)), dim3(hmr::kBlock), 0, stream, po, n,
+                                   offsets, nblocks, seed, offset, low, range, threshold);
+            }
+            return true;
+        });
+    });
+}
+
+}  // extern "C"

@@ -15,10 +15,6 @@ hmr_status unbuilt(const char *name) {
 
 extern "C" {
 
-HMR_UNBUILT(hmr_random_uniform, hmr_context_t, const hmr_tensor_desc *, uint64_t, uint64_t, double, double)
-HMR_UNBUILT(hmr_random_normal, hmr_context_t, const hmr_tensor_desc *, uint64_t, uint64_t, double, double)
-HMR_UNBUILT(hmr_random_int, hmr_context_t, const hmr_tensor_desc *, uint64_t, uint64_t, uint64_t, int64_t, uint64_t,
-            uint64_t, void *)
 HMR_UNBUILT(hmr_index_check, hmr_context_t, const hmr_tensor_desc *, int64_t, int64_t, int32_t, int64_t, uint64_t *)
 HMR_UNBUILT(hmr_index_select, hmr_context_t, const hmr_tensor_desc *, const hmr_tensor_desc *,
             const hmr_tensor_desc *, int32_t, int32_t)

@@ -660,6 +660,67 @@ void addr(const TensorData &out, const TensorData &v1, const TensorData &v2, con
     });
 }
 
+namespace {
+// ref: src/backend/rocm/random.rs:11-19
+bool flat_desc(const char *kernel, const TensorData &out, hmr_tensor_desc &d) {
+    if (!out.layout.is_contiguous()) throw Error(std::string("internal error: ") + kernel + " into a strided tensor");
+    std::vector<hmr_tensor_desc> ds;
+    if (!descs(kernel, {&out}, ds)) return false;
+    d = ds[0];
+    return true;
+}
+}  // namespace
+
+void random_uniform(const TensorData &out, uint64_t seed, uint64_t offset, double from, double to) {
+    if (on_cpu(out)) {
+        hcb_tensor o = cpu_desc(out);
+        cpu_check(cpu_backend("uniform").random_uniform(&o, seed, offset, from, to));
+        return;
+    }
+    hmr_tensor_desc d;
+    if (!flat_desc("uniform", out, d)) return;
+    exec(out, [&](hmr_context_t ctx) { expect(hmr_random_uniform(ctx, &d, seed, offset, from, to)); });
+}
+
+void random_normal(const TensorData &out, uint64_t seed, uint64_t offset, double mean, double std) {
+    if (on_cpu(out)) {
+        hcb_tensor o = cpu_desc(out);
+        cpu_check(cpu_backend("normal").random_normal(&o, seed, offset, mean, std));
+        return;
+    }
+    hmr_tensor_desc d;
+    if (!flat_desc("normal", out, d)) return;
+    exec(out, [&](hmr_context_t ctx) { expect(hmr_random_normal(ctx, &d, seed, offset, mean, std)); });
+}
+
+std::optional<uint64_t> random_int_batch(const TensorData &out, uint64_t seed, uint64_t offset, uint64_t blocks, int64_t low,
+                                         uint64_t range, uint64_t threshold, const TensorData *workspace) {
+    if (on_cpu(out)) {
+        hcb_tensor o = cpu_desc(out);
+        uint64_t accepted = 0;
+        cpu_check(cpu_backend("randint").random_int(&o, seed, offset, blocks, low, range, threshold, &accepted));
+        return accepted;
+    }
+    hmr_tensor_desc d;
+    if (!flat_desc("randint", out, d)) return std::nullopt;
+    const uint64_t tiles = (blocks + HMR_RANDOM_INT_TILE - 1) / HMR_RANDOM_INT_TILE;
+    void *ws = nullptr;
+    if (threshold != 0) {
+        if (!workspace || workspace->layout.offset != 0 || static_cast<uint64_t>(workspace->layout.num_elements()) <= 2 * tiles) {
+            throw Error("internal error: the workspace of randint");
+        }
+        ws = workspace->storage->ptr();
+    }
+    exec(out, [&](hmr_context_t ctx) { expect(hmr_random_int(ctx, &d, seed, offset, blocks, low, range, threshold, ws)); });
+    if (threshold == 0) return std::nullopt;
+    // The batch's count is the workspace's last word: read it back (waits for the device).
+    int64_t count = 0;
+    DeviceState &st = device_state(out.device().index);
+    std::lock_guard<std::recursive_mutex> lock(st.exec);
+    expect(hmr_copy_to_host(st.ctx, &count, static_cast<const char *>(ws) + 2 * tiles * sizeof(int64_t), sizeof count));
+    return static_cast<uint64_t>(count);
+}
+
 void upload(const TensorData &dst, const TensorData &src) {
     if (!src.layout.is_contiguous() || !dst.layout.is_contiguous() || !on_cpu(src) || on_cpu(dst)) {
         throw Error("internal error: upload needs a contiguous CPU source and a contiguous ROCm destination");

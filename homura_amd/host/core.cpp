@@ -64,8 +64,6 @@ std::string Scalar::str() const {
     return s.str();
 }
 
-namespace {
-
 double float_max(DType d) {
     switch (d) {
         case DType::F16: return 65504.0;
@@ -77,6 +75,7 @@ double float_max(DType d) {
 
 void int_range(DType d, int64_t &lo, int64_t &hi) {
     switch (d) {
+        case DType::Bool: lo = 0; hi = 1; break;
         case DType::U8: lo = 0; hi = 255; break;
         case DType::I8: lo = -128; hi = 127; break;
         case DType::I16: lo = -32768; hi = 32767; break;
@@ -84,8 +83,6 @@ void int_range(DType d, int64_t &lo, int64_t &hi) {
         default: lo = INT64_MIN; hi = INT64_MAX; break;
     }
 }
-
-}  // namespace
 
 std::optional<Scalar> Scalar::checked_to(DType dtype) const {
     switch (kind_of(dtype)) {

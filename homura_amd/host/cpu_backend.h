@@ -86,6 +86,15 @@ typedef struct hcb_backend {
     /* ref: src/backend/cpu/reduce.rs:281-324; floating point operands of one shape and dtype */
     int (*exclusive_cumprod)(const hcb_tensor *out, const hcb_tensor *src, int32_t dim,
                              int32_t reverse);
+    /* ref: src/ops/random.rs:29-266: the samples of the Philox blocks from `offset` on under `seed`
+     * into a flat contiguous tensor (floats; I64 for random_int). random_int is one batch of the
+     * rejection sampling over `blocks` blocks and reports how many words it accepted. */
+    int (*random_uniform)(const hcb_tensor *out, uint64_t seed, uint64_t offset, double from,
+                          double to);
+    int (*random_normal)(const hcb_tensor *out, uint64_t seed, uint64_t offset, double mean,
+                         double std);
+    int (*random_int)(const hcb_tensor *out, uint64_t seed, uint64_t offset, uint64_t blocks,
+                      int64_t low, uint64_t range, uint64_t threshold, uint64_t *accepted);
 } hcb_backend;
 
 #ifdef __cplusplus

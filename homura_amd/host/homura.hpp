@@ -77,6 +77,8 @@ class ResultType {
 
 // `value` converted to `dtype` as the CPU's fill converts it, little-endian in the low bytes
 // (ref: src/backend/rocm/copy.rs:253-270).
+double float_max(DType d);                              // the largest finite value of a float dtype
+void int_range(DType d, int64_t &lo, int64_t &hi);      // of an integer or bool dtype
 uint64_t scalar_bits(Scalar value, DType dtype);
 // `value` taken to a floating point dtype's computation type (f32, or f64 for F64), rounded to the dtype,
 // and read back.
@@ -322,6 +324,16 @@ Tensor where_(const Tensor &condition, const Operand &x, const Operand &y);
 // when `reverse`), multiplied in order: what the gradient of `prod` uses for inputs with zeros
 // (ref: src/ops/reduce.rs:158-170).
 Tensor exclusive_cumprod(const Tensor &x, size_t dim, bool reverse);
+// Random sampling from the process-wide Philox4x32-10 generator, shared by all devices: a GPU computes the
+// CPU's uniform samples and integers bit for bit, also when calls on the two alternate
+// (ref: src/ops/random.rs). `uniform` and `normal` are what `uniform_` / `normal_` fill a tensor with.
+void manual_seed(uint64_t seed);
+Tensor rand(const Shape &shape, DType dtype, Device device);
+Tensor randn(const Shape &shape, DType dtype, Device device);
+Tensor randint(int64_t low, int64_t high, const Shape &shape, DType dtype, Device device);
+Tensor uniform(const Shape &shape, double from, double to, DType dtype, Device device);
+Tensor normal(const Shape &shape, double mean, double std, DType dtype, Device device);
+
 // The optimizers' single-rounding steps (ref: src/optim/mod.rs:569-616): new tensors from tensors of one
 // shape, floating point dtype and device. A finite scalar beyond the range of the type it is converted
 // to (the dtype for alpha, the computation type otherwise) is an error.
@@ -388,6 +400,14 @@ void flip(const TensorData &out, const TensorData &src, const std::vector<bool> 
 // values of the dtype (ref: src/backend/mod.rs:562-587).
 void addr(const TensorData &out, const TensorData &v1, const TensorData &v2, const TensorData &input, Scalar alpha,
           Scalar beta);
+// Samples of the Philox blocks from `offset` on under `seed` into a contiguous tensor
+// (ref: src/backend/rocm/random.rs:30-118). random_int_batch is one batch of the integer rejection sampling
+// into the I64 `out`; it returns how many words it accepted (not read back, and `out` filled, when
+// `threshold` is 0 on a ROCm device: then every word is accepted).
+void random_uniform(const TensorData &out, uint64_t seed, uint64_t offset, double from, double to);
+void random_normal(const TensorData &out, uint64_t seed, uint64_t offset, double mean, double std);
+std::optional<uint64_t> random_int_batch(const TensorData &out, uint64_t seed, uint64_t offset, uint64_t blocks, int64_t low,
+                                         uint64_t range, uint64_t threshold, const TensorData *workspace);
 // Host <-> device and device <-> host transfers of contiguous data of one dtype.
 void upload(const TensorData &dst, const TensorData &src);
 void download(const TensorData &dst, const TensorData &src);

@@ -114,6 +114,20 @@ PYBIND11_MODULE(_host, m) {
           py::arg("p"), py::arg("grad"), py::arg("state"), py::arg("lr"), py::arg("beta1") = 0.9, py::arg("beta2") = 0.999,
           py::arg("eps") = 1e-8, py::arg("weight_decay") = 0.0, py::arg("amsgrad") = false, py::arg("maximize") = false,
           py::arg("decoupled_weight_decay") = false);
+    m.def("manual_seed", &manual_seed);
+    m.def("rand", [](const Shape &shape, DType d, const std::string &dev) { return rand(shape, d, parse_device(dev)); },
+          py::arg("shape"), py::arg("dtype") = DType::F32, py::arg("device") = "cpu");
+    m.def("randn", [](const Shape &shape, DType d, const std::string &dev) { return randn(shape, d, parse_device(dev)); },
+          py::arg("shape"), py::arg("dtype") = DType::F32, py::arg("device") = "cpu");
+    m.def("randint", [](int64_t low, int64_t high, const Shape &shape, DType d, const std::string &dev) {
+        return randint(low, high, shape, d, parse_device(dev));
+    }, py::arg("low"), py::arg("high"), py::arg("shape"), py::arg("dtype") = DType::I64, py::arg("device") = "cpu");
+    m.def("uniform", [](const Shape &shape, double from, double to, DType d, const std::string &dev) {
+        return uniform(shape, from, to, d, parse_device(dev));
+    }, py::arg("shape"), py::arg("from_"), py::arg("to"), py::arg("dtype") = DType::F32, py::arg("device") = "cpu");
+    m.def("normal", [](const Shape &shape, double mean, double std, DType d, const std::string &dev) {
+        return normal(shape, mean, std, d, parse_device(dev));
+    }, py::arg("shape"), py::arg("mean"), py::arg("std"), py::arg("dtype") = DType::F32, py::arg("device") = "cpu");
     m.def("exclusive_cumprod", &exclusive_cumprod, py::arg("x"), py::arg("dim"), py::arg("reverse") = false);
     m.def("reduce_plan", [](const Tensor &t, const std::vector<int64_t> &dims) {
         auto p = rocm_reduce_plan(t, dims);

@@ -17,7 +17,7 @@
  *  - enumerations travel as int32_t.
  *
  * Entry points of the reference that belong to other kernel families (gemm, indexing, pooling,
- * random, scans ...) are declared in homura_rocm_unbuilt.h and exported as
+ * convolution windows ...) are declared in homura_rocm_unbuilt.h and exported as
  * stubs that fail with HMR_INVALID, so that the reference crate still links.
  */
 #ifndef HOMURA_ROCM_H
@@ -295,6 +295,36 @@ hmr_status hmr_softmax(hmr_context_t ctx, const hmr_tensor_desc *out_rows,
 hmr_status hmr_exclusive_cumprod(hmr_context_t ctx, const hmr_tensor_desc *out_lines,
                                  const hmr_tensor_desc *src_lines, int64_t n, int64_t out_stride,
                                  int64_t src_stride, int32_t reverse);
+
+/* ---- random sampling ------------------------------------------ ref: csrc/homura_rocm.h:265-295 */
+/* Philox4x32-10 as in src/ops/random.rs:29-91: block n is the counter [n, n >> 32, 0, 0] under the
+ * key [seed, seed >> 32]; the caller reserves the blocks of a call (from `offset` on) as the CPU
+ * does and advances its generator. `out` is flat and contiguous.
+ *
+ * ref :276-279  hmr_random_uniform: from + u * (to - from) in f64 for a float `out`, u from 53
+ * bits (two words, two elements per block) for F64 and from the dtype's significand bits (one
+ * word per element, four per block) otherwise, rounded to the dtype; a result that rounds to `to`
+ * (with from < to) becomes `from`. hmr_random_normal: Box-Muller in f64, two elements per block
+ * (cosine, then sine), rounded to the dtype. */
+hmr_status hmr_random_uniform(hmr_context_t ctx, const hmr_tensor_desc *out, uint64_t seed,
+                              uint64_t offset, double from, double to);
+hmr_status hmr_random_normal(hmr_context_t ctx, const hmr_tensor_desc *out, uint64_t seed,
+                             uint64_t offset, double mean, double std);
+
+/* The Philox blocks of one tile of hmr_random_int. */
+#define HMR_RANDOM_INT_TILE 256
+
+/* ref :284-295  One batch of the CPU's integer rejection sampling (sample_int,
+ * src/ops/random.rs:228-258): the 64-bit words of `blocks` blocks from `offset` on, two per block
+ * in the order [w0 w1] then [w2 w3]; the words >= `threshold`, in that order, become
+ * low + word % range (wrapping) and fill the I64 `out` until it is full, the rest are dropped.
+ * With threshold 0 every word is taken and `workspace` may be NULL. Otherwise `workspace` holds
+ * 2 * tiles + 1 64-bit words of device memory, tiles = ceil(blocks / HMR_RANDOM_INT_TILE), and
+ * the batch's number of words >= threshold (which may exceed out's elements) is left in its last
+ * word. */
+hmr_status hmr_random_int(hmr_context_t ctx, const hmr_tensor_desc *out, uint64_t seed,
+                          uint64_t offset, uint64_t blocks, int64_t low, uint64_t range,
+                          uint64_t threshold, void *workspace);
 
 /* ---- build facts and ABI self-description ------------------- ref: csrc/homura_rocm.h:589-610 */
 /* ';'-separated offload architectures compiled in ("gfx950"). */

@@ -18,16 +18,6 @@
 extern "C" {
 #endif
 
-/* ref :276-295 */
-#define HMR_RANDOM_INT_TILE 256
-hmr_status hmr_random_uniform(hmr_context_t ctx, const hmr_tensor_desc *out, uint64_t seed,
-                              uint64_t offset, double from, double to);
-hmr_status hmr_random_normal(hmr_context_t ctx, const hmr_tensor_desc *out, uint64_t seed,
-                             uint64_t offset, double mean, double std);
-hmr_status hmr_random_int(hmr_context_t ctx, const hmr_tensor_desc *out, uint64_t seed,
-                          uint64_t offset, uint64_t blocks, int64_t low, uint64_t range,
-                          uint64_t threshold, void *workspace);
-
 /* ref :361-426 (indexing) */
 hmr_status hmr_index_check(hmr_context_t ctx, const hmr_tensor_desc *index, int64_t low,
                            int64_t high, int32_t has_exempt, int64_t exempt, uint64_t *slot);

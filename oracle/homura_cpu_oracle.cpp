@@ -1091,6 +1091,123 @@ void exclusive_cumprod(const hcb_tensor &out, const hcb_tensor &src, int dim, bo
     });
 }
 
+// ---- random sampling (ref: src/ops/random.rs:29-226) ---------------------------------------------
+//
+// Philox4x32-10: block n is the counter [n, n >> 32, 0, 0] under the key [seed, seed >> 32]. The
+// caller reserves a call's blocks (from `offset` on) and advances its generator.
+void philox(const uint32_t counter[4], const uint32_t key[2], uint32_t out[4]) {
+    const uint64_t M0 = 0xD2511F53u, M1 = 0xCD9E8D57u;
+    const uint32_t W0 = 0x9E3779B9u, W1 = 0xBB67AE85u;
+    uint32_t c[4] = {counter[0], counter[1], counter[2], counter[3]};
+    uint32_t k[2] = {key[0], key[1]};
+    for (int round = 0; round < 10; ++round) {
+        if (round > 0) {
+            k[0] += W0;
+            k[1] += W1;
+        }
+        const uint64_t p0 = M0 * c[0], p1 = M1 * c[2];
+        const uint32_t n0 = static_cast<uint32_t>(p1 >> 32) ^ c[1] ^ k[0], n1 = static_cast<uint32_t>(p1);
+        const uint32_t n2 = static_cast<uint32_t>(p0 >> 32) ^ c[3] ^ k[1], n3 = static_cast<uint32_t>(p0);
+        c[0] = n0, c[1] = n1, c[2] = n2, c[3] = n3;
+    }
+    for (int i = 0; i < 4; ++i) out[i] = c[i];
+}
+
+struct Blocks {
+    uint64_t seed, start;
+    void operator()(uint64_t i, uint32_t out[4]) const {
+        const uint64_t n = start + i;
+        const uint32_t counter[4] = {static_cast<uint32_t>(n), static_cast<uint32_t>(n >> 32), 0, 0};
+        const uint32_t key[2] = {static_cast<uint32_t>(seed), static_cast<uint32_t>(seed >> 32)};
+        philox(counter, key, out);
+    }
+};
+
+// A uniform f64 in [0, 1) from 53 random bits / from the top `bits` bits of x.
+double unit_f64(uint32_t hi, uint32_t lo) {
+    const uint64_t bits = (static_cast<uint64_t>(hi) << 21) ^ (static_cast<uint64_t>(lo) >> 11);
+    return static_cast<double>(bits) * (1.0 / 9007199254740992.0);
+}
+double unit_bits(uint32_t x, int bits) { return static_cast<double>(x >> (32 - bits)) / static_cast<double>(uint64_t{1} << bits); }
+
+int float_digits(int dtype) { return dtype == HMR_F16 ? 11 : dtype == HMR_BF16 ? 8 : dtype == HMR_F32 ? 24 : 53; }
+
+void check_flat(const hcb_tensor &out) {
+    int64_t expect = 1;
+    for (int d = out.ndim - 1; d >= 0; --d) {
+        if (out.shape[d] != 1 && out.strides[d] != expect) panic("random sampling writes a contiguous tensor");
+        expect *= out.shape[d];
+    }
+}
+
+void random_uniform(const hcb_tensor &out, uint64_t seed, uint64_t offset, double from, double to) {
+    check_flat(out);
+    const int64_t n = num_elements(out);
+    dispatch_float(out.dtype, [&](auto t) {
+        using T = typename decltype(t)::type;
+        T *po = base<T>(out) + out.offset;
+        const int per_block = out.dtype == HMR_F64 ? 2 : 4;  // f64 uses two words per value
+        const int bits = float_digits(out.dtype);
+        const Blocks block{seed, offset};
+        for (int64_t i = 0; i * per_block < n; ++i) {
+            uint32_t b[4];
+            block(static_cast<uint64_t>(i), b);
+            for (int j = 0; j < per_block && i * per_block + j < n; ++j) {
+                const double u = per_block == 2 ? unit_f64(b[2 * j], b[2 * j + 1]) : unit_bits(b[j], bits);
+                const double x = from + u * (to - from);
+                T v = El<T>::from_f64(x);
+                // Rounding can reach the excluded upper bound, which maps to the lower one.
+                if (from < to && El<T>::to_f64(v) >= to) v = El<T>::from_f64(from);
+                po[i * per_block + j] = v;
+            }
+        }
+    });
+}
+
+void random_normal(const hcb_tensor &out, uint64_t seed, uint64_t offset, double mean, double std) {
+    check_flat(out);
+    const int64_t n = num_elements(out);
+    dispatch_float(out.dtype, [&](auto t) {
+        using T = typename decltype(t)::type;
+        T *po = base<T>(out) + out.offset;
+        const Blocks block{seed, offset};
+        for (int64_t i = 0; 2 * i < n; ++i) {  // Box-Muller: each block gives two normals
+            uint32_t b[4];
+            block(static_cast<uint64_t>(i), b);
+            const double u1 = 1.0 - unit_f64(b[0], b[1]), u2 = unit_f64(b[2], b[3]);
+            const double r = std::sqrt(-2.0 * std::log(u1));
+            const double theta = 2.0 * 3.14159265358979323846 * u2;
+            po[2 * i] = El<T>::from_f64(mean + std * r * std::cos(theta));
+            if (2 * i + 1 < n) po[2 * i + 1] = El<T>::from_f64(mean + std * r * std::sin(theta));
+        }
+    });
+}
+
+// One batch of rejection sampling on 64-bit words (two per block: [w0 w1], then [w2 w3]): the words
+// >= threshold become low + word % range and fill the I64 `out` until it is full. Returns how many
+// words of the batch were accepted (which may exceed out's elements).
+uint64_t random_int(const hcb_tensor &out, uint64_t seed, uint64_t offset, uint64_t blocks, int64_t low, uint64_t range,
+                    uint64_t threshold) {
+    check_flat(out);
+    if (out.dtype != HMR_I64) panic("random integers are sampled into an I64 tensor");
+    if (range == 0) panic("random_int: empty range");
+    const uint64_t n = static_cast<uint64_t>(num_elements(out));
+    int64_t *po = base<int64_t>(out) + out.offset;
+    const Blocks block{seed, offset};
+    uint64_t accepted = 0;
+    for (uint64_t i = 0; i < blocks; ++i) {
+        uint32_t b[4];
+        block(i, b);
+        const uint64_t words[2] = {(static_cast<uint64_t>(b[0]) << 32) | b[1], (static_cast<uint64_t>(b[2]) << 32) | b[3]};
+        for (uint64_t w : words) {
+            if (w < threshold) continue;
+            if (accepted < n) po[accepted] = static_cast<int64_t>(static_cast<uint64_t>(low) + w % range);
+            ++accepted;
+        }
+    }
+    return accepted;
+}
+
 template <class F>
 int guarded(F f) {
     try {
@@ -1168,6 +1285,17 @@ int orc_flip(const hcb_tensor *out, const hcb_tensor *src, const uint8_t *mask) 
 int orc_exclusive_cumprod(const hcb_tensor *out, const hcb_tensor *src, int32_t dim, int32_t reverse) {
     return orc::guarded([&] { orc::exclusive_cumprod(*out, *src, dim, reverse != 0); });
 }
+void orc_philox(const uint32_t *counter, const uint32_t *key, uint32_t *out) { orc::philox(counter, key, out); }
+int orc_random_uniform(const hcb_tensor *out, uint64_t seed, uint64_t offset, double from, double to) {
+    return orc::guarded([&] { orc::random_uniform(*out, seed, offset, from, to); });
+}
+int orc_random_normal(const hcb_tensor *out, uint64_t seed, uint64_t offset, double mean, double std) {
+    return orc::guarded([&] { orc::random_normal(*out, seed, offset, mean, std); });
+}
+int orc_random_int(const hcb_tensor *out, uint64_t seed, uint64_t offset, uint64_t blocks, int64_t low, uint64_t range,
+                   uint64_t threshold, uint64_t *accepted) {
+    return orc::guarded([&] { *accepted = orc::random_int(*out, seed, offset, blocks, low, range, threshold); });
+}
 int orc_addr(const hcb_tensor *out, const hcb_tensor *v1, const hcb_tensor *v2, const hcb_tensor *input, hcb_scalar alpha,
              hcb_scalar beta) {
     return orc::guarded([&] { orc::addr(*out, *v1, *v2, *input, alpha, beta); });
@@ -1188,6 +1316,7 @@ const hcb_backend *orc_backend(void) {
         orc_binary,          orc_binary_constant,       orc_binary_scalar,  orc_where,
         orc_where_constant,  orc_reduce,     orc_var,   orc_arg_reduce,     orc_softmax,
         orc_fused,           orc_triangle,   orc_flip,  orc_addr,           orc_exclusive_cumprod,
+        orc_random_uniform,  orc_random_normal,         orc_random_int,
     };
     return &table;
 }
