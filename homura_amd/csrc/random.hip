@@ -28,10 +28,10 @@ __device__ __forceinline__ Word4 philox_block(uint64_t n, uint64_t seed) {
             k0 += W0;
             k1 += W1;
         }
-        const uint32_t h0 = __umulhi(M0, c0), l0 = M0 * c0;
-        const uint32_t h1 = __umulhi(M1, c2), l1 = M1 * c2;
-        const uint32_t n0 = h1 ^ c1 ^ k0, n2 = h0 ^ c3 ^ k1;
-        c0 = n0, c1 = l1, c2 = n2, c3 = l0;
+        // One 32 x 32 -> 64 multiply each (v_mad_u64_u32) rather than a high and a low half.
+        const uint64_t p0 = static_cast<uint64_t>(M0) * c0, p1 = static_cast<uint64_t>(M1) * c2;
+        const uint32_t n0 = static_cast<uint32_t>(p1 >> 32) ^ c1 ^ k0, n2 = static_cast<uint32_t>(p0 >> 32) ^ c3 ^ k1;
+        c0 = n0, c1 = static_cast<uint32_t>(p1), c2 = n2, c3 = static_cast<uint32_t>(p0);
     }
     return Word4{{c0, c1, c2, c3}};
 }
@@ -130,14 +130,27 @@ __device__ __forceinline__ void int_words(const Word4 &b, uint64_t (&w)[2]) {
     w[1] = (static_cast<uint64_t>(b.v[2]) << 32) | b.v[3];
 }
 
+// w % range without a division. A range that rejects nothing divides 2^64, so it is a power of two
+// and the remainder is a mask. Otherwise, with magic = floor(2^64 / range), the quotient estimate
+// floor(w * magic / 2^64) is the quotient or one less (w / range - w * magic / 2^64 < w / 2^64 < 1),
+// so one conditional subtraction finishes; the remainder before it is at most w, which fits.
+struct Modulus {
+    uint64_t range, magic;
+};
+inline Modulus make_modulus(uint64_t range) { return Modulus{range, ~uint64_t{0} / range}; }
+__device__ __forceinline__ uint64_t remainder(uint64_t w, const Modulus &m) {
+    uint64_t r = w - __umul64hi(w, m.magic) * m.range;
+    return r >= m.range ? r - m.range : r;
+}
+
 __global__ void __launch_bounds__(kBlock) int_all_kernel(int64_t *out, int64_t n, int64_t blocks, uint64_t seed,
-                                                         uint64_t offset, int64_t low, uint64_t range) {
+                                                         uint64_t offset, int64_t low, uint64_t mask) {
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; i < blocks;
          i += static_cast<int64_t>(gridDim.x) * kBlock) {
         uint64_t w[2];
         int_words(philox_block(offset + static_cast<uint64_t>(i), seed), w);
-        const int64_t v[2] = {static_cast<int64_t>(static_cast<uint64_t>(low) + w[0] % range),
-                              static_cast<int64_t>(static_cast<uint64_t>(low) + w[1] % range)};
+        const int64_t v[2] = {static_cast<int64_t>(static_cast<uint64_t>(low) + (w[0] & mask)),
+                              static_cast<int64_t>(static_cast<uint64_t>(low) + (w[1] & mask))};
         store_span<int64_t, 2>(out, 2 * i, n, v);
     }
 }
@@ -209,7 +222,7 @@ __global__ void __launch_bounds__(kScanThreads) int_scan_kernel(const uint64_t *
 }
 
 __global__ void __launch_bounds__(kBlock) int_write_kernel(int64_t *out, int64_t n, const uint64_t *offsets, int64_t blocks,
-                                                           uint64_t seed, uint64_t offset, int64_t low, uint64_t range,
+                                                           uint64_t seed, uint64_t offset, int64_t low, Modulus modulus,
                                                            uint64_t threshold) {
     const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
     uint64_t w[2] = {0, 0};
@@ -224,7 +237,7 @@ __global__ void __launch_bounds__(kBlock) int_write_kernel(int64_t *out, int64_t
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         if (!take[j]) continue;
-        if (at < static_cast<uint64_t>(n)) out[at] = static_cast<int64_t>(static_cast<uint64_t>(low) + w[j] % range);
+        if (at < static_cast<uint64_t>(n)) out[at] = static_cast<int64_t>(static_cast<uint64_t>(low) + remainder(w[j], modulus));
         ++at;
     }
 }
@@ -299,6 +312,9 @@ hmr_status hmr_random_int(hmr_context_t ctx, const hmr_tensor_desc *out, uint64_
         if (range == 0) return hmr::fail(HMR_INVALID, "random_int: the range is empty");
         if (blocks > (uint64_t{1} << 62)) return hmr::fail(HMR_INVALID, "random_int: too many blocks");
         if (threshold != 0 && workspace == nullptr) return hmr::fail(HMR_INVALID, "random_int: a workspace is needed to reject words");
+        if (threshold == 0 && (range & (range - 1)) != 0) {
+            return hmr::fail(HMR_INVALID, "random_int: a range that isn't a power of two rejects words below 2^64 mod range");
+        }
         const int64_t nblocks = static_cast<int64_t>(blocks);
         const int64_t tiles = (nblocks + HMR_RANDOM_INT_TILE - 1) / HMR_RANDOM_INT_TILE;
         if (threshold != 0 && tiles > (int64_t{1} << 31) - 1) return hmr::fail(HMR_INVALID, "random_int: too many blocks in one batch");
@@ -307,8 +323,9 @@ hmr_status hmr_random_int(hmr_context_t ctx, const hmr_tensor_desc *out, uint64_
             int64_t *po = reinterpret_cast<int64_t *>(first);
             if (threshold == 0) {
                 if (n == 0) return true;
+                // Nothing is rejected only when the range divides 2^64: a power of two.
                 hipLaunchKernelGGL(hmr::int_all_kernel, dim3(hmr::grid_of(nblocks)), dim3(hmr::kBlock), 0, stream, po, n, nblocks,
-                                   seed, offset, low, range);
+                                   seed, offset, low, range - 1);
                 return true;
             }
             uint64_t *counts = static_cast<uint64_t *>(workspace), *offsets = counts + tiles, *total = counts + 2 * tiles;
@@ -319,7 +336,7 @@ hmr_status hmr_random_int(hmr_context_t ctx, const hmr_tensor_desc *out, uint64_
             hipLaunchKernelGGL(hmr::int_scan_kernel, dim3(1), dim3(hmr::kScanThreads), 0, stream, counts, offsets, total, tiles);
             if (tiles > 0 && n > 0) {
                 hipLaunchKernelGGL(hmr::int_write_kernel, dim3(static_cast<unsigned>(tiles)), dim3(hmr::kBlock), 0, stream, po, n,
-                                   offsets, nblocks, seed, offset, low, range, threshold);
+                                   offsets, nblocks, seed, offset, low, hmr::make_modulus(range), threshold);
             }
             return true;
         });
