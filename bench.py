@@ -294,6 +294,11 @@ def per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP
     add(None, "exclusive_cumprod f32 [16384,4096] dim=1 (a thread per row, sequential)", 8 * N,
         lambda: h.exclusive_cumprod(xf, 1, True), 5)
     del xf
+    y = x.reshape([16384, 4096]).softmax(-1)
+    gy = t2.reshape([16384, 4096])
+    add(None, "softmax backward bf16 [16384,4096] (6 kernels: 2 casts, mul, sum, sub, mul, cast)", 2 * N * (3 + 3 + 6 + 2 + 6 + 6 + 3),
+        lambda: h.grad_softmax(gy, y, -1, False), 10)
+    del y, gy
     shape = [8, 2048, 4096]
     add(None, "rand f32 [8,2048,4096] (Philox on the device, write only)", 4 * N, lambda: h.rand(shape, DT.F32, GPU))
     add(None, "rand bf16 [8,2048,4096]", 2 * N, lambda: h.rand(shape, DT.BF16, GPU))

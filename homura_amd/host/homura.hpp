@@ -324,6 +324,21 @@ Tensor where_(const Tensor &condition, const Operand &x, const Operand &y);
 // when `reverse`), multiplied in order: what the gradient of `prod` uses for inputs with zeros
 // (ref: src/ops/reduce.rs:158-170).
 Tensor exclusive_cumprod(const Tensor &x, size_t dim, bool reverse);
+// The input gradients of the reductions and of softmax for an output gradient `g`, composed from the ops above as
+// the reference's backward nodes compose them outside grad mode (ref: src/autograd/formulas/reduce.rs:160-470,
+// softmax.rs:43-84). `dims` empty = all elements (the full reductions); otherwise the reduced dimensions and
+// whether they were kept. Not here: the gradient of max_dim / min_dim, which scatters through indices.
+namespace grad {
+Tensor sum(const Tensor &g, const Shape &self_shape, const std::vector<int64_t> &dims, bool keepdim);
+Tensor mean(const Tensor &g, const Shape &self_shape, const std::vector<int64_t> &dims, bool keepdim);
+Tensor sum_to_size(const Tensor &g, const Shape &self_shape);
+Tensor prod(const Tensor &g, const Tensor &x, const Tensor &result, std::optional<int64_t> dim, bool keepdim);
+Tensor extremum(const Tensor &g, const Tensor &x, const Tensor &result);  // x.max() / x.min()
+Tensor var_std(const Tensor &g, const Tensor &x, const std::optional<Tensor> &std_result, const std::vector<int64_t> &dims,
+               int64_t correction, bool keepdim);
+Tensor softmax(const Tensor &g, const Tensor &y, int64_t dim, bool log);
+}  // namespace grad
+
 // Random sampling from the process-wide Philox4x32-10 generator, shared by all devices: a GPU computes the
 // CPU's uniform samples and integers bit for bit, also when calls on the two alternate
 // (ref: src/ops/random.rs). `uniform` and `normal` are what `uniform_` / `normal_` fill a tensor with.

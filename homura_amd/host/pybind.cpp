@@ -114,6 +114,13 @@ PYBIND11_MODULE(_host, m) {
           py::arg("p"), py::arg("grad"), py::arg("state"), py::arg("lr"), py::arg("beta1") = 0.9, py::arg("beta2") = 0.999,
           py::arg("eps") = 1e-8, py::arg("weight_decay") = 0.0, py::arg("amsgrad") = false, py::arg("maximize") = false,
           py::arg("decoupled_weight_decay") = false);
+    m.def("grad_sum", &grad::sum);
+    m.def("grad_mean", &grad::mean);
+    m.def("grad_sum_to_size", &grad::sum_to_size);
+    m.def("grad_prod", &grad::prod);
+    m.def("grad_extremum", &grad::extremum);
+    m.def("grad_var_std", &grad::var_std);
+    m.def("grad_softmax", &grad::softmax);
     m.def("manual_seed", &manual_seed);
     m.def("rand", [](const Shape &shape, DType d, const std::string &dev) { return rand(shape, d, parse_device(dev)); },
           py::arg("shape"), py::arg("dtype") = DType::F32, py::arg("device") = "cpu");
