@@ -296,7 +296,7 @@ def per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP
     del xf
     y = x.reshape([16384, 4096]).softmax(-1)
     gy = t2.reshape([16384, 4096])
-    add(None, "softmax backward bf16 [16384,4096] (6 kernels: 2 casts, mul, sum, sub, mul, cast)", 2 * N * (3 + 3 + 6 + 2 + 6 + 6 + 3),
+    add(None, "softmax backward bf16 [16384,4096] (7 kernels: 2 casts, mul, sum, sub, mul, cast)", 2 * N * (3 + 3 + 6 + 2 + 4 + 6 + 3),
         lambda: h.grad_softmax(gy, y, -1, False), 10)
     del y, gy
     shape = [8, 2048, 4096]
