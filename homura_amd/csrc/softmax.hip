@@ -581,8 +581,23 @@ __global__ void __launch_bounds__(kBlock) cumprod_kernel(CumprodArgs a) {
         const T *ps = reinterpret_cast<const T *>(a.src) + a.src_lines.offset(line);
         T *po = reinterpret_cast<T *>(a.out) + a.out_lines.offset(line);
         typename P::A acc = 1;
+        // The chain of multiplications is sequential, the memory accesses need not be: kAhead elements (or
+        // tiles: 128 bytes of the thread's own row) are loaded together, multiplied through in
+        // order and written together.
+        constexpr int kAhead = V == 1 ? 32 : 8;
         if constexpr (V == 1) {
-            for (int64_t k = 0; k < a.n; ++k) {
+            int64_t k = 0;
+            for (; k + kAhead <= a.n; k += kAhead) {
+                T x[kAhead];
+#pragma unroll
+                for (int j = 0; j < kAhead; ++j) x[j] = ps[(a.reverse ? a.n - 1 - (k + j) : k + j) * a.si];
+#pragma unroll
+                for (int j = 0; j < kAhead; ++j) {
+                    po[(a.reverse ? a.n - 1 - (k + j) : k + j) * a.so] = P::narrow(acc);
+                    acc = acc * P::widen(x[j]);
+                }
+            }
+            for (; k < a.n; ++k) {
                 const int64_t at = a.reverse ? a.n - 1 - k : k;
                 const T x = ps[at * a.si];  // read before the write: the operands may be one buffer
                 po[at * a.so] = P::narrow(acc);
@@ -590,10 +605,7 @@ __global__ void __launch_bounds__(kBlock) cumprod_kernel(CumprodArgs a) {
             }
         } else {
             const int64_t tiles = a.n / V;
-            for (int64_t c = 0; c < tiles; ++c) {
-                const int64_t at = (a.reverse ? tiles - 1 - c : c) * V;
-                T r[V], w[V];
-                load_tile<T, V, false>(reinterpret_cast<const char *>(ps + at), r);
+            auto scan_tile = [&](T(&r)[V], T(&w)[V]) {
                 if (a.reverse) {
 #pragma unroll
                     for (int i = V - 1; i >= 0; --i) {
@@ -607,6 +619,26 @@ __global__ void __launch_bounds__(kBlock) cumprod_kernel(CumprodArgs a) {
                         acc = acc * P::widen(r[i]);
                     }
                 }
+            };
+            int64_t c = 0;
+            for (; c + kAhead <= tiles; c += kAhead) {
+                T r[kAhead][V], w[kAhead][V];
+#pragma unroll
+                for (int j = 0; j < kAhead; ++j) {
+                    load_tile<T, V, false>(reinterpret_cast<const char *>(ps + (a.reverse ? tiles - 1 - (c + j) : c + j) * V), r[j]);
+                }
+#pragma unroll
+                for (int j = 0; j < kAhead; ++j) scan_tile(r[j], w[j]);
+#pragma unroll
+                for (int j = 0; j < kAhead; ++j) {
+                    store_tile<T, V, false>(reinterpret_cast<char *>(po + (a.reverse ? tiles - 1 - (c + j) : c + j) * V), w[j]);
+                }
+            }
+            for (; c < tiles; ++c) {
+                const int64_t at = (a.reverse ? tiles - 1 - c : c) * V;
+                T r[V], w[V];
+                load_tile<T, V, false>(reinterpret_cast<const char *>(ps + at), r);
+                scan_tile(r, w);
                 store_tile<T, V, false>(reinterpret_cast<char *>(po + at), w);
             }
         }
