@@ -120,9 +120,10 @@ __global__ void __launch_bounds__(kBlock) normal_kernel(T *out, int64_t n, int64
 // The words of a batch in order are [w0 w1] then [w2 w3] of each block; those >= threshold become
 // low + word % range and fill `out` in that order. With threshold 0 nothing is rejected and word j
 // is element j. Otherwise the batch is compacted in three launches over tiles of
-// HMR_RANDOM_INT_TILE blocks (one workgroup each): count the accepted words per tile, scan the
-// counts (one workgroup), write each tile's accepted words from its offset on. The workspace holds
-// the counts (tiles words), the offsets (tiles words) and the batch's total (one word).
+// HMR_RANDOM_INT_TILE blocks (a workgroup's width): count the accepted words of each group of tiles,
+// scan the counts (one workgroup), write each group's accepted words from its offset on, the
+// blocks being computed again. The workspace holds the counts and the offsets (room for one per
+// tile each) and the batch's total (its last word).
 static_assert(HMR_RANDOM_INT_TILE == kBlock, "a tile is one workgroup's blocks");
 
 __device__ __forceinline__ void int_words(const Word4 &b, uint64_t (&w)[2]) {
@@ -179,14 +180,20 @@ __device__ __forceinline__ uint32_t rank_in_tile(uint32_t mine, uint32_t &total)
     return before + inclusive - mine;
 }
 
+// A workgroup takes kTilesPerGroup tiles one after the other, so that the scan between the two passes
+// has few entries (the workspace has room for one per tile; the first `groups` of each half are used).
+constexpr int kTilesPerGroup = 16;
+
 __global__ void __launch_bounds__(kBlock) int_count_kernel(uint64_t *counts, int64_t blocks, uint64_t seed, uint64_t offset,
                                                            uint64_t threshold) {
-    const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
     uint32_t mine = 0;
-    if (i < blocks) {
-        uint64_t w[2];
-        int_words(philox_block(offset + static_cast<uint64_t>(i), seed), w);
-        mine = (w[0] >= threshold ? 1u : 0u) + (w[1] >= threshold ? 1u : 0u);
+    for (int j = 0; j < kTilesPerGroup; ++j) {
+        const int64_t i = (static_cast<int64_t>(blockIdx.x) * kTilesPerGroup + j) * kBlock + threadIdx.x;
+        if (i < blocks) {
+            uint64_t w[2];
+            int_words(philox_block(offset + static_cast<uint64_t>(i), seed), w);
+            mine += (w[0] >= threshold ? 1u : 0u) + (w[1] >= threshold ? 1u : 0u);
+        }
     }
     uint32_t total;
     rank_in_tile(mine, total);
@@ -224,21 +231,25 @@ __global__ void __launch_bounds__(kScanThreads) int_scan_kernel(const uint64_t *
 __global__ void __launch_bounds__(kBlock) int_write_kernel(int64_t *out, int64_t n, const uint64_t *offsets, int64_t blocks,
                                                            uint64_t seed, uint64_t offset, int64_t low, Modulus modulus,
                                                            uint64_t threshold) {
-    const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
-    uint64_t w[2] = {0, 0};
-    bool take[2] = {false, false};
-    if (i < blocks) {
-        int_words(philox_block(offset + static_cast<uint64_t>(i), seed), w);
-        take[0] = w[0] >= threshold;
-        take[1] = w[1] >= threshold;
-    }
-    uint32_t total;
-    uint64_t at = offsets[blockIdx.x] + rank_in_tile((take[0] ? 1u : 0u) + (take[1] ? 1u : 0u), total);
+    uint64_t running = offsets[blockIdx.x];  // accepted words before this group's first tile
+    for (int j = 0; j < kTilesPerGroup; ++j) {
+        const int64_t i = (static_cast<int64_t>(blockIdx.x) * kTilesPerGroup + j) * kBlock + threadIdx.x;
+        uint64_t w[2] = {0, 0};
+        bool take[2] = {false, false};
+        if (i < blocks) {
+            int_words(philox_block(offset + static_cast<uint64_t>(i), seed), w);
+            take[0] = w[0] >= threshold;
+            take[1] = w[1] >= threshold;
+        }
+        uint32_t total;
+        uint64_t at = running + rank_in_tile((take[0] ? 1u : 0u) + (take[1] ? 1u : 0u), total);
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        if (!take[j]) continue;
-        if (at < static_cast<uint64_t>(n)) out[at] = static_cast<int64_t>(static_cast<uint64_t>(low) + remainder(w[j], modulus));
-        ++at;
+        for (int k = 0; k < 2; ++k) {
+            if (!take[k]) continue;
+            if (at < static_cast<uint64_t>(n)) out[at] = static_cast<int64_t>(static_cast<uint64_t>(low) + remainder(w[k], modulus));
+            ++at;
+        }
+        running += total;
     }
 }
 
@@ -329,13 +340,14 @@ hmr_status hmr_random_int(hmr_context_t ctx, const hmr_tensor_desc *out, uint64_
                 return true;
             }
             uint64_t *counts = static_cast<uint64_t *>(workspace), *offsets = counts + tiles, *total = counts + 2 * tiles;
-            if (tiles > 0) {
-                hipLaunchKernelGGL(hmr::int_count_kernel, dim3(static_cast<unsigned>(tiles)), dim3(hmr::kBlock), 0, stream, counts,
+            const int64_t groups = (tiles + hmr::kTilesPerGroup - 1) / hmr::kTilesPerGroup;
+            if (groups > 0) {
+                hipLaunchKernelGGL(hmr::int_count_kernel, dim3(static_cast<unsigned>(groups)), dim3(hmr::kBlock), 0, stream, counts,
                                    nblocks, seed, offset, threshold);
             }
-            hipLaunchKernelGGL(hmr::int_scan_kernel, dim3(1), dim3(hmr::kScanThreads), 0, stream, counts, offsets, total, tiles);
-            if (tiles > 0 && n > 0) {
-                hipLaunchKernelGGL(hmr::int_write_kernel, dim3(static_cast<unsigned>(tiles)), dim3(hmr::kBlock), 0, stream, po, n,
+            hipLaunchKernelGGL(hmr::int_scan_kernel, dim3(1), dim3(hmr::kScanThreads), 0, stream, counts, offsets, total, groups);
+            if (groups > 0 && n > 0) {
+                hipLaunchKernelGGL(hmr::int_write_kernel, dim3(static_cast<unsigned>(groups)), dim3(hmr::kBlock), 0, stream, po, n,
                                    offsets, nblocks, seed, offset, low, hmr::make_modulus(range), threshold);
             }
             return true;
