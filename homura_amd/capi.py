@@ -90,6 +90,13 @@ PROTOTYPES = {
     "hmr_random_uniform": (c_int32, [CTX, DESC_P, c_uint64, c_uint64, c_double, c_double]),
     "hmr_random_normal": (c_int32, [CTX, DESC_P, c_uint64, c_uint64, c_double, c_double]),
     "hmr_random_int": (c_int32, [CTX, DESC_P, c_uint64, c_uint64, c_uint64, c_int64, c_uint64, c_uint64, c_void_p]),
+    "hmr_index_check": (c_int32, [CTX, DESC_P, c_int64, c_int64, c_int32, c_int64, c_void_p]),
+    "hmr_index_select": (c_int32, [CTX, DESC_P, DESC_P, DESC_P, c_int32, c_int32]),
+    "hmr_gather": (c_int32, [CTX, DESC_P, DESC_P, DESC_P, c_int32]),
+    "hmr_index_add_workspace": (c_int32, [c_int64, c_int64, POINTER(c_int64)]),
+    "hmr_index_add": (c_int32, [CTX, DESC_P, DESC_P, DESC_P, c_int32, c_void_p, c_int64]),
+    "hmr_scatter_add_workspace": (c_int32, [c_int64, POINTER(c_int64)]),
+    "hmr_scatter_add": (c_int32, [CTX, DESC_P, DESC_P, DESC_P, c_int32, c_void_p, c_int64]),
     "hmr_exclusive_cumprod": (c_int32, [CTX, DESC_P, DESC_P, c_int64, c_int64, c_int64, c_int32]),
     "hmr_built_archs": (c_char_p, []),
     "hmr_abi_check": (None, [POINTER(hmr_abi_info)]),
@@ -109,9 +116,7 @@ PROTOTYPES = {
 
 # Exported stubs of other kernel families (include/homura_rocm_unbuilt.h); bound without prototypes.
 UNBUILT = [
-    "hmr_index_check", "hmr_index_select", "hmr_gather",
-    "hmr_index_positions", "hmr_index_overwrite_workspace", "hmr_index_overwrite", "hmr_index_add_workspace",
-    "hmr_index_add", "hmr_scatter_add_workspace", "hmr_scatter_add", "hmr_max_pool2d_backward_workspace",
+    "hmr_index_positions", "hmr_index_overwrite_workspace", "hmr_index_overwrite", "hmr_max_pool2d_backward_workspace",
     "hmr_max_pool2d_backward", "hmr_mask_workspace", "hmr_mask_count", "hmr_mask_coordinates", "hmr_max_pool2d",
     "hmr_max_pool2d_check", "hmr_max_pool2d_gather_backward", "hmr_adaptive_avg_pool2d",
     "hmr_adaptive_avg_pool2d_backward", "hmr_unfold_backward", "hmr_gemm_fold", "hmr_gemm_select",

@@ -1,0 +1,596 @@
+// hmr_index_check, hmr_index_select, hmr_gather, hmr_index_add(+workspace), hmr_scatter_add(+workspace)
+// (ref: csrc/homura_rocm.h:353-404, csrc/index.hip; the semantics are src/backend/cpu/misc.rs:53-127, 213-345).
+//
+// Index tensors are I32 or I64. The caller checks positions first (hmr_index_check in the same
+// critical section), so the other kernels take them as valid.
+//   reads   index_select copies rows of 16-byte tiles when the slices are contiguous (an embedding
+//           lookup: one index load and one row offset per tile, the rest is a copy) and single elements
+//           otherwise; gather is one element per thread.
+//   adds    every element of the output is summed in f64 (wrapping i64 for integers) in the row-major
+//           order of the index positions and rounded once, as the CPU does. Addition is not
+//           associative, so the order is reproduced: each contribution becomes a 64-bit word
+//           (target << 32 | position), the words are sorted (a bitonic network: keys are unique, so any
+//           correct sort gives the one order), and the first word of each target sums its run in
+//           order. Targets run in parallel; index_add also spreads a slice over the lanes.
+#include "ew_common.hpp"
+
+namespace hmr {
+namespace {
+
+constexpr int kMaxIndexDims = HMR_MAX_DIMS;
+
+// The dimensions shared by the operands of a call, innermost first, with up to three stride sets.
+struct Dims {
+    int32_t ndim;
+    int32_t at;  // the indexed dimension, counted from the innermost
+    int64_t size[kMaxIndexDims];
+    int64_t stride[3][kMaxIndexDims];
+};
+
+__device__ __forceinline__ int64_t read_index(const void *base, int is64, int64_t offset) {
+    return is64 ? static_cast<const int64_t *>(base)[offset] : static_cast<int64_t>(static_cast<const int32_t *>(base)[offset]);
+}
+
+// ---- hmr_index_check ------------------------------------------------------------------------------------
+
+__global__ void check_init_kernel(uint64_t *slot) {
+    slot[0] = ~uint64_t{0};
+    slot[1] = 0;
+}
+
+__global__ void __launch_bounds__(kBlock) check_kernel(const void *index, int is64, Dims d, int64_t n, int64_t low, int64_t high,
+                                                       int has_exempt, int64_t exempt, unsigned long long *slot) {
+    unsigned long long first = ~0ull;
+    for (int64_t p = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; p < n; p += static_cast<int64_t>(gridDim.x) * kBlock) {
+        int64_t rest = p, off = 0;
+        for (int k = 0; k < d.ndim; ++k) {
+            const int64_t q = rest / d.size[k];
+            off += (rest - q * d.size[k]) * d.stride[0][k];
+            rest = q;
+        }
+        const int64_t v = read_index(index, is64, off);
+        const bool bad = !(v >= low && v < high) && !(has_exempt && v == exempt);
+        if (bad && static_cast<unsigned long long>(p) < first) first = static_cast<unsigned long long>(p);
+    }
+    // One atomic per wave that found something: the minimum is the same in whatever order they arrive.
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) {
+        const unsigned long long other = (static_cast<unsigned long long>(static_cast<uint32_t>(__shfl_xor(static_cast<int>(first >> 32), m, 64))) << 32) |
+                                         static_cast<uint32_t>(__shfl_xor(static_cast<int>(first), m, 64));
+        first = other < first ? other : first;
+    }
+    if ((threadIdx.x & 63) == 0 && first != ~0ull) atomicMin(slot, first);
+}
+
+__global__ void check_value_kernel(const void *index, int is64, Dims d, uint64_t *slot) {
+    const uint64_t p = slot[0];
+    if (p == ~uint64_t{0}) return;
+    int64_t rest = static_cast<int64_t>(p), off = 0;
+    for (int k = 0; k < d.ndim; ++k) {
+        const int64_t q = rest / d.size[k];
+        off += (rest - q * d.size[k]) * d.stride[0][k];
+        rest = q;
+    }
+    slot[1] = static_cast<uint64_t>(read_index(index, is64, off));
+}
+
+// ---- hmr_index_select / hmr_gather ---------------------------------------------------------------------
+
+// One element per thread. stride[0] out, [1] src, [2] the index (gather: walked like out; index_select:
+// only along `at`). `wrap` adds the source's size along `at` to a negative position.
+template <class W>
+__global__ void __launch_bounds__(kBlock) pick_kernel(W *out, const W *src, const void *index, int is64, Dims d, int64_t n,
+                                                      int64_t wrap) {
+    for (int64_t p = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; p < n; p += static_cast<int64_t>(gridDim.x) * kBlock) {
+        int64_t rest = p, oo = 0, so = 0, io = 0;
+        for (int k = 0; k < d.ndim; ++k) {
+            const int64_t q = rest / d.size[k];
+            const int64_t c = rest - q * d.size[k];
+            rest = q;
+            oo += c * d.stride[0][k];
+            io += c * d.stride[2][k];
+            if (k != d.at) so += c * d.stride[1][k];
+        }
+        int64_t j = read_index(index, is64, io);
+        if (j < 0) j += wrap;
+        out[oo] = src[so + j * d.stride[1][d.at]];
+    }
+}
+
+// index_select of contiguous slices: the innermost dimension is a run of whole 16-byte tiles in both
+// operands; the dimensions outside it (the indexed one among them) are decomposed once per tile.
+struct RowsOfTiles {
+    char *out;
+    const char *src;
+    const void *index;
+    int32_t is64, nouter, at;  // `at` counts outer dimensions from the innermost outer one
+    int64_t n_tiles, wrap, index_stride;
+    uint32_t tiles_per_row;
+    FastDiv tiles_div;
+    FastDiv div[kMaxIndexDims];
+    int64_t stride[2][kMaxIndexDims];  // of the outer dimensions, in elements
+};
+
+template <class W>
+__global__ void __launch_bounds__(kBlock) select_rows_kernel(RowsOfTiles a) {
+    constexpr int V = 16 / static_cast<int>(sizeof(W));
+    constexpr int U = 4;
+    const int64_t first = static_cast<int64_t>(blockIdx.x) * (U * kBlock) + threadIdx.x;
+    W r[U][V];
+    int64_t oo[U];
+    bool valid[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const int64_t t = first + static_cast<int64_t>(u) * kBlock;
+        valid[u] = t < a.n_tiles;
+        const uint32_t tt = static_cast<uint32_t>(valid[u] ? t : a.n_tiles - 1);
+        uint32_t row = divide(tt, a.tiles_div);
+        const int64_t col = static_cast<int64_t>(tt - row * a.tiles_per_row) * V;
+        int64_t o = col, s = col;
+        for (int k = 0; k < a.nouter; ++k) {
+            const uint32_t q = divide(row, a.div[k]);
+            const int64_t c = row - q * a.div[k].div;
+            row = q;
+            o += c * a.stride[0][k];
+            if (k == a.at) {
+                int64_t j = read_index(a.index, a.is64, c * a.index_stride);
+                if (j < 0) j += a.wrap;
+                s += j * a.stride[1][k];
+            } else {
+                s += c * a.stride[1][k];
+            }
+        }
+        oo[u] = o;
+        load_tile<W, V, kStreamLoads>(a.src + s * static_cast<int64_t>(sizeof(W)), r[u]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        if (valid[u]) store_tile<W, V, false>(a.out + oo[u] * static_cast<int64_t>(sizeof(W)), r[u]);
+    }
+}
+
+// ---- sorting 64-bit words (bitonic) -----------------------------------------------------------------------
+//
+// `count` is a power of two >= kSortChunk; a workgroup keeps kSortChunk words in LDS for the steps whose
+// partners lie inside an aligned chunk, the wider steps go through memory one at a time.
+constexpr int kSortChunk = 2048;
+constexpr int kSortThreads = 256;
+
+__device__ __forceinline__ void sort_steps_in_lds(uint64_t *s, uint32_t base, uint32_t k, uint32_t j_first) {
+    for (uint32_t j = j_first; j > 0; j >>= 1) {
+        for (uint32_t t = threadIdx.x; t < kSortChunk / 2; t += kSortThreads) {
+            const uint32_t i = ((t & ~(j - 1)) << 1) | (t & (j - 1));
+            const uint32_t l = i | j;
+            const bool ascending = ((base + i) & k) == 0;
+            const uint64_t x = s[i], y = s[l];
+            if ((x > y) == ascending) {
+                s[i] = y;
+                s[l] = x;
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// Every chunk sorted (k = 2 .. kSortChunk), or, with k > kSortChunk, the last log2(kSortChunk) steps of stage k.
+__global__ void __launch_bounds__(kSortThreads) sort_chunks_kernel(uint64_t *words, uint32_t k_only) {
+    __shared__ uint64_t s[kSortChunk];
+    const uint32_t base = blockIdx.x * kSortChunk;
+    for (uint32_t t = threadIdx.x; t < kSortChunk; t += kSortThreads) s[t] = words[base + t];
+    __syncthreads();
+    if (k_only == 0) {
+        for (uint32_t k = 2; k <= kSortChunk; k <<= 1) sort_steps_in_lds(s, base, k, k >> 1);
+    } else {
+        sort_steps_in_lds(s, base, k_only, kSortChunk >> 1);
+    }
+    for (uint32_t t = threadIdx.x; t < kSortChunk; t += kSortThreads) words[base + t] = s[t];
+}
+
+__global__ void __launch_bounds__(kBlock) sort_step_kernel(uint64_t *words, uint32_t half, uint32_t k, uint32_t j) {
+    const uint32_t t = blockIdx.x * kBlock + threadIdx.x;
+    if (t >= half) return;
+    const uint32_t i = ((t & ~(j - 1)) << 1) | (t & (j - 1));
+    const uint32_t l = i | j;
+    const bool ascending = (i & k) == 0;
+    const uint64_t x = words[i], y = words[l];
+    if ((x > y) == ascending) {
+        words[i] = y;
+        words[l] = x;
+    }
+}
+
+inline int64_t sort_capacity(int64_t n) {
+    int64_t p = kSortChunk;
+    while (p < n) p <<= 1;
+    return p;
+}
+
+void sort_words(uint64_t *words, int64_t count, hipStream_t stream) {
+    const uint32_t n = static_cast<uint32_t>(count);
+    const unsigned chunks = n / kSortChunk;
+    hipLaunchKernelGGL(sort_chunks_kernel, dim3(chunks), dim3(kSortThreads), 0, stream, words, 0u);
+    for (uint32_t k = 2 * kSortChunk; k != 0 && k <= n; k <<= 1) {
+        for (uint32_t j = k >> 1; j >= kSortChunk; j >>= 1) {
+            hipLaunchKernelGGL(sort_step_kernel, dim3(n / 2 / kBlock), dim3(kBlock), 0, stream, words, n / 2, k, j);
+        }
+        hipLaunchKernelGGL(sort_chunks_kernel, dim3(chunks), dim3(kSortThreads), 0, stream, words, k);
+    }
+}
+
+// ---- adds ---------------------------------------------------------------------------------------------------
+
+template <class T>
+struct Sum {
+    static constexpr bool kFloat = Conv<T>::kind == Kind::Float;
+    using A = std::conditional_t<kFloat, double, int64_t>;
+    static __device__ __forceinline__ A widen(T x) {
+        if constexpr (kFloat) return Conv<T>::to_f64(x);
+        else return Conv<T>::to_i64(x);
+    }
+    static __device__ __forceinline__ A add(A acc, T x) {
+        if constexpr (kFloat) return acc + Conv<T>::to_f64(x);
+        else return static_cast<int64_t>(static_cast<uint64_t>(acc) + static_cast<uint64_t>(Conv<T>::to_i64(x)));
+    }
+    static __device__ __forceinline__ T narrow(A acc) {
+        if constexpr (kFloat) return Conv<T>::from_f64(acc);
+        else return Conv<T>::from_i64(acc);
+    }
+};
+
+// scatter_add: word p = (offset of the target in out << 32) | p, for the index's positions p in row-major
+// order; stride[0] the index, [1] out (its stride along `at` multiplies the index value), [2] src.
+__global__ void __launch_bounds__(kBlock) scatter_words_kernel(uint64_t *words, int64_t capacity, const void *index, int is64,
+                                                               Dims d, int64_t n) {
+    for (int64_t p = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; p < capacity;
+         p += static_cast<int64_t>(gridDim.x) * kBlock) {
+        if (p >= n) {
+            words[p] = ~uint64_t{0};
+            continue;
+        }
+        int64_t rest = p, io = 0, oo = 0;
+        for (int k = 0; k < d.ndim; ++k) {
+            const int64_t q = rest / d.size[k];
+            const int64_t c = rest - q * d.size[k];
+            rest = q;
+            io += c * d.stride[0][k];
+            if (k != d.at) oo += c * d.stride[1][k];
+        }
+        oo += read_index(index, is64, io) * d.stride[1][d.at];
+        words[p] = (static_cast<uint64_t>(oo) << 32) | static_cast<uint64_t>(p);
+    }
+}
+
+template <class T>
+__global__ void __launch_bounds__(kBlock) scatter_runs_kernel(T *out, const T *src, const uint64_t *words, Dims d, int64_t n) {
+    using S = Sum<T>;
+    for (int64_t r = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; r < n; r += static_cast<int64_t>(gridDim.x) * kBlock) {
+        const uint64_t target = words[r] >> 32;
+        if (r > 0 && (words[r - 1] >> 32) == target) continue;  // not the first of its run
+        typename S::A acc = S::widen(out[target]);
+        for (int64_t e = r; e < n; ++e) {
+            const uint64_t w = words[e];
+            if ((w >> 32) != target) break;
+            int64_t rest = static_cast<int64_t>(w & 0xFFFFFFFFu), so = 0;
+            for (int k = 0; k < d.ndim; ++k) {
+                const int64_t q = rest / d.size[k];
+                so += (rest - q * d.size[k]) * d.stride[2][k];
+                rest = q;
+            }
+            acc = S::add(acc, src[so]);
+        }
+        out[target] = S::narrow(acc);
+    }
+}
+
+// index_add: word i = (index[i] << 32) | i.
+__global__ void __launch_bounds__(kBlock) index_words_kernel(uint64_t *words, int64_t capacity, const void *index, int is64,
+                                                             int64_t index_stride, int64_t m) {
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; i < capacity;
+         i += static_cast<int64_t>(gridDim.x) * kBlock) {
+        words[i] = i < m ? (static_cast<uint64_t>(read_index(index, is64, i * index_stride)) << 32) | static_cast<uint64_t>(i)
+                         : ~uint64_t{0};
+    }
+}
+
+// A group of `lanes` threads (a power of two up to the workgroup) takes one sorted word; the group of a
+// run's first word sums the run for the elements of the slice, which its lanes share out. `d` holds
+// the slice's dimensions (every dimension but the indexed one): stride[0] out, [1] src.
+template <class T>
+__global__ void __launch_bounds__(kBlock) index_runs_kernel(T *out, const T *src, const uint64_t *words, Dims d, int64_t m,
+                                                            int64_t slice, int64_t out_step, int64_t src_step, int lanes) {
+    using S = Sum<T>;
+    const int per_block = kBlock / lanes;
+    const int lane = threadIdx.x % lanes;
+    for (int64_t r = static_cast<int64_t>(blockIdx.x) * per_block + threadIdx.x / lanes; r < m;
+         r += static_cast<int64_t>(gridDim.x) * per_block) {
+        const uint64_t target = words[r] >> 32;
+        if (r > 0 && (words[r - 1] >> 32) == target) continue;
+        for (int64_t e = lane; e < slice; e += lanes) {
+            int64_t rest = e, oo = 0, so = 0;
+            for (int k = 0; k < d.ndim; ++k) {
+                const int64_t q = rest / d.size[k];
+                const int64_t c = rest - q * d.size[k];
+                rest = q;
+                oo += c * d.stride[0][k];
+                so += c * d.stride[1][k];
+            }
+            T *po = out + oo + static_cast<int64_t>(target) * out_step;
+            typename S::A acc = S::widen(*po);
+            for (int64_t x = r; x < m; ++x) {
+                const uint64_t w = words[x];
+                if ((w >> 32) != target) break;
+                acc = S::add(acc, src[so + static_cast<int64_t>(w & 0xFFFFFFFFu) * src_step]);
+            }
+            *po = S::narrow(acc);
+        }
+    }
+}
+
+// ---- descriptions ---------------------------------------------------------------------------------------------
+
+inline unsigned grid_of(int64_t threads) {
+    const int64_t want = (threads + kBlock - 1) / kBlock;
+    const int64_t cap = int64_t{1} << 20;
+    return static_cast<unsigned>(want < 1 ? 1 : (want < cap ? want : cap));
+}
+
+bool is_index_dtype(int dtype) { return dtype == HMR_I32 || dtype == HMR_I64; }
+
+// The dimensions of `shape_of` (sizes) with the strides of up to three operands, innermost first.
+// `dim` (counted from the outermost, as in the descriptions) becomes `at`.
+Dims dims_of(const hmr_tensor_desc &shape_of, const hmr_tensor_desc *const (&ops)[3], int dim) {
+    Dims d{};
+    d.ndim = shape_of.ndim;
+    d.at = dim < 0 ? -1 : shape_of.ndim - 1 - dim;
+    for (int k = 0; k < shape_of.ndim; ++k) {
+        const int from = shape_of.ndim - 1 - k;
+        d.size[k] = shape_of.sizes[from];
+        for (int o = 0; o < 3; ++o) d.stride[o][k] = ops[o] ? ops[o]->strides[from] : 0;
+    }
+    return d;
+}
+
+char *first_of(const hmr_tensor_desc &d) { return static_cast<char *>(d.data) + d.offset * dtype_size(d.dtype); }
+
+// The largest offset (in elements) a walk over `sizes` with `strides` reaches.
+int64_t reach_of(const hmr_tensor_desc &d) {
+    int64_t reach = 0;
+    for (int k = 0; k < d.ndim; ++k) reach += (d.sizes[k] - 1) * d.strides[k];
+    return reach;
+}
+
+hmr_status check_same_sizes(const hmr_tensor_desc &a, const hmr_tensor_desc &b, int except) {
+    bool same = a.ndim == b.ndim;
+    for (int k = 0; same && k < a.ndim; ++k) same = k == except || a.sizes[k] == b.sizes[k];
+    return same ? HMR_OK : fail(HMR_INVALID, "kernel operands have different sizes");
+}
+
+}  // namespace
+}  // namespace hmr
+
+using hmr::fail;
+using hmr::guarded;
+
+extern "C" {
+
+hmr_status hmr_index_check(hmr_context_t ctx, const hmr_tensor_desc *index, int64_t low, int64_t high, int32_t has_exempt,
+                           int64_t exempt, uint64_t *slot) {
+    return guarded([&] {
+        int64_t n = 0;
+        if (hmr_status s = hmr::check_desc(*index, n)) return s;
+        if (!hmr::is_index_dtype(index->dtype)) return fail(HMR_INVALID, "index_check: unsupported dtype");
+        if (slot == nullptr) return fail(HMR_INVALID, "index_check: no status slot");
+        const hmr_tensor_desc *const ops[3] = {index, nullptr, nullptr};
+        const hmr::Dims d = hmr::dims_of(*index, ops, -1);
+        const void *base = hmr::first_of(*index);
+        const int is64 = index->dtype == HMR_I64;
+        return hmr::launch_on(ctx, "index_check", [&](hipStream_t stream) {
+            hipLaunchKernelGGL(hmr::check_init_kernel, dim3(1), dim3(1), 0, stream, slot);
+            if (n > 0) {
+                hipLaunchKernelGGL(hmr::check_kernel, dim3(hmr::grid_of(n)), dim3(hmr::kBlock), 0, stream, base, is64, d, n, low, high,
+                                   has_exempt, exempt, reinterpret_cast<unsigned long long *>(slot));
+                hipLaunchKernelGGL(hmr::check_value_kernel, dim3(1), dim3(1), 0, stream, base, is64, d, slot);
+            }
+            return true;
+        });
+    });
+}
+
+hmr_status hmr_index_select(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_tensor_desc *src,
+                            const hmr_tensor_desc *index, int32_t dim, int32_t wrap_negative) {
+    return guarded([&] {
+        int64_t n = 0, m = 0, count = 0;
+        if (hmr_status s = hmr::check_desc(*out, n)) return s;
+        if (hmr_status s = hmr::check_desc(*src, m)) return s;
+        if (hmr_status s = hmr::check_desc(*index, count)) return s;
+        if (dim < 0 || dim >= out->ndim) return fail(HMR_INVALID, "index_select: the dimension is out of range");
+        if (hmr_status s = hmr::check_same_sizes(*out, *src, dim)) return s;
+        if (index->ndim != 1 || index->sizes[0] != out->sizes[dim]) return fail(HMR_INVALID, "index_select: the index doesn't match the output");
+        if (!hmr::is_index_dtype(index->dtype)) return fail(HMR_INVALID, "index_select: unsupported dtype");
+        if (n == 0) return HMR_OK;
+        const int is64 = index->dtype == HMR_I64;
+        const int64_t wrap = wrap_negative ? src->sizes[dim] : 0;
+        const int elem = hmr::dtype_size(out->dtype);
+        // The index walks along `dim` only.
+        hmr_tensor_desc walk = *out;
+        for (int k = 0; k < walk.ndim; ++k) walk.strides[k] = k == dim ? index->strides[0] : 0;
+        const hmr_tensor_desc *const ops[3] = {out, src, &walk};
+        const hmr::Dims d = hmr::dims_of(*out, ops, dim);
+        // Rows of whole aligned tiles: the innermost dimension isn't the indexed one and is contiguous in both.
+        const int last = out->ndim - 1;
+        const int vec = 16 / elem;
+        bool rows = last != dim && out->strides[last] == 1 && src->strides[last] == 1 && out->sizes[last] % vec == 0 &&
+                    n < (int64_t{1} << 31) && reinterpret_cast<uintptr_t>(hmr::first_of(*out)) % 16 == 0 &&
+                    reinterpret_cast<uintptr_t>(hmr::first_of(*src)) % 16 == 0;
+        for (int k = 0; rows && k < last; ++k) rows = out->strides[k] % vec == 0 && src->strides[k] % vec == 0;
+        return hmr::launch_on(ctx, "index_select", [&](hipStream_t stream) {
+            if (src->dtype != out->dtype) return false;
+            return hmr::with_word(elem, [&](auto w) {
+                using W = typename decltype(w)::type;
+                if (rows) {
+                    hmr::RowsOfTiles a{};
+                    a.out = hmr::first_of(*out);
+                    a.src = hmr::first_of(*src);
+                    a.index = hmr::first_of(*index);
+                    a.is64 = is64;
+                    a.wrap = wrap;
+                    a.index_stride = index->strides[0];
+                    a.tiles_per_row = static_cast<uint32_t>(out->sizes[last] / vec);
+                    a.tiles_div = hmr::make_fastdiv(a.tiles_per_row);
+                    a.n_tiles = n / vec;
+                    a.nouter = 0;
+                    a.at = -1;
+                    for (int k = last - 1; k >= 0; --k) {
+                        if (k == dim) a.at = a.nouter;
+                        a.div[a.nouter] = hmr::make_fastdiv(static_cast<uint32_t>(out->sizes[k]));
+                        a.stride[0][a.nouter] = out->strides[k];
+                        a.stride[1][a.nouter] = src->strides[k];
+                        ++a.nouter;
+                    }
+                    const int64_t per_block = int64_t{4} * hmr::kBlock;
+                    hipLaunchKernelGGL((hmr::select_rows_kernel<W>), dim3(static_cast<unsigned>((a.n_tiles + per_block - 1) / per_block)),
+                                       dim3(hmr::kBlock), 0, stream, a);
+                } else {
+                    hipLaunchKernelGGL((hmr::pick_kernel<W>), dim3(hmr::grid_of(n)), dim3(hmr::kBlock), 0, stream,
+                                       reinterpret_cast<W *>(hmr::first_of(*out)), reinterpret_cast<const W *>(hmr::first_of(*src)),
+                                       static_cast<const void *>(hmr::first_of(*index)), is64, d, n, wrap);
+                }
+            });
+        });
+    });
+}
+
+hmr_status hmr_gather(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_tensor_desc *src, const hmr_tensor_desc *index,
+                      int32_t dim) {
+    return guarded([&] {
+        int64_t n = 0, m = 0, count = 0;
+        if (hmr_status s = hmr::check_desc(*out, n)) return s;
+        if (hmr_status s = hmr::check_desc(*src, m)) return s;
+        if (hmr_status s = hmr::check_desc(*index, count)) return s;
+        if (dim < 0 || dim >= out->ndim) return fail(HMR_INVALID, "gather: the dimension is out of range");
+        if (hmr_status s = hmr::check_same_sizes(*out, *index, -1)) return s;
+        if (src->ndim != out->ndim) return fail(HMR_INVALID, "kernel operands have different sizes");
+        if (!hmr::is_index_dtype(index->dtype)) return fail(HMR_INVALID, "gather: unsupported dtype");
+        if (n == 0) return HMR_OK;
+        const hmr_tensor_desc *const ops[3] = {out, src, index};
+        const hmr::Dims d = hmr::dims_of(*out, ops, dim);
+        return hmr::launch_on(ctx, "gather", [&](hipStream_t stream) {
+            if (src->dtype != out->dtype) return false;
+            return hmr::with_word(hmr::dtype_size(out->dtype), [&](auto w) {
+                using W = typename decltype(w)::type;
+                hipLaunchKernelGGL((hmr::pick_kernel<W>), dim3(hmr::grid_of(n)), dim3(hmr::kBlock), 0, stream,
+                                   reinterpret_cast<W *>(hmr::first_of(*out)), reinterpret_cast<const W *>(hmr::first_of(*src)),
+                                   static_cast<const void *>(hmr::first_of(*index)), index->dtype == HMR_I64 ? 1 : 0, d, n, int64_t{0});
+            });
+        });
+    });
+}
+
+hmr_status hmr_index_add_workspace(int64_t m, int64_t size, int64_t *bytes) {
+    return guarded([&] {
+        if (m < 0 || size < 0) return fail(HMR_INVALID, "index_add_workspace: negative size");
+        if (m >= (int64_t{1} << 31) || size >= (int64_t{1} << 32)) {
+            return fail(HMR_INVALID, "index_add: more than 2^31 - 1 positions or 2^32 - 1 slices");
+        }
+        *bytes = m == 0 ? 0 : hmr::sort_capacity(m) * 8;
+        return HMR_OK;
+    });
+}
+
+hmr_status hmr_scatter_add_workspace(int64_t n, int64_t *bytes) {
+    return guarded([&] {
+        if (n < 0) return fail(HMR_INVALID, "scatter_add_workspace: negative size");
+        if (n >= (int64_t{1} << 31)) return fail(HMR_INVALID, "scatter_add: more than 2^31 - 1 positions");
+        *bytes = n == 0 ? 0 : hmr::sort_capacity(n) * 8;
+        return HMR_OK;
+    });
+}
+
+hmr_status hmr_index_add(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_tensor_desc *src, const hmr_tensor_desc *index,
+                         int32_t dim, void *workspace, int64_t workspace_bytes) {
+    return guarded([&] {
+        int64_t n = 0, total = 0, m = 0;
+        if (hmr_status s = hmr::check_desc(*out, n)) return s;
+        if (hmr_status s = hmr::check_desc(*src, total)) return s;
+        if (hmr_status s = hmr::check_desc(*index, m)) return s;
+        if (dim < 0 || dim >= out->ndim) return fail(HMR_INVALID, "index_add: the dimension is out of range");
+        if (hmr_status s = hmr::check_same_sizes(*out, *src, dim)) return s;
+        if (index->ndim > 1 || m != src->sizes[dim]) return fail(HMR_INVALID, "index_add: the index doesn't match the source");
+        if (!hmr::is_index_dtype(index->dtype)) return fail(HMR_INVALID, "index_add: unsupported dtype");
+        if (total == 0) return HMR_OK;
+        int64_t need = 0;
+        if (hmr_status s = hmr_index_add_workspace(m, out->sizes[dim], &need)) return s;
+        if (workspace == nullptr || workspace_bytes < need) return fail(HMR_INVALID, "index_add: the workspace is too small");
+        // The slice: every dimension but the indexed one.
+        hmr_tensor_desc so = *out, ss = *src;
+        int kept = 0;
+        for (int k = 0; k < out->ndim; ++k) {
+            if (k == dim) continue;
+            so.sizes[kept] = out->sizes[k];
+            so.strides[kept] = out->strides[k];
+            ss.strides[kept] = src->strides[k];
+            ++kept;
+        }
+        so.ndim = kept;
+        const hmr_tensor_desc *const ops[3] = {&so, &ss, nullptr};
+        const hmr::Dims d = hmr::dims_of(so, ops, -1);
+        const int64_t slice = total / m;
+        int lanes = 1;
+        while (lanes < hmr::kBlock && lanes < slice) lanes <<= 1;
+        const int64_t capacity = hmr::sort_capacity(m);
+        uint64_t *words = static_cast<uint64_t *>(workspace);
+        const int64_t index_stride = index->ndim == 1 ? index->strides[0] : 0;
+        return hmr::launch_on(ctx, "index_add", [&](hipStream_t stream) {
+            if (src->dtype != out->dtype) return false;
+            return hmr::with_any_type(out->dtype, [&](auto t) {
+                using T = typename decltype(t)::type;
+                hipLaunchKernelGGL(hmr::index_words_kernel, dim3(hmr::grid_of(capacity)), dim3(hmr::kBlock), 0, stream, words, capacity,
+                                   static_cast<const void *>(hmr::first_of(*index)), index->dtype == HMR_I64 ? 1 : 0, index_stride, m);
+                hmr::sort_words(words, capacity, stream);
+                const int64_t groups = (m + hmr::kBlock / lanes - 1) / (hmr::kBlock / lanes);
+                const int64_t cap = int64_t{1} << 20;
+                hipLaunchKernelGGL((hmr::index_runs_kernel<T>), dim3(static_cast<unsigned>(groups < cap ? groups : cap)), dim3(hmr::kBlock),
+                                   0, stream, reinterpret_cast<T *>(hmr::first_of(*out)), reinterpret_cast<const T *>(hmr::first_of(*src)),
+                                   static_cast<const uint64_t *>(words), d, m, slice, out->strides[dim], src->strides[dim], lanes);
+            });
+        });
+    });
+}
+
+hmr_status hmr_scatter_add(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_tensor_desc *src, const hmr_tensor_desc *index,
+                           int32_t dim, void *workspace, int64_t workspace_bytes) {
+    return guarded([&] {
+        int64_t n = 0, total = 0, count = 0;
+        if (hmr_status s = hmr::check_desc(*index, n)) return s;
+        if (hmr_status s = hmr::check_desc(*out, total)) return s;
+        if (hmr_status s = hmr::check_desc(*src, count)) return s;
+        if (dim < 0 || dim >= index->ndim) return fail(HMR_INVALID, "scatter_add: the dimension is out of range");
+        if (hmr_status s = hmr::check_same_sizes(*index, *out, dim)) return s;
+        if (hmr_status s = hmr::check_same_sizes(*index, *src, -1)) return s;
+        if (!hmr::is_index_dtype(index->dtype)) return fail(HMR_INVALID, "scatter_add: unsupported dtype");
+        if (n == 0) return HMR_OK;
+        int64_t need = 0;
+        if (hmr_status s = hmr_scatter_add_workspace(n, &need)) return s;
+        if (workspace == nullptr || workspace_bytes < need) return fail(HMR_INVALID, "scatter_add: the workspace is too small");
+        if (hmr::reach_of(*out) >= (int64_t{1} << 32) - 1) return fail(HMR_INVALID, "scatter_add: an output of more than 2^32 - 2 elements");
+        const hmr_tensor_desc *const ops[3] = {index, out, src};
+        const hmr::Dims d = hmr::dims_of(*index, ops, dim);
+        const int64_t capacity = hmr::sort_capacity(n);
+        uint64_t *words = static_cast<uint64_t *>(workspace);
+        return hmr::launch_on(ctx, "scatter_add", [&](hipStream_t stream) {
+            if (src->dtype != out->dtype) return false;
+            return hmr::with_any_type(out->dtype, [&](auto t) {
+                using T = typename decltype(t)::type;
+                hipLaunchKernelGGL(hmr::scatter_words_kernel, dim3(hmr::grid_of(capacity)), dim3(hmr::kBlock), 0, stream, words, capacity,
+                                   static_cast<const void *>(hmr::first_of(*index)), index->dtype == HMR_I64 ? 1 : 0, d, n);
+                hmr::sort_words(words, capacity, stream);
+                hipLaunchKernelGGL((hmr::scatter_runs_kernel<T>), dim3(hmr::grid_of(n)), dim3(hmr::kBlock), 0, stream,
+                                   reinterpret_cast<T *>(hmr::first_of(*out)), reinterpret_cast<const T *>(hmr::first_of(*src)),
+                                   static_cast<const uint64_t *>(words), d, n);
+            });
+        });
+    });
+}
+
+}  // extern "C"

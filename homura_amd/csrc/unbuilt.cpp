@@ -15,21 +15,10 @@ hmr_status unbuilt(const char *name) {
 
 extern "C" {
 
-HMR_UNBUILT(hmr_index_check, hmr_context_t, const hmr_tensor_desc *, int64_t, int64_t, int32_t, int64_t, uint64_t *)
-HMR_UNBUILT(hmr_index_select, hmr_context_t, const hmr_tensor_desc *, const hmr_tensor_desc *,
-            const hmr_tensor_desc *, int32_t, int32_t)
-HMR_UNBUILT(hmr_gather, hmr_context_t, const hmr_tensor_desc *, const hmr_tensor_desc *, const hmr_tensor_desc *,
-            int32_t)
 HMR_UNBUILT(hmr_index_positions, hmr_context_t, const hmr_tensor_desc *, const hmr_tensor_desc *, int64_t, int64_t,
             int32_t)
 HMR_UNBUILT(hmr_index_overwrite_workspace, int64_t, int64_t *)
 HMR_UNBUILT(hmr_index_overwrite, hmr_context_t, const hmr_tensor_desc *, const hmr_tensor_desc *,
-            const hmr_tensor_desc *, int32_t, void *, int64_t)
-HMR_UNBUILT(hmr_index_add_workspace, int64_t, int64_t, int64_t *)
-HMR_UNBUILT(hmr_index_add, hmr_context_t, const hmr_tensor_desc *, const hmr_tensor_desc *, const hmr_tensor_desc *,
-            int32_t, void *, int64_t)
-HMR_UNBUILT(hmr_scatter_add_workspace, int64_t, int64_t *)
-HMR_UNBUILT(hmr_scatter_add, hmr_context_t, const hmr_tensor_desc *, const hmr_tensor_desc *,
             const hmr_tensor_desc *, int32_t, void *, int64_t)
 HMR_UNBUILT(hmr_max_pool2d_backward_workspace, int64_t, int64_t *)
 HMR_UNBUILT(hmr_max_pool2d_backward, hmr_context_t, const hmr_tensor_desc *, const hmr_tensor_desc *,

@@ -660,6 +660,171 @@ void addr(const TensorData &out, const TensorData &v1, const TensorData &v2, con
     });
 }
 
+// ---- indexing (ref: src/backend/rocm/index.rs) -----------------------------------------------------------------
+
+namespace {
+
+// The strides of an operand walked over a shape it shares with the others of a call (but along `dim`).
+struct Walked {
+    const TensorData *data;
+    Strides strides;
+    int64_t offset;
+};
+
+// The descriptions of `operands` over `shape`, with the dimensions before `dim` and those after it merged as
+// the CPU merges them and `dim` kept in between; `at` is its position among them
+// (ref: src/backend/rocm/index.rs:62-88). `shape` has elements.
+std::vector<hmr_tensor_desc> around(const char *kernel, const std::vector<Walked> &operands, const Shape &shape, size_t dim,
+                                    int &at) {
+    auto part = [&](size_t from, size_t to) {
+        Shape sub(shape.begin() + from, shape.begin() + to);
+        std::vector<Strides> cut;
+        for (const Walked &w : operands) cut.emplace_back(w.strides.begin() + from, w.strides.begin() + to);
+        std::vector<const Strides *> ptrs;
+        for (const Strides &c : cut) ptrs.push_back(&c);
+        auto merged = merge_dims(sub, ptrs);
+        return merged ? *merged : std::vector<MergedDim>{};
+    };
+    std::vector<MergedDim> dims = part(0, dim);
+    at = static_cast<int>(dims.size());
+    MergedDim middle{shape[dim], {}};
+    for (const Walked &w : operands) middle.strides.push_back(w.strides[dim]);
+    dims.push_back(middle);
+    for (const MergedDim &d : part(dim + 1, shape.size())) dims.push_back(d);
+    std::vector<hmr_tensor_desc> out;
+    for (size_t k = 0; k < operands.size(); ++k) out.push_back(desc_with_dims(kernel, *operands[k].data, operands[k].offset, dims, k));
+    return out;
+}
+
+Walked walked(const TensorData &t) { return Walked{&t, walk_strides(t.layout), t.layout.offset}; }
+
+// The description of `data` with its own dimensions merged (ref: index.rs:36-45); false without elements.
+bool own_desc(const char *kernel, const TensorData &data, hmr_tensor_desc &d) {
+    std::vector<hmr_tensor_desc> ds;
+    if (!descs(kernel, {&data}, ds)) return false;
+    d = ds[0];
+    return true;
+}
+
+std::string out_of_bounds(int64_t value, size_t dim, int64_t size) {
+    return "index " + std::to_string(value) + " is out of bounds for dimension " + std::to_string(dim) + " with size " +
+           std::to_string(size);
+}
+
+// Inside the execution lock of `on`'s device: checks the positions of `index` against a dimension `dim` of
+// `size` on the device, reads the verdict back (a synchronization) and, if every position is in range, queues
+// `then`: the check and the kernel see the same index data (ref: index.rs:118-215).
+template <class F>
+void run_checked(const char *kernel, const TensorData &on, const TensorData &index, size_t dim, int64_t size, Bounds bounds,
+                 F then) {
+    hmr_tensor_desc check{};
+    const bool checks = bounds != Bounds::Valid && own_desc(kernel, index, check);
+    std::shared_ptr<Storage> slots = checks ? workspace(16, on.device()) : nullptr;
+    exec(on, [&](hmr_context_t ctx) {
+        if (checks) {
+            const int64_t low = bounds == Bounds::AllowNegative ? -size : 0;
+            uint64_t words[2] = {0, 0};
+            expect(hmr_index_check(ctx, &check, low, size, 0, 0, static_cast<uint64_t *>(slots->ptr())));
+            expect(hmr_copy_to_host(ctx, words, slots->ptr(), sizeof words));
+            if (words[0] != ~uint64_t{0}) throw Error(out_of_bounds(static_cast<int64_t>(words[1]), dim, size));
+        }
+        then(ctx);
+    });
+}
+
+}  // namespace
+
+void index_select(const TensorData &out, const TensorData &src, size_t dim, const TensorData &index, Bounds bounds) {
+    if (on_cpu(out)) {
+        hcb_tensor o = cpu_desc(out), s = cpu_desc(src), i = cpu_desc(index);
+        cpu_check(cpu_backend("index_select").index_select(&o, &s, static_cast<int32_t>(dim), &i, static_cast<int32_t>(bounds)));
+        return;
+    }
+    const int64_t size = src.layout.shape[dim];
+    const Shape &shape = out.layout.shape;
+    std::vector<hmr_tensor_desc> d;
+    int at = 0;
+    const bool work = out.layout.num_elements() > 0;
+    if (work) {
+        // The index walked along `dim` of out, its other strides 0.
+        Strides along(shape.size(), 0);
+        const Strides own = walk_strides(index.layout);
+        along[dim] = own.empty() ? 0 : own[0];
+        d = around("index_select", {walked(out), walked(src), Walked{&index, along, index.layout.offset}}, shape, dim, at);
+        d[1].sizes[at] = size;
+    }
+    run_checked("index_select", out, index, dim, size, bounds, [&](hmr_context_t ctx) {
+        if (!work) return;
+        hmr_tensor_desc i = d[2];  // the 1-D index: its walk along `dim`
+        i.ndim = 1;
+        i.sizes[0] = d[2].sizes[at];
+        i.strides[0] = d[2].strides[at];
+        expect(hmr_index_select(ctx, &d[0], &d[1], &i, at, bounds == Bounds::AllowNegative ? 1 : 0));
+    });
+}
+
+void gather(const TensorData &out, const TensorData &src, size_t dim, const TensorData &index) {
+    if (on_cpu(out)) {
+        hcb_tensor o = cpu_desc(out), s = cpu_desc(src), i = cpu_desc(index);
+        cpu_check(cpu_backend("gather").gather(&o, &s, static_cast<int32_t>(dim), &i));
+        return;
+    }
+    const int64_t size = src.layout.shape[dim];
+    std::vector<hmr_tensor_desc> d;
+    int at = 0;
+    const bool work = out.layout.num_elements() > 0;
+    if (work) d = around("gather", {walked(out), walked(src), walked(index)}, out.layout.shape, dim, at);
+    run_checked("gather", out, index, dim, size, Bounds::NonNegative, [&](hmr_context_t ctx) {
+        if (work) expect(hmr_gather(ctx, &d[0], &d[1], &d[2], at));
+    });
+}
+
+void index_add(const TensorData &out, size_t dim, const TensorData &index, const TensorData &src, Bounds bounds) {
+    if (on_cpu(out)) {
+        hcb_tensor o = cpu_desc(out), s = cpu_desc(src), i = cpu_desc(index);
+        cpu_check(cpu_backend("index_add").index_add(&o, static_cast<int32_t>(dim), &i, &s, static_cast<int32_t>(bounds)));
+        return;
+    }
+    if (bounds == Bounds::AllowNegative) throw Error("internal error: index_add on ROCm takes positions counted from the start");
+    const int64_t size = out.layout.shape[dim], m = index.layout.num_elements();
+    const bool work = src.layout.num_elements() > 0;
+    std::vector<hmr_tensor_desc> d;
+    hmr_tensor_desc idx{};
+    int at = 0;
+    int64_t bytes = 0;
+    if (work) {
+        d = around("index_add", {walked(out), walked(src)}, out.layout.shape, dim, at);
+        d[1].sizes[at] = m;
+        own_desc("index_add", index, idx);
+        expect(hmr_index_add_workspace(m, size, &bytes));
+    }
+    std::shared_ptr<Storage> ws = workspace(bytes, out.device());
+    run_checked("index_add", out, index, dim, size, bounds, [&](hmr_context_t ctx) {
+        if (work) expect(hmr_index_add(ctx, &d[0], &d[1], &idx, at, ws ? ws->ptr() : nullptr, bytes));
+    });
+}
+
+void scatter_add(const TensorData &out, size_t dim, const TensorData &index, const TensorData &src) {
+    if (on_cpu(out)) {
+        hcb_tensor o = cpu_desc(out), s = cpu_desc(src), i = cpu_desc(index);
+        cpu_check(cpu_backend("scatter_add").scatter_add(&o, static_cast<int32_t>(dim), &i, &s));
+        return;
+    }
+    const int64_t size = out.layout.shape[dim], n = index.layout.num_elements();
+    std::vector<hmr_tensor_desc> d;
+    int at = 0;
+    int64_t bytes = 0;
+    if (n > 0) {
+        d = around("scatter_add", {walked(index), walked(out), walked(src)}, index.layout.shape, dim, at);
+        d[1].sizes[at] = size;
+        expect(hmr_scatter_add_workspace(n, &bytes));
+    }
+    std::shared_ptr<Storage> ws = workspace(bytes, out.device());
+    run_checked("scatter_add", out, index, dim, size, Bounds::NonNegative, [&](hmr_context_t ctx) {
+        if (n > 0) expect(hmr_scatter_add(ctx, &d[1], &d[2], &d[0], at, ws ? ws->ptr() : nullptr, bytes));
+    });
+}
+
 namespace {
 // ref: src/backend/rocm/random.rs:11-19
 bool flat_desc(const char *kernel, const TensorData &out, hmr_tensor_desc &d) {

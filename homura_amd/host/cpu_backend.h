@@ -95,6 +95,20 @@ typedef struct hcb_backend {
                          double std);
     int (*random_int)(const hcb_tensor *out, uint64_t seed, uint64_t offset, uint64_t blocks,
                       int64_t low, uint64_t range, uint64_t threshold, uint64_t *accepted);
+    /* ref: src/backend/cpu/misc.rs:53-127, 213-345. `index` is I32 or I64; `bounds`: 0 the positions
+     * are valid, 1 none may be negative, 2 negative ones count from the end; the first position
+     * out of range fails the call with "index {v} is out of bounds for dimension {dim} with size
+     * {size}". index_add and scatter_add add into a contiguous `out` that shares no memory with
+     * `src`, each element summed in f64 (wrapping i64 for integers) in row-major order of the
+     * index and rounded once. */
+    int (*index_select)(const hcb_tensor *out, const hcb_tensor *src, int32_t dim,
+                        const hcb_tensor *index, int32_t bounds);
+    int (*gather)(const hcb_tensor *out, const hcb_tensor *src, int32_t dim,
+                  const hcb_tensor *index);
+    int (*index_add)(const hcb_tensor *out, int32_t dim, const hcb_tensor *index,
+                     const hcb_tensor *src, int32_t bounds);
+    int (*scatter_add)(const hcb_tensor *out, int32_t dim, const hcb_tensor *index,
+                       const hcb_tensor *src);
 } hcb_backend;
 
 #ifdef __cplusplus

@@ -296,6 +296,11 @@ class Tensor {
     // ref: src/ops/composite.rs:10-27
     Tensor softmax(int64_t dim) const;
     Tensor log_softmax(int64_t dim) const;
+    // Gathering and scattering (ref: src/tensor/index.rs:712-755, src/ops/scatter.rs:42-234).
+    Tensor index_select(int64_t dim, const Tensor &index) const;
+    Tensor gather(int64_t dim, const Tensor &index) const;
+    Tensor index_add(int64_t dim, const Tensor &index, const Tensor &source) const;
+    Tensor scatter_add(int64_t dim, const Tensor &index, const Tensor &src) const;
     // ref: src/ops/shape_ops.rs:182-263
     Tensor triu(int64_t diagonal) const;
     Tensor tril(int64_t diagonal) const;
@@ -382,6 +387,9 @@ Tensor adam_step(const Tensor &p, const Tensor &grad, std::optional<AdamState> &
 
 // ---- backend dispatch (ref: src/backend/mod.rs:298-534) ---------------------------------------------
 
+// How the positions of an index tensor are checked (ref: src/backend/mod.rs:360-373).
+enum class Bounds { Valid = 0, NonNegative = 1, AllowNegative = 2 };
+
 // The optimizers' fused steps (ref: src/backend/cpu/mod.rs:509-530).
 struct Fused {
     enum Kind { ScaledAdd = 0, Lerp = 1, Addcmul = 2, Addcdiv = 3 } kind;
@@ -408,6 +416,12 @@ void arg_reduce(const TensorData *values, const TensorData &indices, const Tenso
                 bool is_max);
 void softmax(const TensorData &out, const TensorData &src, size_t dim, bool log);
 void exclusive_cumprod(const TensorData &out, const TensorData &src, size_t dim, bool reverse);
+// Indexing (ref: src/backend/mod.rs:375-430). `index` is I32 or I64; a position out of range is an Error with
+// the CPU's message. index_add and scatter_add add into `out`, a new contiguous tensor.
+void index_select(const TensorData &out, const TensorData &src, size_t dim, const TensorData &index, Bounds bounds);
+void gather(const TensorData &out, const TensorData &src, size_t dim, const TensorData &index);
+void index_add(const TensorData &out, size_t dim, const TensorData &index, const TensorData &src, Bounds bounds);
+void scatter_add(const TensorData &out, size_t dim, const TensorData &index, const TensorData &src);
 void fused(const Fused &op, const TensorData &out, const TensorData &a, const TensorData &b, const TensorData *c);
 void triangle(const TensorData &out, const TensorData &src, int64_t diagonal, bool upper);
 void flip(const TensorData &out, const TensorData &src, const std::vector<bool> &mask);

@@ -255,6 +255,10 @@ PYBIND11_MODULE(_host, m) {
     T.def("any_dim", [](const Tensor &t, const py::handle &d, bool k) { return t.any_dim(to_dims(d), k); });
     T.def("softmax", &Tensor::softmax);
     T.def("log_softmax", &Tensor::log_softmax);
+    T.def("index_select", &Tensor::index_select);
+    T.def("gather", &Tensor::gather);
+    T.def("index_add", &Tensor::index_add);
+    T.def("scatter_add", &Tensor::scatter_add);
     T.def("triu", &Tensor::triu, py::arg("diagonal") = 0);
     T.def("tril", &Tensor::tril, py::arg("diagonal") = 0);
     T.def("flip", &Tensor::flip);

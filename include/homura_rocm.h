@@ -16,8 +16,8 @@
  *    previous device back before it returns;
  *  - enumerations travel as int32_t.
  *
- * Entry points of the reference that belong to other kernel families (gemm, indexing, pooling,
- * convolution windows ...) are declared in homura_rocm_unbuilt.h and exported as
+ * Entry points of the reference that belong to other kernel families (gemm, pooling, convolution
+ * windows, the rest of indexing ...) are declared in homura_rocm_unbuilt.h and exported as
  * stubs that fail with HMR_INVALID, so that the reference crate still links.
  */
 #ifndef HOMURA_ROCM_H
@@ -325,6 +325,49 @@ hmr_status hmr_random_normal(hmr_context_t ctx, const hmr_tensor_desc *out, uint
 hmr_status hmr_random_int(hmr_context_t ctx, const hmr_tensor_desc *out, uint64_t seed,
                           uint64_t offset, uint64_t blocks, int64_t low, uint64_t range,
                           uint64_t threshold, void *workspace);
+
+/* ---- indexing -------------------------------------------------- ref: csrc/homura_rocm.h:353-404 */
+/* Index tensors are I32 or I64; positions are checked before they are used (hmr_index_check, in the
+ * same critical section of the caller), so the other entry points take them as valid.
+ *
+ * ref :358-363  The first element of `index`, in row-major order of its logical positions, that is
+ * outside [low, high) and, if has_exempt, not equal to `exempt`: queues writing its position to
+ * slot[0] (UINT64_MAX if there is none) and its value to slot[1]. `slot` is two words of device
+ * memory. */
+hmr_status hmr_index_check(hmr_context_t ctx, const hmr_tensor_desc *index, int64_t low,
+                           int64_t high, int32_t has_exempt, int64_t exempt, uint64_t *slot);
+
+/* ref :365-370  cpu::index_select (src/backend/cpu/misc.rs:74-105): out (src's sizes but the 1-D
+ * `index`'s length along dim) gets the slices of src along dim at the positions of `index`,
+ * negative ones counted from the end if wrap_negative. */
+hmr_status hmr_index_select(hmr_context_t ctx, const hmr_tensor_desc *out,
+                            const hmr_tensor_desc *src, const hmr_tensor_desc *index, int32_t dim,
+                            int32_t wrap_negative);
+
+/* ref :372-375  cpu::gather (misc.rs:313-345): out (index's sizes) gets src at each index position
+ * with the coordinate along dim replaced by the index element. */
+hmr_status hmr_gather(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_tensor_desc *src,
+                      const hmr_tensor_desc *index, int32_t dim);
+
+/* ref :392-399  cpu::index_add (misc.rs:254-290): slice i of src along dim is added into slice
+ * index[i] of out, each element of out summed in f64 (floats; integers wrap in i64, bools are
+ * or-ed) in the order of i and rounded once. The workspace has hmr_index_add_workspace bytes for
+ * `m` positions (`size`, out's size along dim, bounds them). Here: m < 2^31, size < 2^32. */
+hmr_status hmr_index_add_workspace(int64_t m, int64_t size, int64_t *bytes);
+hmr_status hmr_index_add(hmr_context_t ctx, const hmr_tensor_desc *out,
+                         const hmr_tensor_desc *src, const hmr_tensor_desc *index, int32_t dim,
+                         void *workspace, int64_t workspace_bytes);
+
+/* ref :401-408  cpu::scatter_add (misc.rs:292-311): src at each index position is added into out
+ * at that position with the coordinate along dim replaced by the index element, summed as
+ * hmr_index_add sums, in row-major order of the index positions. `index`, `out` and `src` are
+ * described over the index's sizes (out with its own size along dim). The workspace has
+ * hmr_scatter_add_workspace bytes for the index's number of elements. Here: fewer than 2^31
+ * positions, an output of fewer than 2^32 - 1 elements. */
+hmr_status hmr_scatter_add_workspace(int64_t n, int64_t *bytes);
+hmr_status hmr_scatter_add(hmr_context_t ctx, const hmr_tensor_desc *out,
+                           const hmr_tensor_desc *src, const hmr_tensor_desc *index, int32_t dim,
+                           void *workspace, int64_t workspace_bytes);
 
 /* ---- build facts and ABI self-description ------------------- ref: csrc/homura_rocm.h:589-610 */
 /* ';'-separated offload architectures compiled in ("gfx950"). */

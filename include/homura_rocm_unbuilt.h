@@ -18,14 +18,7 @@
 extern "C" {
 #endif
 
-/* ref :361-426 (indexing) */
-hmr_status hmr_index_check(hmr_context_t ctx, const hmr_tensor_desc *index, int64_t low,
-                           int64_t high, int32_t has_exempt, int64_t exempt, uint64_t *slot);
-hmr_status hmr_index_select(hmr_context_t ctx, const hmr_tensor_desc *out,
-                            const hmr_tensor_desc *src, const hmr_tensor_desc *index, int32_t dim,
-                            int32_t wrap_negative);
-hmr_status hmr_gather(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_tensor_desc *src,
-                      const hmr_tensor_desc *index, int32_t dim);
+/* ref :376-390, 412-426 (the rest of indexing: positions of advanced indexing, overwriting puts, masks) */
 hmr_status hmr_index_positions(hmr_context_t ctx, const hmr_tensor_desc *out,
                                const hmr_tensor_desc *coord, int64_t size, int64_t stride,
                                int32_t first);
@@ -33,14 +26,6 @@ hmr_status hmr_index_overwrite_workspace(int64_t size, int64_t *bytes);
 hmr_status hmr_index_overwrite(hmr_context_t ctx, const hmr_tensor_desc *out,
                                const hmr_tensor_desc *src, const hmr_tensor_desc *positions,
                                int32_t dim, void *workspace, int64_t workspace_bytes);
-hmr_status hmr_index_add_workspace(int64_t m, int64_t size, int64_t *bytes);
-hmr_status hmr_index_add(hmr_context_t ctx, const hmr_tensor_desc *out,
-                         const hmr_tensor_desc *src, const hmr_tensor_desc *index, int32_t dim,
-                         void *workspace, int64_t workspace_bytes);
-hmr_status hmr_scatter_add_workspace(int64_t n, int64_t *bytes);
-hmr_status hmr_scatter_add(hmr_context_t ctx, const hmr_tensor_desc *out,
-                           const hmr_tensor_desc *src, const hmr_tensor_desc *index, int32_t dim,
-                           void *workspace, int64_t workspace_bytes);
 hmr_status hmr_max_pool2d_backward_workspace(int64_t n, int64_t *bytes);
 hmr_status hmr_max_pool2d_backward(hmr_context_t ctx, const hmr_tensor_desc *out,
                                    const hmr_tensor_desc *grad, const hmr_tensor_desc *indices,

@@ -1208,6 +1208,150 @@ uint64_t random_int(const hcb_tensor &out, uint64_t seed, uint64_t offset, uint6
     return accepted;
 }
 
+// ---- indexing (ref: src/backend/cpu/misc.rs:53-127, 213-345; src/backend/mod.rs:360-378) ----------
+//
+// `bounds`: 0 the positions are valid, 1 none may be negative, 2 negative ones count from the end.
+// The first position out of range, in row-major order of the index, is the error.
+std::vector<int64_t> positions(const hcb_tensor &index, int dim, int64_t size, int bounds) {
+    std::vector<int64_t> out;
+    const int64_t n = num_elements(index);
+    out.reserve(static_cast<size_t>(n));
+    const int64_t low = bounds == 2 ? -size : 0;
+    auto take = [&](int64_t v) {
+        if (bounds != 0 && !(v >= low && v < size)) {
+            panic("index " + std::to_string(v) + " is out of bounds for dimension " + std::to_string(dim) + " with size " +
+                  std::to_string(size));
+        }
+        out.push_back(v < 0 ? v + size : v);
+    };
+    const int64_t *const st[1] = {index.strides};
+    Plan<1> plan(index.ndim, index.shape, st);
+    const int64_t b[1] = {index.offset};
+    if (index.dtype == HMR_I64) {
+        const int64_t *p = base<int64_t>(index);
+        plan.for_each(b, [&](const int64_t(&o)[1]) { take(p[o[0]]); });
+    } else if (index.dtype == HMR_I32) {
+        const int32_t *p = base<int32_t>(index);
+        plan.for_each(b, [&](const int64_t(&o)[1]) { take(p[o[0]]); });
+    } else {
+        panic("an index tensor is I32 or I64");
+    }
+    return out;
+}
+
+// out = the slices of src along dim picked by the 1-D index (ref: misc.rs:74-105).
+void index_select(const hcb_tensor &out, const hcb_tensor &src, int dim, const hcb_tensor &index, int bounds) {
+    const std::vector<int64_t> picked = positions(index, dim, src.shape[dim], bounds);
+    if (num_elements(out) == 0) return;
+    std::vector<int64_t> shape, so, ss;
+    for (int d = 0; d < out.ndim; ++d) {
+        if (d == dim) continue;
+        shape.push_back(out.shape[d]);
+        so.push_back(out.strides[d]);
+        ss.push_back(src.strides[d]);
+    }
+    dispatch_all(src.dtype, [&](auto t) {
+        using T = typename decltype(t)::type;
+        T *po = base<T>(out);
+        const T *ps = base<T>(src);
+        const int64_t *const st[2] = {so.data(), ss.data()};
+        Plan<2> slice(static_cast<int>(shape.size()), shape.data(), st);
+        for (size_t j = 0; j < picked.size(); ++j) {
+            const int64_t b[2] = {out.offset + static_cast<int64_t>(j) * out.strides[dim], src.offset + picked[j] * src.strides[dim]};
+            slice.for_each(b, [&](const int64_t(&o)[2]) { po[o[0]] = ps[o[1]]; });
+        }
+    });
+}
+
+// out[p] = src[.., index[p], ..] for every position p of the contiguous out, which has the index's shape
+// (ref: misc.rs:313-345).
+void gather(const hcb_tensor &out, const hcb_tensor &src, int dim, const hcb_tensor &index) {
+    const std::vector<int64_t> picked = positions(index, dim, src.shape[dim], 1);
+    if (picked.empty()) return;
+    std::vector<int64_t> walk(src.strides, src.strides + src.ndim);
+    walk[dim] = 0;  // the index value replaces the position along dim
+    dispatch_all(src.dtype, [&](auto t) {
+        using T = typename decltype(t)::type;
+        T *po = base<T>(out);
+        const T *ps = base<T>(src);
+        const int64_t *const st[2] = {out.strides, walk.data()};
+        Plan<2> plan(out.ndim, out.shape, st);
+        const int64_t b[2] = {out.offset, src.offset};
+        size_t k = 0;
+        plan.for_each(b, [&](const int64_t(&o)[2]) { po[o[0]] = ps[o[1] + picked[k++] * src.strides[dim]]; });
+    });
+}
+
+// out[o] += src[s] for the pairs `pairs` reports in order: each element of the contiguous out is
+// accumulated in f64 (floats) or wrapping i64 (integers; an or for bools) and rounded once at the end
+// (ref: misc.rs:213-252).
+template <class Pairs>
+void add_at(const hcb_tensor &out, const hcb_tensor &src, Pairs pairs) {
+    const int64_t n = num_elements(out);
+    if (n == 0) return;
+    if (out.dtype != src.dtype) panic("add_at: the operands have different dtypes");
+    dispatch_all(out.dtype, [&](auto t) {
+        using T = typename decltype(t)::type;
+        T *elements = base<T>(out) + out.offset;
+        const T *ps = base<T>(src);
+        if (is_float(out.dtype)) {
+            std::vector<double> acc(static_cast<size_t>(n));
+            for (int64_t i = 0; i < n; ++i) acc[i] = El<T>::to_f64(elements[i]);
+            pairs([&](int64_t o, int64_t s) { acc[o] += El<T>::to_f64(ps[s]); });
+            for (int64_t i = 0; i < n; ++i) elements[i] = El<T>::from_f64(acc[i]);
+        } else {
+            std::vector<int64_t> acc(static_cast<size_t>(n));
+            for (int64_t i = 0; i < n; ++i) acc[i] = El<T>::to_i64(elements[i]);
+            pairs([&](int64_t o, int64_t s) { acc[o] = wadd<int64_t>(acc[o], El<T>::to_i64(ps[s])); });
+            for (int64_t i = 0; i < n; ++i) elements[i] = El<T>::from_i64(acc[i]);
+        }
+    });
+}
+
+std::vector<int64_t> contiguous_strides_of(const int64_t *shape, int ndim) {
+    std::vector<int64_t> st(static_cast<size_t>(ndim), 1);
+    for (int d = ndim - 2; d >= 0; --d) st[d] = st[d + 1] * shape[d + 1];
+    return st;
+}
+
+// Adds slice i of src along dim into slice index[i] of the contiguous out (ref: misc.rs:254-290).
+void index_add(const hcb_tensor &out, int dim, const hcb_tensor &index, const hcb_tensor &src, int bounds) {
+    const std::vector<int64_t> picked = positions(index, dim, out.shape[dim], bounds);
+    if (num_elements(src) == 0) return;
+    const std::vector<int64_t> out_strides = contiguous_strides_of(out.shape, out.ndim);
+    std::vector<int64_t> shape, so, ss;
+    for (int d = 0; d < src.ndim; ++d) {
+        if (d == dim) continue;
+        shape.push_back(src.shape[d]);
+        so.push_back(out_strides[d]);
+        ss.push_back(src.strides[d]);
+    }
+    const int64_t *const st[2] = {so.data(), ss.data()};
+    Plan<2> plan(static_cast<int>(shape.size()), shape.data(), st);
+    add_at(out, src, [&](auto f) {
+        for (size_t i = 0; i < picked.size(); ++i) {
+            const int64_t b[2] = {picked[i] * out_strides[dim], src.offset + static_cast<int64_t>(i) * src.strides[dim]};
+            plan.for_each(b, [&](const int64_t(&o)[2]) { f(o[0], o[1]); });
+        }
+    });
+}
+
+// out[.., index[p], ..] += src[p] for every position p of the index (ref: misc.rs:292-311).
+void scatter_add(const hcb_tensor &out, int dim, const hcb_tensor &index, const hcb_tensor &src) {
+    const std::vector<int64_t> picked = positions(index, dim, out.shape[dim], 1);
+    if (picked.empty()) return;
+    const std::vector<int64_t> out_strides = contiguous_strides_of(out.shape, out.ndim);
+    std::vector<int64_t> walk = out_strides;
+    walk[dim] = 0;
+    const int64_t *const st[2] = {walk.data(), src.strides};
+    Plan<2> plan(index.ndim, index.shape, st);
+    add_at(out, src, [&](auto f) {
+        size_t k = 0;
+        const int64_t b[2] = {0, src.offset};
+        plan.for_each(b, [&](const int64_t(&o)[2]) { f(o[0] + picked[k++] * out_strides[dim], o[1]); });
+    });
+}
+
 template <class F>
 int guarded(F f) {
     try {
@@ -1296,6 +1440,18 @@ int orc_random_int(const hcb_tensor *out, uint64_t seed, uint64_t offset, uint64
                    uint64_t threshold, uint64_t *accepted) {
     return orc::guarded([&] { *accepted = orc::random_int(*out, seed, offset, blocks, low, range, threshold); });
 }
+int orc_index_select(const hcb_tensor *out, const hcb_tensor *src, int32_t dim, const hcb_tensor *index, int32_t bounds) {
+    return orc::guarded([&] { orc::index_select(*out, *src, dim, *index, bounds); });
+}
+int orc_gather(const hcb_tensor *out, const hcb_tensor *src, int32_t dim, const hcb_tensor *index) {
+    return orc::guarded([&] { orc::gather(*out, *src, dim, *index); });
+}
+int orc_index_add(const hcb_tensor *out, int32_t dim, const hcb_tensor *index, const hcb_tensor *src, int32_t bounds) {
+    return orc::guarded([&] { orc::index_add(*out, dim, *index, *src, bounds); });
+}
+int orc_scatter_add(const hcb_tensor *out, int32_t dim, const hcb_tensor *index, const hcb_tensor *src) {
+    return orc::guarded([&] { orc::scatter_add(*out, dim, *index, *src); });
+}
 int orc_addr(const hcb_tensor *out, const hcb_tensor *v1, const hcb_tensor *v2, const hcb_tensor *input, hcb_scalar alpha,
              hcb_scalar beta) {
     return orc::guarded([&] { orc::addr(*out, *v1, *v2, *input, alpha, beta); });
@@ -1317,6 +1473,7 @@ const hcb_backend *orc_backend(void) {
         orc_where_constant,  orc_reduce,     orc_var,   orc_arg_reduce,     orc_softmax,
         orc_fused,           orc_triangle,   orc_flip,  orc_addr,           orc_exclusive_cumprod,
         orc_random_uniform,  orc_random_normal,         orc_random_int,
+        orc_index_select,    orc_gather,     orc_index_add,         orc_scatter_add,
     };
     return &table;
 }

@@ -106,6 +106,6 @@ def test_out_of_scope_entry_points_fail_loudly():
     lib = ctypes.CDLL(capi.LIB_PATH)
     lib.hmr_last_error.restype = ctypes.c_char_p
     lib.hmr_gemm_path_name.restype = ctypes.c_char_p
-    rc = lib.hmr_gather(None, None, None, None, 0, 0)
+    rc = lib.hmr_max_pool2d_check(None, None, None, None, None, None, None, None)
     assert rc == 2
-    assert lib.hmr_last_error() == b"hmr_gather: not built in this library"
+    assert lib.hmr_last_error() == b"hmr_max_pool2d_check: not built in this library"
