@@ -299,6 +299,25 @@ def per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP
     add(None, "softmax backward bf16 [16384,4096] (7 kernels: 2 casts, mul, sum, sub, mul, cast)", 2 * N * (3 + 3 + 6 + 2 + 4 + 6 + 3),
         lambda: h.grad_softmax(gy, y, -1, False), 10)
     del y, gy
+    # Indexing: an embedding lookup and its gradient (vocabulary 32 768 x 4096 bf16, 16 384 tokens), gather and
+    # scatter_add along the rows of the f32 matrix. Bytes: rows moved + indices (+ the target's read and write).
+    vocab, hidden, tokens = 32768, 4096, 16384
+    table = x.reshape([16384, 4096]).narrow(0, 0, 1).expand([2, 16384, 4096]).reshape([vocab, hidden]).contiguous()
+    ids = tensor((words(0x5EED0600, tokens) % np.uint64(vocab)).astype(np.int64), DT.I64, [tokens], GPU)
+    add(None, "index_select bf16 [32768,4096] rows by 16384 ids (embedding lookup)", 4 * tokens * hidden + 8 * tokens,
+        lambda: table.index_select(0, ids), 10)
+    grads = x.reshape([16384, 4096])
+    zeros = h.full([vocab, hidden], 0.0, DT.BF16, GPU)
+    add(None, "index_add bf16 16384 rows into [32768,4096] (embedding gradient: copy, check, sort, ordered sums)",
+        4 * vocab * hidden + 2 * tokens * hidden + 4 * tokens * hidden, lambda: zeros.index_add(0, ids, grads), 5)
+    del table, grads, zeros
+    mat = residual.reshape([16384, 4096])
+    cols = tensor((words(0x5EED0601, 16384 * 512) % np.uint64(4096)).astype(np.int32), DT.I32, [16384, 512], GPU)
+    add(None, "gather f32 [16384,4096] dim 1 by i32 [16384,512]", (4 + 4 + 4) * 16384 * 512, lambda: mat.gather(1, cols), 10)
+    vals = mat.narrow(1, 0, 512)
+    add(None, "scatter_add f32 [16384,512] into [16384,4096] dim 1 (copy, check, sort, ordered sums)",
+        8 * N + (4 + 4 + 8) * 16384 * 512, lambda: mat.scatter_add(1, cols, vals), 3)
+    del mat, cols, vals
     shape = [8, 2048, 4096]
     add(None, "rand f32 [8,2048,4096] (Philox on the device, write only)", 4 * N, lambda: h.rand(shape, DT.F32, GPU))
     add(None, "rand bf16 [8,2048,4096]", 2 * N, lambda: h.rand(shape, DT.BF16, GPU))

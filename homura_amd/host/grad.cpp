@@ -85,6 +85,15 @@ Tensor extremum(const Tensor &g, const Tensor &x, const Tensor &result) {
     return Tensor::full(x.shape(), Scalar::of_int(0), g.dtype(), g.device()).masked_fill(mask, share);
 }
 
+// ref: reduce.rs:353-380
+Tensor extremum_dim(const Tensor &g_in, const Tensor &indices_in, const Shape &self_shape, int64_t dim, bool keepdim) {
+    const size_t d = normalize_dim(dim, self_shape.size());
+    Tensor g = unreduce(g_in, self_shape, {static_cast<int64_t>(d)}, keepdim);
+    Tensor indices = unreduce(indices_in, self_shape, {static_cast<int64_t>(d)}, keepdim);
+    Tensor zeros = Tensor::full(self_shape, Scalar::of_int(0), g.dtype(), g.device());
+    return zeros.scatter_add(static_cast<int64_t>(d), indices, g);
+}
+
 // ref: reduce.rs:382-424
 Tensor var_std(const Tensor &g_in, const Tensor &x, const std::optional<Tensor> &std_result, const std::vector<int64_t> &dims_in,
                int64_t correction_in, bool keepdim) {

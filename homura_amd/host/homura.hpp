@@ -332,13 +332,15 @@ Tensor exclusive_cumprod(const Tensor &x, size_t dim, bool reverse);
 // The input gradients of the reductions and of softmax for an output gradient `g`, composed from the ops above as
 // the reference's backward nodes compose them outside grad mode (ref: src/autograd/formulas/reduce.rs:160-470,
 // softmax.rs:43-84). `dims` empty = all elements (the full reductions); otherwise the reduced dimensions and
-// whether they were kept. Not here: the gradient of max_dim / min_dim, which scatters through indices.
+// whether they were kept.
 namespace grad {
 Tensor sum(const Tensor &g, const Shape &self_shape, const std::vector<int64_t> &dims, bool keepdim);
 Tensor mean(const Tensor &g, const Shape &self_shape, const std::vector<int64_t> &dims, bool keepdim);
 Tensor sum_to_size(const Tensor &g, const Shape &self_shape);
 Tensor prod(const Tensor &g, const Tensor &x, const Tensor &result, std::optional<int64_t> dim, bool keepdim);
 Tensor extremum(const Tensor &g, const Tensor &x, const Tensor &result);  // x.max() / x.min()
+// x.max_dim / x.min_dim (values): g scattered to the positions the saved indices name.
+Tensor extremum_dim(const Tensor &g, const Tensor &indices, const Shape &self_shape, int64_t dim, bool keepdim);
 Tensor var_std(const Tensor &g, const Tensor &x, const std::optional<Tensor> &std_result, const std::vector<int64_t> &dims,
                int64_t correction, bool keepdim);
 Tensor softmax(const Tensor &g, const Tensor &y, int64_t dim, bool log);

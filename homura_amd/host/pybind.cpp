@@ -119,6 +119,7 @@ PYBIND11_MODULE(_host, m) {
     m.def("grad_sum_to_size", &grad::sum_to_size);
     m.def("grad_prod", &grad::prod);
     m.def("grad_extremum", &grad::extremum);
+    m.def("grad_extremum_dim", &grad::extremum_dim);
     m.def("grad_var_std", &grad::var_std);
     m.def("grad_softmax", &grad::softmax);
     m.def("manual_seed", &manual_seed);

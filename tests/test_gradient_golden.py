@@ -7,8 +7,8 @@ broadcast gradients (expand, sum_to_size), mean / var / std scaling, the tie and
 y * (g - sum(g * y)) with f32 intermediates for the halves. For an input with zeros the gradient of prod is g times
 exclusive_cumprod(x) * exclusive_cumprod(x, reverse): the `special.prod*` cases compare exactly (ref:
 tests/autograd_golden.rs:236-246) and fix that kernel's multiplication order, accumulation type and rounding point.
-On the CPU this pins the oracle's exclusive_cumprod; on the GPU everything runs on the HIP kernels.
-Not covered: max_dim / min_dim, whose gradient scatters through the indices (the indexing family is not built).
+The gradient of max_dim / min_dim scatters g through the saved indices (scatter_add). On the CPU this pins the oracle's
+exclusive_cumprod; on the GPU everything runs on the HIP kernels.
 """
 import os
 
@@ -38,6 +38,8 @@ OPS = {
     "prod_dim_keep": lambda x, g: h.grad_prod(g, x, x.prod_dim(0, True), 0, True),
     "max": lambda x, g: h.grad_extremum(g, x, x.max()),
     "min": lambda x, g: h.grad_extremum(g, x, x.min()),
+    "max_dim": lambda x, g: h.grad_extremum_dim(g, x.max_dim(1, False)[1], x.shape, 1, False),
+    "min_dim_keep": lambda x, g: h.grad_extremum_dim(g, x.min_dim(0, True)[1], x.shape, 0, True),
     "var": lambda x, g: h.grad_var_std(g, x, None, [], 1, False),
     "var_c2": lambda x, g: h.grad_var_std(g, x, None, [], 2, False),
     "var_c4": lambda x, g: h.grad_var_std(g, x, None, [], 4, False),
@@ -59,7 +61,6 @@ ALIASES = {"prod_zero": "prod", "prod_two_zeros": "prod", "prod_overflow": "prod
            "prod_dim_order_f32": "prod_dim", "prod_dim_order_f16": "prod_dim", "prod_dim_order_bf16": "prod_dim",
            "max_ties": "max", "softmax_masked": "softmax_last", "softmax_opmath_f16": "softmax_last",
            "log_softmax_masked": "log_softmax_last", "log_softmax_opmath_bf16": "log_softmax_last"}
-SCATTERED = {"max_dim", "min_dim_keep"}
 FAMILIES = ("sum", "mean", "prod", "max", "min", "var", "std", "softmax", "log_softmax")
 
 
@@ -68,7 +69,7 @@ def on_the_path(case):
     return any(op == f or op.startswith(f + "_") for f in FAMILIES)
 
 
-CASES = sorted(c for c in GOLDEN if on_the_path(c) and c.partition(".")[2] not in SCATTERED)
+CASES = sorted(c for c in GOLDEN if on_the_path(c))
 
 
 def check(case, device):
@@ -94,9 +95,7 @@ def check(case, device):
 
 
 def test_every_reduction_and_softmax_gradient_of_the_fixture_is_handled():
-    assert len(CASES) == 65
-    skipped = sorted(c for c in GOLDEN if on_the_path(c) and c.partition(".")[2] in SCATTERED)
-    assert len(skipped) == 6  # max_dim in four dtypes and categories, min_dim_keep in two
+    assert len(CASES) == 71
     # The cases that reach the cumulative products: every dtype's accumulation order, overflowing partial products,
     # one zero and two.
     with_zeros = {c for c in CASES if "prod" in c and (GOLDEN[c]["x"][0] == 0).any()}
