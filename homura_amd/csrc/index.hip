@@ -327,6 +327,40 @@ __global__ void __launch_bounds__(kBlock) index_runs_kernel(T *out, const T *src
     }
 }
 
+// The same when a slice is one contiguous run of whole aligned 16-byte tiles in both operands (the rows of
+// an embedding table): a lane owns a tile and keeps its V sums in registers.
+template <class T>
+__global__ void __launch_bounds__(kBlock) index_runs_tiles_kernel(T *out, const T *src, const uint64_t *words, int64_t m,
+                                                                  int64_t tiles, int64_t out_step, int64_t src_step, int lanes) {
+    using S = Sum<T>;
+    constexpr int V = 16 / static_cast<int>(sizeof(T));
+    const int per_block = kBlock / lanes;
+    const int lane = threadIdx.x % lanes;
+    for (int64_t r = static_cast<int64_t>(blockIdx.x) * per_block + threadIdx.x / lanes; r < m;
+         r += static_cast<int64_t>(gridDim.x) * per_block) {
+        const uint64_t target = words[r] >> 32;
+        if (r > 0 && (words[r - 1] >> 32) == target) continue;
+        for (int64_t t = lane; t < tiles; t += lanes) {
+            T *po = out + static_cast<int64_t>(target) * out_step + t * V;
+            T v[V];
+            typename S::A acc[V];
+            load_tile<T, V, false>(reinterpret_cast<const char *>(po), v);
+#pragma unroll
+            for (int i = 0; i < V; ++i) acc[i] = S::widen(v[i]);
+            for (int64_t x = r; x < m; ++x) {
+                const uint64_t w = words[x];
+                if ((w >> 32) != target) break;
+                load_tile<T, V, false>(reinterpret_cast<const char *>(src + static_cast<int64_t>(w & 0xFFFFFFFFu) * src_step + t * V), v);
+#pragma unroll
+                for (int i = 0; i < V; ++i) acc[i] = S::add(acc[i], v[i]);
+            }
+#pragma unroll
+            for (int i = 0; i < V; ++i) v[i] = S::narrow(acc[i]);
+            store_tile<T, V, false>(reinterpret_cast<char *>(po), v);
+        }
+    }
+}
+
 // ---- descriptions ---------------------------------------------------------------------------------------------
 
 inline unsigned grid_of(int64_t threads) {
@@ -548,11 +582,27 @@ hmr_status hmr_index_add(hmr_context_t ctx, const hmr_tensor_desc *out, const hm
                 hipLaunchKernelGGL(hmr::index_words_kernel, dim3(hmr::grid_of(capacity)), dim3(hmr::kBlock), 0, stream, words, capacity,
                                    static_cast<const void *>(hmr::first_of(*index)), index->dtype == HMR_I64 ? 1 : 0, index_stride, m);
                 hmr::sort_words(words, capacity, stream);
-                const int64_t groups = (m + hmr::kBlock / lanes - 1) / (hmr::kBlock / lanes);
                 const int64_t cap = int64_t{1} << 20;
-                hipLaunchKernelGGL((hmr::index_runs_kernel<T>), dim3(static_cast<unsigned>(groups < cap ? groups : cap)), dim3(hmr::kBlock),
-                                   0, stream, reinterpret_cast<T *>(hmr::first_of(*out)), reinterpret_cast<const T *>(hmr::first_of(*src)),
-                                   static_cast<const uint64_t *>(words), d, m, slice, out->strides[dim], src->strides[dim], lanes);
+                constexpr int V = 16 / static_cast<int>(sizeof(T));
+                T *po = reinterpret_cast<T *>(hmr::first_of(*out));
+                const T *ps = reinterpret_cast<const T *>(hmr::first_of(*src));
+                // One contiguous run of whole aligned tiles per slice, in both operands?
+                const bool tiles = (d.ndim == 0 || (d.ndim == 1 && d.stride[0][0] == 1 && d.stride[1][0] == 1)) && slice % V == 0 &&
+                                   reinterpret_cast<uintptr_t>(po) % 16 == 0 && reinterpret_cast<uintptr_t>(ps) % 16 == 0 &&
+                                   out->strides[dim] % V == 0 && src->strides[dim] % V == 0;
+                if (tiles) {
+                    int group = 1;
+                    while (group < hmr::kBlock && group < slice / V) group <<= 1;
+                    const int64_t groups = (m + hmr::kBlock / group - 1) / (hmr::kBlock / group);
+                    hipLaunchKernelGGL((hmr::index_runs_tiles_kernel<T>), dim3(static_cast<unsigned>(groups < cap ? groups : cap)),
+                                       dim3(hmr::kBlock), 0, stream, po, ps, static_cast<const uint64_t *>(words), m, slice / V,
+                                       out->strides[dim], src->strides[dim], group);
+                } else {
+                    const int64_t groups = (m + hmr::kBlock / lanes - 1) / (hmr::kBlock / lanes);
+                    hipLaunchKernelGGL((hmr::index_runs_kernel<T>), dim3(static_cast<unsigned>(groups < cap ? groups : cap)),
+                                       dim3(hmr::kBlock), 0, stream, po, ps, static_cast<const uint64_t *>(words), d, m, slice,
+                                       out->strides[dim], src->strides[dim], lanes);
+                }
             });
         });
     });
