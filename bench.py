@@ -310,6 +310,12 @@ def per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP
     zeros = h.full([vocab, hidden], 0.0, DT.BF16, GPU)
     add(None, "index_add bf16 16384 rows into [32768,4096] (embedding gradient: copy, check, sort, ordered sums)",
         4 * vocab * hidden + 2 * tokens * hidden + 4 * tokens * hidden, lambda: zeros.index_add(0, ids, grads), 5)
+    # Advanced indexing: the same rows through index tensors (check, positions, rows of tiles) and written back
+    # (copy of the table, winners per row, the winners' rows).
+    add(None, "x[ids] bf16 [32768,4096] by 16384 ids (advanced indexing: check, positions, rows)",
+        4 * tokens * hidden + 24 * tokens, lambda: table.index_tensors([ids]), 10)
+    add(None, "index_put bf16 16384 rows into [32768,4096] (copy, check, positions, last write wins)",
+        4 * vocab * hidden + 4 * tokens * hidden + 24 * tokens, lambda: table.index_put_tensors([ids], grads, False), 5)
     del table, grads, zeros
     mat = residual.reshape([16384, 4096])
     cols = tensor((words(0x5EED0601, 16384 * 512) % np.uint64(4096)).astype(np.int32), DT.I32, [16384, 512], GPU)
@@ -317,7 +323,15 @@ def per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP
     vals = mat.narrow(1, 0, 512)
     add(None, "scatter_add f32 [16384,512] into [16384,4096] dim 1 (copy, check, sort, ordered sums)",
         8 * N + (4 + 4 + 8) * 16384 * 512, lambda: mat.scatter_add(1, cols, vals), 3)
-    del mat, cols, vals
+    # A boolean mask over the f32 matrix, 60 % true: the coordinates (count, scan, write; two i64 per true element),
+    # then the selected elements (positions, one element per pick).
+    keep = tensor((words(0x5EED0602, N) % np.uint64(5) < 3).astype(np.uint8), DT.Bool, [16384, 4096], GPU)
+    kept = int((words(0x5EED0602, N) % np.uint64(5) < 3).sum())
+    add(None, "mask coordinates bool [16384,4096], 60 % true (count, scan, coordinates)", 2 * N + 16 * kept,
+        lambda: keep.mask_coordinates(), 5)
+    add(None, "x[mask] f32 [16384,4096], 60 % true (coordinates, check, positions, picks)", 2 * N + 88 * kept,
+        lambda: mat.index_tensors([keep]), 3)
+    del mat, cols, vals, keep
     shape = [8, 2048, 4096]
     add(None, "rand f32 [8,2048,4096] (Philox on the device, write only)", 4 * N, lambda: h.rand(shape, DT.F32, GPU))
     add(None, "rand bf16 [8,2048,4096]", 2 * N, lambda: h.rand(shape, DT.BF16, GPU))

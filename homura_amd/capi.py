@@ -97,6 +97,12 @@ PROTOTYPES = {
     "hmr_index_add": (c_int32, [CTX, DESC_P, DESC_P, DESC_P, c_int32, c_void_p, c_int64]),
     "hmr_scatter_add_workspace": (c_int32, [c_int64, POINTER(c_int64)]),
     "hmr_scatter_add": (c_int32, [CTX, DESC_P, DESC_P, DESC_P, c_int32, c_void_p, c_int64]),
+    "hmr_index_positions": (c_int32, [CTX, DESC_P, DESC_P, c_int64, c_int64, c_int32]),
+    "hmr_index_overwrite_workspace": (c_int32, [c_int64, POINTER(c_int64)]),
+    "hmr_index_overwrite": (c_int32, [CTX, DESC_P, DESC_P, DESC_P, c_int32, c_void_p, c_int64]),
+    "hmr_mask_workspace": (c_int32, [c_int64, POINTER(c_int64), POINTER(c_int64)]),
+    "hmr_mask_count": (c_int32, [CTX, DESC_P, c_void_p, c_int64]),
+    "hmr_mask_coordinates": (c_int32, [CTX, DESC_P, c_void_p, c_int64, DESC_P]),
     "hmr_exclusive_cumprod": (c_int32, [CTX, DESC_P, DESC_P, c_int64, c_int64, c_int64, c_int32]),
     "hmr_built_archs": (c_char_p, []),
     "hmr_abi_check": (None, [POINTER(hmr_abi_info)]),
@@ -116,8 +122,7 @@ PROTOTYPES = {
 
 # Exported stubs of other kernel families (include/homura_rocm_unbuilt.h); bound without prototypes.
 UNBUILT = [
-    "hmr_index_positions", "hmr_index_overwrite_workspace", "hmr_index_overwrite", "hmr_max_pool2d_backward_workspace",
-    "hmr_max_pool2d_backward", "hmr_mask_workspace", "hmr_mask_count", "hmr_mask_coordinates", "hmr_max_pool2d",
+    "hmr_max_pool2d_backward_workspace", "hmr_max_pool2d_backward", "hmr_max_pool2d",
     "hmr_max_pool2d_check", "hmr_max_pool2d_gather_backward", "hmr_adaptive_avg_pool2d",
     "hmr_adaptive_avg_pool2d_backward", "hmr_unfold_backward", "hmr_gemm_fold", "hmr_gemm_select",
     "hmr_gemm_path_name", "hmr_gemm_workspace", "hmr_gemm", "hmr_test_index_value", "hmr_test_wide_pool",

@@ -15,17 +15,9 @@ hmr_status unbuilt(const char *name) {
 
 extern "C" {
 
-HMR_UNBUILT(hmr_index_positions, hmr_context_t, const hmr_tensor_desc *, const hmr_tensor_desc *, int64_t, int64_t,
-            int32_t)
-HMR_UNBUILT(hmr_index_overwrite_workspace, int64_t, int64_t *)
-HMR_UNBUILT(hmr_index_overwrite, hmr_context_t, const hmr_tensor_desc *, const hmr_tensor_desc *,
-            const hmr_tensor_desc *, int32_t, void *, int64_t)
 HMR_UNBUILT(hmr_max_pool2d_backward_workspace, int64_t, int64_t *)
 HMR_UNBUILT(hmr_max_pool2d_backward, hmr_context_t, const hmr_tensor_desc *, const hmr_tensor_desc *,
             const hmr_tensor_desc *, void *, int64_t)
-HMR_UNBUILT(hmr_mask_workspace, int64_t, int64_t *, int64_t *)
-HMR_UNBUILT(hmr_mask_count, hmr_context_t, const hmr_tensor_desc *, void *, int64_t)
-HMR_UNBUILT(hmr_mask_coordinates, hmr_context_t, const hmr_tensor_desc *, void *, int64_t, const hmr_tensor_desc *)
 HMR_UNBUILT(hmr_max_pool2d, hmr_context_t, const hmr_tensor_desc *, const hmr_tensor_desc *,
             const hmr_tensor_desc *, const int64_t *)
 HMR_UNBUILT(hmr_max_pool2d_check, hmr_context_t, const hmr_tensor_desc *, int64_t, int64_t, const int64_t *,

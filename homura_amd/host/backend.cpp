@@ -706,10 +706,15 @@ bool own_desc(const char *kernel, const TensorData &data, hmr_tensor_desc &d) {
     return true;
 }
 
+}  // namespace
+
+// ref: src/backend/mod.rs:375-378
 std::string out_of_bounds(int64_t value, size_t dim, int64_t size) {
     return "index " + std::to_string(value) + " is out of bounds for dimension " + std::to_string(dim) + " with size " +
            std::to_string(size);
 }
+
+namespace {
 
 // Inside the execution lock of `on`'s device: checks the positions of `index` against a dimension `dim` of
 // `size` on the device, reads the verdict back (a synchronization) and, if every position is in range, queues
@@ -823,6 +828,140 @@ void scatter_add(const TensorData &out, size_t dim, const TensorData &index, con
     run_checked("scatter_add", out, index, dim, size, Bounds::NonNegative, [&](hmr_context_t ctx) {
         if (n > 0) expect(hmr_scatter_add(ctx, &d[1], &d[2], &d[0], at, ws ? ws->ptr() : nullptr, bytes));
     });
+}
+
+// ref: src/backend/rocm/index.rs:299-336
+void index_overwrite(const TensorData &out, size_t dim, const TensorData &index, const TensorData &src) {
+    if (on_cpu(out)) {
+        hcb_tensor o = cpu_desc(out), s = cpu_desc(src), i = cpu_desc(index);
+        cpu_check(cpu_backend("index_overwrite").index_overwrite(&o, static_cast<int32_t>(dim), &i, &s));
+        return;
+    }
+    if (src.layout.num_elements() == 0) return;
+    if (!index.layout.is_contiguous() || index.dtype != DType::I64) {
+        throw Error("internal error: index_overwrite with positions that aren't contiguous I64");
+    }
+    const int64_t size = out.layout.shape[dim], m = index.layout.num_elements();
+    int at = 0;
+    std::vector<hmr_tensor_desc> d = around("index_overwrite", {walked(src), walked(out)}, src.layout.shape, dim, at);
+    d[1].sizes[at] = size;
+    // One dimension even for a single position, as the kernel expects.
+    const std::vector<MergedDim> flat{MergedDim{m, {1}}};
+    const hmr_tensor_desc positions = desc_with_dims("index_overwrite", index, index.layout.offset, flat, 0);
+    int64_t bytes = 0;
+    expect(hmr_index_overwrite_workspace(size, &bytes));
+    std::shared_ptr<Storage> ws = workspace(bytes, out.device());
+    exec(out, [&](hmr_context_t ctx) {
+        expect(hmr_index_overwrite(ctx, &d[1], &d[0], &positions, at, ws ? ws->ptr() : nullptr, bytes));
+    });
+}
+
+// ref: src/backend/rocm/index.rs:560-612: the count, its read-back and the coordinates in one critical section,
+// so that both passes see the same mask.
+std::vector<TensorData> mask_coordinates(const TensorData &mask) {
+    const size_t nd = mask.layout.shape.size();
+    const int64_t n = mask.layout.num_elements();
+    const Device device = mask.device();
+    auto rows_of = [&](const Tensor &coords) {
+        std::vector<TensorData> rows;
+        for (size_t d = 0; d < nd; ++d) rows.push_back(coords.select(0, static_cast<int64_t>(d)).data());
+        return rows;
+    };
+    if (on_cpu(mask)) {
+        hcb_tensor m = cpu_desc(mask);
+        int64_t count = 0;
+        cpu_check(cpu_backend("mask_coordinates").mask_coordinates(&m, nullptr, &count));
+        Tensor coords = Tensor::uninit_on(Shape{static_cast<int64_t>(nd), count}, DType::I64, device);
+        hcb_tensor o = cpu_desc(coords.data());
+        cpu_check(cpu_backend("mask_coordinates").mask_coordinates(&m, &o, &count));
+        return rows_of(coords);
+    }
+    if (n == 0) return rows_of(Tensor::uninit_on(Shape{static_cast<int64_t>(nd), 0}, DType::I64, device));
+    // Every dimension of the mask, unmerged: the kernel reports coordinates along each.
+    std::vector<MergedDim> dims;
+    const Strides strides = walk_strides(mask.layout);
+    for (size_t d = 0; d < nd; ++d) dims.push_back(MergedDim{mask.layout.shape[d], {strides[d]}});
+    const hmr_tensor_desc desc = desc_with_dims("mask_coordinates", mask, mask.layout.offset, dims, 0);
+    int64_t bytes = 0, total_word = 0;
+    expect(hmr_mask_workspace(n, &bytes, &total_word));
+    std::shared_ptr<Storage> ws = workspace(bytes, device);
+    Tensor coords;
+    exec(mask, [&](hmr_context_t ctx) {
+        expect(hmr_mask_count(ctx, &desc, ws->ptr(), bytes));
+        uint64_t count = 0;
+        expect(hmr_copy_to_host(ctx, &count, static_cast<const uint64_t *>(ws->ptr()) + total_word, sizeof count));
+        coords = Tensor::uninit_on(Shape{static_cast<int64_t>(nd), static_cast<int64_t>(count)}, DType::I64, device);
+        const TensorData &out = coords.data();
+        const std::vector<MergedDim> rows{MergedDim{static_cast<int64_t>(nd), {static_cast<int64_t>(count)}},
+                                          MergedDim{static_cast<int64_t>(count), {1}}};
+        const hmr_tensor_desc o = desc_with_dims("mask_coordinates", out, out.layout.offset, rows, 0);
+        expect(hmr_mask_coordinates(ctx, &desc, ws->ptr(), bytes, &o));
+    });
+    return rows_of(coords);
+}
+
+// ref: src/backend/rocm/index.rs:614-668: the indices are checked and, without a position out of range, `out`
+// written, in one critical section.
+std::optional<std::pair<size_t, int64_t>> index_positions(const TensorData *out, const std::vector<TensorData> &coords,
+                                                          const std::vector<int64_t> &sizes) {
+    const TensorData *first = out ? out : (coords.empty() ? nullptr : &coords[0]);
+    if (first == nullptr) return std::nullopt;
+    if (on_cpu(*first)) {
+        std::vector<hcb_tensor> descs_;
+        for (const TensorData &c : coords) descs_.push_back(cpu_desc(c));
+        std::vector<const hcb_tensor *> ptrs;
+        for (const hcb_tensor &c : descs_) ptrs.push_back(&c);
+        hcb_tensor o{};
+        if (out) o = cpu_desc(*out);
+        int32_t bad = -1;
+        int64_t value = 0;
+        cpu_check(cpu_backend("index_positions")
+                      .index_positions(out ? &o : nullptr, static_cast<int32_t>(coords.size()), ptrs.data(), sizes.data(), &bad, &value));
+        if (bad >= 0) return std::make_pair(static_cast<size_t>(bad), value);
+        return std::nullopt;
+    }
+    // The checks: one per index with elements.
+    std::vector<hmr_tensor_desc> checks(coords.size());
+    std::vector<bool> has(coords.size(), false);
+    for (size_t k = 0; k < coords.size(); ++k) has[k] = own_desc("index_positions", coords[k], checks[k]);
+    // The positions: one pass per index over the broadcast shape.
+    Strides strides(sizes.size(), 1);
+    for (size_t k = sizes.size(); k-- > 1;) strides[k - 1] = strides[k] * sizes[k];
+    struct Pass {
+        hmr_tensor_desc out, coord;
+    };
+    std::vector<Pass> passes;
+    std::vector<TensorData> expanded;
+    if (out && out->layout.num_elements() > 0) {
+        for (const TensorData &c : coords) expanded.push_back(c.expand_to(out->layout.shape));
+        for (const TensorData &c : expanded) {
+            std::vector<hmr_tensor_desc> d;
+            if (!descs("index_positions", {out, &c}, d)) throw Error("internal error: index_positions over an empty shape");
+            passes.push_back(Pass{d[0], d[1]});
+        }
+    }
+    std::shared_ptr<Storage> slots = workspace(static_cast<int64_t>(16 * (coords.empty() ? 1 : coords.size())), first->device());
+    std::optional<std::pair<size_t, int64_t>> bad;
+    exec(*first, [&](hmr_context_t ctx) {
+        std::vector<uint64_t> words(2 * coords.size(), 0);
+        bool any = false;
+        for (size_t k = 0; k < coords.size(); ++k) {
+            if (!has[k]) continue;
+            any = true;
+            expect(hmr_index_check(ctx, &checks[k], -sizes[k], sizes[k], 0, 0, static_cast<uint64_t *>(slots->ptr()) + 2 * k));
+        }
+        if (any) expect(hmr_copy_to_host(ctx, words.data(), slots->ptr(), words.size() * sizeof(uint64_t)));
+        for (size_t k = 0; k < coords.size(); ++k) {
+            if (has[k] && words[2 * k] != ~uint64_t{0}) {
+                bad = std::make_pair(k, static_cast<int64_t>(words[2 * k + 1]));
+                return;
+            }
+        }
+        for (size_t k = 0; k < passes.size(); ++k) {
+            expect(hmr_index_positions(ctx, &passes[k].out, &passes[k].coord, sizes[k], strides[k], k == 0 ? 1 : 0));
+        }
+    });
+    return bad;
 }
 
 namespace {

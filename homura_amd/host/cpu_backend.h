@@ -109,6 +109,21 @@ typedef struct hcb_backend {
                      const hcb_tensor *src, int32_t bounds);
     int (*scatter_add)(const hcb_tensor *out, int32_t dim, const hcb_tensor *index,
                        const hcb_tensor *src);
+    /* ref: src/backend/cpu/misc.rs:104-126. Slice i of src along dim is copied to slice index[i]
+     * (valid positions) of out, in order: the last of repeated positions wins. */
+    int (*index_overwrite)(const hcb_tensor *out, int32_t dim, const hcb_tensor *index,
+                           const hcb_tensor *src);
+    /* ref: src/backend/cpu/misc.rs:128-148. *count = the number of true elements of the BOOL mask;
+     * with `out` (I64, contiguous, the mask's rank x that number) coordinate d of the k-th true
+     * element in row-major order goes to out[d][k]. */
+    int (*mask_coordinates)(const hcb_tensor *mask, const hcb_tensor *out, int64_t *count);
+    /* ref: src/backend/cpu/misc.rs:150-203. The `n` indices (I32 or I64) are checked in order to lie
+     * in -sizes[k]..sizes[k]: the first value out of range is left in (*bad_index, *bad_value) and
+     * nothing is written; otherwise *bad_index = -1 and, with `out` (I64, contiguous, the shape the
+     * indices broadcast to), every element gets its row-major position in the subspace of
+     * `sizes`, negative coordinates counting from the end. */
+    int (*index_positions)(const hcb_tensor *out, int32_t n, const hcb_tensor *const *coords,
+                           const int64_t *sizes, int32_t *bad_index, int64_t *bad_value);
 } hcb_backend;
 
 #ifdef __cplusplus

@@ -301,6 +301,10 @@ class Tensor {
     Tensor gather(int64_t dim, const Tensor &index) const;
     Tensor index_add(int64_t dim, const Tensor &index, const Tensor &source) const;
     Tensor scatter_add(int64_t dim, const Tensor &index, const Tensor &src) const;
+    // Advanced indexing with one optional index tensor (I32 / I64 positions or a bool mask) per leading
+    // dimension; nullopt keeps the dimension (ref: src/ops/advanced_index.rs:403-440).
+    Tensor index_tensors(const std::vector<std::optional<Tensor>> &indices) const;
+    Tensor index_put_tensors(const std::vector<std::optional<Tensor>> &indices, const Tensor &values, bool accumulate) const;
     // ref: src/ops/shape_ops.rs:182-263
     Tensor triu(int64_t diagonal) const;
     Tensor tril(int64_t diagonal) const;
@@ -420,10 +424,23 @@ void softmax(const TensorData &out, const TensorData &src, size_t dim, bool log)
 void exclusive_cumprod(const TensorData &out, const TensorData &src, size_t dim, bool reverse);
 // Indexing (ref: src/backend/mod.rs:375-430). `index` is I32 or I64; a position out of range is an Error with
 // the CPU's message. index_add and scatter_add add into `out`, a new contiguous tensor.
+std::string out_of_bounds(int64_t value, size_t dim, int64_t size);
 void index_select(const TensorData &out, const TensorData &src, size_t dim, const TensorData &index, Bounds bounds);
 void gather(const TensorData &out, const TensorData &src, size_t dim, const TensorData &index);
 void index_add(const TensorData &out, size_t dim, const TensorData &index, const TensorData &src, Bounds bounds);
 void scatter_add(const TensorData &out, size_t dim, const TensorData &index, const TensorData &src);
+// Copies slice i of src along dim into slice index[i] of out, the last of repeated positions winning; `index`
+// holds valid positions (contiguous I64) (ref: src/backend/mod.rs:391-396).
+void index_overwrite(const TensorData &out, size_t dim, const TensorData &index, const TensorData &src);
+// The coordinates of the true elements of a bool tensor in row-major order: one I64 vector per dimension, on
+// the mask's device (ref: src/backend/mod.rs:398-403).
+std::vector<TensorData> mask_coordinates(const TensorData &mask);
+// The positions of advanced indexing: checks each index, in order, to lie in -size..size for its size in `sizes`
+// and returns the first value out of range as (k, value). Without one, and with `out` (I64, the shape the indices
+// broadcast to), writes the row-major position in the subspace of `sizes` of every element, negative coordinates
+// counting from the end (ref: src/backend/mod.rs:425-447).
+std::optional<std::pair<size_t, int64_t>> index_positions(const TensorData *out, const std::vector<TensorData> &coords,
+                                                          const std::vector<int64_t> &sizes);
 void fused(const Fused &op, const TensorData &out, const TensorData &a, const TensorData &b, const TensorData *c);
 void triangle(const TensorData &out, const TensorData &src, int64_t diagonal, bool upper);
 void flip(const TensorData &out, const TensorData &src, const std::vector<bool> &mask);

@@ -1,5 +1,7 @@
 // Gathering and scattering through index tensors: the checks of the front end
 // (ref: src/tensor/index.rs:712-755, src/ops/scatter.rs:13-234).
+#include <algorithm>
+
 #include "homura.hpp"
 
 namespace homura {
@@ -128,6 +130,268 @@ Tensor Tensor::scatter_add(int64_t dim, const Tensor &index, const Tensor &src) 
     TensorData out = copy_of(*this);
     backend::scatter_add(at_least_1d(out), d, idx, source);
     return Tensor(out);
+}
+
+// ---- advanced indexing (ref: src/ops/advanced_index.rs) ---------------------------------------------------------
+//
+// Masks are expanded into one coordinate vector per dimension they cover, the indices are broadcast together, and
+// when the indexed dimensions are not adjacent they move to the front of the result. Reading and writing both
+// fold the target, its dimensions in that order, into [before, indexed, after] and pick or write slices along
+// the middle dimension at the linear positions the indices give in the indexed subspace.
+
+namespace {
+
+// One index after masks are expanded: positions on the device of the target.
+struct Coords {
+    Shape shape;
+    TensorData values;
+};
+
+// nullopt if the shapes don't broadcast together (ref: advanced_index.rs:79-97).
+std::optional<Shape> broadcast_of(const Shape &a, const Shape &b) {
+    const size_t n = std::max(a.size(), b.size());
+    auto dim = [&](const Shape &s, size_t i) { return i < n - s.size() ? int64_t{1} : s[i - (n - s.size())]; };
+    Shape out;
+    for (size_t i = 0; i < n; ++i) {
+        const int64_t x = dim(a, i), y = dim(b, i);
+        if (x == y || y == 1) out.push_back(x);
+        else if (x == 1) out.push_back(y);
+        else return std::nullopt;
+    }
+    return out;
+}
+
+// Indices on the CPU are copied to the target's device first (ref: advanced_index.rs:46-57).
+TensorData on_device(const TensorData &data, Device device) {
+    if (data.device() == Device::cpu() && device != Device::cpu()) return Tensor(data).to(device).data();
+    return data;
+}
+
+int64_t product(const Shape &s, size_t from, size_t to) {
+    int64_t n = 1;
+    for (size_t k = from; k < to; ++k) n *= s[k];
+    return n;
+}
+
+class AdvancedIndex {
+  public:
+    // ref: advanced_index.rs:99-231 (ATen's make_info): index dtypes, then devices, mask shapes, the number of
+    // indices, broadcasting, and indices into empty dimensions.
+    AdvancedIndex(const TensorData &target, const std::vector<std::optional<Tensor>> &indices) {
+        const Device device = target.device();
+        const Shape &shape = target.layout.shape;
+        const size_t nd = shape.size();
+        for (const auto &t : indices) {
+            if (!t) continue;
+            const DType d = t->dtype();
+            if (d != DType::I64 && d != DType::I32 && d != DType::Bool) {
+                throw Error(std::string("tensors used as indices must be i64, i32 or bool tensors, got ") + name_of(d) +
+                            (d == DType::U8 ? "; use a bool tensor for a mask" : ""));
+            }
+        }
+        for (const auto &t : indices) {
+            if (t && t->device() != Device::cpu() && t->device() != device) {
+                throw Error("indices should be either on cpu or on the same device as the indexed tensor (" + device.str() + ")");
+            }
+        }
+        size_t count = 0;
+        for (const auto &t : indices) count += t && t->dtype() == DType::Bool ? t->num_dims() : 1;
+        if (count > nd) {
+            throw Error("too many indices for tensor of dimension " + std::to_string(nd) + " (got " + std::to_string(count) + ")");
+        }
+        std::vector<std::optional<Coords>> slots;
+        for (const auto &t : indices) {
+            if (!t) {
+                slots.push_back(std::nullopt);
+                continue;
+            }
+            const TensorData &data = t->data();
+            if (t->dtype() != DType::Bool) {
+                slots.push_back(Coords{data.layout.shape, on_device(data, device)});
+                continue;
+            }
+            const Shape &mask_shape = data.layout.shape;
+            if (mask_shape.empty()) throw Error("indexing with a zero-dimensional bool tensor is not supported");
+            const size_t start = slots.size();
+            for (size_t j = 0; j < mask_shape.size(); ++j) {
+                if (mask_shape[j] != shape[start + j]) {
+                    throw Error("The shape of the mask " + shape_str(mask_shape) + " at index " + std::to_string(j) +
+                                " does not match the shape of the indexed tensor " + shape_str(shape) + " at index " +
+                                std::to_string(start + j));
+                }
+            }
+            for (const TensorData &values : backend::mask_coordinates(data)) {
+                slots.push_back(Coords{values.layout.shape, on_device(values, device)});
+            }
+        }
+        while (!slots.empty() && !slots.back()) slots.pop_back();
+        std::vector<size_t> defined;
+        for (size_t k = 0; k < slots.size(); ++k) {
+            if (slots[k]) defined.push_back(k);
+        }
+        if (defined.empty()) throw Error("advanced indexing needs at least one index tensor");
+        bool adjacent = true;
+        for (size_t k = defined.front(); k <= defined.back(); ++k) adjacent = adjacent && slots[k].has_value();
+        slots.resize(nd);
+        if (adjacent) {
+            for (size_t k = 0; k < nd; ++k) perm_.push_back(k);
+            first_ = defined.front();
+        } else {
+            perm_ = defined;
+            for (size_t k = 0; k < nd; ++k) {
+                if (!slots[k]) perm_.push_back(k);
+            }
+            first_ = 0;
+        }
+        for (size_t k : perm_) shape_.push_back(shape[k]);
+        for (size_t k : perm_) {
+            if (slots[k]) coords_.push_back(std::move(*slots[k]));
+        }
+        std::optional<Shape> together = Shape{};
+        for (const Coords &c : coords_) {
+            together = broadcast_of(*together, c.shape);
+            if (!together) {
+                std::string shapes;
+                for (const Coords &each : coords_) shapes += (shapes.empty() ? "" : ", ") + shape_str(each.shape);
+                throw Error("shape mismatch: indexing tensors could not be broadcast together with shapes " + shapes);
+            }
+        }
+        broadcast_ = *together;
+        const size_t n = coords_.size();
+        bool empty_dimension = false;
+        for (size_t k = first_; k < first_ + n; ++k) empty_dimension = empty_dimension || shape_[k] == 0;
+        if (product(broadcast_, 0, broadcast_.size()) > 0 && empty_dimension) {
+            throw Error("index is out of bounds for dimension with size 0");
+        }
+        out_shape_.assign(shape_.begin(), shape_.begin() + first_);
+        out_shape_.insert(out_shape_.end(), broadcast_.begin(), broadcast_.end());
+        out_shape_.insert(out_shape_.end(), shape_.begin() + first_ + n, shape_.end());
+    }
+
+    const Shape &out_shape() const { return out_shape_; }
+
+    // The indexing result: a new contiguous tensor of out_shape (ref: advanced_index.rs:293-316).
+    Tensor gather(const TensorData &target) const {
+        Tensor out = Tensor::uninit_on(out_shape_, target.dtype, target.device());
+        if (out.num_elements() == 0) {
+            check_and_place(nullptr);
+            return out;
+        }
+        const TensorData where = positions(target.device());
+        const int64_t count = where.layout.num_elements();
+        const Tensor src = Tensor(permuted(target)).reshape(folded());
+        TensorData shaped = out.data();
+        shaped.layout = Layout::contiguous(Shape{before(), count, after()});
+        backend::index_select(shaped, src.data(), 1, where, Bounds::Valid);
+        return out;
+    }
+
+    // ref: advanced_index.rs:318-343
+    void check_values(const TensorData &target, const TensorData &values) const {
+        if (values.dtype != target.dtype) {
+            throw Error(std::string("Index put requires the source and destination dtypes match, got ") + name_of(target.dtype) +
+                        " for the destination and " + name_of(values.dtype) + " for the source.");
+        }
+        if (values.device() != target.device()) {
+            throw Error("Expected all tensors to be on the same device, but found at least two devices, " + target.device().str() +
+                        " and " + values.device().str() + "!");
+        }
+        const Shape &v = values.layout.shape, &o = out_shape_;
+        bool fits = v.size() <= o.size();
+        for (size_t k = 0; fits && k < v.size(); ++k) {
+            const int64_t b = o[o.size() - v.size() + k];
+            fits = v[k] == b || v[k] == 1;
+        }
+        if (!fits) {
+            throw Error("shape mismatch: value tensor of shape " + shape_str(v) + " cannot be broadcast to indexing result of shape " +
+                        shape_str(o));
+        }
+    }
+
+    // A copy of the target with `values` written at the indexed positions: added with `accumulate`, otherwise
+    // copied, the last of repeated positions winning. The work happens on a contiguous copy with the dimensions
+    // in the order of perm, which the result sees in the original order (ref: advanced_index.rs:345-387).
+    Tensor scatter(const TensorData &target, const TensorData &values, bool accumulate) const {
+        const TensorData work = copy_of(Tensor(permuted(target)));
+        if (product(out_shape_, 0, out_shape_.size()) == 0) {
+            check_and_place(nullptr);
+        } else {
+            const TensorData where = positions(target.device());
+            const int64_t count = where.layout.num_elements();
+            TensorData shaped = work;
+            shaped.layout = Layout::contiguous(folded());
+            const Tensor src = Tensor(values.expand_to(out_shape_)).reshape(Shape{before(), count, after()});
+            if (accumulate) backend::index_add(shaped, 1, where, src.data(), Bounds::Valid);
+            else backend::index_overwrite(shaped, 1, where, src.data());
+        }
+        const size_t nd = perm_.size();
+        TensorData result = work;
+        result.layout.shape.assign(nd, 0);
+        result.layout.strides.assign(nd, 0);
+        for (size_t k = 0; k < nd; ++k) {
+            result.layout.shape[perm_[k]] = work.layout.shape[k];
+            result.layout.strides[perm_[k]] = work.layout.strides[k];
+        }
+        return Tensor(result);
+    }
+
+  private:
+    int64_t before() const { return product(shape_, 0, first_); }
+    int64_t indexed() const { return product(shape_, first_, first_ + coords_.size()); }
+    int64_t after() const { return product(shape_, first_ + coords_.size(), shape_.size()); }
+    Shape folded() const { return Shape{before(), indexed(), after()}; }
+
+    // Checks every position to be in range along its dimension, the indices in order; with `out`, then writes
+    // the linear position in the indexed subspace of every element of the broadcast shape (ref: :241-262).
+    void check_and_place(const TensorData *out) const {
+        std::vector<TensorData> values;
+        for (const Coords &c : coords_) values.push_back(c.values);
+        const std::vector<int64_t> sizes(shape_.begin() + first_, shape_.begin() + first_ + coords_.size());
+        if (auto bad = backend::index_positions(out, values, sizes)) {
+            throw Error(backend::out_of_bounds(bad->second, bad->first, sizes[bad->first]));
+        }
+    }
+
+    // ref: advanced_index.rs:264-279
+    TensorData positions(Device device) const {
+        const int64_t n = product(broadcast_, 0, broadcast_.size());
+        const TensorData out = Tensor::uninit_on(Shape{n}, DType::I64, device).data();
+        TensorData shaped = out;
+        shaped.layout = Layout::contiguous(broadcast_);
+        check_and_place(&shaped);
+        return out;
+    }
+
+    TensorData permuted(const TensorData &data) const {
+        TensorData d = data;
+        d.layout.shape.clear();
+        d.layout.strides.clear();
+        for (size_t k : perm_) {
+            d.layout.shape.push_back(data.layout.shape[k]);
+            d.layout.strides.push_back(data.layout.strides[k]);
+        }
+        return d;
+    }
+
+    std::vector<size_t> perm_;  // the target's dimensions in working order: the indexed ones first unless adjacent
+    Shape shape_;               // the target's shape in that order
+    size_t first_ = 0;          // the first indexed dimension in shape_
+    std::vector<Coords> coords_;
+    Shape broadcast_;           // what the indices broadcast to
+    Shape out_shape_;           // before + broadcast + after
+};
+
+}  // namespace
+
+Tensor Tensor::index_tensors(const std::vector<std::optional<Tensor>> &indices) const {
+    const AdvancedIndex info(d_, indices);
+    return info.gather(d_);
+}
+
+Tensor Tensor::index_put_tensors(const std::vector<std::optional<Tensor>> &indices, const Tensor &values, bool accumulate) const {
+    const AdvancedIndex info(d_, indices);
+    info.check_values(d_, values.data());
+    return info.scatter(d_, values.data(), accumulate);
 }
 
 }  // namespace homura

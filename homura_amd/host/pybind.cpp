@@ -260,6 +260,13 @@ PYBIND11_MODULE(_host, m) {
     T.def("gather", &Tensor::gather);
     T.def("index_add", &Tensor::index_add);
     T.def("scatter_add", &Tensor::scatter_add);
+    T.def("index_tensors", &Tensor::index_tensors);
+    T.def("index_put_tensors", &Tensor::index_put_tensors);
+    T.def("mask_coordinates", [](const Tensor &mask) {
+        std::vector<Tensor> out;
+        for (const homura::TensorData &d : homura::backend::mask_coordinates(mask.data())) out.emplace_back(d);
+        return out;
+    });
     T.def("triu", &Tensor::triu, py::arg("diagonal") = 0);
     T.def("tril", &Tensor::tril, py::arg("diagonal") = 0);
     T.def("flip", &Tensor::flip);

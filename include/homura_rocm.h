@@ -369,6 +369,33 @@ hmr_status hmr_scatter_add(hmr_context_t ctx, const hmr_tensor_desc *out,
                            const hmr_tensor_desc *src, const hmr_tensor_desc *index, int32_t dim,
                            void *workspace, int64_t workspace_bytes);
 
+/* ref :376-380  One indexed dimension of advanced indexing (cpu::index_positions, misc.rs:150-203):
+ * out (I64) = (if first) or += coord * stride, the coordinate (I32 or I64) wrapped by `size` when
+ * negative; `coord` has out's sizes (broadcast through zero strides). */
+hmr_status hmr_index_positions(hmr_context_t ctx, const hmr_tensor_desc *out,
+                               const hmr_tensor_desc *coord, int64_t size, int64_t stride,
+                               int32_t first);
+
+/* ref :382-389  cpu::index_overwrite (misc.rs:104-126): slice i of src along dim is copied to slice
+ * positions[i] of out, the last of repeated positions winning. `positions` is a 1-D tensor of valid
+ * positions; out and src are described as for hmr_index_add. The workspace has
+ * hmr_index_overwrite_workspace bytes for out's size along dim (a word per position). */
+hmr_status hmr_index_overwrite_workspace(int64_t size, int64_t *bytes);
+hmr_status hmr_index_overwrite(hmr_context_t ctx, const hmr_tensor_desc *out,
+                               const hmr_tensor_desc *src, const hmr_tensor_desc *positions,
+                               int32_t dim, void *workspace, int64_t workspace_bytes);
+
+/* ref :416-426  cpu::mask_coordinates (misc.rs:128-148) in two calls: hmr_mask_count queues counting
+ * the true elements of the BOOL mask (any layout), whose number it leaves at word total_word of the
+ * workspace (hmr_mask_workspace bytes for the mask's number of elements: a 64-bit word per tile of
+ * 4096 elements and one for the total); hmr_mask_coordinates then writes coordinate d of the k-th
+ * true element, in row-major order, to out[d][k] (I64, the mask's rank x the number). */
+hmr_status hmr_mask_workspace(int64_t n, int64_t *bytes, int64_t *total_word);
+hmr_status hmr_mask_count(hmr_context_t ctx, const hmr_tensor_desc *mask, void *workspace,
+                          int64_t workspace_bytes);
+hmr_status hmr_mask_coordinates(hmr_context_t ctx, const hmr_tensor_desc *mask, void *workspace,
+                                int64_t workspace_bytes, const hmr_tensor_desc *out);
+
 /* ---- build facts and ABI self-description ------------------- ref: csrc/homura_rocm.h:589-610 */
 /* ';'-separated offload architectures compiled in ("gfx950"). */
 const char *hmr_built_archs(void);

@@ -1,7 +1,6 @@
 /*
  * homura_rocm_unbuilt.h -- entry points of the reference's C ABI that belong to kernel families
- * this library does not implement (fused optimiser steps, outer product, triangle, flip, random
- * sampling, cumulative product, indexing, pooling, matrix products). They are exported so that
+ * this library does not implement (pooling, unfold, matrix products). They are exported so that
  * the reference crate's 77 `extern "C"` declarations (ref: src/backend/rocm/ffi.rs) all resolve
  * at link time; each one fails with HMR_INVALID and the message
  * "<name>: not built in this library". The size queries among them (`*_workspace`) fail the same
@@ -18,23 +17,11 @@
 extern "C" {
 #endif
 
-/* ref :376-390, 412-426 (the rest of indexing: positions of advanced indexing, overwriting puts, masks) */
-hmr_status hmr_index_positions(hmr_context_t ctx, const hmr_tensor_desc *out,
-                               const hmr_tensor_desc *coord, int64_t size, int64_t stride,
-                               int32_t first);
-hmr_status hmr_index_overwrite_workspace(int64_t size, int64_t *bytes);
-hmr_status hmr_index_overwrite(hmr_context_t ctx, const hmr_tensor_desc *out,
-                               const hmr_tensor_desc *src, const hmr_tensor_desc *positions,
-                               int32_t dim, void *workspace, int64_t workspace_bytes);
+/* ref :407-414 (the backward of max pooling through sorted positions) */
 hmr_status hmr_max_pool2d_backward_workspace(int64_t n, int64_t *bytes);
 hmr_status hmr_max_pool2d_backward(hmr_context_t ctx, const hmr_tensor_desc *out,
                                    const hmr_tensor_desc *grad, const hmr_tensor_desc *indices,
                                    void *workspace, int64_t workspace_bytes);
-hmr_status hmr_mask_workspace(int64_t n, int64_t *bytes, int64_t *total_word);
-hmr_status hmr_mask_count(hmr_context_t ctx, const hmr_tensor_desc *mask, void *workspace,
-                          int64_t workspace_bytes);
-hmr_status hmr_mask_coordinates(hmr_context_t ctx, const hmr_tensor_desc *mask, void *workspace,
-                                int64_t workspace_bytes, const hmr_tensor_desc *out);
 
 /* ref :434-466 (pooling) */
 hmr_status hmr_max_pool2d(hmr_context_t ctx, const hmr_tensor_desc *out,

@@ -1352,6 +1352,131 @@ void scatter_add(const hcb_tensor &out, int dim, const hcb_tensor &index, const 
     });
 }
 
+// The elements of an I32 or I64 tensor in row-major order, as i64 (ref: misc.rs read_host::<i64>).
+std::vector<int64_t> integers_of(const hcb_tensor &t) {
+    std::vector<int64_t> out;
+    out.reserve(static_cast<size_t>(num_elements(t)));
+    const int64_t *const st[1] = {t.strides};
+    Plan<1> plan(t.ndim, t.shape, st);
+    const int64_t b[1] = {t.offset};
+    if (t.dtype == HMR_I64) {
+        const int64_t *p = base<int64_t>(t);
+        plan.for_each(b, [&](const int64_t(&o)[1]) { out.push_back(p[o[0]]); });
+    } else if (t.dtype == HMR_I32) {
+        const int32_t *p = base<int32_t>(t);
+        plan.for_each(b, [&](const int64_t(&o)[1]) { out.push_back(p[o[0]]); });
+    } else {
+        panic("an index tensor is I32 or I64");
+    }
+    return out;
+}
+
+// Copies slice i of src along dim into slice index[i] of out, in order, so that the last of repeated
+// positions wins (ref: misc.rs:104-126). The positions are valid.
+void index_overwrite(const hcb_tensor &out, int dim, const hcb_tensor &index, const hcb_tensor &src) {
+    if (num_elements(src) == 0) return;
+    const std::vector<int64_t> picked = positions(index, dim, out.shape[dim], 0);
+    std::vector<int64_t> shape, so, ss;
+    for (int d = 0; d < src.ndim; ++d) {
+        if (d == dim) continue;
+        shape.push_back(src.shape[d]);
+        so.push_back(out.strides[d]);
+        ss.push_back(src.strides[d]);
+    }
+    dispatch_all(src.dtype, [&](auto t) {
+        using T = typename decltype(t)::type;
+        T *po = base<T>(out);
+        const T *ps = base<T>(src);
+        const int64_t *const st[2] = {so.data(), ss.data()};
+        Plan<2> slice(static_cast<int>(shape.size()), shape.data(), st);
+        for (size_t i = 0; i < picked.size(); ++i) {
+            const int64_t b[2] = {out.offset + picked[i] * out.strides[dim], src.offset + static_cast<int64_t>(i) * src.strides[dim]};
+            slice.for_each(b, [&](const int64_t(&o)[2]) { po[o[0]] = ps[o[1]]; });
+        }
+    });
+}
+
+// The number of true elements of a BOOL mask and, with `out` (I64, contiguous, the mask's rank x that number),
+// coordinate d of the k-th of them in row-major order at out[d][k] (ref: misc.rs:128-148).
+int64_t mask_coordinates(const hcb_tensor &mask, const hcb_tensor *out) {
+    if (mask.dtype != HMR_BOOL) panic("a mask is a BOOL tensor");
+    const boolean *p = base<boolean>(mask);
+    const int64_t *const st[1] = {mask.strides};
+    Plan<1> plan(mask.ndim, mask.shape, st);
+    const int64_t b[1] = {mask.offset};
+    int64_t count = 0;
+    plan.for_each(b, [&](const int64_t(&o)[1]) { count += p[o[0]].v != 0; });
+    if (out == nullptr) return count;
+    int64_t *po = base<int64_t>(*out) + out->offset;
+    std::vector<int64_t> at(static_cast<size_t>(mask.ndim), 0);
+    int64_t k = 0;
+    plan.for_each(b, [&](const int64_t(&o)[1]) {
+        if (p[o[0]].v != 0) {
+            for (int d = 0; d < mask.ndim; ++d) po[d * count + k] = at[d];
+            ++k;
+        }
+        for (int d = mask.ndim - 1; d >= 0; --d) {
+            if (++at[d] < mask.shape[d]) break;
+            at[d] = 0;
+        }
+    });
+    return count;
+}
+
+// Checks each of the `n` indices, in order and each in row-major order, to lie in -size..size for its size
+// in `sizes`; the first one out of range is reported as (bad_index, bad_value) and nothing is written.
+// Otherwise (bad_index = -1), and with `out` (I64, contiguous, the shape the indices broadcast to), the linear
+// position in the indexed subspace (row-major over `sizes`) of every element goes to out, negative coordinates
+// counting from the end (ref: misc.rs:150-203).
+void index_positions(const hcb_tensor *out, int n, const hcb_tensor *const *coords, const int64_t *sizes, int32_t *bad_index,
+                     int64_t *bad_value) {
+    *bad_index = -1;
+    *bad_value = 0;
+    std::vector<std::vector<int64_t>> values;
+    for (int k = 0; k < n; ++k) values.push_back(integers_of(*coords[k]));
+    for (int k = 0; k < n; ++k) {
+        for (int64_t v : values[static_cast<size_t>(k)]) {
+            if (v < -sizes[k] || v >= sizes[k]) {
+                *bad_index = k;
+                *bad_value = v;
+                return;
+            }
+        }
+    }
+    if (out == nullptr) return;
+    const std::vector<int64_t> strides = contiguous_strides_of(sizes, n);
+    // Every index, contiguous over its own shape, walked over out's shape (right-aligned, 1 -> stride 0).
+    std::vector<std::vector<int64_t>> walks;
+    for (int k = 0; k < n; ++k) {
+        const hcb_tensor &c = *coords[k];
+        const std::vector<int64_t> own = contiguous_strides_of(c.shape, c.ndim);
+        std::vector<int64_t> walk(static_cast<size_t>(out->ndim), 0);
+        for (int d = 0; d < c.ndim; ++d) {
+            const int to = out->ndim - c.ndim + d;
+            if (to < 0) panic("index_positions: an index has more dimensions than the positions");
+            walk[static_cast<size_t>(to)] = c.shape[d] == 1 ? 0 : own[static_cast<size_t>(d)];
+        }
+        walks.push_back(walk);
+    }
+    int64_t *po = base<int64_t>(*out) + out->offset;
+    const int64_t total = num_elements(*out);
+    std::vector<int64_t> at(static_cast<size_t>(out->ndim), 0);
+    for (int64_t e = 0; e < total; ++e) {
+        int64_t position = 0;
+        for (int k = 0; k < n; ++k) {
+            int64_t offset = 0;
+            for (int d = 0; d < out->ndim; ++d) offset += at[d] * walks[static_cast<size_t>(k)][static_cast<size_t>(d)];
+            const int64_t v = values[static_cast<size_t>(k)][static_cast<size_t>(offset)];
+            position += (v < 0 ? v + sizes[k] : v) * strides[static_cast<size_t>(k)];
+        }
+        po[e] = position;
+        for (int d = out->ndim - 1; d >= 0; --d) {
+            if (++at[d] < out->shape[d]) break;
+            at[d] = 0;
+        }
+    }
+}
+
 template <class F>
 int guarded(F f) {
     try {
@@ -1452,6 +1577,16 @@ int orc_index_add(const hcb_tensor *out, int32_t dim, const hcb_tensor *index, c
 int orc_scatter_add(const hcb_tensor *out, int32_t dim, const hcb_tensor *index, const hcb_tensor *src) {
     return orc::guarded([&] { orc::scatter_add(*out, dim, *index, *src); });
 }
+int orc_index_overwrite(const hcb_tensor *out, int32_t dim, const hcb_tensor *index, const hcb_tensor *src) {
+    return orc::guarded([&] { orc::index_overwrite(*out, dim, *index, *src); });
+}
+int orc_mask_coordinates(const hcb_tensor *mask, const hcb_tensor *out, int64_t *count) {
+    return orc::guarded([&] { *count = orc::mask_coordinates(*mask, out); });
+}
+int orc_index_positions(const hcb_tensor *out, int32_t n, const hcb_tensor *const *coords, const int64_t *sizes, int32_t *bad_index,
+                        int64_t *bad_value) {
+    return orc::guarded([&] { orc::index_positions(out, n, coords, sizes, bad_index, bad_value); });
+}
 int orc_addr(const hcb_tensor *out, const hcb_tensor *v1, const hcb_tensor *v2, const hcb_tensor *input, hcb_scalar alpha,
              hcb_scalar beta) {
     return orc::guarded([&] { orc::addr(*out, *v1, *v2, *input, alpha, beta); });
@@ -1474,6 +1609,7 @@ const hcb_backend *orc_backend(void) {
         orc_fused,           orc_triangle,   orc_flip,  orc_addr,           orc_exclusive_cumprod,
         orc_random_uniform,  orc_random_normal,         orc_random_int,
         orc_index_select,    orc_gather,     orc_index_add,         orc_scatter_add,
+        orc_index_overwrite, orc_mask_coordinates,      orc_index_positions,
     };
     return &table;
 }
