@@ -183,11 +183,20 @@ __global__ void __launch_bounds__(kScanBlock) mask_scan_kernel(uint64_t *counts,
     if (threadIdx.x == 0) counts[tiles] = carry;
 }
 
-// out[dim][k] at out + dim * out_row + k * out_col.
-template <bool FLAT>
-__global__ void __launch_bounds__(kBlock) mask_write_kernel(const uint8_t *mask, Dims d, int64_t n, int64_t tiles, const uint64_t *offsets,
-                                                            int64_t *out, int64_t count, int64_t out_row, int64_t out_col) {
+// Division by the mask's sizes (innermost first) for positions below 2^31.
+struct MaskDivs {
+    FastDiv d[kMaxIndexDims];
+};
+
+// out[dim][k] at out + dim * out_row + k * out_col. The true elements of a tile are first compacted into LDS
+// (their places inside the tile, in order), then lane j takes the tile's j-th, j + 256-th, ... of them: the
+// stores of a wave fill whole lines of each row of out. SMALL: n < 2^31, coordinates by multiplication.
+template <bool FLAT, bool SMALL>
+__global__ void __launch_bounds__(kBlock) mask_write_kernel(const uint8_t *mask, Dims d, MaskDivs divs, int64_t n, int64_t tiles,
+                                                            const uint64_t *offsets, int64_t *out, int64_t count, int64_t out_row,
+                                                            int64_t out_col) {
     __shared__ uint32_t lds[kBlock / 64];
+    __shared__ uint16_t place[kMaskTile];
     const int lane = threadIdx.x & 63, wave = threadIdx.x / 64;
     for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
         const int64_t first = tile * kMaskTile + static_cast<int64_t>(threadIdx.x) * kMaskPerThread;
@@ -199,19 +208,38 @@ __global__ void __launch_bounds__(kBlock) mask_write_kernel(const uint8_t *mask,
             const uint32_t y = static_cast<uint32_t>(__shfl_up(static_cast<int>(x), off, 64));
             if (lane >= off) x += y;
         }
-        __syncthreads();
+        __syncthreads();  // lds and place are reused from tile to tile
         if (lane == 63) lds[wave] = x;
         __syncthreads();
-        uint32_t before = 0;
-        for (int w = 0; w < wave; ++w) before += lds[w];
-        int64_t k = static_cast<int64_t>(offsets[tile]) + before + x - c;
-        for (uint32_t rest_bits = bits; rest_bits != 0; rest_bits &= rest_bits - 1, ++k) {
+        uint32_t rank = x - c;
+        for (int w = 0; w < wave; ++w) rank += lds[w];
+        for (uint32_t rest_bits = bits; rest_bits != 0; rest_bits &= rest_bits - 1) {
+            place[rank++] = static_cast<uint16_t>(threadIdx.x * kMaskPerThread + (__ffs(rest_bits) - 1));
+        }
+        __syncthreads();
+        const int64_t k0 = static_cast<int64_t>(offsets[tile]);
+        const uint32_t in_tile = static_cast<uint32_t>(offsets[tile + 1] - offsets[tile]);
+        for (uint32_t j = threadIdx.x; j < in_tile; j += kBlock) {
+            const int64_t k = k0 + j;
             if (k >= count) break;
-            int64_t rest = first + (__ffs(rest_bits) - 1);
-            for (int dd = 0; dd < d.ndim; ++dd) {
-                const int64_t q = rest / d.size[dd];
-                out[(d.ndim - 1 - dd) * out_row + k * out_col] = rest - q * d.size[dd];
-                rest = q;
+            const int64_t linear = tile * kMaskTile + place[j];
+            int64_t *po = out + k * out_col;
+            if constexpr (SMALL) {
+                uint32_t rest = static_cast<uint32_t>(linear);
+                for (int dd = 0; dd < d.ndim - 1; ++dd) {
+                    const uint32_t q = divide(rest, divs.d[dd]);
+                    po[(d.ndim - 1 - dd) * out_row] = rest - q * divs.d[dd].div;
+                    rest = q;
+                }
+                if (d.ndim > 0) po[0] = rest;
+            } else {
+                int64_t rest = linear;
+                for (int dd = 0; dd < d.ndim - 1; ++dd) {
+                    const int64_t q = rest / d.size[dd];
+                    po[(d.ndim - 1 - dd) * out_row] = rest - q * d.size[dd];
+                    rest = q;
+                }
+                if (d.ndim > 0) po[0] = rest;
             }
         }
     }
@@ -379,16 +407,21 @@ hmr_status hmr_mask_coordinates(hmr_context_t ctx, const hmr_tensor_desc *mask, 
         const uint64_t *offsets = static_cast<const uint64_t *>(workspace);
         int64_t *po = reinterpret_cast<int64_t *>(hmr::first_of(*out));
         const bool flat = hmr::mask_is_flat(*mask);
+        const bool small = n < (int64_t{1} << 31);
+        hmr::MaskDivs divs{};
+        for (int k = 0; small && k < d.ndim; ++k) divs.d[k] = hmr::make_fastdiv(static_cast<uint32_t>(d.size[k]));
         const int64_t cap = int64_t{1} << 20;
         return hmr::launch_on(ctx, "mask_coordinates", [&](hipStream_t stream) {
             const dim3 grid(static_cast<unsigned>(tiles < cap ? tiles : cap));
-            if (flat) {
-                hipLaunchKernelGGL((hmr::mask_write_kernel<true>), grid, dim3(hmr::kBlock), 0, stream, base, d, n, tiles, offsets, po,
-                                   out->sizes[1], out->strides[0], out->strides[1]);
-            } else {
-                hipLaunchKernelGGL((hmr::mask_write_kernel<false>), grid, dim3(hmr::kBlock), 0, stream, base, d, n, tiles, offsets, po,
-                                   out->sizes[1], out->strides[0], out->strides[1]);
-            }
+            auto run = [&](auto flat_tag, auto small_tag) {
+                hipLaunchKernelGGL((hmr::mask_write_kernel<decltype(flat_tag)::value, decltype(small_tag)::value>), grid,
+                                   dim3(hmr::kBlock), 0, stream, base, d, divs, n, tiles, offsets, po, out->sizes[1], out->strides[0],
+                                   out->strides[1]);
+            };
+            if (flat && small) run(std::true_type{}, std::true_type{});
+            else if (flat) run(std::true_type{}, std::false_type{});
+            else if (small) run(std::false_type{}, std::true_type{});
+            else run(std::false_type{}, std::false_type{});
             return true;
         });
     });
