@@ -9,10 +9,11 @@
 //   adds    every element of the output is summed in f64 (wrapping i64 for integers) in the row-major
 //           order of the index positions and rounded once, as the CPU does. Addition is not
 //           associative, so the order is reproduced: each contribution becomes a 64-bit word
-//           (target << 32 | position), the words are sorted (a bitonic network: keys are unique, so any
-//           correct sort gives the one order), and the first word of each target sums its run in
-//           order. Targets run in parallel; index_add also spreads a slice over the lanes.
+//           (target << 32 | position), the words are sorted by target with a stable radix sort (sort.hpp;
+//           positions ascend on input, so each target's stay in order), and the first word of each target
+//           sums its run in order. Targets run in parallel; index_add also spreads a slice over the lanes.
 #include "index.hpp"
+#include "sort.hpp"
 
 namespace hmr {
 namespace {
@@ -136,74 +137,6 @@ __global__ void __launch_bounds__(kBlock) select_rows_kernel(RowsOfTiles a) {
     }
 }
 
-// ---- sorting 64-bit words (bitonic) -----------------------------------------------------------------------
-//
-// `count` is a power of two >= kSortChunk; a workgroup keeps kSortChunk words in LDS for the steps whose
-// partners lie inside an aligned chunk, the wider steps go through memory one at a time.
-constexpr int kSortChunk = 2048;
-constexpr int kSortThreads = 256;
-
-__device__ __forceinline__ void sort_steps_in_lds(uint64_t *s, uint32_t base, uint32_t k, uint32_t j_first) {
-    for (uint32_t j = j_first; j > 0; j >>= 1) {
-        for (uint32_t t = threadIdx.x; t < kSortChunk / 2; t += kSortThreads) {
-            const uint32_t i = ((t & ~(j - 1)) << 1) | (t & (j - 1));
-            const uint32_t l = i | j;
-            const bool ascending = ((base + i) & k) == 0;
-            const uint64_t x = s[i], y = s[l];
-            if ((x > y) == ascending) {
-                s[i] = y;
-                s[l] = x;
-            }
-        }
-        __syncthreads();
-    }
-}
-
-// Every chunk sorted (k = 2 .. kSortChunk), or, with k > kSortChunk, the last log2(kSortChunk) steps of stage k.
-__global__ void __launch_bounds__(kSortThreads) sort_chunks_kernel(uint64_t *words, uint32_t k_only) {
-    __shared__ uint64_t s[kSortChunk];
-    const uint32_t base = blockIdx.x * kSortChunk;
-    for (uint32_t t = threadIdx.x; t < kSortChunk; t += kSortThreads) s[t] = words[base + t];
-    __syncthreads();
-    if (k_only == 0) {
-        for (uint32_t k = 2; k <= kSortChunk; k <<= 1) sort_steps_in_lds(s, base, k, k >> 1);
-    } else {
-        sort_steps_in_lds(s, base, k_only, kSortChunk >> 1);
-    }
-    for (uint32_t t = threadIdx.x; t < kSortChunk; t += kSortThreads) words[base + t] = s[t];
-}
-
-__global__ void __launch_bounds__(kBlock) sort_step_kernel(uint64_t *words, uint32_t half, uint32_t k, uint32_t j) {
-    const uint32_t t = blockIdx.x * kBlock + threadIdx.x;
-    if (t >= half) return;
-    const uint32_t i = ((t & ~(j - 1)) << 1) | (t & (j - 1));
-    const uint32_t l = i | j;
-    const bool ascending = (i & k) == 0;
-    const uint64_t x = words[i], y = words[l];
-    if ((x > y) == ascending) {
-        words[i] = y;
-        words[l] = x;
-    }
-}
-
-inline int64_t sort_capacity(int64_t n) {
-    int64_t p = kSortChunk;
-    while (p < n) p <<= 1;
-    return p;
-}
-
-void sort_words(uint64_t *words, int64_t count, hipStream_t stream) {
-    const uint32_t n = static_cast<uint32_t>(count);
-    const unsigned chunks = n / kSortChunk;
-    hipLaunchKernelGGL(sort_chunks_kernel, dim3(chunks), dim3(kSortThreads), 0, stream, words, 0u);
-    for (uint32_t k = 2 * kSortChunk; k != 0 && k <= n; k <<= 1) {
-        for (uint32_t j = k >> 1; j >= kSortChunk; j >>= 1) {
-            hipLaunchKernelGGL(sort_step_kernel, dim3(n / 2 / kBlock), dim3(kBlock), 0, stream, words, n / 2, k, j);
-        }
-        hipLaunchKernelGGL(sort_chunks_kernel, dim3(chunks), dim3(kSortThreads), 0, stream, words, k);
-    }
-}
-
 // ---- adds ---------------------------------------------------------------------------------------------------
 
 template <class T>
@@ -226,14 +159,8 @@ struct Sum {
 
 // scatter_add: word p = (offset of the target in out << 32) | p, for the index's positions p in row-major
 // order; stride[0] the index, [1] out (its stride along `at` multiplies the index value), [2] src.
-__global__ void __launch_bounds__(kBlock) scatter_words_kernel(uint64_t *words, int64_t capacity, const void *index, int is64,
-                                                               Dims d, int64_t n) {
-    for (int64_t p = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; p < capacity;
-         p += static_cast<int64_t>(gridDim.x) * kBlock) {
-        if (p >= n) {
-            words[p] = ~uint64_t{0};
-            continue;
-        }
+__global__ void __launch_bounds__(kBlock) scatter_words_kernel(uint64_t *words, const void *index, int is64, Dims d, int64_t n) {
+    for (int64_t p = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; p < n; p += static_cast<int64_t>(gridDim.x) * kBlock) {
         int64_t rest = p, io = 0, oo = 0;
         for (int k = 0; k < d.ndim; ++k) {
             const int64_t q = rest / d.size[k];
@@ -270,12 +197,10 @@ __global__ void __launch_bounds__(kBlock) scatter_runs_kernel(T *out, const T *s
 }
 
 // index_add: word i = (index[i] << 32) | i.
-__global__ void __launch_bounds__(kBlock) index_words_kernel(uint64_t *words, int64_t capacity, const void *index, int is64,
-                                                             int64_t index_stride, int64_t m) {
-    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; i < capacity;
-         i += static_cast<int64_t>(gridDim.x) * kBlock) {
-        words[i] = i < m ? (static_cast<uint64_t>(read_index(index, is64, i * index_stride)) << 32) | static_cast<uint64_t>(i)
-                         : ~uint64_t{0};
+__global__ void __launch_bounds__(kBlock) index_words_kernel(uint64_t *words, const void *index, int is64, int64_t index_stride,
+                                                             int64_t m) {
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; i < m; i += static_cast<int64_t>(gridDim.x) * kBlock) {
+        words[i] = (static_cast<uint64_t>(read_index(index, is64, i * index_stride)) << 32) | static_cast<uint64_t>(i);
     }
 }
 
@@ -474,7 +399,7 @@ hmr_status hmr_index_add_workspace(int64_t m, int64_t size, int64_t *bytes) {
         if (m >= (int64_t{1} << 31) || size >= (int64_t{1} << 32)) {
             return fail(HMR_INVALID, "index_add: more than 2^31 - 1 positions or 2^32 - 1 slices");
         }
-        *bytes = m == 0 ? 0 : hmr::sort_capacity(m) * 8;
+        *bytes = m == 0 ? 0 : hmr::sort_layout(m).bytes;
         return HMR_OK;
     });
 }
@@ -483,7 +408,7 @@ hmr_status hmr_scatter_add_workspace(int64_t n, int64_t *bytes) {
     return guarded([&] {
         if (n < 0) return fail(HMR_INVALID, "scatter_add_workspace: negative size");
         if (n >= (int64_t{1} << 31)) return fail(HMR_INVALID, "scatter_add: more than 2^31 - 1 positions");
-        *bytes = n == 0 ? 0 : hmr::sort_capacity(n) * 8;
+        *bytes = n == 0 ? 0 : hmr::sort_layout(n).bytes;
         return HMR_OK;
     });
 }
@@ -519,16 +444,16 @@ hmr_status hmr_index_add(hmr_context_t ctx, const hmr_tensor_desc *out, const hm
         const int64_t slice = total / m;
         int lanes = 1;
         while (lanes < hmr::kBlock && lanes < slice) lanes <<= 1;
-        const int64_t capacity = hmr::sort_capacity(m);
         uint64_t *words = static_cast<uint64_t *>(workspace);
+        const int key_bits = hmr::bits_for(static_cast<uint64_t>(out->sizes[dim] > 0 ? out->sizes[dim] - 1 : 0));
         const int64_t index_stride = index->ndim == 1 ? index->strides[0] : 0;
         return hmr::launch_on(ctx, "index_add", [&](hipStream_t stream) {
             if (src->dtype != out->dtype) return false;
             return hmr::with_any_type(out->dtype, [&](auto t) {
                 using T = typename decltype(t)::type;
-                hipLaunchKernelGGL(hmr::index_words_kernel, dim3(hmr::grid_of(capacity)), dim3(hmr::kBlock), 0, stream, words, capacity,
+                hipLaunchKernelGGL(hmr::index_words_kernel, dim3(hmr::grid_of(m)), dim3(hmr::kBlock), 0, stream, words,
                                    static_cast<const void *>(hmr::first_of(*index)), index->dtype == HMR_I64 ? 1 : 0, index_stride, m);
-                hmr::sort_words(words, capacity, stream);
+                const uint64_t *sorted = hmr::sort_words(workspace, m, key_bits, stream);
                 const int64_t cap = int64_t{1} << 20;
                 constexpr int V = 16 / static_cast<int>(sizeof(T));
                 T *po = reinterpret_cast<T *>(hmr::first_of(*out));
@@ -542,12 +467,12 @@ hmr_status hmr_index_add(hmr_context_t ctx, const hmr_tensor_desc *out, const hm
                     while (group < hmr::kBlock && group < slice / V) group <<= 1;
                     const int64_t groups = (m + hmr::kBlock / group - 1) / (hmr::kBlock / group);
                     hipLaunchKernelGGL((hmr::index_runs_tiles_kernel<T>), dim3(static_cast<unsigned>(groups < cap ? groups : cap)),
-                                       dim3(hmr::kBlock), 0, stream, po, ps, static_cast<const uint64_t *>(words), m, slice / V,
+                                       dim3(hmr::kBlock), 0, stream, po, ps, sorted, m, slice / V,
                                        out->strides[dim], src->strides[dim], group);
                 } else {
                     const int64_t groups = (m + hmr::kBlock / lanes - 1) / (hmr::kBlock / lanes);
                     hipLaunchKernelGGL((hmr::index_runs_kernel<T>), dim3(static_cast<unsigned>(groups < cap ? groups : cap)),
-                                       dim3(hmr::kBlock), 0, stream, po, ps, static_cast<const uint64_t *>(words), d, m, slice,
+                                       dim3(hmr::kBlock), 0, stream, po, ps, sorted, d, m, slice,
                                        out->strides[dim], src->strides[dim], lanes);
                 }
             });
@@ -573,18 +498,17 @@ hmr_status hmr_scatter_add(hmr_context_t ctx, const hmr_tensor_desc *out, const 
         if (hmr::reach_of(*out) >= (int64_t{1} << 32) - 1) return fail(HMR_INVALID, "scatter_add: an output of more than 2^32 - 2 elements");
         const hmr_tensor_desc *const ops[3] = {index, out, src};
         const hmr::Dims d = hmr::dims_of(*index, ops, dim);
-        const int64_t capacity = hmr::sort_capacity(n);
         uint64_t *words = static_cast<uint64_t *>(workspace);
+        const int key_bits = hmr::bits_for(static_cast<uint64_t>(hmr::reach_of(*out)));
         return hmr::launch_on(ctx, "scatter_add", [&](hipStream_t stream) {
             if (src->dtype != out->dtype) return false;
             return hmr::with_any_type(out->dtype, [&](auto t) {
                 using T = typename decltype(t)::type;
-                hipLaunchKernelGGL(hmr::scatter_words_kernel, dim3(hmr::grid_of(capacity)), dim3(hmr::kBlock), 0, stream, words, capacity,
+                hipLaunchKernelGGL(hmr::scatter_words_kernel, dim3(hmr::grid_of(n)), dim3(hmr::kBlock), 0, stream, words,
                                    static_cast<const void *>(hmr::first_of(*index)), index->dtype == HMR_I64 ? 1 : 0, d, n);
-                hmr::sort_words(words, capacity, stream);
+                const uint64_t *sorted = hmr::sort_words(workspace, n, key_bits, stream);
                 hipLaunchKernelGGL((hmr::scatter_runs_kernel<T>), dim3(hmr::grid_of(n)), dim3(hmr::kBlock), 0, stream,
-                                   reinterpret_cast<T *>(hmr::first_of(*out)), reinterpret_cast<const T *>(hmr::first_of(*src)),
-                                   static_cast<const uint64_t *>(words), d, n);
+                                   reinterpret_cast<T *>(hmr::first_of(*out)), reinterpret_cast<const T *>(hmr::first_of(*src)), sorted, d, n);
             });
         });
     });
