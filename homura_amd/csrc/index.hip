@@ -29,11 +29,14 @@ __global__ void __launch_bounds__(kBlock) check_kernel(const void *index, int is
                                                        int has_exempt, int64_t exempt, unsigned long long *slot) {
     unsigned long long first = ~0ull;
     for (int64_t p = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; p < n; p += static_cast<int64_t>(gridDim.x) * kBlock) {
-        int64_t rest = p, off = 0;
-        for (int k = 0; k < d.ndim; ++k) {
-            const int64_t q = rest / d.size[k];
-            off += (rest - q * d.size[k]) * d.stride[0][k];
-            rest = q;
+        int64_t rest = p, off = p * d.stride[0][0];
+        if (d.ndim > 1) {
+            off = 0;
+            for (int k = 0; k < d.ndim; ++k) {
+                const int64_t q = rest / d.size[k];
+                off += (rest - q * d.size[k]) * d.stride[0][k];
+                rest = q;
+            }
         }
         const int64_t v = read_index(index, is64, off);
         const bool bad = !(v >= low && v < high) && !(has_exempt && v == exempt);
@@ -47,6 +50,60 @@ __global__ void __launch_bounds__(kBlock) check_kernel(const void *index, int is
         first = other < first ? other : first;
     }
     if ((threadIdx.x & 63) == 0 && first != ~0ull) atomicMin(slot, first);
+}
+
+// The whole check in one workgroup, for indices of a few thousand elements (three launches otherwise).
+constexpr int kCheckBlock = 1024;
+constexpr int64_t kCheckSmall = 64 * kCheckBlock;
+__global__ void __launch_bounds__(kCheckBlock) check_small_kernel(const void *index, int is64, Dims d, int64_t n, int64_t low, int64_t high,
+                                                                  int has_exempt, int64_t exempt, uint64_t *slot) {
+    __shared__ unsigned long long firsts[kCheckBlock / 64];
+    __shared__ long long values[kCheckBlock / 64];
+    unsigned long long first = ~0ull;
+    long long value = 0;
+    for (int64_t p = threadIdx.x; p < n; p += kCheckBlock) {
+        int64_t rest = p, off = p * d.stride[0][0];
+        if (d.ndim > 1) {
+            off = 0;
+            for (int k = 0; k < d.ndim; ++k) {
+                const int64_t q = rest / d.size[k];
+                off += (rest - q * d.size[k]) * d.stride[0][k];
+                rest = q;
+            }
+        }
+        const int64_t v = read_index(index, is64, off);
+        const bool bad = !(v >= low && v < high) && !(has_exempt && v == exempt);
+        if (bad && static_cast<unsigned long long>(p) < first) {
+            first = static_cast<unsigned long long>(p);
+            value = v;
+        }
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) {
+        const unsigned long long other = (static_cast<unsigned long long>(static_cast<uint32_t>(__shfl_xor(static_cast<int>(first >> 32), m, 64))) << 32) |
+                                         static_cast<uint32_t>(__shfl_xor(static_cast<int>(first), m, 64));
+        const long long theirs = static_cast<long long>((static_cast<unsigned long long>(static_cast<uint32_t>(__shfl_xor(static_cast<int>(value >> 32), m, 64))) << 32) |
+                                                        static_cast<uint32_t>(__shfl_xor(static_cast<int>(value), m, 64)));
+        if (other < first) {
+            first = other;
+            value = theirs;
+        }
+    }
+    if ((threadIdx.x & 63) == 0) {
+        firsts[threadIdx.x / 64] = first;
+        values[threadIdx.x / 64] = value;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < kCheckBlock / 64; ++w) {
+            if (firsts[w] < first) {
+                first = firsts[w];
+                value = values[w];
+            }
+        }
+        slot[0] = first;
+        slot[1] = first == ~0ull ? 0 : static_cast<uint64_t>(value);
+    }
 }
 
 __global__ void check_value_kernel(const void *index, int is64, Dims d, uint64_t *slot) {
@@ -292,6 +349,11 @@ hmr_status hmr_index_check(hmr_context_t ctx, const hmr_tensor_desc *index, int6
         const void *base = hmr::first_of(*index);
         const int is64 = index->dtype == HMR_I64;
         return hmr::launch_on(ctx, "index_check", [&](hipStream_t stream) {
+            if (n <= hmr::kCheckSmall) {
+                hipLaunchKernelGGL(hmr::check_small_kernel, dim3(1), dim3(hmr::kCheckBlock), 0, stream, base, is64, d, n, low, high,
+                                   has_exempt, exempt, slot);
+                return true;
+            }
             hipLaunchKernelGGL(hmr::check_init_kernel, dim3(1), dim3(1), 0, stream, slot);
             if (n > 0) {
                 hipLaunchKernelGGL(hmr::check_kernel, dim3(hmr::grid_of(n)), dim3(hmr::kBlock), 0, stream, base, is64, d, n, low, high,

@@ -248,6 +248,26 @@ def test_the_c_abi_of_the_index_kernels():
         capi.check(L.hmr_index_check(ctx.handle, byref(transposed), 0, 10, 1, -4, slot.ptr))  # -4 is exempt
         ctx.synchronize()
         assert slot.download(np.int64, 2).tolist() == [2, 99]
+        # More elements than the single-workgroup form takes: the first offender of several, then none.
+        big = (np.arange(200000) % 1000).astype(np.int32)
+        big[[77777, 150000, 199999]] = [1000, -1, 5000]
+        db = ctx.upload(big)
+        B = capi.make_desc(db.ptr, capi.I32, [200000], [1], 0)
+        capi.check(L.hmr_index_check(ctx.handle, byref(B), 0, 1000, 0, 0, slot.ptr))
+        ctx.synchronize()
+        assert slot.download(np.int64, 2).tolist() == [77777, 1000]
+        capi.check(L.hmr_index_check(ctx.handle, byref(B), -1, 5001, 0, 0, slot.ptr))
+        ctx.synchronize()
+        assert slot.download(np.uint64, 2).tolist() == [2 ** 64 - 1, 0]
+        # The last element of a single-workgroup check, and of a wave's share.
+        for n, bad in ((65536, 65535), (65536, 1023), (1000, 999)):
+            small = np.zeros(n, dtype=np.int64)
+            small[bad] = 7
+            dsm = ctx.upload(small)
+            S_ = capi.make_desc(dsm.ptr, capi.I64, [n], [1], 0)
+            capi.check(L.hmr_index_check(ctx.handle, byref(S_), 0, 7, 0, 0, slot.ptr))
+            ctx.synchronize()
+            assert slot.download(np.int64, 2).tolist() == [bad, 7]
         f = capi.make_desc(di.ptr, capi.F64, [6], [1], 0)
         assert L.hmr_index_check(ctx.handle, byref(f), 0, 1, 0, 0, slot.ptr) == capi.HMR_INVALID
         assert L.hmr_last_error().decode() == "index_check: unsupported dtype"
