@@ -149,14 +149,17 @@ def main():
         cb = tensor(host_bias, DT.BF16, [H])
         cs = tensor(host_scale, DT.BF16, [B, S, 1])
         cr = tensor(host_res, DT.F32, [B, S, H])
-        t0 = time.perf_counter()
-        cx.add(cb).mul(cs).add(cr)
-        dt = time.perf_counter() - t0
+        dt = None
+        for _ in range(5):  # the first pass also pages the buffers in; the best of five is reported
+            t0 = time.perf_counter()
+            cx.add(cb).mul(cs).add(cr)
+            took = time.perf_counter() - t0
+            dt = took if dt is None else min(dt, took)
         # The CPU path follows the reference: the bf16 intermediate is cast to f32 by a separate copy.
         cpu = {"value": round(chain_bytes / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
                "host_cores_available": os.cpu_count(),
-               "sample": "one full pass of configs[1] (67 108 864 elements per op), C++ port of homura's "
-                         "single-threaded CPU backend, g++ -O2 -ffp-contract=off",
+               "sample": "the whole of configs[1] (67 108 864 elements per op), best of five passes, C++ port of "
+                         "homura's single-threaded CPU backend, g++ -O2 -ffp-contract=off",
                "seconds": round(dt, 3), "gpu_speedup": round(value / (chain_bytes / dt / 1e9), 1)}
 
     line = {
