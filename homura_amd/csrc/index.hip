@@ -61,21 +61,32 @@ __global__ void __launch_bounds__(kCheckBlock) check_small_kernel(const void *in
     __shared__ long long values[kCheckBlock / 64];
     unsigned long long first = ~0ull;
     long long value = 0;
-    for (int64_t p = threadIdx.x; p < n; p += kCheckBlock) {
-        int64_t rest = p, off = p * d.stride[0][0];
-        if (d.ndim > 1) {
-            off = 0;
-            for (int k = 0; k < d.ndim; ++k) {
-                const int64_t q = rest / d.size[k];
-                off += (rest - q * d.size[k]) * d.stride[0][k];
-                rest = q;
+    constexpr int kAhead = 8;  // loads in flight per lane
+    for (int64_t p0 = threadIdx.x; p0 < n; p0 += static_cast<int64_t>(kAhead) * kCheckBlock) {
+        int64_t v[kAhead];
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) {
+            const int64_t p = p0 + static_cast<int64_t>(u) * kCheckBlock;
+            const int64_t q = p < n ? p : n - 1;  // past the end: the last element again, left out below
+            int64_t rest = q, off = q * d.stride[0][0];
+            if (d.ndim > 1) {
+                off = 0;
+                for (int k = 0; k < d.ndim; ++k) {
+                    const int64_t w = rest / d.size[k];
+                    off += (rest - w * d.size[k]) * d.stride[0][k];
+                    rest = w;
+                }
             }
+            v[u] = read_index(index, is64, off);
         }
-        const int64_t v = read_index(index, is64, off);
-        const bool bad = !(v >= low && v < high) && !(has_exempt && v == exempt);
-        if (bad && static_cast<unsigned long long>(p) < first) {
-            first = static_cast<unsigned long long>(p);
-            value = v;
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) {
+            const int64_t p = p0 + static_cast<int64_t>(u) * kCheckBlock;
+            const bool bad = p < n && !(v[u] >= low && v[u] < high) && !(has_exempt && v[u] == exempt);
+            if (bad && static_cast<unsigned long long>(p) < first) {
+                first = static_cast<unsigned long long>(p);
+                value = v[u];
+            }
         }
     }
 #pragma unroll

@@ -153,16 +153,24 @@ __global__ void __launch_bounds__(kBlock) mask_count_kernel(const uint8_t *mask,
     }
 }
 
-// One workgroup: counts[0 .. tiles) become their exclusive prefix sums and counts[tiles] the total.
+// One workgroup: counts[0 .. tiles) become their exclusive prefix sums and counts[tiles] the total. A lane takes
+// eight adjacent counts per step.
 constexpr int kScanBlock = 1024;
+constexpr int kScanPer = 8;
 __global__ void __launch_bounds__(kScanBlock) mask_scan_kernel(uint64_t *counts, int64_t tiles) {
     __shared__ uint64_t lds[kScanBlock / 64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x / 64;
     uint64_t carry = 0;
-    for (int64_t base = 0; base < tiles; base += kScanBlock) {
-        const int64_t i = base + threadIdx.x;
-        const uint64_t v = i < tiles ? counts[i] : 0;
-        uint64_t x = v;
+    for (int64_t base = 0; base < tiles; base += static_cast<int64_t>(kScanBlock) * kScanPer) {
+        const int64_t first = base + static_cast<int64_t>(threadIdx.x) * kScanPer;
+        uint64_t v[kScanPer];
+        uint64_t sum = 0;
+#pragma unroll
+        for (int i = 0; i < kScanPer; ++i) {
+            v[i] = first + i < tiles ? counts[first + i] : 0;
+            sum += v[i];
+        }
+        uint64_t x = sum;
 #pragma unroll
         for (int off = 1; off < 64; off <<= 1) {
             const uint64_t lo = static_cast<uint32_t>(__shfl_up(static_cast<int>(x), off, 64));
@@ -171,12 +179,16 @@ __global__ void __launch_bounds__(kScanBlock) mask_scan_kernel(uint64_t *counts,
         }
         if (lane == 63) lds[wave] = x;
         __syncthreads();
-        uint64_t before = 0, total = 0;
+        uint64_t before = carry + x - sum, total = 0;
         for (int w = 0; w < kScanBlock / 64; ++w) {
             before += w < wave ? lds[w] : 0;
             total += lds[w];
         }
-        if (i < tiles) counts[i] = carry + before + x - v;
+#pragma unroll
+        for (int i = 0; i < kScanPer; ++i) {
+            if (first + i < tiles) counts[first + i] = before;
+            before += v[i];
+        }
         carry += total;
         __syncthreads();
     }
