@@ -213,6 +213,8 @@ VIEWS = [
     ("inner broadcast [7, 48]", 48, lambda t: t.reshape([1, 48]).expand([7, 48])),
     ("row broadcast [6, 40]", 6, lambda t: t.reshape([6, 1]).expand([6, 40])),
     ("permuted heads [2, 4, 3, 32]", 2 * 3 * 4 * 32, lambda t: t.reshape([2, 3, 4, 32]).permute([0, 2, 1, 3])),
+    # Large enough for the rows kernel to walk the transposed pair of dimensions in tiles of 8.
+    ("permuted heads [2, 8, 24, 32]", 2 * 24 * 8 * 32, lambda t: t.reshape([2, 24, 8, 32]).permute([0, 2, 1, 3])),
 ]
 
 
