@@ -535,6 +535,26 @@ Tensor Tensor::narrow(int64_t dim, int64_t start, int64_t length) const {
     return Tensor(TensorData{d_.storage, l, d_.dtype});
 }
 
+// ref: src/tensor/view.rs:32-58, 317-333: a Python-style slice start:end:step; bounds may be negative and are
+// clamped into 0..=size.
+Tensor Tensor::slice(int64_t dim, std::optional<int64_t> start, std::optional<int64_t> end, int64_t step) const {
+    Layout l = d_.layout;
+    if (l.shape.empty()) throw Error("slice() cannot be applied to a 0-dim tensor.");
+    if (step <= 0) throw Error("slice step must be positive");
+    const size_t d = normalize_dim(dim, l.shape.size());
+    const int64_t size = l.shape[d];
+    auto clamp = [&](int64_t v) {
+        if (v < 0) v += size;
+        return v < 0 ? int64_t{0} : (v > size ? size : v);
+    };
+    const int64_t from = clamp(start.value_or(0)), to = clamp(end.value_or(size));
+    const int64_t len = to > from ? (to - from - 1) / step + 1 : 0;
+    l.offset += from * l.strides[d];
+    l.shape[d] = len;
+    l.strides[d] *= step;
+    return Tensor(TensorData{d_.storage, l, d_.dtype});
+}
+
 Tensor Tensor::select(int64_t dim, int64_t index) const {
     const Layout &l = d_.layout;
     if (l.shape.empty()) throw Error("select() cannot be applied to a 0-dim tensor.");

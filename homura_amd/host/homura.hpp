@@ -220,6 +220,7 @@ class Tensor {
     Tensor unsqueeze(int64_t dim) const;
     Tensor narrow(int64_t dim, int64_t start, int64_t length) const;
     Tensor select(int64_t dim, int64_t index) const;
+    Tensor slice(int64_t dim, std::optional<int64_t> start, std::optional<int64_t> end, int64_t step) const;
     Tensor flatten(int64_t start_dim, int64_t end_dim) const;
 
     // Unary (ref: src/ops/unary.rs).

@@ -260,6 +260,7 @@ PYBIND11_MODULE(_host, m) {
     T.def("gather", &Tensor::gather);
     T.def("index_add", &Tensor::index_add);
     T.def("scatter_add", &Tensor::scatter_add);
+    T.def("slice", &Tensor::slice, py::arg("dim"), py::arg("start") = py::none(), py::arg("end") = py::none(), py::arg("step") = 1);
     T.def("index_tensors", &Tensor::index_tensors);
     T.def("index_put_tensors", &Tensor::index_put_tensors);
     T.def("mask_coordinates", [](const Tensor &mask) {
