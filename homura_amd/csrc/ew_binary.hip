@@ -7,10 +7,6 @@ namespace {
 
 using CompareOps = std::integer_sequence<int, HMR_BINARY_GREATER, HMR_BINARY_GREATER_EQUAL, HMR_BINARY_LESS,
                                          HMR_BINARY_LESS_EQUAL, HMR_BINARY_EQUAL, HMR_BINARY_NOT_EQUAL>;
-using IntOps = std::integer_sequence<int, HMR_BINARY_ADD, HMR_BINARY_SUB, HMR_BINARY_MUL, HMR_BINARY_POW,
-                                     HMR_BINARY_MAXIMUM, HMR_BINARY_MINIMUM, HMR_BINARY_BITWISE_AND>;
-using FloatOps = std::integer_sequence<int, HMR_BINARY_ADD, HMR_BINARY_SUB, HMR_BINARY_MUL, HMR_BINARY_DIV,
-                                       HMR_BINARY_POW, HMR_BINARY_MAXIMUM, HMR_BINARY_MINIMUM>;
 using MixedOps = std::integer_sequence<int, HMR_BINARY_ADD, HMR_BINARY_SUB, HMR_BINARY_MUL, HMR_BINARY_DIV>;
 
 bool is_float(int d) { return d >= HMR_F16 && d <= HMR_F64; }
@@ -58,17 +54,9 @@ bool pick_binary(int op, int out_dtype, int a_dtype, int b_dtype, const MapCall 
             default: return false;
         }
     }
-    if (with_int_type(dtype, [&](auto t) {
-            using T = typename decltype(t)::type;
-            done = with_code(op, IntOps{}, [&](auto o) { launch_map<IntBinary<decltype(o)::value, T>>(call, stream); });
-        })) {
-        return done;
-    }
-    with_float_type(dtype, [&](auto t) {
-        using T = typename decltype(t)::type;
-        done = with_code(op, FloatOps{}, [&](auto o) { launch_map<FloatBinary<decltype(o)::value, T>>(call, stream); });
-    });
-    return done;
+    // Same-dtype arithmetic: the integer and the float kernels are translation units of their own.
+    if (dtype >= HMR_U8 && dtype <= HMR_I64) return launch_int_binary(op, dtype, call, stream);
+    return launch_float_binary(op, dtype, call, stream);
 }
 
 }  // namespace

@@ -1,0 +1,17 @@
+// The same-dtype float kernels of hmr_binary / hmr_binary_constant (see ew_binary.hip).
+#include "ew_common.hpp"
+
+namespace hmr {
+
+bool launch_float_binary(int op, int dtype, const MapCall &call, hipStream_t stream) {
+    using FloatOps = std::integer_sequence<int, HMR_BINARY_ADD, HMR_BINARY_SUB, HMR_BINARY_MUL, HMR_BINARY_DIV,
+                                           HMR_BINARY_POW, HMR_BINARY_MAXIMUM, HMR_BINARY_MINIMUM>;
+    bool done = false;
+    with_float_type(dtype, [&](auto t) {
+        using T = typename decltype(t)::type;
+        done = with_code(op, FloatOps{}, [&](auto o) { launch_map<FloatBinary<decltype(o)::value, T>>(call, stream); });
+    });
+    return done;
+}
+
+}  // namespace hmr

@@ -28,4 +28,9 @@ hmr_status run_map(hmr_context_t ctx, const char *what, int count, const hmr_ten
     return run_map(ctx, what, count, descs, bits, pick, [](const MapCall &) { return HMR_OK; });
 }
 
+// The same-dtype arithmetic kernels of hmr_binary, one translation unit per family (ew_binary_int.hip,
+// ew_binary_float.hip); false when there is no kernel for the op and dtype.
+bool launch_int_binary(int op, int dtype, const MapCall &call, hipStream_t stream);
+bool launch_float_binary(int op, int dtype, const MapCall &call, hipStream_t stream);
+
 }  // namespace hmr

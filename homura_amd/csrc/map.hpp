@@ -300,14 +300,14 @@ struct Chunk<Unused, V> {
 
 // Loads the chunk at `p` (dense) or the aligned chunk containing the element at `p` (splat);
 // `low` is the element's byte offset inside that chunk.
-template <class T, int V>
+template <class T, int V, bool STREAM = kStreamLoads>
 __device__ __forceinline__ typename Chunk<T, V>::Raw load_chunk(const char *p, bool splat, int &low) {
     using Raw = typename Chunk<T, V>::Raw;
     constexpr int bytes = Chunk<T, V>::bytes;
     // Pointer arithmetic only: an integer-to-pointer cast would lose the global address space.
     low = static_cast<int>(reinterpret_cast<uintptr_t>(p) & static_cast<uintptr_t>(bytes - 1));
     const Raw *q = reinterpret_cast<const Raw *>(splat ? p - low : p);
-    if constexpr (kStreamLoads) return __builtin_nontemporal_load(q);
+    if constexpr (STREAM) return __builtin_nontemporal_load(q);
     else return *q;
 }
 
@@ -376,7 +376,10 @@ __device__ __forceinline__ void read_ragged(T (&r)[V], const char *base, uint64_
 
 // FLAT: one dimension (contiguous / scalar-broadcast operands); its last tile may be ragged.
 // Otherwise the innermost size is a multiple of V and rows never straddle a tile.
-template <class F, bool FLAT>
+// CACHED: bit k set = input k is loaded through the caches (a broadcast operand, read by many waves); the other
+// inputs stream past them with nontemporal loads. The choice has to be made at compile time: loads that differ
+// only in the hint are folded into one plain load.
+template <class F, bool FLAT, int CACHED = 0>
 __global__ void __launch_bounds__(kBlock) map_rows_kernel(RowsArgs<F::N + 1> a) {
     using T = MapTraits<F>;
     constexpr int V = T::V, U = T::U, N = F::N;
@@ -434,12 +437,12 @@ __global__ void __launch_bounds__(kBlock) map_rows_kernel(RowsArgs<F::N + 1> a) 
                 Off off[4];
                 offsets(t0 + static_cast<int64_t>(u) * kBlock, off);
                 oo[u] = off[0];
-                wa[u] = load_chunk<A, V>(a.ptr[1] + static_cast<int64_t>(off[1]) * static_cast<int64_t>(sizeof(A)), s0, la[u]);
+                wa[u] = load_chunk<A, V, kStreamLoads && !(CACHED & 1)>(a.ptr[1] + static_cast<int64_t>(off[1]) * static_cast<int64_t>(sizeof(A)), s0, la[u]);
                 if constexpr (N >= 2) {
-                    wb[u] = load_chunk<B, V>(a.ptr[2] + static_cast<int64_t>(off[2]) * static_cast<int64_t>(sizeof(B)), s1, lb[u]);
+                    wb[u] = load_chunk<B, V, kStreamLoads && !(CACHED & 2)>(a.ptr[2] + static_cast<int64_t>(off[2]) * static_cast<int64_t>(sizeof(B)), s1, lb[u]);
                 }
                 if constexpr (N >= 3) {
-                    wc[u] = load_chunk<C, V>(a.ptr[3] + static_cast<int64_t>(off[3]) * static_cast<int64_t>(sizeof(C)), s2, lc[u]);
+                    wc[u] = load_chunk<C, V, kStreamLoads && !(CACHED & 4)>(a.ptr[3] + static_cast<int64_t>(off[3]) * static_cast<int64_t>(sizeof(C)), s2, lc[u]);
                 }
             }
 #pragma unroll
@@ -682,8 +685,36 @@ void launch_map(const MapCall &c, hipStream_t stream) {
         RowsArgs<NOPS> a = rows_args<F>(c, variant);
         int64_t tiles = (c.n + T::V - 1) / T::V;
         unsigned grid = grid_for(tiles, int64_t{T::U} * kBlock);
-        if (variant == 0) hipLaunchKernelGGL((map_rows_kernel<F, true>), dim3(grid), dim3(kBlock), 0, stream, a);
-        else hipLaunchKernelGGL((map_rows_kernel<F, false>), dim3(grid), dim3(kBlock), 0, stream, a);
+        // Which inputs are broadcast (a zero stride in some dimension). Three patterns get kernels of their own:
+        // every input (an outer product), the first one only, the second one only (x + bias, x * scale).
+        int reused = 0, inputs = 0;
+        for (int k = 1; k < NOPS; ++k) {
+            if (c.is_const[k]) continue;
+            inputs |= 1 << (k - 1);
+            for (int d = 0; d < c.ndim; ++d) {
+                if (c.stride[k][d] == 0) reused |= 1 << (k - 1);
+            }
+        }
+        auto run = [&](auto flat) {
+            constexpr bool kFlat = decltype(flat)::value;
+            if constexpr (F::N >= 2) {
+                if (inputs != 0 && reused == inputs) {
+                    hipLaunchKernelGGL((map_rows_kernel<F, kFlat, 7>), dim3(grid), dim3(kBlock), 0, stream, a);
+                    return;
+                }
+                if (reused == 1) {
+                    hipLaunchKernelGGL((map_rows_kernel<F, kFlat, 1>), dim3(grid), dim3(kBlock), 0, stream, a);
+                    return;
+                }
+                if (reused == 2) {
+                    hipLaunchKernelGGL((map_rows_kernel<F, kFlat, 2>), dim3(grid), dim3(kBlock), 0, stream, a);
+                    return;
+                }
+            }
+            hipLaunchKernelGGL((map_rows_kernel<F, kFlat, 0>), dim3(grid), dim3(kBlock), 0, stream, a);
+        };
+        if (variant == 0) run(std::true_type{});
+        else run(std::false_type{});
         return;
     }
     unsigned grid = grid_for(c.n, kBlock);
