@@ -250,7 +250,8 @@ struct SoftmaxArgs {
 //
 // WALK = false: the rows form one dimension (row r starts r * stride elements in), which is what a
 // contiguous tensor gives; WALK = true: up to 25 row dimensions, decoded per row.
-template <class T, int G, int C, bool LOG, bool WALK>
+// NTSTORE: nontemporal stores, for outputs far larger than the memory-side cache.
+template <class T, int G, int C, bool LOG, bool WALK, bool NTSTORE = false>
 __global__ void __launch_bounds__(G > kBlock ? G : kBlock) softmax_regs_kernel(SoftmaxArgs a) {
     using M = SoftmaxMath<T>;
     using X = typename M::X;
@@ -356,7 +357,7 @@ __global__ void __launch_bounds__(G > kBlock ? G : kBlock) softmax_regs_kernel(S
             }
             if (live && tile < nvec) {
                 u32x4 *q = reinterpret_cast<u32x4 *>(reinterpret_cast<char *>(out) + static_cast<uint32_t>(tile) * 16u);
-                if constexpr (kStreamStores) __builtin_nontemporal_store(M::pack(res), q);
+                if constexpr (kStreamStores || NTSTORE) __builtin_nontemporal_store(M::pack(res), q);
                 else *q = M::pack(res);
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -495,7 +496,9 @@ void launch_softmax(const SoftmaxPlan &p, const SoftmaxArgs &a, bool out_ok, hip
         auto run = [&](auto g, auto c) {
             constexpr int G = decltype(g)::value, C = decltype(c)::value;
             constexpr int kThreads = G > kBlock ? G : kBlock;
-            if (a.src_rows.ndim <= 1) {
+            if (a.src_rows.ndim <= 1 && a.nrows * a.n * static_cast<int64_t>(sizeof(T)) >= kStreamStoreBytes) {
+                hipLaunchKernelGGL((softmax_regs_kernel<T, G, C, LOG, false, true>), blocks(kThreads / G), dim3(kThreads), 0, stream, a);
+            } else if (a.src_rows.ndim <= 1) {
                 hipLaunchKernelGGL((softmax_regs_kernel<T, G, C, LOG, false>), blocks(kThreads / G), dim3(kThreads), 0, stream, a);
             } else {
                 hipLaunchKernelGGL((softmax_regs_kernel<T, G, C, LOG, true>), blocks(kThreads / G), dim3(kThreads), 0, stream, a);
