@@ -47,6 +47,8 @@ constexpr int64_t kStreamBytes = int64_t{32} << 20;
 // Outputs from this size on are stored with the nontemporal hint (measured: 537 MB outputs of i64 ops and of the
 // f32 softmax gain 3-6 %, 268 MB outputs lose 3-5 %; the memory-side cache holds 256 MB).
 constexpr int64_t kStreamStoreBytes = int64_t{384} << 20;
+// Calls that move no more than this in all go through the caches (the memory-side cache holds 256 MB).
+constexpr int64_t kCacheResidentBytes = int64_t{224} << 20;
 
 struct Unused {};
 
@@ -702,7 +704,14 @@ void launch_map(const MapCall &c, hipStream_t stream) {
         auto run = [&](auto flat) {
             constexpr bool kFlat = decltype(flat)::value;
             if constexpr (F::N >= 2) {
-                if (inputs != 0 && reused == inputs) {
+                // A call whose operands all fit in the memory-side cache together: what the previous kernel left
+                // there (or this one, called again) is found again only by cached loads.
+                constexpr int sizes[4] = {T::so, T::s0, T::s1, T::s2};
+                int64_t bytes = c.n * sizes[0];
+                for (int k = 1; k < NOPS; ++k) {
+                    if (!c.is_const[k] && !(reused & (1 << (k - 1)))) bytes += c.n * sizes[k];
+                }
+                if ((inputs != 0 && reused == inputs) || bytes <= kCacheResidentBytes) {
                     hipLaunchKernelGGL((map_rows_kernel<F, kFlat, 7>), dim3(grid), dim3(kBlock), 0, stream, a);
                     return;
                 }

@@ -47,6 +47,11 @@ def test_config_1_broadcast_chain_with_promotion_is_bit_exact():
     # Each intermediate too: two bf16 roundings.
     assert_same(gx.add(gb), x.add(bias), "cfg1 step 1")
     assert_same(gx.add(gb).mul(gs), x.add(bias).mul(scale), "cfg1 step 2")
+    # The broadcast operand first (another form of the kernel: which inputs go through the caches is chosen per
+    # launch), and both operands broadcast (an outer sum of the bias and the scale).
+    assert_same(gb.add(gx), x.add(bias), "cfg1 step 1, bias first")
+    assert_same(gs.mul(gx.add(gb)), x.add(bias).mul(scale), "cfg1 step 2, scale first")
+    assert_same(gs.add(gb), scale.add(bias), "bias + scale, both broadcast")
 
 
 def test_config_2_reductions_stay_within_one_ulp():

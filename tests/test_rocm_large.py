@@ -27,6 +27,10 @@ def test_more_than_two_to_the_31_elements():
     got = array(x.add(y))
     assert got.shape == (N,) and np.array_equal(got, a + b)
     del got
+    # A conversion (one input; the output is large enough for the streaming stores).
+    got = array(x.to(DT.I8))
+    assert np.array_equal(got, a.astype(np.int8))
+    del got
     # A comparison into bool.
     got = array(x.greater(y))
     assert np.array_equal(got, (a > b).astype(np.uint8))
