@@ -165,9 +165,10 @@ def main():
     line = {
         "metric": METRIC, "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "bf16+f32", "data": "synthetic",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "configs[1]: ((x_bf16[8,2048,4096] + bias_bf16[4096]) * scale_bf16[8,2048,1]) + "
                                "residual_f32[8,2048,4096] -> f32; 3 kernel launches per step",
+                   "storage": "bf16 operands and intermediates, f32 residual and result; every op computes in f32",
                    "algorithmic_bytes_per_step": chain_bytes, "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
                    "seeds": "SplitMix64 0x5EED0001..4"},
         "roofline": roofline, "cpu_baseline": cpu, "ops": ops,
