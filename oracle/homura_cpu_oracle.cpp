@@ -14,7 +14,20 @@
 //   int_pow, erf                         ref: src/backend/cpu/num.rs:160-219
 //   fold, reduce, var, arg_reduce        ref: src/backend/cpu/reduce.rs:10-225
 //   softmax                              ref: src/backend/cpu/misc.rs:13-51
+//   fused optimizer steps                ref: src/backend/cpu/mod.rs:509-569
+//   addr                                 ref: src/backend/cpu/linalg.rs:224-388
+//   triangle, flip                       ref: src/backend/cpu/misc.rs:347-411
+//   exclusive_cumprod                    ref: src/backend/cpu/reduce.rs:286-324
+//   Philox blocks, uniform, normal, int  ref: src/ops/random.rs:29-226
+//   positions, index_select, gather,     ref: src/backend/cpu/misc.rs:53-127, 213-345
+//   index_add, scatter_add (add_at)
+//   index_overwrite, mask_coordinates,   ref: src/backend/cpu/misc.rs:104-203
+//   index_positions
 //   element conversions                  elements.hpp
+//
+// What pins each part (golden vectors of the reference, known answers, independent arithmetic) is listed
+// beside the tests that do it: tests/test_golden_ops.py, test_optim_golden.py, test_gradient_golden.py,
+// test_oracle_kats.py, test_random.py, test_advanced_index.py.
 //
 // Transcendental functions: Rust's f32/f64 methods (exp, ln, sin, cos, tanh, powf, ln_1p) lower
 // to the platform libm; this file calls the same glibc functions. Their last-bit behaviour is
