@@ -303,6 +303,30 @@ def test_tails_and_alignments():
             assert_bitwise(gv.mul(scale.to(GPU)), v.mul(scale), f"scale {dtype} {cols}/{pitch}")
 
 
+def test_transposed_outer_dimensions_in_every_depth():
+    """Views whose two innermost outer dimensions are swapped, under one to four more dimensions: the rows kernel
+    walks such a pair in tiles, which splits a dimension (up to its five outer dimensions), or not at all when
+    there is no room; with a second operand that is contiguous, broadcast or permuted the other way."""
+    shapes = [([16, 8, 32], [1, 0, 2]), ([3, 16, 8, 32], [0, 2, 1, 3]), ([2, 3, 16, 8, 32], [0, 1, 3, 2, 4]),
+              ([2, 2, 3, 16, 8, 32], [0, 1, 2, 4, 3, 5]), ([2, 2, 2, 3, 16, 8, 32], [0, 1, 2, 3, 5, 4, 6]),
+              ([24, 9, 16], [1, 0, 2]), ([40, 8, 8], [1, 0, 2])]
+    for dtype in (DT.BF16, DT.F32, DT.I64):
+        for shape, perm in shapes:
+            n = int(np.prod(shape))
+            a, b = tensor(values(dtype, n, 81), dtype, shape), tensor(values(dtype, n, 82), dtype, shape)
+            ga, gb = a.to(GPU), b.to(GPU)
+            pa, pga = a.permute(perm), ga.permute(perm)
+            out_shape = pa.shape
+            name = "add"
+            what = f"{dtype} {shape} permuted {perm}"
+            assert_bitwise(pga.contiguous(), pa.contiguous(), f"copy of {what}")
+            assert_bitwise(getattr(pga, name)(gb.reshape(out_shape)), getattr(pa, name)(b.reshape(out_shape)), f"{what} + contiguous")
+            assert_bitwise(getattr(pga, name)(gb.permute(perm)), getattr(pa, name)(b.permute(perm)), f"{what} + the same view")
+            last = tensor(values(dtype, out_shape[-1], 83), dtype, [out_shape[-1]])
+            assert_bitwise(getattr(pga, name)(last.to(GPU)), getattr(pa, name)(last), f"{what} + bias")
+            assert_bitwise(pga.neg() if dtype != DT.I64 else pga.abs(), pa.neg() if dtype != DT.I64 else pa.abs(), f"unary of {what}")
+
+
 def test_uniform_operands_in_every_position():
     """An operand broadcast from one element, in each position (ref: rocm_elementwise.rs:864-937)."""
     for dtype in (DT.F32, DT.BF16, DT.I32):
