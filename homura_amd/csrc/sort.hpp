@@ -2,7 +2,7 @@
 // deterministic adds of the indexing kernels: word = (target << 32) | position, positions ascending on input, so
 // sorting stably by the target's bits alone leaves every target's positions in order.
 //
-// A pass handles 8 bits. Workgroups take tiles of 4096 words:
+// A pass handles 8 bits. Workgroups take tiles of 2048 words:
 //   count    the tile's digit histogram into hist[digit][tile] (digit-major, so that one exclusive scan of the whole
 //            table gives, for every digit and tile, where the tile's words of that digit go);
 //   scan     the table in chunks of 4096 entries, then the chunks' totals by one workgroup;
@@ -17,7 +17,7 @@
 namespace hmr {
 
 constexpr int kSortThreads = 256;
-constexpr int kSortRounds = 16;  // words per thread
+constexpr int kSortRounds = 8;  // words per thread (4 and 16 measured slower)
 constexpr int kSortTile = kSortThreads * kSortRounds;
 constexpr int kSortDigits = 256;
 constexpr int kSortWaves = kSortThreads / 64;

@@ -224,9 +224,9 @@ def test_positions_out_of_range_report_what_the_cpu_reports():
 
 
 def sort_bytes(n):
-    """The workspace of the adds: two buffers of n 64-bit words, a 256-entry histogram per tile of 4096 words and a
+    """The workspace of the adds: two buffers of n 64-bit words, a 256-entry histogram per tile of 2048 words and a
     word per 4096 histogram entries, rounded up to 256 bytes."""
-    tiles = -(-n // 4096)
+    tiles = -(-n // 2048)
     chunks = -(-tiles * 256 // 4096)
     return -(-(16 * n + 4 * 256 * tiles + 4 * chunks) // 256) * 256
 
@@ -275,7 +275,7 @@ def test_the_c_abi_of_the_index_kernels():
         n = 5000
         need = c_int64()
         capi.check(L.hmr_scatter_add_workspace(n, byref(need)))
-        assert need.value == sort_bytes(n) == 82176
+        assert need.value == sort_bytes(n) == 83200
         capi.check(L.hmr_index_add_workspace(100, 7, byref(need)))
         assert need.value == sort_bytes(100) == 2816
         assert L.hmr_index_add_workspace(1 << 31, 7, byref(need)) == capi.HMR_INVALID
