@@ -64,12 +64,19 @@ static __global__ void __launch_bounds__(kSortThreads) radix_count_kernel(const 
     counts[threadIdx.x] = 0;
     __syncthreads();
     const int64_t base = static_cast<int64_t>(blockIdx.x) * kSortTile;
+    uint64_t word[kSortRounds];
+#pragma unroll
+    for (int r = 0; r < kSortRounds; ++r) {  // every load is out before the first ballot waits for one
+        const int64_t i = base + r * kSortThreads + threadIdx.x;
+        word[r] = i < n ? words[i] : 0;
+    }
+#pragma unroll
     for (int r = 0; r < kSortRounds; ++r) {
         const int64_t i = base + r * kSortThreads + threadIdx.x;
         const bool valid = i < n;
         const uint64_t lanes = __builtin_amdgcn_ballot_w64(valid);
         if (valid) {
-            const uint32_t digit = static_cast<uint32_t>(words[i] >> shift) & 0xFFu;
+            const uint32_t digit = static_cast<uint32_t>(word[r] >> shift) & 0xFFu;
             const uint64_t peers = same_digit(digit, lanes);
             if (lanes_below(peers) == 0) atomicAdd(&counts[digit], static_cast<uint32_t>(__popcll(peers)));
         }
