@@ -9,8 +9,6 @@ using CompareOps = std::integer_sequence<int, HMR_BINARY_GREATER, HMR_BINARY_GRE
                                          HMR_BINARY_LESS_EQUAL, HMR_BINARY_EQUAL, HMR_BINARY_NOT_EQUAL>;
 using MixedOps = std::integer_sequence<int, HMR_BINARY_ADD, HMR_BINARY_SUB, HMR_BINARY_MUL, HMR_BINARY_DIV>;
 
-bool is_float(int d) { return d >= HMR_F16 && d <= HMR_F64; }
-
 // Mixed float inputs (extension): a half with F32, output F32.
 template <class A, class B>
 bool pick_mixed(int op, const MapCall &call, hipStream_t stream) {

@@ -36,8 +36,6 @@ int64_t build_walk(const hmr_tensor_desc &d, Walk &w) {
 
 int64_t ceil_div(int64_t a, int64_t b) { return a / b + (a % b != 0); }
 
-int64_t clamp64(int64_t v, int64_t lo, int64_t hi) { return v < lo ? lo : (v > hi ? hi : v); }
-
 // Cuts nred into at most `want` slices of a multiple of `quantum` elements.
 void cut(ReducePlan &p, int64_t want, int64_t quantum) {
     int64_t nred = p.args.nred;

@@ -75,12 +75,35 @@ def test_every_symbol_binds_through_ctypes():
     assert set(capi.PROTOTYPES) | set(capi.UNBUILT) >= set(RUST_FFI)
 
 
-def test_static_archive_is_built_beside_the_shared_library():
-    archive = os.path.join(os.path.dirname(capi.LIB_PATH), "libhomura_rocm.a")
-    assert os.path.exists(archive), "the Rust build links libhomura_rocm.a (ref: build.rs:60-70)"
-    out = subprocess.check_output(["nm", "--defined-only", "-g", archive], text=True, stderr=subprocess.DEVNULL)
+ARCHIVE = os.path.join(os.path.dirname(capi.LIB_PATH), "libhomura_rocm.a")
+
+
+def test_static_archive_is_one_object_with_only_hmr_symbols_global():
+    """The Rust build links libhomura_rocm.a: one relocatable object in which only hmr_* stay global
+    (ref: build.rs:231-250; linked at build.rs:60-70)."""
+    assert os.path.exists(ARCHIVE)
+    members = subprocess.check_output(["ar", "t", ARCHIVE], text=True).split()
+    assert members == ["homura_rocm.o"], members
+    out = subprocess.check_output(["nm", "--defined-only", "-g", ARCHIVE], text=True, stderr=subprocess.DEVNULL)
     have = {line.split()[-1] for line in out.splitlines() if len(line.split()) == 3}
     assert set(RUST_FFI) <= have
+    stray = {s for s in have if not s.startswith("hmr_")}
+    assert not stray, sorted(stray)[:20]
+    # Nothing is left for the linker to find except what the Rust build links beside it: the HIP runtime,
+    # the C++ runtime and libc / libm.
+    out = subprocess.check_output(["nm", "--undefined-only", ARCHIVE], text=True, stderr=subprocess.DEVNULL)
+    undefined = {line.split()[-1] for line in out.splitlines() if len(line.split()) == 2}
+    assert not {s for s in undefined if s.startswith("hmr_")}, "an hmr_* symbol is not defined in the archive"
+
+
+def test_a_c_program_links_statically_against_the_archive(tmp_path):
+    """Linked here from source, so the test fails if the archive needs anything but amdhip64 and stdc++."""
+    exe = tmp_path / "static_check"
+    source = os.path.join(ROOT, "homura_amd", "csrc", "static_check.c")
+    subprocess.check_call(["gcc", "-O1", "-I", INCLUDE, source, ARCHIVE, "-L/opt/rocm/lib", "-lamdhip64", "-lstdc++",
+                           "-lm", "-lpthread", "-Wl,-rpath,/opt/rocm/lib", "-o", str(exe)])
+    out = subprocess.check_output([str(exe)], text=True)
+    assert out.startswith("archs gfx950, desc 424 bytes, max dims 25")
 
 
 def test_abi_layout():
