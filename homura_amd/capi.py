@@ -83,6 +83,7 @@ PROTOTYPES = {
     "hmr_flip": (c_int32, [CTX, DESC_P, DESC_P]),
     "hmr_reduce_workspace": (c_int32, [DESC_P, DESC_P, c_int32, POINTER(c_int64)]),
     "hmr_reduce": (c_int32, [CTX, c_int32, DESC_P, DESC_P, DESC_P, c_void_p, c_int64]),
+    "hmr_reduce_static": (c_int32, [CTX, c_int32, DESC_P, DESC_P, DESC_P]),
     "hmr_var": (c_int32, [CTX, DESC_P, DESC_P, DESC_P, c_double, c_int32, c_void_p, c_int64]),
     "hmr_arg_reduce": (c_int32, [CTX, DESC_P, DESC_P, DESC_P, DESC_P, c_int32, c_void_p, c_int64]),
     "hmr_softmax_workspace": (c_int32, [DESC_P, c_int64, c_int64, POINTER(c_int64)]),

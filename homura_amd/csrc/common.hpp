@@ -24,6 +24,9 @@ struct hmr_context {
     std::mutex table_lock;
     void *tables = nullptr;
     uint64_t tables_filled = 0;  // bit per table
+    // Device address, on this context's GPU, of the library's static block for partial results
+    // (hmr_reduce_static). Each GPU holds its own copy of the block at its own address.
+    void *reduce_scratch = nullptr;
 };
 
 namespace hmr {
@@ -46,6 +49,10 @@ hmr_status hip_fail(hipError_t error, const char *call) noexcept;
         hipError_t hmr_hip_e_ = (expr);                                       \
         if (hmr_hip_e_ != hipSuccess) return ::hmr::hip_fail(hmr_hip_e_, #expr); \
     } while (0)
+
+// Looks up where the static block of hmr_reduce_static lives on the current device and keeps the address
+// in the context. Called once per context, with its device current (defined beside the block, reduce.hip).
+hmr_status bind_reduce_scratch(hmr_context &ctx);
 
 // Consumes one failure armed by hmr_test_fail_data, if any: returns its status, else HMR_OK.
 hmr_status injected_data_failure(const char *call) noexcept;

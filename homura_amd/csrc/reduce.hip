@@ -2,6 +2,12 @@
 // hmr_test_reduce_plan (ref: csrc/homura_rocm.h:297-336, csrc/reduce.hip:133-170, 432-517).
 #include "reduce_plan.hpp"
 
+// Where hmr_reduce_static stages its partial results: a block inside the library's code object, so each
+// GPU the library runs on holds its own copy at its own address until the process ends. In host code this
+// name is only a handle for hipGetSymbolAddress (bind_reduce_scratch below); every use goes through the
+// address that call returns, kept in the context.
+static __device__ __align__(256) unsigned char scratch[HMR_REDUCE_STATIC_BYTES];
+
 namespace hmr {
 namespace {
 
@@ -172,7 +178,49 @@ void *element0(const hmr_tensor_desc &d) { return static_cast<char *>(d.data) + 
 
 bool is_float(int d) { return d >= HMR_F16 && d <= HMR_F64; }
 
+// One reduction, planned and queued; the body of hmr_reduce and hmr_reduce_static.
+hmr_status run_reduce(hmr_context_t ctx, int32_t op, const hmr_tensor_desc *out, const hmr_tensor_desc *kept,
+                      const ReducePlan &p, void *partials) {
+    if (p.args.nout == 0) return HMR_OK;
+    if ((op == HMR_REDUCE_MAX || op == HMR_REDUCE_MIN) && p.args.nred == 0) {
+        return fail(HMR_INVALID, "reduction over an empty dimension");
+    }
+    return launch_on(ctx, "reduce", [&](hipStream_t stream) {
+        const int dtype = kept->dtype;
+        void *o = element0(*out);
+        switch (op) {
+            case HMR_REDUCE_SUM:
+            case HMR_REDUCE_PROD:
+            case HMR_REDUCE_MEAN:
+                if (is_float(dtype)) {
+                    if (out->dtype != dtype) return false;
+                    return launch_float_reduce(op, dtype, p, partials, o, stream);
+                }
+                if (op == HMR_REDUCE_MEAN || out->dtype != HMR_I64) return false;
+                return launch_int_reduce(op, dtype, p, partials, o, stream);
+            case HMR_REDUCE_MAX:
+            case HMR_REDUCE_MIN:
+                if (out->dtype != dtype) return false;
+                return launch_extreme_reduce(op == HMR_REDUCE_MAX, dtype, p, partials, o, nullptr, stream);
+            case HMR_REDUCE_ALL:
+            case HMR_REDUCE_ANY:
+                if (out->dtype != (dtype == HMR_U8 ? HMR_U8 : HMR_BOOL)) return false;
+                return launch_truth_reduce(op, dtype, p, partials, o, stream);
+            default: return false;
+        }
+    });
+}
+
 }  // namespace
+
+hmr_status bind_reduce_scratch(hmr_context &ctx) {
+    void *address = nullptr;
+    HMR_HIP(hipGetSymbolAddress(&address, HIP_SYMBOL(::scratch)));
+    if (address == nullptr) return fail(HMR_INTERNAL_ERROR, "the static reduction block has no device address");
+    ctx.reduce_scratch = address;
+    return HMR_OK;
+}
+
 }  // namespace hmr
 
 using hmr::guarded;
@@ -208,34 +256,25 @@ hmr_status hmr_reduce(hmr_context_t ctx, int32_t op, const hmr_tensor_desc *out,
         if (hmr_status s = hmr::plan_reduction(out, *kept, *red, p)) return s;
         void *partials = nullptr;
         if (hmr_status s = hmr::take_workspace(p, false, workspace, workspace_bytes, partials)) return s;
-        if (p.args.nout == 0) return HMR_OK;
-        if ((op == HMR_REDUCE_MAX || op == HMR_REDUCE_MIN) && p.args.nred == 0) {
-            return hmr::fail(HMR_INVALID, "reduction over an empty dimension");
+        return hmr::run_reduce(ctx, op, out, kept, p, partials);
+    });
+}
+
+hmr_status hmr_reduce_static(hmr_context_t ctx, int32_t op, const hmr_tensor_desc *out, const hmr_tensor_desc *kept,
+                             const hmr_tensor_desc *red) {
+    return guarded([&] {
+        hmr::ReducePlan p;
+        if (hmr_status s = hmr::plan_reduction(out, *kept, *red, p)) return s;
+        const int64_t need = hmr::partial_bytes(p, false);
+        if (need > HMR_REDUCE_STATIC_BYTES) {
+            return hmr::fail(HMR_INVALID, "hmr_reduce_static: this reduction stages " + std::to_string(need) +
+                                              " bytes of partial results, the library's block holds " +
+                                              std::to_string(HMR_REDUCE_STATIC_BYTES) +
+                                              "; call hmr_reduce with a workspace");
         }
-        return hmr::launch_on(ctx, "reduce", [&](hipStream_t stream) {
-            const int dtype = kept->dtype;
-            void *o = hmr::element0(*out);
-            switch (op) {
-                case HMR_REDUCE_SUM:
-                case HMR_REDUCE_PROD:
-                case HMR_REDUCE_MEAN:
-                    if (hmr::is_float(dtype)) {
-                        if (out->dtype != dtype) return false;
-                        return hmr::launch_float_reduce(op, dtype, p, partials, o, stream);
-                    }
-                    if (op == HMR_REDUCE_MEAN || out->dtype != HMR_I64) return false;
-                    return hmr::launch_int_reduce(op, dtype, p, partials, o, stream);
-                case HMR_REDUCE_MAX:
-                case HMR_REDUCE_MIN:
-                    if (out->dtype != dtype) return false;
-                    return hmr::launch_extreme_reduce(op == HMR_REDUCE_MAX, dtype, p, partials, o, nullptr, stream);
-                case HMR_REDUCE_ALL:
-                case HMR_REDUCE_ANY:
-                    if (out->dtype != (dtype == HMR_U8 ? HMR_U8 : HMR_BOOL)) return false;
-                    return hmr::launch_truth_reduce(op, dtype, p, partials, o, stream);
-                default: return false;
-            }
-        });
+        // Every partial result the second kernel reads is written by the first one of the same call, so
+        // what an earlier call left in the block needs no clearing.
+        return hmr::run_reduce(ctx, op, out, kept, p, need > 0 ? ctx->reduce_scratch : nullptr);
     });
 }
 

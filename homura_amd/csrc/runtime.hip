@@ -235,6 +235,7 @@ hmr_status hmr_context_create(int32_t device, hmr_context_t *out) {
             --hmr::t_fail_late;
             throw std::bad_alloc();
         }
+        if (hmr_status s = hmr::bind_reduce_scratch(*ctx)) return s;
         ctx->device = device;
         ctx->compute_units = p.multiProcessorCount > 0 ? p.multiProcessorCount : 256;
         ctx->stream = holder.take();

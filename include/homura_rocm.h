@@ -265,6 +265,18 @@ hmr_status hmr_reduce(hmr_context_t ctx, int32_t op, const hmr_tensor_desc *out,
                       const hmr_tensor_desc *kept, const hmr_tensor_desc *red, void *workspace,
                       int64_t workspace_bytes);
 
+/* No counterpart in the reference. hmr_reduce for callers that cannot allocate device memory (code
+ * under HIP graph capture, serving loops, harnesses that forbid hipMalloc) and so have no workspace
+ * to pass: the partial results go to HMR_REDUCE_STATIC_BYTES of device memory that the library's
+ * code object holds on every GPU it runs on, bound when the context is created. Same results as
+ * hmr_reduce, bit for bit. HMR_INVALID, with nothing queued, when the reduction's plan needs more
+ * than that (hmr_reduce_workspace reports the need). Allocates nothing. Every call on a GPU uses
+ * that GPU's one block: calls on the same GPU must not overlap (two contexts, two threads), or their
+ * partial results race. */
+#define HMR_REDUCE_STATIC_BYTES (8 * 1024 * 1024)
+hmr_status hmr_reduce_static(hmr_context_t ctx, int32_t op, const hmr_tensor_desc *out,
+                             const hmr_tensor_desc *kept, const hmr_tensor_desc *red);
+
 /* ref :327  cpu::var (src/backend/cpu/reduce.rs:135-170): f64 variance about the f64 mean,
  * divided by max(0, n - correction); NaN for n == 0; sqrt of it with take_sqrt. */
 hmr_status hmr_var(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_tensor_desc *kept,
