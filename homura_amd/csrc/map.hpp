@@ -43,7 +43,6 @@ constexpr int kMaxOperands = 4;  // output + 3 inputs
 // one plain access.
 constexpr bool kStreamLoads = true;
 constexpr bool kStreamStores = false;
-constexpr int64_t kStreamBytes = int64_t{32} << 20;
 // Outputs from this size on are stored with the nontemporal hint (measured: 537 MB outputs of i64 ops and of the
 // f32 softmax gain 3-6 %, 268 MB outputs lose 3-5 %; the memory-side cache holds 256 MB).
 constexpr int64_t kStreamStoreBytes = int64_t{384} << 20;
@@ -110,7 +109,6 @@ struct RowsArgs {
     uint64_t cbits[NOPS];
     uint32_t const_mask;   // bit k: operand k is a constant
     uint32_t bcast_mask;   // bit k: operand k has inner stride 0
-    uint32_t stream;       // nonzero: nontemporal loads and stores (large, read-once operands)
     int64_t n;             // elements
     uint32_t inner;        // size of the innermost dimension
     int32_t nouter;        // outer dimensions (0 for contiguous)
@@ -622,7 +620,6 @@ int resolve_variant(const MapCall &c) {
 // Kernel arguments of the rows kernel for a call of variant 0 (flat) or 1 (outer dimensions).
 template <class F>
 RowsArgs<F::N + 1> rows_args(const MapCall &c, int variant) {
-    using T = MapTraits<F>;
     constexpr int NOPS = F::N + 1;
     RowsArgs<NOPS> a{};
     a.n = c.n;
@@ -635,7 +632,6 @@ RowsArgs<F::N + 1> rows_args(const MapCall &c, int variant) {
         if (c.is_const[k]) a.const_mask |= 1u << k;
         else if (c.ndim == 0 || c.stride[k][last] == 0) a.bcast_mask |= k == 0 ? 0u : 1u << k;
     }
-    a.stream = c.n * (T::so + T::s0 + T::s1 + T::s2) >= kStreamBytes ? 1u : 0u;
     if (variant == 0) {
         a.inner = static_cast<uint32_t>(c.n < (int64_t{1} << 31) ? c.n : 0);
         a.nouter = 0;

@@ -1,5 +1,7 @@
 // Reduction plans and the entry points hmr_reduce_workspace, hmr_reduce, hmr_var, hmr_arg_reduce,
 // hmr_test_reduce_plan (ref: csrc/homura_rocm.h:297-336, csrc/reduce.hip:133-170, 432-517).
+#include <algorithm>
+
 #include "reduce_plan.hpp"
 
 // Where hmr_reduce_static stages its partial results: a block inside the library's code object, so each
@@ -90,7 +92,6 @@ hmr_status plan_reduction(const hmr_tensor_desc *out, const hmr_tensor_desc &kep
     p.rstride = 0;
     p.inner = 0;
     p.across = 4;
-    a.stream = 0;
     if (a.nout == 0 || a.nred == 0) return HMR_OK;  // nothing to read: one lane per output writes the identity
 
     const bool base_aligned = reinterpret_cast<uintptr_t>(a.src) % 16 == 0;
@@ -102,13 +103,6 @@ hmr_status plan_reduction(const hmr_tensor_desc *out, const hmr_tensor_desc &kep
     };
     const bool red_contiguous = a.red.ndim == 1 && a.red.stride[0] == 1;
     const int vec = 16 / elem;
-    // Read-once sources far larger than an XCD's L2 stream past the caches. (A broadcast source,
-    // whose elements are visited repeatedly, is smaller than nout*nred and stays cached.)
-    bool dense = true;
-    for (int d = 0; d < a.kept.ndim; ++d) dense = dense && a.kept.stride[d] != 0;
-    for (int d = 0; d < a.red.ndim; ++d) dense = dense && a.red.stride[d] != 0;
-    a.stream = dense && a.nout * a.nred >= kStreamSourceBytes / elem ? 1u : 0u;
-
     // Rows: one contiguous run per output.
     if (red_contiguous && a.nred >= 256 && base_aligned && strides_aligned(a.kept, 0)) {
         p.kind = ReduceKind::Rows;
@@ -120,11 +114,11 @@ hmr_status plan_reduction(const hmr_tensor_desc *out, const hmr_tensor_desc &kep
         }
         return HMR_OK;
     }
-    // Cols: a contiguous run of outputs, one strided reduced dimension.
-    if (a.red.ndim == 1 && a.kept.ndim >= 1 && a.kept.stride[0] == 1 && a.kept.size[0] >= 32 && base_aligned &&
-        (a.red.stride[0] * elem) % 16 == 0 && strides_aligned(a.kept, 1)) {
+    // Cols: a contiguous run of outputs, one strided reduced dimension (fewer than 2^31 rows: the kernel
+    // counts rows in 32 bits).
+    if (a.red.ndim == 1 && a.nred < (int64_t{1} << 31) && a.kept.ndim >= 1 && a.kept.stride[0] == 1 &&
+        a.kept.size[0] >= 32 && base_aligned && (a.red.stride[0] * elem) % 16 == 0 && strides_aligned(a.kept, 1)) {
         p.kind = ReduceKind::Cols;
-        p.group = kBlock / kWave;
         p.rstride = a.red.stride[0];
         p.inner = a.kept.size[0];
         // The kernel walks the outer kept dimensions only.
@@ -135,14 +129,24 @@ hmr_status plan_reduction(const hmr_tensor_desc *out, const hmr_tensor_desc &kep
         a.kept.ndim -= 1;
         // As many waves side by side as the run of outputs fills (wide spans read best).
         p.across = p.inner > 2 * kWave * vec ? 4 : (p.inner > kWave * vec ? 2 : 1);
-        int64_t tiles = ceil_div(p.inner, int64_t{p.across} * kWave * vec) * (a.nout / p.inner);
-        if (elem >= 4 && p.across == 4 && tiles < 256 && a.nred >= 4096) {
-            // Few tiles of long columns: 1024-lane workgroups, one per compute unit.
-            p.group = 1024 / kWave;
-            cut(p, ceil_div(256, tiles), 128);
-        } else {
-            cut(p, ceil_div(4 * 256, tiles), 32);
-        }
+        const int64_t tiles = ceil_div(p.inner, int64_t{p.across} * kWave * vec) * (a.nout / p.inner);
+        // 1024-lane workgroups (16 / across row groups that meet in LDS: a sixteenth of the partial results
+        // of single waves) where the columns are long enough to feed them and the tile's states fit LDS
+        // (elements of four bytes or more).
+        const bool big = a.nred >= 512 && elem >= 4;
+        p.group = (big ? 1024 : kBlock) / kWave;
+        const int64_t rgroups = p.group / p.across;
+        // How many workgroups stream at once decides the rate, and more is not better: on 16384 x 4096 f32
+        // (4 tiles) 32 slices run at 46 us, 44 to 48 at 39 us, 56 at 40.6, 64 (a workgroup on every compute
+        // unit) at 40.4-41.8, 96 at 47. The plan aims at 184 workgroups of 1024 lanes (the same number of
+        // waves with 256-lane workgroups), and keeps a slice long enough that its partial results stay
+        // small beside the rows it read.
+        const int64_t target = big ? 184 : 736;
+        const int64_t min_rows = std::max<int64_t>(8 * rgroups, 256 / elem);
+        int64_t want = (target + tiles / 2) / tiles;
+        want = std::min(want, a.nred / min_rows);
+        p.splits = want > 1 ? want : 1;
+        p.chunk = ceil_div(a.nred, p.splits);  // rows per slice (they are interleaved, not consecutive)
         return HMR_OK;
     }
     // Any layout.

@@ -227,6 +227,13 @@ struct Moments {
     double n, mean, m2;
 };
 
+// 1 / x for a count x through the hardware reciprocal refined once (relative error about 2^-52). A true
+// f64 division is some thirty instructions; the weights of a merge and the mean of a lane do not need it.
+__device__ __forceinline__ double count_reciprocal(double x) {
+    const double r = __builtin_amdgcn_rcp(x);
+    return __builtin_fma(__builtin_fma(-x, r, 1.0), r, r);
+}
+
 template <class T>
 struct MomentsFold {
     using In = T;
@@ -253,9 +260,10 @@ struct MomentsFold {
     __device__ __forceinline__ Acc combine(Acc a, Acc b) const {
         if (b.n == 0.0) return a;
         if (a.n == 0.0) return b;
-        double n = a.n + b.n;
-        double delta = b.mean - a.mean;
-        return Acc{n, a.mean + delta * (b.n / n), a.m2 + b.m2 + delta * delta * (a.n * b.n / n)};
+        const double n = a.n + b.n;
+        const double delta = b.mean - a.mean;
+        const double wb = b.n * count_reciprocal(n);
+        return Acc{n, a.mean + delta * wb, a.m2 + b.m2 + delta * delta * (a.n * wb)};
     }
 };
 
@@ -326,12 +334,12 @@ struct ReduceArgs {
     int64_t splits;   // slices of the reduced range
     int64_t chunk;    // reduced elements per slice
     void *partials;   // workspace for splits > 1
-    uint32_t stream;  // nonzero: nontemporal loads (a source much larger than the caches, read once)
 };
 
+// Sources are read once: every vector load carries the nontemporal hint (a compile-time property of the load;
+// a run-time choice between the two forms is merged by the compiler into one plain load).
 template <class T, int V>
-__device__ __forceinline__ void load_tile_rt(const char *p, T (&r)[V], bool nt) {
-    (void)nt;  // a run-time choice would be merged into one plain load; the hint is compile-time
+__device__ __forceinline__ void load_stream(const char *p, T (&r)[V]) {
     load_tile<T, V, kStreamLoads>(p, r);
 }
 
@@ -378,14 +386,14 @@ __global__ void __launch_bounds__(kBlock) reduce_any_kernel(ReduceArgs a, Op op,
 // Folds the slices of each output, in an order fixed by the sizes alone. A workgroup takes OUTS
 // adjacent outputs (64, 16, 4 or 1: the fewer outputs there are, the fewer each workgroup takes, so
 // that the grid still covers the GPU); its 256 lanes are 256/OUTS slice lanes per output. A lane folds
-// every (256/OUTS)-th slice, eight loads in flight; the slice lanes of an output that share a wave meet
+// every (256/OUTS)-th slice, four loads in flight; the slice lanes of an output that share a wave meet
 // by shuffles, the four waves through LDS.
 template <class Op, class Sink, int OUTS>
 __global__ void __launch_bounds__(kBlock) combine_kernel(ReduceArgs a, Op op, Sink sink) {
     using Acc = typename Op::Acc;
     constexpr int kWaves = kBlock / kWave;
     constexpr int L = kBlock / OUTS;  // slice lanes per output
-    constexpr int U = 8;
+    constexpr int U = 4;
     __shared__ Acc lds[kWaves - 1][kWave];
     const Acc *partials = static_cast<const Acc *>(a.partials);
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
@@ -395,15 +403,20 @@ __global__ void __launch_bounds__(kBlock) combine_kernel(ReduceArgs a, Op op, Si
         const int64_t o = g * OUTS + ol;
         Acc acc = op.init();
         if (o < a.nout) {
-            int64_t s = sl;
-            for (; s + (U - 1) * L < a.splits; s += U * L) {
+            // Batches of U loads, all issued before the first is folded (a slice past the end reads the last
+            // slice again and is left out): a lane's slices cost one trip to memory per batch, not one each.
+            for (int64_t s = sl; s < a.splits; s += U * L) {
                 Acc t[U];
 #pragma unroll
-                for (int u = 0; u < U; ++u) t[u] = partials[(s + u * L) * a.nout + o];
+                for (int u = 0; u < U; ++u) {
+                    const int64_t k = s + u * L < a.splits ? s + u * L : a.splits - 1;
+                    t[u] = partials[k * a.nout + o];
+                }
 #pragma unroll
-                for (int u = 0; u < U; ++u) acc = op.combine(acc, t[u]);
+                for (int u = 0; u < U; ++u) {
+                    if (s + u * L < a.splits) acc = op.combine(acc, t[u]);
+                }
             }
-            for (; s < a.splits; s += L) acc = op.combine(acc, partials[s * a.nout + o]);
         }
         // Slice lanes of one output inside a wave sit OUTS lanes apart.
 #pragma unroll
@@ -435,7 +448,6 @@ __global__ void __launch_bounds__(kBlock) reduce_rows_kernel(ReduceArgs a, Op op
     constexpr int U = 4;  // loads in flight per lane
     __shared__ Acc lds[WAVES == 4 ? 4 : 1];
     const int lane = threadIdx.x % G;
-    const bool nt = a.stream != 0;
     const int64_t split = blockIdx.y;
     const int64_t begin = split * a.chunk;
     const int64_t end = begin + a.chunk < a.nred ? begin + a.chunk : a.nred;
@@ -454,7 +466,7 @@ __global__ void __launch_bounds__(kBlock) reduce_rows_kernel(ReduceArgs a, Op op
                 T r[U][V];
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
-                    load_tile_rt<T, V>(reinterpret_cast<const char *>(p + begin + (k + u * G) * V), r[u], nt);
+                    load_stream<T, V>(reinterpret_cast<const char *>(p + begin + (k + u * G) * V), r[u]);
                 }
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
@@ -464,7 +476,7 @@ __global__ void __launch_bounds__(kBlock) reduce_rows_kernel(ReduceArgs a, Op op
             }
             for (; k < nvec; k += G) {
                 T r[V];
-                load_tile_rt<T, V>(reinterpret_cast<const char *>(p + begin + k * V), r, nt);
+                load_stream<T, V>(reinterpret_cast<const char *>(p + begin + k * V), r);
 #pragma unroll
                 for (int i = 0; i < V; ++i) op.lane_add(state, r[i], begin + k * V + i, ctx);
             }
@@ -487,15 +499,81 @@ __global__ void __launch_bounds__(kBlock) reduce_rows_kernel(ReduceArgs a, Op op
     }
 }
 
-// Contiguous outputs ("columns"), one strided reduced dimension. `rstride` is that stride and
-// `inner` the length of the contiguous run of outputs (the innermost kept dimension); a.kept
-// holds the remaining, outer kept dimensions. Every row of every tile starts 16-byte aligned.
-// `across` (1, 2 or 4) waves of the workgroup sit side by side on a span of across*64*V columns;
-// the other 4/across wave groups take interleaved rows of the slice.
+// ---- the column kernel ----------------------------------------------------------------------------
 //
-// BLOCK = 256, or 1024 with across = 4: sixteen waves, four row groups on one 4 KB-wide span. The big
-// workgroup is for few column tiles and long columns: the same number of waves per compute unit reads
-// the same spans, but a slice is four times as long, so four times fewer partial results are staged.
+// Per-column state of a lane of the column kernel. The kernel feeds a lane the rows of its columns in
+// increasing order, the first one through `first`, which seeds the state, so that the update of the
+// following rows tests nothing about emptiness; row numbers are 32-bit (the plan keeps the column kernel
+// below 2^31 rows) and the kernel knows how many rows it fed when it asks for the accumulator.
+template <class Op, class = void>
+struct ColState {
+    using T = typename Op::In;
+    typename Op::Lane s;
+    __device__ __forceinline__ void first(const Op &op, T x, int32_t r, typename Op::Ctx c) {
+        s = op.lane_init();
+        op.lane_add(s, x, r, c);
+    }
+    __device__ __forceinline__ void next(const Op &op, T x, int32_t r, typename Op::Ctx c) { op.lane_add(s, x, r, c); }
+    __device__ __forceinline__ typename Op::Acc done(const Op &op, int32_t) const { return op.lane_done(s); }
+};
+
+template <class T, bool MAX>
+struct ColState<ExtremeFold<T, MAX>> {
+    using Op = ExtremeFold<T, MAX>;
+    T v;
+    int32_t i;
+    __device__ __forceinline__ void first(const Op &, T x, int32_t r, NoCtx) {
+        v = x;
+        i = r;
+    }
+    // ref: src/backend/cpu/reduce.rs:75-86 with positions that only grow: a held NaN sticks (a == a fails),
+    // otherwise a NaN or a strictly better value replaces ("not (b <= a)" is true for both).
+    __device__ __forceinline__ void next(const Op &, T x, int32_t r, NoCtx) {
+        auto a = Op::key(v), b = Op::key(x);
+        const bool take = a == a && !(MAX ? b <= a : b >= a);
+        v = take ? x : v;
+        i = take ? r : i;
+    }
+    __device__ __forceinline__ Best<T> done(const Op &, int32_t) const { return Best<T>{v, static_cast<int64_t>(i)}; }
+};
+
+// Sums of (x - K) and (x - K)^2 about the lane's first element K (see MomentsFold): the count is the
+// kernel's, the squares go through one fused multiply-add (nothing here has to match the CPU's roundings;
+// the result is judged against its two-pass value).
+template <class T>
+struct ColState<MomentsFold<T>> {
+    using Op = MomentsFold<T>;
+    double k, s1, s2;
+    __device__ __forceinline__ void first(const Op &, T x, int32_t, NoCtx) {
+        k = Conv<T>::to_f64(x);
+        s1 = 0.0;
+        s2 = 0.0;
+    }
+    __device__ __forceinline__ void next(const Op &, T x, int32_t, NoCtx) {
+        const double d = Conv<T>::to_f64(x) - k;
+        s1 += d;
+        s2 = __builtin_fma(d, d, s2);
+    }
+    __device__ __forceinline__ Moments done(const Op &, int32_t count) const {
+        const double n = static_cast<double>(count);
+        const double mean_shift = s1 * count_reciprocal(n);
+        const double m2 = s2 - s1 * mean_shift;
+        return Moments{n, k + mean_shift, m2 > 0.0 ? m2 : 0.0};
+    }
+};
+
+// Contiguous outputs ("columns"), one strided reduced dimension of fewer than 2^31 rows. `rstride` is that
+// stride and `inner` the length of the contiguous run of outputs (the innermost kept dimension); a.kept holds
+// the remaining, outer kept dimensions. Every row of every tile starts 16-byte aligned.
+//
+// A lane owns V adjacent columns (one 16-byte load per row) and keeps their states in registers; `across`
+// (1, 2 or 4) waves of the workgroup sit side by side on a span of across*64*V columns and the BLOCK/64/across
+// row groups take interleaved rows. The S = gridDim.y slices are interleaved as well: row group g of slice s
+// takes rows s*RG + g, s*RG + g + S*RG, ... - so all workgroups of a launch together sweep ONE band of
+// S*RG consecutive rows through the source, the way a copy would. (Measured on 16384 x 4096 f32: slices that
+// are blocks of consecutive rows, i.e. S streams 4 MB apart, 45.4 us; interleaved 43.1 us.)
+// The loop is software-pipelined two rows deep: the next two loads are issued before the last two are folded
+// (two rows per step 40.5 us, four 41.8, one 44.1 in that shape).
 template <class Op, class Sink, int BLOCK>
 __global__ void __launch_bounds__(BLOCK)
     reduce_cols_kernel(ReduceArgs a, int64_t rstride, int64_t inner, int across, Op op, Sink sink) {
@@ -503,15 +581,18 @@ __global__ void __launch_bounds__(BLOCK)
     using Acc = typename Op::Acc;
     constexpr int V = 16 / static_cast<int>(sizeof(T));
     constexpr int kWaves = BLOCK / kWave;
-    constexpr int U = 4;
-    constexpr int kMinAcross = BLOCK == kBlock ? 1 : 4;
-    __shared__ Acc lds[kWaves - kMinAcross][kWave * V];
-    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    constexpr int U = 2;
+    __shared__ Acc lds[kWaves][kWave * V];  // a wave's accumulators, for the fold across row groups
+    // The wave's number is the same in all its lanes; said so, the row bookkeeping below (first row, count,
+    // the loop itself) stays in scalar registers.
+    const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) / kWave), lane = threadIdx.x % kWave;
     const int cgroup = wave % across, rgroup = wave / across, rgroups = kWaves / across;
-    const bool nt = a.stream != 0;
-    const int64_t split = blockIdx.y;
-    const int64_t begin = split * a.chunk;
-    const int64_t end = begin + a.chunk < a.nred ? begin + a.chunk : a.nred;
+    // Rows of this wave: first, first + stride, ...
+    const int32_t nred = static_cast<int32_t>(a.nred);
+    const int32_t stride = static_cast<int32_t>(gridDim.y) * rgroups;
+    const int32_t first = static_cast<int32_t>(blockIdx.y) * rgroups + rgroup;
+    const int32_t count = first < nred ? (nred - first + stride - 1) / stride : 0;
+    const int64_t step = static_cast<int64_t>(stride) * rstride * static_cast<int64_t>(sizeof(T));  // bytes
     const int64_t span = static_cast<int64_t>(across) * kWave * V;
     const int64_t tiles_inner = (inner + span - 1) / span;
     const int64_t tiles = tiles_inner * (a.nout / inner);
@@ -521,64 +602,111 @@ __global__ void __launch_bounds__(BLOCK)
         const int64_t obase = outer * inner;                                                    // first output of the run
         const T *src = reinterpret_cast<const T *>(a.src) + a.kept.offset(outer);
         const int valid = inner - col >= V ? V : (inner > col ? static_cast<int>(inner - col) : 0);
-        typename Op::Lane state[V];
+        ColState<Op> state[V];
         typename Op::Ctx ctx[V];
 #pragma unroll
-        for (int i = 0; i < V; ++i) {
-            state[i] = op.lane_init();
-            ctx[i] = op.context(i < valid ? obase + col + i : 0);
-        }
-        if (valid == V) {
-            int64_t r = begin + rgroup;
-            for (; r + (U - 1) * rgroups < end; r += U * rgroups) {
-                T t[U][V];
-#pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    load_tile_rt<T, V>(reinterpret_cast<const char *>(src + (r + u * rgroups) * rstride + col), t[u], nt);
-                }
-#pragma unroll
-                for (int u = 0; u < U; ++u) {
-#pragma unroll
-                    for (int i = 0; i < V; ++i) op.lane_add(state[i], t[u][i], r + u * rgroups, ctx[i]);
-                }
-            }
-            for (; r < end; r += rgroups) {
+        for (int i = 0; i < V; ++i) ctx[i] = op.context(i < valid ? obase + col + i : 0);
+        Acc acc[V];
+        if (count > 0 && valid == V) {
+            const char *p = reinterpret_cast<const char *>(src + static_cast<int64_t>(first) * rstride + col);
+            int32_t r = first, n = count - 1;
+            {
                 T t[V];
-                load_tile_rt<T, V>(reinterpret_cast<const char *>(src + r * rstride + col), t, nt);
+                load_stream<T, V>(p, t);
+                p += step;
 #pragma unroll
-                for (int i = 0; i < V; ++i) op.lane_add(state[i], t[i], r, ctx[i]);
+                for (int i = 0; i < V; ++i) state[i].first(op, t[i], r, ctx[i]);
+                r += stride;
             }
-        } else if (valid > 0) {
-            for (int64_t r = begin + rgroup; r < end; r += rgroups) {
+            auto fold = [&](const T(&t)[V]) {
+#pragma unroll
+                for (int i = 0; i < V; ++i) state[i].next(op, t[i], r, ctx[i]);
+                r += stride;
+            };
+            // The next U rows are requested before the last U are folded, and handed over by a register copy
+            // that waits for them: at most U loads are out per wave at any time. (Two buffers that swap roles keep
+            // up to 2 U loads out and measured 1 us slower on 16384 x 4096: this access pattern runs best with
+            // little in flight.)
+            if (n >= U) {
+                T cur[U][V];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    load_stream<T, V>(p, cur[u]);
+                    p += step;
+                }
+                for (n -= U; n >= U; n -= U) {
+                    T nxt[U][V];
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        load_stream<T, V>(p, nxt[u]);
+                        p += step;
+                    }
+#pragma unroll
+                    for (int u = 0; u < U; ++u) fold(cur[u]);
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+#pragma unroll
+                        for (int i = 0; i < V; ++i) cur[u][i] = nxt[u][i];
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < U; ++u) fold(cur[u]);
+            }
+            for (; n > 0; --n) {
+                T t[V];
+                load_stream<T, V>(p, t);
+                p += step;
+                fold(t);
+            }
+#pragma unroll
+            for (int i = 0; i < V; ++i) acc[i] = state[i].done(op, count);
+        } else if (count > 0 && valid > 0) {
+            // The ragged last lane of a run of outputs: element by element.
+            const T *q = src + static_cast<int64_t>(first) * rstride + col;
+            const int64_t estep = static_cast<int64_t>(stride) * rstride;
+#pragma unroll
+            for (int i = 0; i < V; ++i) {
+                if (i < valid) state[i].first(op, q[i], first, ctx[i]);
+            }
+            int32_t r = first + stride;
+            for (int32_t n = count - 1; n > 0; --n, r += stride) {
+                q += estep;
 #pragma unroll
                 for (int i = 0; i < V; ++i) {
-                    if (i < valid) op.lane_add(state[i], src[r * rstride + col + i], r, ctx[i]);
+                    if (i < valid) state[i].next(op, q[i], r, ctx[i]);
                 }
             }
-        }
-        Acc acc[V];
 #pragma unroll
-        for (int i = 0; i < V; ++i) acc[i] = op.lane_done(state[i]);
+            for (int i = 0; i < V; ++i) acc[i] = i < valid ? state[i].done(op, count) : op.init();
+        } else {
+#pragma unroll
+            for (int i = 0; i < V; ++i) acc[i] = op.init();
+        }
+        const int64_t tile_col = (tile - outer * tiles_inner) * span;  // first column of the tile, within the run
         if (rgroups > 1) {
-            // Row groups 1.. hand their accumulators to row group 0, which folds them in order.
-            __syncthreads();
-            if (rgroup > 0) {
+            // Every wave leaves its accumulators in LDS; then the row groups share the fold: of the 64*V columns
+            // of its column group, row group g folds columns [g, g + 1) * 64*V / rgroups, a column per lane, the
+            // row groups' values in order. All waves work, and a wave's results are consecutive outputs.
+            __syncthreads();  // the previous tile's fold has read LDS
 #pragma unroll
-                for (int i = 0; i < V; ++i) lds[wave - across][lane * V + i] = acc[i];
-            }
+            for (int i = 0; i < V; ++i) lds[wave][lane * V + i] = acc[i];
             __syncthreads();
-            if (rgroup == 0) {
-                for (int g = 1; g < rgroups; ++g) {
-#pragma unroll
-                    for (int i = 0; i < V; ++i) acc[i] = op.combine(acc[i], lds[g * across + cgroup - across][lane * V + i]);
+            const int share = kWave * V / rgroups;
+            for (int j = lane; j < share; j += kWave) {
+                const int c = rgroup * share + j;  // column within the column group
+                Acc folded = lds[cgroup][c];
+                for (int g = 1; g < rgroups; ++g) folded = op.combine(folded, lds[g * across + cgroup][c]);
+                const int64_t column = tile_col + cgroup * (kWave * V) + c;
+                if (column < inner) {
+                    if (a.splits > 1) put_partial(a.partials, a.nout, static_cast<int64_t>(blockIdx.y), obase + column, folded);
+                    else sink.put(obase + column, folded, a.nred);
                 }
             }
-        }
-        if (rgroup == 0) {
+        } else {
 #pragma unroll
             for (int i = 0; i < V; ++i) {
                 if (i < valid) {
-                    if (a.splits > 1) put_partial(a.partials, a.nout, split, obase + col + i, acc[i]);
+                    if (a.splits > 1) put_partial(a.partials, a.nout, static_cast<int64_t>(blockIdx.y), obase + col + i, acc[i]);
                     else sink.put(obase + col + i, acc[i], a.nred);
                 }
             }

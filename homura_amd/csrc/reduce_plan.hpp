@@ -25,8 +25,6 @@ struct ReducePlan {
 // pair at most, or for hmr_var a (count, mean, M2) triple.
 constexpr int64_t kPartialBytes = 16;
 constexpr int64_t kVarPartialBytes = 32;
-// A source at least this large is read with nontemporal loads (see load_tile in map.hpp).
-constexpr int64_t kStreamSourceBytes = int64_t{32} << 20;
 // Machine width the plans aim at: lanes of a full MI355X at 4 waves per SIMD.
 constexpr int64_t kTargetLanes = 256 * 4 * 4 * 64;
 
@@ -72,7 +70,7 @@ void launch_reduce(const ReducePlan &plan, void *partials, Op op, Sink sink, hip
             int64_t tiles = (plan.inner + span - 1) / span * (a.nout / plan.inner);
             dim3 grid(capped(tiles, cap), ysplits);
             if (plan.group == 1024 / kWave) {
-                // Planned for 4- and 8-byte elements only (wider tiles would not fit LDS).
+                // Planned for elements of four bytes or more (the states of wider tiles would not fit LDS).
                 if constexpr (sizeof(typename Op::In) >= 4) {
                     hipLaunchKernelGGL((reduce_cols_kernel<Op, Sink, 1024>), grid, dim3(1024), 0, stream, a,
                                        plan.rstride, plan.inner, plan.across, op, sink);

@@ -305,9 +305,10 @@ PLAN_SHAPES = [
     ([4, 100000], [1], 256, True),          # rows cut into slices
     ([1 << 21], [0], 256, True),            # a full reduction
     ([8, 1 << 20], [0], 4, False),          # columns, one slice
-    ([5000, 256], [0], 4, True),            # columns cut into row slices
+    ([400, 256], [0], 4, True),             # short columns cut into row slices: 256-lane workgroups
+    ([5000, 256], [0], 16, True),           # long narrow columns: 1024-lane workgroups, sixteen row groups
     ([8192, 2048], [0], 16, True),          # long columns in few tiles: 1024-lane workgroups, four row groups
-    ([6, 700, 96], [1], 4, True),           # columns under an outer kept dimension
+    ([6, 700, 96], [1], 16, True),          # columns under an outer kept dimension
     ([5000, 20], [1], 1, False),            # short rows: a lane per output
     ([9, 2, 3000], [0, 2], 256, True),      # two reduced dimensions: any layout, 256 lanes
     ([70, 600, 70], [0, 2], 256, False),    # ... without slices

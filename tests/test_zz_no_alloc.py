@@ -113,20 +113,21 @@ def test_integer_sums_and_the_other_dtypes(ctx):
 
 
 def test_a_plan_beyond_the_block_is_refused_and_queues_nothing(ctx):
-    rows, cols = 2048, 65536
-    src = ctx.malloc(rows * cols * 4)
-    kept, red, nout = matrix_reduction(src, capi.F32, rows, cols, 0)
+    # Many one-byte columns: 64 slices of 32 768 partial sums of 16 bytes.
+    rows, cols = 16384, 32768
+    src = ctx.malloc(rows * cols)
+    kept, red, nout = matrix_reduction(src, capi.I8, rows, cols, 0)
     need = workspace_bytes(kept, red)
     assert need > LIMIT, "this shape is meant to stage more than the block holds; pick a wider one if the plan changed"
-    out = ctx.malloc(nout * 4)
-    capi.check(L.hmr_memset(ctx.handle, out.ptr, 0x5C, nout * 4))
-    o = capi.make_desc(out.ptr, capi.F32, [nout], [1])
+    out = ctx.malloc(nout * 8)
+    capi.check(L.hmr_memset(ctx.handle, out.ptr, 0x5C, nout * 8))
+    o = capi.make_desc(out.ptr, capi.I64, [nout], [1])
     assert L.hmr_reduce_static(ctx.handle, capi.REDUCE["sum"], byref(o), byref(kept), byref(red)) == capi.HMR_INVALID
     message = L.hmr_last_error().decode()
     assert message.startswith("hmr_reduce_static: this reduction stages %d bytes" % need) and str(LIMIT) in message
     ctx.synchronize()
-    assert (out.download(np.uint8, nout * 4) == 0x5C).all()
+    assert (out.download(np.uint8, nout * 8) == 0x5C).all()
     # The same errors as hmr_reduce for a bad call.
-    bad = capi.make_desc(out.ptr, capi.F32, [nout + 1], [1])
+    bad = capi.make_desc(out.ptr, capi.I64, [nout + 1], [1])
     assert L.hmr_reduce_static(ctx.handle, capi.REDUCE["sum"], byref(bad), byref(kept), byref(red)) == capi.HMR_INVALID
     assert L.hmr_last_error().decode() == "a reduction's output is not contiguous with its sizes"
