@@ -114,6 +114,7 @@ PROTOTYPES = {
     "hmr_test_reduce_plan": (c_int32, [DESC_P, DESC_P, POINTER(c_int64), POINTER(c_int64), POINTER(c_int64)]),
     "hmr_test_softmax_plan": (c_int32, [DESC_P, c_int64, c_int64, POINTER(c_int32), POINTER(c_int32),
                                         POINTER(c_int32)]),
+    "hmr_test_index_value": (c_int32, [CTX, DESC_P, c_void_p]),
     "hmr_test_live_streams": (c_int32, []),
     "hmr_test_current_device": (c_int32, [POINTER(c_int32)]),
     "hmr_test_set_current_device": (c_int32, [c_int32]),
@@ -126,7 +127,7 @@ UNBUILT = [
     "hmr_max_pool2d_backward_workspace", "hmr_max_pool2d_backward", "hmr_max_pool2d",
     "hmr_max_pool2d_check", "hmr_max_pool2d_gather_backward", "hmr_adaptive_avg_pool2d",
     "hmr_adaptive_avg_pool2d_backward", "hmr_unfold_backward", "hmr_gemm_fold", "hmr_gemm_select",
-    "hmr_gemm_path_name", "hmr_gemm_workspace", "hmr_gemm", "hmr_test_index_value", "hmr_test_wide_pool",
+    "hmr_gemm_path_name", "hmr_gemm_workspace", "hmr_gemm", "hmr_test_wide_pool",
     "hmr_test_force_gemm_path", "hmr_test_pool_candidates",
 ]
 

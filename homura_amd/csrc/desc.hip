@@ -12,11 +12,15 @@ hmr_status check_desc(const hmr_tensor_desc &d, int64_t &n, bool negative_stride
         return fail(HMR_INVALID, "invalid number of dimensions " + std::to_string(d.ndim));
     }
     n = 1;
+    bool empty = false, wraps = false;
     for (int k = 0; k < d.ndim; ++k) {
         if (d.sizes[k] < 0) return fail(HMR_INVALID, "negative size");
         if (d.strides[k] < 0 && !negative_strides) return fail(HMR_INVALID, "negative stride");
-        n *= d.sizes[k];
+        empty = empty || d.sizes[k] == 0;
+        wraps = __builtin_mul_overflow(n, d.sizes[k], &n) || wraps;
     }
+    if (empty) n = 0;  // whatever the other sizes are
+    else if (wraps) return fail(HMR_INVALID, "the number of elements does not fit 64 bits");
     return HMR_OK;
 }
 

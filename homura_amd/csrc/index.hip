@@ -376,6 +376,34 @@ hmr_status hmr_index_check(hmr_context_t ctx, const hmr_tensor_desc *index, int6
     });
 }
 
+// The second step of hmr_index_check alone (ref: csrc/homura_rocm.h:631-657, csrc/index.hip:465-479): the caller
+// sets slot[0] to a logical position of `index`; unless that is UINT64_MAX the value there goes to slot[1].
+// Positions reach 2^63 - 1 in views with zero strides, whose element count no longer fits 64 bits, so the
+// description is checked dimension by dimension and no product is formed.
+hmr_status hmr_test_index_value(hmr_context_t ctx, const hmr_tensor_desc *index, uint64_t *slot) {
+    return guarded([&] {
+        if (index == nullptr || slot == nullptr) return fail(HMR_INVALID, "index value: null argument");
+        if (index->dtype < HMR_BOOL || index->dtype > HMR_F64) return fail(HMR_INVALID, "invalid dtype " + std::to_string(index->dtype));
+        if (index->ndim < 0 || index->ndim > HMR_MAX_DIMS) {
+            return fail(HMR_INVALID, "invalid number of dimensions " + std::to_string(index->ndim));
+        }
+        for (int k = 0; k < index->ndim; ++k) {
+            if (index->sizes[k] < 0) return fail(HMR_INVALID, "negative size");
+            if (index->strides[k] < 0) return fail(HMR_INVALID, "negative stride");
+            if (index->sizes[k] == 0) return fail(HMR_INVALID, "index value: the index is empty");
+        }
+        if (!hmr::is_index_dtype(index->dtype)) return fail(HMR_INVALID, "index tensors must be I32 or I64");
+        const hmr_tensor_desc *const ops[3] = {index, nullptr, nullptr};
+        const hmr::Dims d = hmr::dims_of(*index, ops, -1);
+        const void *base = hmr::first_of(*index);
+        const int is64 = index->dtype == HMR_I64;
+        return hmr::launch_on(ctx, "index value", [&](hipStream_t stream) {
+            hipLaunchKernelGGL(hmr::check_value_kernel, dim3(1), dim3(1), 0, stream, base, is64, d, slot);
+            return true;
+        });
+    });
+}
+
 hmr_status hmr_index_select(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_tensor_desc *src,
                             const hmr_tensor_desc *index, int32_t dim, int32_t wrap_negative) {
     return guarded([&] {

@@ -109,6 +109,7 @@ struct RowsArgs {
     uint64_t cbits[NOPS];
     uint32_t const_mask;   // bit k: operand k is a constant
     uint32_t bcast_mask;   // bit k: operand k has inner stride 0
+    uint32_t gather;       // nonzero: 2-byte output tiles of eight lanes leave as one 16-byte store (2: nontemporal)
     int64_t n;             // elements
     uint32_t inner;        // size of the innermost dimension
     int32_t nouter;        // outer dimensions (0 for contiguous)
@@ -192,6 +193,30 @@ __device__ __forceinline__ void store_tile(char *p, const T (&r)[V]) {
     } else {
         static_assert(bytes == 1, "tile size");
         __builtin_memcpy(p, r, 1);
+    }
+}
+
+// A 2-byte tile per lane (a bool mask computed from 8-byte operands) would leave as 2-byte stores, 128 bytes
+// per instruction. Eight consecutive lanes hold eight consecutive tiles, so their sixteen bytes are gathered
+// into the first of them with data-parallel moves inside the row of 16 lanes and leave as one 16-byte store:
+//   pair      lanes 2k:  own bytes + those of lane 2k+1        (quad_perm [1,0,3,2])
+//   next_pair lanes 4k:  the pair of lane 4k+2                 (quad_perm [2,3,0,1])
+//   far       lanes 8k:  pair and next_pair of lane 8k+4       (row_shl:4)
+template <bool NT>
+__device__ __forceinline__ void store_eight_lanes(char *p, uint16_t own) {
+    constexpr int kSwapPairs = 1 | (0 << 2) | (3 << 4) | (2 << 6), kSwapHalves = 2 | (3 << 2) | (0 << 4) | (1 << 6);
+    constexpr int kRowShl4 = 0x104;
+    const int x = static_cast<int>(own);
+    const int pair = x | (__builtin_amdgcn_mov_dpp(x, kSwapPairs, 0xF, 0xF, true) << 16);
+    const int next_pair = __builtin_amdgcn_mov_dpp(pair, kSwapHalves, 0xF, 0xF, true);
+    const int far0 = __builtin_amdgcn_mov_dpp(pair, kRowShl4, 0xF, 0xF, true);
+    const int far1 = __builtin_amdgcn_mov_dpp(next_pair, kRowShl4, 0xF, 0xF, true);
+    if ((threadIdx.x & 7u) == 0) {
+        u32x4 w = {static_cast<uint32_t>(pair), static_cast<uint32_t>(next_pair), static_cast<uint32_t>(far0),
+                   static_cast<uint32_t>(far1)};
+        u32x4 *q = reinterpret_cast<u32x4 *>(p);
+        if constexpr (NT) __builtin_nontemporal_store(w, q);
+        else *q = w;
     }
 }
 
@@ -460,7 +485,19 @@ __global__ void __launch_bounds__(kBlock) map_rows_kernel(RowsArgs<F::N + 1> a) 
                 Out ro[V];
 #pragma unroll
                 for (int i = 0; i < V; ++i) ro[i] = apply(f, ra[i], rb[i], rc[i]);
-                store_tile<Out, V, kStreamStores || NTSTORE>(a.ptr[0] + static_cast<int64_t>(oo[u]) * static_cast<int64_t>(sizeof(Out)), ro);
+                char *po = a.ptr[0] + static_cast<int64_t>(oo[u]) * static_cast<int64_t>(sizeof(Out));
+                if constexpr (V * sizeof(Out) == 2) {
+                    if (a.gather) {
+                        uint16_t w;
+                        __builtin_memcpy(&w, ro, 2);
+                        // Two forms, as the hint is a property of the instruction: a call larger than the
+                        // memory-side cache stores past it (i64 > i64 over 67M elements: 185 -> 176 us).
+                        if (a.gather == 2) store_eight_lanes<true>(po, w);
+                        else store_eight_lanes<false>(po, w);
+                        continue;
+                    }
+                }
+                store_tile<Out, V, kStreamStores || NTSTORE>(po, ro);
             }
         } else {
             // Ragged pass (the last workgroup): tile by tile, partial tiles element by element.
@@ -631,6 +668,17 @@ RowsArgs<F::N + 1> rows_args(const MapCall &c, int variant) {
         a.cbits[k] = c.cbits[k];
         if (c.is_const[k]) a.const_mask |= 1u << k;
         else if (c.ndim == 0 || c.stride[k][last] == 0) a.bcast_mask |= k == 0 ? 0u : 1u << k;
+    }
+    // Eight consecutive tiles are sixteen consecutive output bytes when the output is one run (variant 0) or
+    // its rows hold a multiple of eight tiles; the output's base is 16-byte aligned then (pick_variant checks
+    // 2-byte alignment only).
+    using T = MapTraits<F>;
+    a.gather = 0;
+    if (T::V * T::so == 2 && reinterpret_cast<uintptr_t>(c.ptr[0]) % 16 == 0) {
+        bool whole = variant == 0 || c.size[last] % (8 * T::V) == 0;
+        for (int d = 0; whole && variant != 0 && d < last; ++d) whole = (c.stride[0][d] * T::so) % 16 == 0;
+        const int64_t moved = c.n * (T::so + T::s0 + T::s1 + T::s2);
+        a.gather = whole ? (moved > kCacheResidentBytes ? 2u : 1u) : 0u;
     }
     if (variant == 0) {
         a.inner = static_cast<uint32_t>(c.n < (int64_t{1} << 31) ? c.n : 0);

@@ -33,7 +33,6 @@ HMR_UNBUILT(hmr_gemm_select, const hmr_gemm_desc *, int32_t *, int32_t *)
 HMR_UNBUILT(hmr_gemm_path_name, int32_t, const char **)
 HMR_UNBUILT(hmr_gemm_workspace, const hmr_gemm_desc *, int32_t, int64_t *)
 HMR_UNBUILT(hmr_gemm, hmr_context_t, const hmr_gemm_desc *, int32_t, void *, int64_t)
-HMR_UNBUILT(hmr_test_index_value, hmr_context_t, const hmr_tensor_desc *, uint64_t *)
 HMR_UNBUILT(hmr_test_pool_candidates, const int64_t *, int64_t, int64_t, int64_t, int64_t, int64_t *)
 
 void hmr_test_wide_pool(int32_t) {}

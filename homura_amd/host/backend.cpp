@@ -5,6 +5,8 @@
 #include <cstring>
 #include <map>
 #include <mutex>
+#include <utility>
+#include <vector>
 
 #include "homura.hpp"
 #include "homura_rocm.h"
@@ -264,14 +266,20 @@ Storage::~Storage() {
 void register_cpu_backend(const hcb_backend *table) { g_cpu = table; }
 
 void empty_cache() {
-    std::lock_guard<std::mutex> lock(g_registry);
-    for (auto &kv : g_devices) {
-        DeviceState &st = *kv.second;
-        std::lock_guard<std::recursive_mutex> run(st.exec);
-        expect(hmr_context_synchronize(st.ctx));
-        std::lock_guard<std::mutex> a(st.alloc);
-        for (auto &b : st.cache) expect(hmr_free(kv.first, b.second));
-        st.cache.clear();
+    // Lock order everywhere is exec -> registry (an op allocates its outputs, and so looks its device up,
+    // inside the execution lock), so the registry lock is dropped before any execution lock is taken.
+    // Device states live until the process ends: the pointers stay valid.
+    std::vector<std::pair<int, DeviceState *>> devices;
+    {
+        std::lock_guard<std::mutex> lock(g_registry);
+        for (auto &kv : g_devices) devices.emplace_back(kv.first, kv.second.get());
+    }
+    for (auto &[index, st] : devices) {
+        std::lock_guard<std::recursive_mutex> run(st->exec);
+        expect(hmr_context_synchronize(st->ctx));
+        std::lock_guard<std::mutex> a(st->alloc);
+        for (auto &b : st->cache) expect(hmr_free(index, b.second));
+        st->cache.clear();
     }
 }
 

@@ -69,7 +69,7 @@ PYBIND11_MODULE(_host, m) {
     });
     m.def("register_cpu_backend", [](uintptr_t table) { register_cpu_backend(reinterpret_cast<const hcb_backend *>(table)); },
           "Registers the hcb_backend table at this address for kernels on CPU tensors (0 unregisters).");
-    m.def("empty_cache", &empty_cache);
+    m.def("empty_cache", &empty_cache, py::call_guard<py::gil_scoped_release>());
     m.def("set_fused_promotion", &set_fused_promotion);
     m.def("synchronize", [](const std::string &d) {
         py::gil_scoped_release release;
@@ -261,13 +261,13 @@ PYBIND11_MODULE(_host, m) {
     T.def("index_add", &Tensor::index_add);
     T.def("scatter_add", &Tensor::scatter_add);
     T.def("slice", &Tensor::slice, py::arg("dim"), py::arg("start") = py::none(), py::arg("end") = py::none(), py::arg("step") = 1);
-    T.def("index_tensors", &Tensor::index_tensors);
+    T.def("index_tensors", &Tensor::index_tensors, py::call_guard<py::gil_scoped_release>());
     T.def("index_put_tensors", &Tensor::index_put_tensors);
     T.def("mask_coordinates", [](const Tensor &mask) {
         std::vector<Tensor> out;
         for (const homura::TensorData &d : homura::backend::mask_coordinates(mask.data())) out.emplace_back(d);
         return out;
-    });
+    }, py::call_guard<py::gil_scoped_release>());
     T.def("triu", &Tensor::triu, py::arg("diagonal") = 0);
     T.def("tril", &Tensor::tril, py::arg("diagonal") = 0);
     T.def("flip", &Tensor::flip);

@@ -451,6 +451,10 @@ hmr_status hmr_test_reduce_plan(const hmr_tensor_desc *kept, const hmr_tensor_de
  *   streamed twice instead). */
 hmr_status hmr_test_softmax_plan(const hmr_tensor_desc *src_rows, int64_t n, int64_t src_stride,
                                  int32_t *split, int32_t *group, int32_t *cache);
+/* ref :631-657  The second step of hmr_index_check alone: unless slot[0] (a logical position of `index`,
+ * set by the caller) is UINT64_MAX, the value there goes to slot[1]. For positions far beyond what a
+ * check could reach in a test (2^60 and more, in views with zero strides). */
+hmr_status hmr_test_index_value(hmr_context_t ctx, const hmr_tensor_desc *index, uint64_t *slot);
 int32_t hmr_test_live_streams(void);
 hmr_status hmr_test_current_device(int32_t *device);
 hmr_status hmr_test_set_current_device(int32_t device);

@@ -72,8 +72,6 @@ hmr_status hmr_gemm(hmr_context_t ctx, const hmr_gemm_desc *desc, int32_t path, 
                     int64_t workspace_bytes);
 
 /* ref :657-662 (test hooks of the families above) */
-hmr_status hmr_test_index_value(hmr_context_t ctx, const hmr_tensor_desc *index,
-                                uint64_t *slot);
 void hmr_test_wide_pool(int32_t on);
 void hmr_test_force_gemm_path(int32_t path);
 hmr_status hmr_test_pool_candidates(const int64_t *geometry, int64_t height, int64_t width,

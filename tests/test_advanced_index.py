@@ -402,3 +402,32 @@ def test_the_c_abi_of_positions_masks_and_overwrites():
         assert x.download(np.float32, 10).tolist() == [0.0, 1.0, 2.0, 2.0, 4.0, 5.0, 6.0, 3.0, 8.0, 9.0]
     finally:
         ctx.close()
+
+
+@pytest.mark.gpu
+def test_masked_reads_and_empty_cache_from_two_threads_do_not_deadlock():
+    """`x[mask]` allocates inside the device's execution lock (and so looks the device up) while empty_cache walks
+    the devices and takes each execution lock: the two orders must not cross. The thread is joined with a
+    time limit, so a regression fails here instead of hanging the run."""
+    import threading
+
+    x = tensor(values(DT.F32, 4096, 77), DT.F32, [64, 64]).to(GPU)
+    keep = bools(mask([64, 64], 78)).to(GPU)
+    want = array(x.index_tensors([keep]))
+    failures = []
+
+    def reads():
+        try:
+            for _ in range(200):
+                if not same(array(x.index_tensors([keep])), want):
+                    failures.append("a masked read changed")
+        except Exception as e:  # pragma: no cover
+            failures.append(repr(e))
+
+    worker = threading.Thread(target=reads, daemon=True)
+    worker.start()
+    for _ in range(200):
+        h.empty_cache()
+    worker.join(timeout=60)
+    assert not worker.is_alive(), "x[mask] and empty_cache wait for each other"
+    assert not failures, failures

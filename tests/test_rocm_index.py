@@ -294,3 +294,52 @@ def test_the_c_abi_of_the_index_kernels():
         np.testing.assert_array_equal(out.download(np.float32, 16), want)
     finally:
         ctx.close()
+
+
+def test_values_are_read_at_large_logical_positions():
+    """hmr_test_index_value: the second step of a position check alone, at logical positions as large as a shape
+    allows (below 2^63) in two-element views with zero strides; the kernel computes offsets in 64 bits
+    (ref: src/backend/rocm/tests.rs:1213-1261, the same five cases)."""
+    import ctypes
+
+    from homura_amd import capi
+
+    ctx = capi.Context(0)
+    try:
+        for np_dtype, code in ((np.int64, capi.I64), (np.int32, capi.I32)):
+            base = ctx.upload(np.array([11, 22], dtype=np_dtype))
+            cases = [([2, 1 << 60], [1, 0], 1 << 60, 22), ([2, 1 << 60], [1, 0], (1 << 60) - 1, 11),
+                     ([2, 1 << 60], [1, 0], (1 << 61) - 1, 22), ([1 << 62, 2], [0, 1], (1 << 63) - 1, 22),
+                     ([1 << 62, 2], [0, 1], (1 << 63) - 2, 11)]
+            for shape, strides, position, expected in cases:
+                slots = ctx.upload(np.array([position, 0], dtype=np.uint64))
+                desc = capi.make_desc(base.ptr, code, shape, strides)
+                capi.check(capi.lib.hmr_test_index_value(ctx.handle, ctypes.byref(desc), slots.ptr))
+                ctx.synchronize()
+                assert list(slots.download(np.uint64, 2)) == [position, expected], (shape, position)
+            # UINT64_MAX means "no position": nothing is written.
+            slots = ctx.upload(np.array([2**64 - 1, 7], dtype=np.uint64))
+            desc = capi.make_desc(base.ptr, code, [2], [1])
+            capi.check(capi.lib.hmr_test_index_value(ctx.handle, ctypes.byref(desc), slots.ptr))
+            ctx.synchronize()
+            assert list(slots.download(np.uint64, 2)) == [2**64 - 1, 7]
+        bad = capi.make_desc(base.ptr, capi.F32, [2], [1])
+        assert capi.lib.hmr_test_index_value(ctx.handle, ctypes.byref(bad), slots.ptr) == capi.HMR_INVALID
+        assert capi.lib.hmr_last_error().decode() == "index tensors must be I32 or I64"
+    finally:
+        ctx.close()
+
+
+def test_a_sort_whose_histogram_table_needs_several_rounds_of_the_totals_scan():
+    """34.6 M positions are 16 895 tiles of 2048 words, so the digit histogram has 4.3 M entries in 1056 chunks of
+    4096: more than the 1024 totals one round of the last scan takes, which then carries over. Order-sensitive f64
+    values into a few targets: a word out of place or out of order changes a sum."""
+    n, size = 34_600_000, 300
+    pattern = np.array([2.0 ** 53, 1.0, 1.0, -(2.0 ** 53)])
+    src = tensor(np.tile(pattern, n // 4), DT.F64)
+    picks = tensor(random_positions(n, size, 91).astype(np.int32), DT.I32, [n])
+    x = h.full([size], 0.0, DT.F64, "cpu")
+    want = array(x.scatter_add(0, picks, src))
+    got = array(x.to(GPU).scatter_add(0, picks.to(GPU), src.to(GPU)))
+    wrong = np.flatnonzero(got.view(np.uint64) != want.view(np.uint64))
+    assert wrong.size == 0, f"first difference at target {wrong[0]}: {got[wrong[0]]} != {want[wrong[0]]}"
