@@ -1,6 +1,9 @@
-// Shared by every translation unit of the library: the context, the per-thread error channel,
-// the exception fence of the C ABI and the current-device guard.
-// Conventions follow ref: csrc/common.hpp:12-87 and csrc/homura_rocm.h:1-15.
+// What every translation unit of the library shares: the context, the calling thread's failure text and
+// `Visit`, the object that stands for one entry point's stay inside the library.
+//
+// The contract these serve is the C ABI's (ref: csrc/homura_rocm.h:1-15): a status per call, a message that
+// belongs to the calling thread, no C++ exception across the boundary, the caller's current device put back,
+// and no failed HIP call left behind in hipGetLastError.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -15,9 +18,9 @@
 
 // What hmr_context_t points at. One per device.
 struct hmr_context {
-    int device;
-    hipStream_t stream;
-    int compute_units;  // multiProcessorCount of the device (256 on MI355X), for grid sizing
+    int device = -1;
+    hipStream_t stream = nullptr;
+    int compute_units = 256;  // multiProcessorCount of the device (256 on MI355X), for grid sizing
     // Result tables of the 16-bit unary operations (one 128 KiB table per operation and dtype, every
     // input pattern -> its output pattern). The block is allocated at the first use and lives as long
     // as the context; a table is filled, on `stream`, by the first call that needs it.
@@ -31,37 +34,86 @@ struct hmr_context {
 
 namespace hmr {
 
-// Stores `message` as the calling thread's last error and hands `status` back.
+// ---- failures ------------------------------------------------------------------------------------------
+
+// Makes `message` the calling thread's failure text and hands `status` back, so that a failure reads
+// `return fail(HMR_INVALID, "...")`.
 hmr_status fail(hmr_status status, std::string message);
 
-// Same for a string literal; allocates nothing, so it is safe where memory may be exhausted.
+// The same for a string literal. Nothing is allocated, so it works when memory is what ran out.
 hmr_status fail_static(hmr_status status, const char *message) noexcept;
 
 const char *last_error_text() noexcept;
 
-// Reports a failed HIP call: out of memory maps to HMR_OUT_OF_MEMORY, everything else to
-// HMR_HIP_ERROR. Also clears HIP's sticky per-thread error so that a later launch check does not
-// see this failure again.
-hmr_status hip_fail(hipError_t error, const char *call) noexcept;
-
-#define HMR_HIP(expr)                                                         \
-    do {                                                                      \
-        hipError_t hmr_hip_e_ = (expr);                                       \
-        if (hmr_hip_e_ != hipSuccess) return ::hmr::hip_fail(hmr_hip_e_, #expr); \
-    } while (0)
+// The failure of a HIP call as a status: out of memory is its own status, anything else HMR_HIP_ERROR, the
+// text "<what>: <HIP's description>". HIP keeps the last error per thread until it is read; it is read here,
+// so that the check after a later launch does not meet this failure again.
+hmr_status hip_failure(hipError_t error, const char *what) noexcept;
 
 // Looks up where the static block of hmr_reduce_static lives on the current device and keeps the address
 // in the context. Called once per context, with its device current (defined beside the block, reduce.hip).
 hmr_status bind_reduce_scratch(hmr_context &ctx);
 
-// Consumes one failure armed by hmr_test_fail_data, if any: returns its status, else HMR_OK.
-hmr_status injected_data_failure(const char *call) noexcept;
+// ---- one entry point's stay in the library ---------------------------------------------------------------
 
-// Runs `body`; no exception gets past it.
-template <class F>
-hmr_status guarded(F body) noexcept {
+class Visit {
+  public:
+    Visit() noexcept = default;
+    Visit(const Visit &) = delete;
+    Visit &operator=(const Visit &) = delete;
+    // Leaves the calling thread on the device it came with.
+    ~Visit() {
+        if (moved_) (void)hipSetDevice(home_);
+    }
+
+    // Makes `device` current for the rest of the visit.
+    hmr_status use_device(int device) noexcept {
+        if (home_ < 0) {
+            if (hmr_status s = hip(hipGetDevice(&home_), "hipGetDevice(&previous_)")) return s;
+            now_ = home_;
+        }
+        if (device == now_) return HMR_OK;
+        if (hmr_status s = hip(hipSetDevice(device), "hipSetDevice(device)")) return s;
+        moved_ = true;
+        now_ = device;
+        return HMR_OK;
+    }
+
+    // HMR_OK for hipSuccess; otherwise the call's failure, recorded.
+    hmr_status hip(hipError_t result, const char *what) noexcept {
+        return result == hipSuccess ? HMR_OK : hip_failure(result, what);
+    }
+
+    // A test can arm the next data-moving steps of the calling thread to fail (hmr_test_fail_data). Each such
+    // step asks here first, naming the HIP call it stands for, and fails the way that call would have.
+    hmr_status armed_failure(const char *what) noexcept;
+
+    // Queues one call's kernels on the context's stream. `queue(stream)` launches them and returns false,
+    // having launched nothing, when it has no kernel for the dtype / operation. Around it: the device is made
+    // current, an armed failure fires before anything is queued, HIP's last error is cleared and, afterwards,
+    // read: that is where a launch that could not be queued shows.
+    template <class Queue>
+    hmr_status kernels(hmr_context_t ctx, const char *what, Queue queue) {
+        if (hmr_status s = use_device(ctx->device)) return s;
+        if (hmr_status s = armed_failure("hipGetLastError()")) return s;
+        (void)hipGetLastError();
+        if (!queue(ctx->stream)) return fail(HMR_INVALID, std::string(what) + ": unsupported dtype");
+        return hip(hipGetLastError(), "hipGetLastError()");
+    }
+
+  private:
+    int home_ = -1;  // the caller's device, once asked for
+    int now_ = -1;   // the calling thread's current device
+    bool moved_ = false;
+};
+
+// The exception fence of the C ABI: runs `body(visit)` with a fresh Visit and turns anything thrown into a
+// status (a failed allocation of host memory is HMR_OUT_OF_MEMORY, the rest HMR_INTERNAL_ERROR).
+template <class Body>
+hmr_status visit(Body body) noexcept {
     try {
-        return body();
+        Visit v;
+        return body(v);
     } catch (const std::bad_alloc &) {
         return fail_static(HMR_OUT_OF_MEMORY, "host allocation failed");
     } catch (const std::exception &e) {
@@ -75,41 +127,17 @@ hmr_status guarded(F body) noexcept {
     }
 }
 
-// Makes `device` current for the calling thread and restores the previous device on scope exit.
-class DeviceGuard {
-  public:
-    DeviceGuard() = default;
-    DeviceGuard(const DeviceGuard &) = delete;
-    DeviceGuard &operator=(const DeviceGuard &) = delete;
-    ~DeviceGuard() {
-        if (switched_) (void)hipSetDevice(previous_);
-    }
-    hmr_status enter(int device) {
-        HMR_HIP(hipGetDevice(&previous_));
-        if (previous_ != device) {
-            HMR_HIP(hipSetDevice(device));
-            switched_ = true;
-        }
-        return HMR_OK;
-    }
+// The two forms most entry points need, for code that has no use for the Visit itself: the fence alone, and
+// the kernels of one call (a Visit of its own; the device goes back when they are queued).
+template <class Body>
+hmr_status fenced(Body body) noexcept {
+    return visit([&](Visit &) { return body(); });
+}
 
-  private:
-    int previous_ = -1;
-    bool switched_ = false;
-};
-
-// Brackets the launches `body(stream)` makes: device made current, an armed test failure fires
-// before anything is queued, and hipGetLastError is checked afterwards. `body` returns false,
-// having queued nothing, when it has no kernel for the dtype/op pair.
-template <class F>
-hmr_status launch_on(hmr_context_t ctx, const char *what, F body) {
-    DeviceGuard guard;
-    if (hmr_status s = guard.enter(ctx->device)) return s;
-    if (hmr_status s = injected_data_failure("hipGetLastError()")) return s;
-    (void)hipGetLastError();
-    if (!body(ctx->stream)) return fail(HMR_INVALID, std::string(what) + ": unsupported dtype");
-    HMR_HIP(hipGetLastError());
-    return HMR_OK;
+template <class Queue>
+hmr_status queue_on(hmr_context_t ctx, const char *what, Queue queue) {
+    Visit v;
+    return v.kernels(ctx, what, queue);
 }
 
 }  // namespace hmr

@@ -64,7 +64,7 @@ extern "C" {
 
 hmr_status hmr_binary(hmr_context_t ctx, int32_t op, const hmr_tensor_desc *out, const hmr_tensor_desc *a,
                       const hmr_tensor_desc *b) {
-    return hmr::guarded([&] {
+    return hmr::fenced([&] {
         const hmr_tensor_desc *descs[3] = {out, a, b};
         return hmr::run_map(ctx, "binary", 3, descs, nullptr, [&](const hmr::MapCall &call, hipStream_t stream) {
             return hmr::pick_binary(op, out->dtype, a->dtype, b->dtype, call, stream);
@@ -74,7 +74,7 @@ hmr_status hmr_binary(hmr_context_t ctx, int32_t op, const hmr_tensor_desc *out,
 
 hmr_status hmr_binary_constant(hmr_context_t ctx, int32_t op, const hmr_tensor_desc *out, const hmr_tensor_desc *a,
                                uint64_t bits, int32_t constant_first) {
-    return hmr::guarded([&] {
+    return hmr::fenced([&] {
         const hmr_tensor_desc *descs[3] = {out, constant_first ? nullptr : a, constant_first ? a : nullptr};
         const uint64_t cbits[3] = {0, bits, bits};
         return hmr::run_map(ctx, "binary_constant", 3, descs, cbits,

@@ -19,7 +19,7 @@ hmr_status run_map(hmr_context_t ctx, const char *what, int count, const hmr_ten
     if (call.n == 0) return HMR_OK;
     call.compute_units = ctx->compute_units;
     if (hmr_status s = before(call)) return s;
-    return launch_on(ctx, what, [&](hipStream_t stream) { return pick(call, stream); });
+    return queue_on(ctx, what, [&](hipStream_t stream) { return pick(call, stream); });
 }
 
 template <class Pick>

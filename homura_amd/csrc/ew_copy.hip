@@ -2,7 +2,7 @@
 #include "ew_common.hpp"
 
 extern "C" hmr_status hmr_copy(hmr_context_t ctx, const hmr_tensor_desc *dst, const hmr_tensor_desc *src) {
-    return hmr::guarded([&] {
+    return hmr::fenced([&] {
         const hmr_tensor_desc *descs[2] = {dst, src};
         return hmr::run_map(ctx, "copy", 2, descs, nullptr, [&](const hmr::MapCall &call, hipStream_t stream) {
             if (dst->dtype == src->dtype) {

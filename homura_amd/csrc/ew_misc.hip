@@ -60,7 +60,7 @@ extern "C" {
 
 hmr_status hmr_binary_scalar(hmr_context_t ctx, int32_t op, const hmr_tensor_desc *out, const hmr_tensor_desc *a,
                              double s, int32_t scalar_first) {
-    return hmr::guarded([&] {
+    return hmr::fenced([&] {
         if (op != HMR_BINARY_MUL && op != HMR_BINARY_DIV) {
             return hmr::fail(HMR_INVALID, "binary_scalar: only Mul and Div keep their scalar unrounded");
         }
@@ -87,7 +87,7 @@ hmr_status hmr_binary_scalar(hmr_context_t ctx, int32_t op, const hmr_tensor_des
 hmr_status hmr_where_constant(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_tensor_desc *cond,
                               const hmr_tensor_desc *x, uint64_t x_bits, const hmr_tensor_desc *y,
                               uint64_t y_bits) {
-    return hmr::guarded([&] {
+    return hmr::fenced([&] {
         const hmr_tensor_desc *descs[4] = {out, cond, x, y};
         const uint64_t cbits[4] = {0, 0, x_bits, y_bits};
         return hmr::run_map(ctx, "where", 4, descs, cbits, [&](const hmr::MapCall &call, hipStream_t stream) {
@@ -107,7 +107,7 @@ hmr_status hmr_where(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_te
 }
 
 hmr_status hmr_fill(hmr_context_t ctx, const hmr_tensor_desc *dst, uint64_t bits) {
-    return hmr::guarded([&] {
+    return hmr::fenced([&] {
         const hmr_tensor_desc *descs[2] = {dst, nullptr};
         const uint64_t cbits[2] = {0, bits};
         return hmr::run_map(ctx, "fill", 2, descs, cbits, [&](const hmr::MapCall &call, hipStream_t stream) {

@@ -227,7 +227,7 @@ extern "C" {
 
 hmr_status hmr_fused(hmr_context_t ctx, int32_t op, const hmr_tensor_desc *out, const hmr_tensor_desc *a,
                      const hmr_tensor_desc *b, const hmr_tensor_desc *c, double coefficient, int32_t small) {
-    return hmr::guarded([&] {
+    return hmr::fenced([&] {
         if (op < HMR_FUSED_SCALED_ADD || op > HMR_FUSED_ADDCDIV) return hmr::fail(HMR_INVALID, "fused: unknown step");
         const bool three = op >= HMR_FUSED_ADDCMUL;
         if (three != (c != nullptr)) {
@@ -259,7 +259,7 @@ hmr_status hmr_fused(hmr_context_t ctx, int32_t op, const hmr_tensor_desc *out, 
 
 hmr_status hmr_addr(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_tensor_desc *v1, const hmr_tensor_desc *v2,
                     const hmr_tensor_desc *input, double alpha, double beta, int64_t alpha_int, int64_t beta_int) {
-    return hmr::guarded([&] {
+    return hmr::fenced([&] {
         const bool is_float = out->dtype >= HMR_F16 && out->dtype <= HMR_F64;
         const bool is_bool = out->dtype == HMR_BOOL;
         // The coefficients as the kernels take them: bits of the computation type, i64, or 0 / 1.
@@ -304,7 +304,7 @@ hmr_status hmr_addr(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_ten
 
 hmr_status hmr_triangle(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_tensor_desc *src, int64_t diagonal,
                         int32_t upper) {
-    return hmr::guarded([&] {
+    return hmr::fenced([&] {
         int64_t n = 0, m = 0;
         if (hmr_status s = hmr::check_desc(*out, n)) return s;
         if (hmr_status s = hmr::check_desc(*src, m)) return s;
@@ -314,7 +314,7 @@ hmr_status hmr_triangle(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr
         if (out->ndim < 2) return hmr::fail(HMR_INVALID, "triangle needs two dimensions");
         if (n == 0) return HMR_OK;
         if (n >= (int64_t{1} << 31)) return hmr::fail(HMR_INVALID, "triangle: more than 2^31 - 1 elements");
-        return hmr::launch_on(ctx, "triangle", [&](hipStream_t stream) {
+        return hmr::queue_on(ctx, "triangle", [&](hipStream_t stream) {
             if (src->dtype != out->dtype) return false;
             return hmr::with_word(hmr::dtype_size(out->dtype), [&](auto w) {
                 hmr::launch_triangle<typename decltype(w)::type>(*out, *src, n, diagonal, upper != 0, stream);
@@ -324,7 +324,7 @@ hmr_status hmr_triangle(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr
 }
 
 hmr_status hmr_flip(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_tensor_desc *src) {
-    return hmr::guarded([&] {
+    return hmr::fenced([&] {
         const hmr_tensor_desc *descs[2] = {out, src};
         return hmr::run_map(
             ctx, "flip", 2, descs, nullptr,

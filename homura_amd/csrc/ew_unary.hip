@@ -20,10 +20,10 @@ int table_slot(int op, int dtype) { return (dtype == HMR_BF16 ? kTableOps : 0) +
 hmr_status ensure_tables(hmr_context_t ctx) {
     std::lock_guard<std::mutex> lock(ctx->table_lock);
     if (ctx->tables != nullptr) return HMR_OK;
-    DeviceGuard guard;
-    if (hmr_status s = guard.enter(ctx->device)) return s;
+    Visit v;
+    if (hmr_status s = v.use_device(ctx->device)) return s;
     void *p = nullptr;
-    HMR_HIP(hipMalloc(&p, kTableSlots * kTableBytes));
+    if (hmr_status s = v.hip(hipMalloc(&p, kTableSlots * kTableBytes), "hipMalloc(&p, kTableSlots * kTableBytes)")) return s;
     ctx->tables = p;
     ctx->tables_filled = 0;
     return HMR_OK;
@@ -89,7 +89,7 @@ bool pick_unary(hmr_context_t ctx, int op, int out_dtype, int dtype, const MapCa
 
 extern "C" hmr_status hmr_unary(hmr_context_t ctx, int32_t op, const hmr_tensor_desc *out,
                                 const hmr_tensor_desc *src) {
-    return hmr::guarded([&] {
+    return hmr::fenced([&] {
         const hmr_tensor_desc *descs[2] = {out, src};
         return hmr::run_map(
             ctx, "unary", 2, descs, nullptr,

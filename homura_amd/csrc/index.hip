@@ -340,17 +340,129 @@ __global__ void __launch_bounds__(kBlock) index_runs_tiles_kernel(T *out, const 
     }
 }
 
+// ---- lines: gather and scatter_add along a dimension never leave their line -------------------------------------
+//
+// A line is the indexed dimension under one choice of all other coordinates. gather reads a line of the source
+// at the index's positions; scatter_add adds a line of contributions into a line of the output. Lines do not
+// interact, so a workgroup takes a line at a time and keeps what is accessed at random in LDS.
+
+// The offsets of line `line` (row-major over every dimension but `at`) in the three operands.
+__device__ __forceinline__ void line_bases(const Dims &d, int64_t line, int64_t (&base)[3]) {
+    base[0] = base[1] = base[2] = 0;
+    for (int k = 0; k < d.ndim; ++k) {
+        if (k == d.at) continue;
+        const int64_t q = line / d.size[k];
+        const int64_t c = line - q * d.size[k];
+        line = q;
+        base[0] += c * d.stride[0][k];
+        base[1] += c * d.stride[1][k];
+        base[2] += c * d.stride[2][k];
+    }
+}
+
+// gather: the source's line (contiguous, `length` elements) is staged in LDS with coalesced loads, the picks hit
+// LDS and leave as coalesced stores. stride[0] out, [1] src, [2] index; `count` positions per line.
+// Every 4-byte pick straight from memory costs a 64-byte sector and one address per lane in the texture path;
+// 512 picks from a 16 KB line touch nearly all of its sectors anyway.
+template <class W>
+__global__ void __launch_bounds__(kBlock) gather_lines_kernel(W *out, const W *src, const void *index, int is64, Dims d,
+                                                              int64_t lines, int64_t count, int64_t length) {
+    extern __shared__ __align__(16) unsigned char staged_raw[];
+    W *staged = reinterpret_cast<W *>(staged_raw);
+    constexpr int V = 16 / static_cast<int>(sizeof(W));
+    const int64_t out_step = d.stride[0][d.at], index_step = d.stride[2][d.at];
+    for (int64_t line = blockIdx.x; line < lines; line += gridDim.x) {
+        int64_t base[3];
+        line_bases(d, line, base);
+        const W *from = src + base[1];
+        __syncthreads();  // the previous line's picks have read LDS
+        if (reinterpret_cast<uintptr_t>(from) % 16 == 0 && length % V == 0) {
+            const u32x4 *q = reinterpret_cast<const u32x4 *>(from);
+            u32x4 *to = reinterpret_cast<u32x4 *>(staged);
+            for (int64_t t = threadIdx.x; t < length / V; t += kBlock) to[t] = __builtin_nontemporal_load(q + t);
+        } else {
+            for (int64_t e = threadIdx.x; e < length; e += kBlock) staged[e] = from[e];
+        }
+        __syncthreads();
+        W *to = out + base[0];
+        for (int64_t j = threadIdx.x; j < count; j += kBlock) {
+            to[j * out_step] = staged[read_index(index, is64, base[2] + j * index_step)];
+        }
+    }
+}
+
+// Sorts keys[0, N) ascending in LDS (N a power of two, every thread of the workgroup calls this).
+template <int N>
+__device__ __forceinline__ void sort_in_lds(uint64_t *keys) {
+    for (int k = 2; k <= N; k <<= 1) {
+        for (int j = k >> 1; j > 0; j >>= 1) {
+            for (int i = threadIdx.x; i < N; i += kBlock) {
+                const int partner = i ^ j;
+                if (partner > i) {
+                    const uint64_t a = keys[i], b = keys[partner];
+                    const bool ascending = (i & k) == 0;
+                    if ((a > b) == ascending) {
+                        keys[i] = b;
+                        keys[partner] = a;
+                    }
+                }
+            }
+            __syncthreads();
+        }
+    }
+}
+
+// scatter_add of lines of at most N positions: the line's words (target << 32 | position in the line) are sorted in
+// LDS - positions are distinct, so the order of equal targets is the order of their positions, the CPU's - and the
+// first word of each target sums its run, in that order, into the output element (f64 or wrapping i64 accumulation,
+// one rounding). stride[0] index, [1] out, [2] src, as for the kernels above.
+template <class T, int N>
+__global__ void __launch_bounds__(kBlock) scatter_lines_kernel(T *out, const T *src, const void *index, int is64, Dims d,
+                                                               int64_t lines, int count) {
+    using S = Sum<T>;
+    __shared__ uint64_t keys[N];
+    const int64_t index_step = d.stride[0][d.at], out_step = d.stride[1][d.at], src_step = d.stride[2][d.at];
+    for (int64_t line = blockIdx.x; line < lines; line += gridDim.x) {
+        int64_t base[3];
+        line_bases(d, line, base);
+        __syncthreads();  // the previous line's sums have read the keys
+        for (int j = threadIdx.x; j < N; j += kBlock) {
+            keys[j] = j < count ? (static_cast<uint64_t>(read_index(index, is64, base[0] + j * index_step)) << 32) | static_cast<uint32_t>(j)
+                                : ~uint64_t{0};
+        }
+        __syncthreads();
+        sort_in_lds<N>(keys);
+        for (int p = threadIdx.x; p < count; p += kBlock) {
+            const uint64_t target = keys[p] >> 32;
+            if (p > 0 && (keys[p - 1] >> 32) == target) continue;  // not the first of its run
+            T *po = out + base[1] + static_cast<int64_t>(target) * out_step;
+            typename S::A acc = S::widen(*po);
+            for (int e = p; e < count; ++e) {
+                const uint64_t w = keys[e];
+                if ((w >> 32) != target) break;
+                acc = S::add(acc, src[base[2] + static_cast<int64_t>(w & 0xFFFFFFFFu) * src_step]);
+            }
+            *po = S::narrow(acc);
+        }
+    }
+}
+
+// Lines worth a workgroup each: enough of them to cover the GPU, and positions per line in the range the LDS sort
+// takes. The index and the source run along the line with stride 1 (their loads are coalesced then).
+constexpr int64_t kMinLines = 128;
+constexpr int kMaxLinePositions = 2048;
+
 }  // namespace
 }  // namespace hmr
 
 using hmr::fail;
-using hmr::guarded;
+using hmr::fenced;
 
 extern "C" {
 
 hmr_status hmr_index_check(hmr_context_t ctx, const hmr_tensor_desc *index, int64_t low, int64_t high, int32_t has_exempt,
                            int64_t exempt, uint64_t *slot) {
-    return guarded([&] {
+    return fenced([&] {
         int64_t n = 0;
         if (hmr_status s = hmr::check_desc(*index, n)) return s;
         if (!hmr::is_index_dtype(index->dtype)) return fail(HMR_INVALID, "index_check: unsupported dtype");
@@ -359,7 +471,7 @@ hmr_status hmr_index_check(hmr_context_t ctx, const hmr_tensor_desc *index, int6
         const hmr::Dims d = hmr::dims_of(*index, ops, -1);
         const void *base = hmr::first_of(*index);
         const int is64 = index->dtype == HMR_I64;
-        return hmr::launch_on(ctx, "index_check", [&](hipStream_t stream) {
+        return hmr::queue_on(ctx, "index_check", [&](hipStream_t stream) {
             if (n <= hmr::kCheckSmall) {
                 hipLaunchKernelGGL(hmr::check_small_kernel, dim3(1), dim3(hmr::kCheckBlock), 0, stream, base, is64, d, n, low, high,
                                    has_exempt, exempt, slot);
@@ -381,7 +493,7 @@ hmr_status hmr_index_check(hmr_context_t ctx, const hmr_tensor_desc *index, int6
 // Positions reach 2^63 - 1 in views with zero strides, whose element count no longer fits 64 bits, so the
 // description is checked dimension by dimension and no product is formed.
 hmr_status hmr_test_index_value(hmr_context_t ctx, const hmr_tensor_desc *index, uint64_t *slot) {
-    return guarded([&] {
+    return fenced([&] {
         if (index == nullptr || slot == nullptr) return fail(HMR_INVALID, "index value: null argument");
         if (index->dtype < HMR_BOOL || index->dtype > HMR_F64) return fail(HMR_INVALID, "invalid dtype " + std::to_string(index->dtype));
         if (index->ndim < 0 || index->ndim > HMR_MAX_DIMS) {
@@ -397,7 +509,7 @@ hmr_status hmr_test_index_value(hmr_context_t ctx, const hmr_tensor_desc *index,
         const hmr::Dims d = hmr::dims_of(*index, ops, -1);
         const void *base = hmr::first_of(*index);
         const int is64 = index->dtype == HMR_I64;
-        return hmr::launch_on(ctx, "index value", [&](hipStream_t stream) {
+        return hmr::queue_on(ctx, "index value", [&](hipStream_t stream) {
             hipLaunchKernelGGL(hmr::check_value_kernel, dim3(1), dim3(1), 0, stream, base, is64, d, slot);
             return true;
         });
@@ -406,7 +518,7 @@ hmr_status hmr_test_index_value(hmr_context_t ctx, const hmr_tensor_desc *index,
 
 hmr_status hmr_index_select(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_tensor_desc *src,
                             const hmr_tensor_desc *index, int32_t dim, int32_t wrap_negative) {
-    return guarded([&] {
+    return fenced([&] {
         int64_t n = 0, m = 0, count = 0;
         if (hmr_status s = hmr::check_desc(*out, n)) return s;
         if (hmr_status s = hmr::check_desc(*src, m)) return s;
@@ -431,7 +543,7 @@ hmr_status hmr_index_select(hmr_context_t ctx, const hmr_tensor_desc *out, const
                     n < (int64_t{1} << 31) && reinterpret_cast<uintptr_t>(hmr::first_of(*out)) % 16 == 0 &&
                     reinterpret_cast<uintptr_t>(hmr::first_of(*src)) % 16 == 0;
         for (int k = 0; rows && k < last; ++k) rows = out->strides[k] % vec == 0 && src->strides[k] % vec == 0;
-        return hmr::launch_on(ctx, "index_select", [&](hipStream_t stream) {
+        return hmr::queue_on(ctx, "index_select", [&](hipStream_t stream) {
             if (src->dtype != out->dtype) return false;
             return hmr::with_word(elem, [&](auto w) {
                 using W = typename decltype(w)::type;
@@ -470,7 +582,7 @@ hmr_status hmr_index_select(hmr_context_t ctx, const hmr_tensor_desc *out, const
 
 hmr_status hmr_gather(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_tensor_desc *src, const hmr_tensor_desc *index,
                       int32_t dim) {
-    return guarded([&] {
+    return fenced([&] {
         int64_t n = 0, m = 0, count = 0;
         if (hmr_status s = hmr::check_desc(*out, n)) return s;
         if (hmr_status s = hmr::check_desc(*src, m)) return s;
@@ -482,10 +594,25 @@ hmr_status hmr_gather(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_t
         if (n == 0) return HMR_OK;
         const hmr_tensor_desc *const ops[3] = {out, src, index};
         const hmr::Dims d = hmr::dims_of(*out, ops, dim);
-        return hmr::launch_on(ctx, "gather", [&](hipStream_t stream) {
+        // Lines of the source staged in LDS: the source runs along `dim` with stride 1, a line fits 64 KB, there
+        // are enough lines to cover the GPU, and the picks are dense enough that most of a line's 64-byte sectors
+        // would be fetched anyway.
+        const int elem = hmr::dtype_size(out->dtype);
+        const int64_t picks = out->sizes[dim], length = src->sizes[dim], lines = n / picks;
+        const bool by_lines = src->strides[dim] == 1 && length * elem <= 65536 && lines >= hmr::kMinLines &&
+                              picks * 64 >= length * elem / 2 && picks >= 64;
+        return hmr::queue_on(ctx, "gather", [&](hipStream_t stream) {
             if (src->dtype != out->dtype) return false;
-            return hmr::with_word(hmr::dtype_size(out->dtype), [&](auto w) {
+            return hmr::with_word(elem, [&](auto w) {
                 using W = typename decltype(w)::type;
+                if (by_lines) {
+                    const unsigned grid = static_cast<unsigned>(lines < (int64_t{1} << 20) ? lines : (int64_t{1} << 20));
+                    hipLaunchKernelGGL((hmr::gather_lines_kernel<W>), dim3(grid), dim3(hmr::kBlock), static_cast<size_t>(length * elem),
+                                       stream, reinterpret_cast<W *>(hmr::first_of(*out)), reinterpret_cast<const W *>(hmr::first_of(*src)),
+                                       static_cast<const void *>(hmr::first_of(*index)), index->dtype == HMR_I64 ? 1 : 0, d, lines, picks,
+                                       length);
+                    return;
+                }
                 hipLaunchKernelGGL((hmr::pick_kernel<W>), dim3(hmr::grid_of(n)), dim3(hmr::kBlock), 0, stream,
                                    reinterpret_cast<W *>(hmr::first_of(*out)), reinterpret_cast<const W *>(hmr::first_of(*src)),
                                    static_cast<const void *>(hmr::first_of(*index)), index->dtype == HMR_I64 ? 1 : 0, d, n, int64_t{0});
@@ -495,7 +622,7 @@ hmr_status hmr_gather(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_t
 }
 
 hmr_status hmr_index_add_workspace(int64_t m, int64_t size, int64_t *bytes) {
-    return guarded([&] {
+    return fenced([&] {
         if (m < 0 || size < 0) return fail(HMR_INVALID, "index_add_workspace: negative size");
         if (m >= (int64_t{1} << 31) || size >= (int64_t{1} << 32)) {
             return fail(HMR_INVALID, "index_add: more than 2^31 - 1 positions or 2^32 - 1 slices");
@@ -506,7 +633,7 @@ hmr_status hmr_index_add_workspace(int64_t m, int64_t size, int64_t *bytes) {
 }
 
 hmr_status hmr_scatter_add_workspace(int64_t n, int64_t *bytes) {
-    return guarded([&] {
+    return fenced([&] {
         if (n < 0) return fail(HMR_INVALID, "scatter_add_workspace: negative size");
         if (n >= (int64_t{1} << 31)) return fail(HMR_INVALID, "scatter_add: more than 2^31 - 1 positions");
         *bytes = n == 0 ? 0 : hmr::sort_layout(n).bytes;
@@ -516,7 +643,7 @@ hmr_status hmr_scatter_add_workspace(int64_t n, int64_t *bytes) {
 
 hmr_status hmr_index_add(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_tensor_desc *src, const hmr_tensor_desc *index,
                          int32_t dim, void *workspace, int64_t workspace_bytes) {
-    return guarded([&] {
+    return fenced([&] {
         int64_t n = 0, total = 0, m = 0;
         if (hmr_status s = hmr::check_desc(*out, n)) return s;
         if (hmr_status s = hmr::check_desc(*src, total)) return s;
@@ -548,7 +675,7 @@ hmr_status hmr_index_add(hmr_context_t ctx, const hmr_tensor_desc *out, const hm
         uint64_t *words = static_cast<uint64_t *>(workspace);
         const int key_bits = hmr::bits_for(static_cast<uint64_t>(out->sizes[dim] > 0 ? out->sizes[dim] - 1 : 0));
         const int64_t index_stride = index->ndim == 1 ? index->strides[0] : 0;
-        return hmr::launch_on(ctx, "index_add", [&](hipStream_t stream) {
+        return hmr::queue_on(ctx, "index_add", [&](hipStream_t stream) {
             if (src->dtype != out->dtype) return false;
             return hmr::with_any_type(out->dtype, [&](auto t) {
                 using T = typename decltype(t)::type;
@@ -583,7 +710,7 @@ hmr_status hmr_index_add(hmr_context_t ctx, const hmr_tensor_desc *out, const hm
 
 hmr_status hmr_scatter_add(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_tensor_desc *src, const hmr_tensor_desc *index,
                            int32_t dim, void *workspace, int64_t workspace_bytes) {
-    return guarded([&] {
+    return fenced([&] {
         int64_t n = 0, total = 0, count = 0;
         if (hmr_status s = hmr::check_desc(*index, n)) return s;
         if (hmr_status s = hmr::check_desc(*out, total)) return s;
@@ -601,10 +728,29 @@ hmr_status hmr_scatter_add(hmr_context_t ctx, const hmr_tensor_desc *out, const 
         const hmr::Dims d = hmr::dims_of(*index, ops, dim);
         uint64_t *words = static_cast<uint64_t *>(workspace);
         const int key_bits = hmr::bits_for(static_cast<uint64_t>(hmr::reach_of(*out)));
-        return hmr::launch_on(ctx, "scatter_add", [&](hipStream_t stream) {
+        // Lines sorted in LDS (no global sort, no workspace traffic) when there are enough lines of a size the
+        // workgroup's sort takes; one long line, or many tiny ones, go through the global sort.
+        const int64_t positions = index->sizes[dim], lines = n / positions;
+        const bool by_lines = lines >= hmr::kMinLines && positions >= 64 && positions <= hmr::kMaxLinePositions &&
+                              index->strides[dim] == 1 && src->strides[dim] == 1;
+        return hmr::queue_on(ctx, "scatter_add", [&](hipStream_t stream) {
             if (src->dtype != out->dtype) return false;
             return hmr::with_any_type(out->dtype, [&](auto t) {
                 using T = typename decltype(t)::type;
+                if (by_lines) {
+                    const unsigned grid = static_cast<unsigned>(lines < (int64_t{1} << 20) ? lines : (int64_t{1} << 20));
+                    auto run = [&](auto padded) {
+                        constexpr int N = decltype(padded)::value;
+                        hipLaunchKernelGGL((hmr::scatter_lines_kernel<T, N>), dim3(grid), dim3(hmr::kBlock), 0, stream,
+                                           reinterpret_cast<T *>(hmr::first_of(*out)), reinterpret_cast<const T *>(hmr::first_of(*src)),
+                                           static_cast<const void *>(hmr::first_of(*index)), index->dtype == HMR_I64 ? 1 : 0, d, lines,
+                                           static_cast<int>(positions));
+                    };
+                    if (positions <= 128) run(hmr::IntTag<128>{});
+                    else if (positions <= 512) run(hmr::IntTag<512>{});
+                    else run(hmr::IntTag<2048>{});
+                    return;
+                }
                 hipLaunchKernelGGL(hmr::scatter_words_kernel, dim3(hmr::grid_of(n)), dim3(hmr::kBlock), 0, stream, words,
                                    static_cast<const void *>(hmr::first_of(*index)), index->dtype == HMR_I64 ? 1 : 0, d, n);
                 const uint64_t *sorted = hmr::sort_words(workspace, n, key_bits, stream);

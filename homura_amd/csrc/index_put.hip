@@ -272,13 +272,13 @@ bool mask_is_flat(const hmr_tensor_desc &mask) {
 }  // namespace hmr
 
 using hmr::fail;
-using hmr::guarded;
+using hmr::fenced;
 
 extern "C" {
 
 hmr_status hmr_index_positions(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_tensor_desc *coord, int64_t size, int64_t stride,
                                int32_t first) {
-    return guarded([&] {
+    return fenced([&] {
         int64_t n = 0, m = 0;
         if (hmr_status s = hmr::check_desc(*out, n)) return s;
         if (hmr_status s = hmr::check_desc(*coord, m)) return s;
@@ -288,7 +288,7 @@ hmr_status hmr_index_positions(hmr_context_t ctx, const hmr_tensor_desc *out, co
         if (n == 0) return HMR_OK;
         const hmr_tensor_desc *const ops[3] = {out, coord, nullptr};
         const hmr::Dims d = hmr::dims_of(*out, ops, -1);
-        return hmr::launch_on(ctx, "index_positions", [&](hipStream_t stream) {
+        return hmr::queue_on(ctx, "index_positions", [&](hipStream_t stream) {
             hipLaunchKernelGGL(hmr::positions_kernel, dim3(hmr::grid_of(n)), dim3(hmr::kBlock), 0, stream,
                                reinterpret_cast<int64_t *>(hmr::first_of(*out)), static_cast<const void *>(hmr::first_of(*coord)),
                                coord->dtype == HMR_I64 ? 1 : 0, d, n, size, stride, first);
@@ -298,7 +298,7 @@ hmr_status hmr_index_positions(hmr_context_t ctx, const hmr_tensor_desc *out, co
 }
 
 hmr_status hmr_index_overwrite_workspace(int64_t size, int64_t *bytes) {
-    return guarded([&] {
+    return fenced([&] {
         if (size < 0) return fail(HMR_INVALID, "index_overwrite_workspace: negative size");
         *bytes = size * 8;
         return HMR_OK;
@@ -307,7 +307,7 @@ hmr_status hmr_index_overwrite_workspace(int64_t size, int64_t *bytes) {
 
 hmr_status hmr_index_overwrite(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_tensor_desc *src,
                                const hmr_tensor_desc *positions, int32_t dim, void *workspace, int64_t workspace_bytes) {
-    return guarded([&] {
+    return fenced([&] {
         int64_t n = 0, total = 0, m = 0;
         if (hmr_status s = hmr::check_desc(*out, n)) return s;
         if (hmr_status s = hmr::check_desc(*src, total)) return s;
@@ -343,7 +343,7 @@ hmr_status hmr_index_overwrite(hmr_context_t ctx, const hmr_tensor_desc *out, co
                            reinterpret_cast<uintptr_t>(hmr::first_of(*out)) % 16 == 0 &&
                            reinterpret_cast<uintptr_t>(hmr::first_of(*src)) % 16 == 0 && out->strides[dim] % vec == 0 &&
                            src->strides[dim] % vec == 0;
-        return hmr::launch_on(ctx, "index_overwrite", [&](hipStream_t stream) {
+        return hmr::queue_on(ctx, "index_overwrite", [&](hipStream_t stream) {
             hipLaunchKernelGGL(hmr::winners_clear_kernel, dim3(hmr::grid_of(size)), dim3(hmr::kBlock), 0, stream, winners, size);
             hipLaunchKernelGGL(hmr::winners_kernel, dim3(hmr::grid_of(m)), dim3(hmr::kBlock), 0, stream, winners, pos, is64, position_stride,
                                m);
@@ -366,7 +366,7 @@ hmr_status hmr_index_overwrite(hmr_context_t ctx, const hmr_tensor_desc *out, co
 }
 
 hmr_status hmr_mask_workspace(int64_t n, int64_t *bytes, int64_t *total_word) {
-    return guarded([&] {
+    return fenced([&] {
         if (n < 0) return fail(HMR_INVALID, "mask_workspace: negative size");
         const int64_t tiles = hmr::mask_tiles(n);
         *bytes = (tiles + 1) * 8;
@@ -376,7 +376,7 @@ hmr_status hmr_mask_workspace(int64_t n, int64_t *bytes, int64_t *total_word) {
 }
 
 hmr_status hmr_mask_count(hmr_context_t ctx, const hmr_tensor_desc *mask, void *workspace, int64_t workspace_bytes) {
-    return guarded([&] {
+    return fenced([&] {
         int64_t n = 0;
         if (hmr_status s = hmr::check_desc(*mask, n)) return s;
         if (mask->dtype != HMR_BOOL) return fail(HMR_INVALID, "mask_count: the mask is BOOL");
@@ -388,7 +388,7 @@ hmr_status hmr_mask_count(hmr_context_t ctx, const hmr_tensor_desc *mask, void *
         uint64_t *counts = static_cast<uint64_t *>(workspace);
         const bool flat = hmr::mask_is_flat(*mask);
         const int64_t cap = int64_t{1} << 20;
-        return hmr::launch_on(ctx, "mask_count", [&](hipStream_t stream) {
+        return hmr::queue_on(ctx, "mask_count", [&](hipStream_t stream) {
             if (tiles > 0) {
                 const dim3 grid(static_cast<unsigned>(tiles < cap ? tiles : cap));
                 if (flat) hipLaunchKernelGGL((hmr::mask_count_kernel<true>), grid, dim3(hmr::kBlock), 0, stream, base, d, n, tiles, counts);
@@ -402,7 +402,7 @@ hmr_status hmr_mask_count(hmr_context_t ctx, const hmr_tensor_desc *mask, void *
 
 hmr_status hmr_mask_coordinates(hmr_context_t ctx, const hmr_tensor_desc *mask, void *workspace, int64_t workspace_bytes,
                                 const hmr_tensor_desc *out) {
-    return guarded([&] {
+    return fenced([&] {
         int64_t n = 0, total = 0;
         if (hmr_status s = hmr::check_desc(*mask, n)) return s;
         if (hmr_status s = hmr::check_desc(*out, total)) return s;
@@ -423,7 +423,7 @@ hmr_status hmr_mask_coordinates(hmr_context_t ctx, const hmr_tensor_desc *mask, 
         hmr::MaskDivs divs{};
         for (int k = 0; small && k < d.ndim; ++k) divs.d[k] = hmr::make_fastdiv(static_cast<uint32_t>(d.size[k]));
         const int64_t cap = int64_t{1} << 20;
-        return hmr::launch_on(ctx, "mask_coordinates", [&](hipStream_t stream) {
+        return hmr::queue_on(ctx, "mask_coordinates", [&](hipStream_t stream) {
             const dim3 grid(static_cast<unsigned>(tiles < cap ? tiles : cap));
             auto run = [&](auto flat_tag, auto small_tag) {
                 hipLaunchKernelGGL((hmr::mask_write_kernel<decltype(flat_tag)::value, decltype(small_tag)::value>), grid,

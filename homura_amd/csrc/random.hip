@@ -278,12 +278,12 @@ extern "C" {
 
 hmr_status hmr_random_uniform(hmr_context_t ctx, const hmr_tensor_desc *out, uint64_t seed, uint64_t offset, double from,
                               double to) {
-    return hmr::guarded([&] {
+    return hmr::fenced([&] {
         int64_t n = 0;
         char *first = nullptr;
         if (hmr_status s = hmr::flat_output(*out, n, first)) return s;
         if (n == 0) return HMR_OK;
-        return hmr::launch_on(ctx, "random_uniform", [&](hipStream_t stream) {
+        return hmr::queue_on(ctx, "random_uniform", [&](hipStream_t stream) {
             return hmr::with_float_type(out->dtype, [&](auto t) {
                 using T = typename decltype(t)::type;
                 const int64_t per = std::is_same_v<T, double> ? 2 : 4;
@@ -297,12 +297,12 @@ hmr_status hmr_random_uniform(hmr_context_t ctx, const hmr_tensor_desc *out, uin
 
 hmr_status hmr_random_normal(hmr_context_t ctx, const hmr_tensor_desc *out, uint64_t seed, uint64_t offset, double mean,
                              double std) {
-    return hmr::guarded([&] {
+    return hmr::fenced([&] {
         int64_t n = 0;
         char *first = nullptr;
         if (hmr_status s = hmr::flat_output(*out, n, first)) return s;
         if (n == 0) return HMR_OK;
-        return hmr::launch_on(ctx, "random_normal", [&](hipStream_t stream) {
+        return hmr::queue_on(ctx, "random_normal", [&](hipStream_t stream) {
             return hmr::with_float_type(out->dtype, [&](auto t) {
                 using T = typename decltype(t)::type;
                 const int64_t blocks = (n + 1) / 2;
@@ -315,7 +315,7 @@ hmr_status hmr_random_normal(hmr_context_t ctx, const hmr_tensor_desc *out, uint
 
 hmr_status hmr_random_int(hmr_context_t ctx, const hmr_tensor_desc *out, uint64_t seed, uint64_t offset, uint64_t blocks,
                           int64_t low, uint64_t range, uint64_t threshold, void *workspace) {
-    return hmr::guarded([&] {
+    return hmr::fenced([&] {
         int64_t n = 0;
         char *first = nullptr;
         if (hmr_status s = hmr::flat_output(*out, n, first)) return s;
@@ -330,7 +330,7 @@ hmr_status hmr_random_int(hmr_context_t ctx, const hmr_tensor_desc *out, uint64_
         const int64_t tiles = (nblocks + HMR_RANDOM_INT_TILE - 1) / HMR_RANDOM_INT_TILE;
         if (threshold != 0 && tiles > (int64_t{1} << 31) - 1) return hmr::fail(HMR_INVALID, "random_int: too many blocks in one batch");
         if (blocks == 0 && threshold == 0) return HMR_OK;
-        return hmr::launch_on(ctx, "random_int", [&](hipStream_t stream) {
+        return hmr::queue_on(ctx, "random_int", [&](hipStream_t stream) {
             int64_t *po = reinterpret_cast<int64_t *>(first);
             if (threshold == 0) {
                 if (n == 0) return true;

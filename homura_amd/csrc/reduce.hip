@@ -189,7 +189,7 @@ hmr_status run_reduce(hmr_context_t ctx, int32_t op, const hmr_tensor_desc *out,
     if ((op == HMR_REDUCE_MAX || op == HMR_REDUCE_MIN) && p.args.nred == 0) {
         return fail(HMR_INVALID, "reduction over an empty dimension");
     }
-    return launch_on(ctx, "reduce", [&](hipStream_t stream) {
+    return queue_on(ctx, "reduce", [&](hipStream_t stream) {
         const int dtype = kept->dtype;
         void *o = element0(*out);
         switch (op) {
@@ -219,7 +219,8 @@ hmr_status run_reduce(hmr_context_t ctx, int32_t op, const hmr_tensor_desc *out,
 
 hmr_status bind_reduce_scratch(hmr_context &ctx) {
     void *address = nullptr;
-    HMR_HIP(hipGetSymbolAddress(&address, HIP_SYMBOL(::scratch)));
+    const hipError_t found = hipGetSymbolAddress(&address, HIP_SYMBOL(::scratch));
+    if (found != hipSuccess) return hip_failure(found, "hipGetSymbolAddress(&address, HIP_SYMBOL(scratch))");
     if (address == nullptr) return fail(HMR_INTERNAL_ERROR, "the static reduction block has no device address");
     ctx.reduce_scratch = address;
     return HMR_OK;
@@ -227,13 +228,13 @@ hmr_status bind_reduce_scratch(hmr_context &ctx) {
 
 }  // namespace hmr
 
-using hmr::guarded;
+using hmr::fenced;
 
 extern "C" {
 
 hmr_status hmr_reduce_workspace(const hmr_tensor_desc *kept, const hmr_tensor_desc *red, int32_t var,
                                 int64_t *bytes) {
-    return guarded([&] {
+    return fenced([&] {
         hmr::ReducePlan p;
         if (hmr_status s = hmr::plan_reduction(nullptr, *kept, *red, p)) return s;
         *bytes = hmr::means_bytes(p, var != 0) + hmr::partial_bytes(p, var != 0);
@@ -243,7 +244,7 @@ hmr_status hmr_reduce_workspace(const hmr_tensor_desc *kept, const hmr_tensor_de
 
 hmr_status hmr_test_reduce_plan(const hmr_tensor_desc *kept, const hmr_tensor_desc *red, int64_t *group,
                                 int64_t *splits, int64_t *chunk) {
-    return guarded([&] {
+    return fenced([&] {
         hmr::ReducePlan p;
         if (hmr_status s = hmr::plan_reduction(nullptr, *kept, *red, p)) return s;
         *group = p.group;
@@ -255,7 +256,7 @@ hmr_status hmr_test_reduce_plan(const hmr_tensor_desc *kept, const hmr_tensor_de
 
 hmr_status hmr_reduce(hmr_context_t ctx, int32_t op, const hmr_tensor_desc *out, const hmr_tensor_desc *kept,
                       const hmr_tensor_desc *red, void *workspace, int64_t workspace_bytes) {
-    return guarded([&] {
+    return fenced([&] {
         hmr::ReducePlan p;
         if (hmr_status s = hmr::plan_reduction(out, *kept, *red, p)) return s;
         void *partials = nullptr;
@@ -266,7 +267,7 @@ hmr_status hmr_reduce(hmr_context_t ctx, int32_t op, const hmr_tensor_desc *out,
 
 hmr_status hmr_reduce_static(hmr_context_t ctx, int32_t op, const hmr_tensor_desc *out, const hmr_tensor_desc *kept,
                              const hmr_tensor_desc *red) {
-    return guarded([&] {
+    return fenced([&] {
         hmr::ReducePlan p;
         if (hmr_status s = hmr::plan_reduction(out, *kept, *red, p)) return s;
         const int64_t need = hmr::partial_bytes(p, false);
@@ -285,13 +286,13 @@ hmr_status hmr_reduce_static(hmr_context_t ctx, int32_t op, const hmr_tensor_des
 hmr_status hmr_var(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_tensor_desc *kept,
                    const hmr_tensor_desc *red, double correction, int32_t take_sqrt, void *workspace,
                    int64_t workspace_bytes) {
-    return guarded([&] {
+    return fenced([&] {
         hmr::ReducePlan p;
         if (hmr_status s = hmr::plan_reduction(out, *kept, *red, p)) return s;
         void *partials = nullptr;
         if (hmr_status s = hmr::take_workspace(p, true, workspace, workspace_bytes, partials)) return s;
         if (p.args.nout == 0) return HMR_OK;
-        return hmr::launch_on(ctx, "var", [&](hipStream_t stream) {
+        return hmr::queue_on(ctx, "var", [&](hipStream_t stream) {
             if (out->dtype != kept->dtype || !hmr::is_float(kept->dtype)) return false;
             double *means = static_cast<double *>(workspace);
             double divisor = static_cast<double>(p.args.nred) - correction;
@@ -310,7 +311,7 @@ hmr_status hmr_var(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_tens
 hmr_status hmr_arg_reduce(hmr_context_t ctx, const hmr_tensor_desc *values, const hmr_tensor_desc *indices,
                           const hmr_tensor_desc *kept, const hmr_tensor_desc *red, int32_t is_max, void *workspace,
                           int64_t workspace_bytes) {
-    return guarded([&] {
+    return fenced([&] {
         hmr::ReducePlan p;
         if (hmr_status s = hmr::plan_reduction(indices, *kept, *red, p)) return s;
         if (values != nullptr) {
@@ -321,7 +322,7 @@ hmr_status hmr_arg_reduce(hmr_context_t ctx, const hmr_tensor_desc *values, cons
         if (hmr_status s = hmr::take_workspace(p, false, workspace, workspace_bytes, partials)) return s;
         if (p.args.nred == 0) return hmr::fail(HMR_INVALID, "arg reduction of an empty dimension");
         if (p.args.nout == 0) return HMR_OK;
-        return hmr::launch_on(ctx, "arg_reduce", [&](hipStream_t stream) {
+        return hmr::queue_on(ctx, "arg_reduce", [&](hipStream_t stream) {
             if (indices->dtype != HMR_I64) return false;
             if (values != nullptr && values->dtype != kept->dtype) return false;
             return hmr::launch_extreme_reduce(is_max != 0, kept->dtype, p, partials,

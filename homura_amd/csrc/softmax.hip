@@ -665,12 +665,12 @@ void launch_cumprod(const CumprodArgs &a, hipStream_t stream) {
 }  // namespace
 }  // namespace hmr
 
-using hmr::guarded;
+using hmr::fenced;
 
 extern "C" {
 
 hmr_status hmr_softmax_workspace(const hmr_tensor_desc *src_rows, int64_t n, int64_t src_stride, int64_t *bytes) {
-    return guarded([&] {
+    return fenced([&] {
         int64_t nrows = 0;
         if (hmr_status s = hmr::check_rows(*src_rows, *src_rows, n, 0, src_stride, nrows)) return s;
         *bytes = 0;  // no plan of this library cuts a row across workgroups
@@ -680,7 +680,7 @@ hmr_status hmr_softmax_workspace(const hmr_tensor_desc *src_rows, int64_t n, int
 
 hmr_status hmr_test_softmax_plan(const hmr_tensor_desc *src_rows, int64_t n, int64_t src_stride, int32_t *split,
                                  int32_t *group, int32_t *cache) {
-    return guarded([&] {
+    return fenced([&] {
         int64_t nrows = 0;
         if (hmr_status s = hmr::check_rows(*src_rows, *src_rows, n, 0, src_stride, nrows)) return s;
         hmr::Walk wo, ws;
@@ -698,7 +698,7 @@ hmr_status hmr_softmax(hmr_context_t ctx, const hmr_tensor_desc *out_rows, const
                        int64_t workspace_bytes) {
     (void)workspace;
     (void)workspace_bytes;
-    return guarded([&] {
+    return fenced([&] {
         int64_t nrows = 0;
         if (hmr_status s = hmr::check_rows(*out_rows, *src_rows, n, out_stride, src_stride, nrows)) return s;
         if (nrows == 0 || n == 0) return HMR_OK;
@@ -713,7 +713,7 @@ hmr_status hmr_softmax(hmr_context_t ctx, const hmr_tensor_desc *out_rows, const
         hmr::SoftmaxPlan plan = hmr::plan_softmax(*src_rows, n, src_stride, a.src_rows);
         bool out_ok = (n == 1 || out_stride == 1) && reinterpret_cast<uintptr_t>(a.out) % 16 == 0;
         for (int d = 0; out_ok && d < a.out_rows.ndim; ++d) out_ok = (a.out_rows.stride[d] * elem) % 16 == 0;
-        return hmr::launch_on(ctx, "softmax", [&](hipStream_t stream) {
+        return hmr::queue_on(ctx, "softmax", [&](hipStream_t stream) {
             if (out_rows->dtype != src_rows->dtype) return false;
             return hmr::with_float_type(out_rows->dtype, [&](auto t) {
                 using T = typename decltype(t)::type;
@@ -726,7 +726,7 @@ hmr_status hmr_softmax(hmr_context_t ctx, const hmr_tensor_desc *out_rows, const
 
 hmr_status hmr_exclusive_cumprod(hmr_context_t ctx, const hmr_tensor_desc *out_lines, const hmr_tensor_desc *src_lines,
                                  int64_t n, int64_t out_stride, int64_t src_stride, int32_t reverse) {
-    return guarded([&] {
+    return fenced([&] {
         int64_t nlines = 0;
         if (hmr_status s = hmr::check_rows(*out_lines, *src_lines, n, out_stride, src_stride, nlines)) return s;
         if (nlines == 0 || n == 0) return HMR_OK;
@@ -739,7 +739,7 @@ hmr_status hmr_exclusive_cumprod(hmr_context_t ctx, const hmr_tensor_desc *out_l
         a.so = out_stride;
         a.si = src_stride;
         a.reverse = reverse != 0;
-        return hmr::launch_on(ctx, "exclusive_cumprod", [&](hipStream_t stream) {
+        return hmr::queue_on(ctx, "exclusive_cumprod", [&](hipStream_t stream) {
             if (out_lines->dtype != src_lines->dtype) return false;
             return hmr::with_float_type(out_lines->dtype, [&](auto t) {
                 hmr::launch_cumprod<typename decltype(t)::type>(a, stream);

@@ -6,7 +6,7 @@
 
 namespace {
 hmr_status unbuilt(const char *name) {
-    return hmr::guarded([&] { return hmr::fail(HMR_INVALID, std::string(name) + ": not built in this library"); });
+    return hmr::fenced([&] { return hmr::fail(HMR_INVALID, std::string(name) + ": not built in this library"); });
 }
 }  // namespace
 
