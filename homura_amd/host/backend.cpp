@@ -786,7 +786,10 @@ void gather(const TensorData &out, const TensorData &src, size_t dim, const Tens
     std::vector<hmr_tensor_desc> d;
     int at = 0;
     const bool work = out.layout.num_elements() > 0;
-    if (work) d = around("gather", {walked(out), walked(src), walked(index)}, out.layout.shape, dim, at);
+    if (work) {
+        d = around("gather", {walked(out), walked(src), walked(index)}, out.layout.shape, dim, at);
+        d[1].sizes[at] = size;  // the source's own length along `dim`, as for index_select
+    }
     run_checked("gather", out, index, dim, size, Bounds::NonNegative, [&](hmr_context_t ctx) {
         if (work) expect(hmr_gather(ctx, &d[0], &d[1], &d[2], at));
     });
