@@ -180,7 +180,7 @@ def per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP
     """[{cfg, op, bytes, us, gbs, frac}] for the ops of BASELINE.json configs[0..4] (cfg = index)."""
     rows = []
 
-    def add(cfg, op, nbytes, fns, iters=20):
+    def add(cfg, op, nbytes, fns, iters=50):
         """fns: one callable, or several over disjoint buffers that are cycled so that a working set
         smaller than the 256 MB Infinity Cache is read from HBM every time."""
         fns = fns if isinstance(fns, list) else [fns]
@@ -343,6 +343,20 @@ def per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP
     add(None, "randint [0, 1024) i64 [8,2048,4096] (no rejection)", 8 * N, lambda: h.randint(0, 1024, shape, DT.I64, GPU), 10)
     add(None, "randint [-5, 6) i64 [8,2048,4096] (rejection: count, scan, write + a read-back)", 8 * N,
         lambda: h.randint(-5, 6, shape, DT.I64, GPU), 5)
+    # General layouts: transposed and permuted views made contiguous or combined with a contiguous operand (a tile
+    # of the two dimensions goes through LDS), and every other column (one element per lane).
+    sqm = residual.reshape([8192, 8192])
+    sqt = sqm.transpose(0, 1)
+    add(None, "transpose f32 [8192,8192] -> contiguous (tiles through LDS)", 8 * N, lambda: sqt.contiguous(), 10)
+    add(None, "transposed + contiguous f32 [8192,8192] (tiles through LDS)", 12 * N, lambda: sqt.add(sqm), 10)
+    sqb = x.reshape([8192, 8192]).transpose(0, 1)
+    add(None, "transpose bf16 [8192,8192] -> contiguous (tiles through LDS)", 4 * N, lambda: sqb.contiguous(), 10)
+    cube = residual.reshape([64, 1024, 1024]).permute([2, 0, 1])
+    add(None, "permute(2,0,1) f32 [64,1024,1024] -> contiguous (tiles through LDS)", 8 * N, lambda: cube.contiguous(), 10)
+    halfcols = sqm.slice(1, 0, 8192, 2)
+    add(None, "every other column f32 [8192,4096] -> contiguous (general kernel, an element per lane)", 4 * N,
+        lambda: halfcols.contiguous(), 10)
+    del sqm, sqt, sqb, cube, halfcols
     sq = residual.reshape([16, 2048, 2048])
     add(None, "triu(1) f32 [16,2048,2048] (reads the kept half)", 6 * N, lambda: sq.triu(1))
     add(None, "tril(0) f32 [16,2048,2048] (reads the kept half)", 6 * N, lambda: sq.tril(0))
