@@ -10,6 +10,7 @@
 #include <cmath>
 
 #include "ew_common.hpp"
+#include "normal_math.hpp"
 
 namespace hmr {
 namespace {
@@ -100,17 +101,28 @@ __global__ void __launch_bounds__(kBlock) uniform_kernel(T *out, int64_t n, int6
     }
 }
 
+struct HardwareSeeds {
+    static __device__ __forceinline__ double rcp(double x) { return __builtin_amdgcn_rcp(x); }
+    static __device__ __forceinline__ double rsq(double x) { return __builtin_amdgcn_rsq(x); }
+};
+
 template <class T>
 __global__ void __launch_bounds__(kBlock) normal_kernel(T *out, int64_t n, int64_t blocks, uint64_t seed, uint64_t offset,
                                                         double mean, double std) {
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; i < blocks;
          i += static_cast<int64_t>(gridDim.x) * kBlock) {
         const Word4 b = philox_block(offset + static_cast<uint64_t>(i), seed);
-        // Box-Muller in f64: each block gives two normals, the cosine first.
+        // Box-Muller in f64: each block gives two normals, the cosine first. Outputs narrower than f64 take
+        // the short polynomials of normal_math.hpp.
         const double u1 = 1.0 - unit_f64(b.v[0], b.v[1]), u2 = unit_f64(b.v[2], b.v[3]);
-        const double r = sqrt(-2.0 * log(u1));
-        const double theta = 2.0 * 3.14159265358979323846 * u2;
-        const T v[2] = {Conv<T>::from_f64(mean + std * r * cos(theta)), Conv<T>::from_f64(mean + std * r * sin(theta))};
+        double r, c, s;
+        if constexpr (std::is_same_v<T, double>) {
+            const double theta = 2.0 * 3.14159265358979323846 * u2;
+            r = sqrt(-2.0 * log(u1)), c = cos(theta), s = sin(theta);
+        } else {
+            normal_polar<HardwareSeeds>(u1, u2, r, c, s);
+        }
+        const T v[2] = {Conv<T>::from_f64(mean + std * r * c), Conv<T>::from_f64(mean + std * r * s)};
         store_span<T, 2>(out, 2 * i, n, v);
     }
 }
@@ -122,8 +134,9 @@ __global__ void __launch_bounds__(kBlock) normal_kernel(T *out, int64_t n, int64
 // is element j. Otherwise the batch is compacted in three launches over tiles of
 // HMR_RANDOM_INT_TILE blocks (a workgroup's width): count the accepted words of each group of tiles,
 // scan the counts (one workgroup), write each group's accepted words from its offset on, the
-// blocks being computed again. The workspace holds the counts and the offsets (room for one per
-// tile each) and the batch's total (its last word).
+// blocks being computed again. The first launch also writes the elements as if nothing were rejected
+// and the third returns at once when the total says so, which is the usual case. The workspace holds
+// the counts and the offsets (room for one per tile each) and the batch's total (its last word).
 static_assert(HMR_RANDOM_INT_TILE == kBlock, "a tile is one workgroup's blocks");
 
 __device__ __forceinline__ void int_words(const Word4 &b, uint64_t (&w)[2]) {
@@ -184,7 +197,11 @@ __device__ __forceinline__ uint32_t rank_in_tile(uint32_t mine, uint32_t &total)
 // has few entries (the workspace has room for one per tile; the first `groups` of each half are used).
 constexpr int kTilesPerGroup = 16;
 
-__global__ void __launch_bounds__(kBlock) int_count_kernel(uint64_t *counts, int64_t blocks, uint64_t seed, uint64_t offset,
+// Counts the accepted words of each group and, on the way, writes word j as element j: right as it
+// stands when the batch rejects nothing, which is all but certain for a small range (a word is rejected
+// with probability range / 2^64 or so). int_write_kernel puts the elements where they belong otherwise.
+__global__ void __launch_bounds__(kBlock) int_count_kernel(uint64_t *counts, int64_t *out, int64_t n, int64_t blocks,
+                                                           uint64_t seed, uint64_t offset, int64_t low, Modulus modulus,
                                                            uint64_t threshold) {
     uint32_t mine = 0;
     for (int j = 0; j < kTilesPerGroup; ++j) {
@@ -193,6 +210,11 @@ __global__ void __launch_bounds__(kBlock) int_count_kernel(uint64_t *counts, int
             uint64_t w[2];
             int_words(philox_block(offset + static_cast<uint64_t>(i), seed), w);
             mine += (w[0] >= threshold ? 1u : 0u) + (w[1] >= threshold ? 1u : 0u);
+            if (2 * i < n) {
+                const int64_t v[2] = {static_cast<int64_t>(static_cast<uint64_t>(low) + remainder(w[0], modulus)),
+                                      static_cast<int64_t>(static_cast<uint64_t>(low) + remainder(w[1], modulus))};
+                store_span<int64_t, 2>(out, 2 * i, n, v);
+            }
         }
     }
     uint32_t total;
@@ -230,7 +252,8 @@ __global__ void __launch_bounds__(kScanThreads) int_scan_kernel(const uint64_t *
 
 __global__ void __launch_bounds__(kBlock) int_write_kernel(int64_t *out, int64_t n, const uint64_t *offsets, int64_t blocks,
                                                            uint64_t seed, uint64_t offset, int64_t low, Modulus modulus,
-                                                           uint64_t threshold) {
+                                                           uint64_t threshold, const uint64_t *total_accepted) {
+    if (*total_accepted == 2 * static_cast<uint64_t>(blocks)) return;  // nothing rejected: int_count_kernel wrote it all
     uint64_t running = offsets[blockIdx.x];  // accepted words before this group's first tile
     for (int j = 0; j < kTilesPerGroup; ++j) {
         const int64_t i = (static_cast<int64_t>(blockIdx.x) * kTilesPerGroup + j) * kBlock + threadIdx.x;
@@ -343,12 +366,12 @@ hmr_status hmr_random_int(hmr_context_t ctx, const hmr_tensor_desc *out, uint64_
             const int64_t groups = (tiles + hmr::kTilesPerGroup - 1) / hmr::kTilesPerGroup;
             if (groups > 0) {
                 hipLaunchKernelGGL(hmr::int_count_kernel, dim3(static_cast<unsigned>(groups)), dim3(hmr::kBlock), 0, stream, counts,
-                                   nblocks, seed, offset, threshold);
+                                   po, n, nblocks, seed, offset, low, hmr::make_modulus(range), threshold);
             }
             hipLaunchKernelGGL(hmr::int_scan_kernel, dim3(1), dim3(hmr::kScanThreads), 0, stream, counts, offsets, total, groups);
             if (groups > 0 && n > 0) {
                 hipLaunchKernelGGL(hmr::int_write_kernel, dim3(static_cast<unsigned>(groups)), dim3(hmr::kBlock), 0, stream, po, n,
-                                   offsets, nblocks, seed, offset, low, hmr::make_modulus(range), threshold);
+                                   offsets, nblocks, seed, offset, low, hmr::make_modulus(range), threshold, total);
             }
             return true;
         });
