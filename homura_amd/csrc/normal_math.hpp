@@ -40,10 +40,11 @@ __host__ __device__ __forceinline__ double normal_log(double u) {
     return __builtin_fma(static_cast<double>(e), 0.6931471805599453, log_m);
 }
 
-// sqrt(x) for a finite x >= 0: the estimate of 1 / sqrt(x) refined once (2^-44 at least).
+// sqrt(x) for a finite x >= 0: the estimate of 1 / sqrt(x) refined once (2^-44 at least). Zero, which only
+// u1 = 1 gives, is taken for 1e-300: its root, 1e-150, vanishes in every output narrower than f64.
 template <class Seeds>
-__host__ __device__ __forceinline__ double normal_sqrt(double x) {
-    if (!(x > 0.0)) return 0.0;
+__host__ __device__ __forceinline__ double normal_sqrt(double x_in) {
+    const double x = __builtin_fmax(x_in, 1e-300);
     const double y = Seeds::rsq(x), g = x * y;
     return __builtin_fma(__builtin_fma(-g, g, x), 0.5 * y, g);
 }

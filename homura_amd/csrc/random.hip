@@ -37,10 +37,14 @@ __device__ __forceinline__ Word4 philox_block(uint64_t n, uint64_t seed) {
     return Word4{{c0, c1, c2, c3}};
 }
 
-// A uniform f64 in [0, 1) from 53 random bits / from the top BITS bits of x (exact in f64).
+// A uniform f64 in [0, 1) from 53 random bits: (hi * 2^21 + (lo >> 11)) * 2^-53, built from two 32-bit
+// conversions; every step is exact. unit_complement is 1 minus it, exact as well (a multiple of 2^-53 in (0, 1]).
 __device__ __forceinline__ double unit_f64(uint32_t hi, uint32_t lo) {
-    const uint64_t bits = (static_cast<uint64_t>(hi) << 21) ^ (static_cast<uint64_t>(lo) >> 11);
-    return static_cast<double>(bits) * (1.0 / 9007199254740992.0);
+    return __builtin_fma(static_cast<double>(lo >> 11), 1.0 / 9007199254740992.0, static_cast<double>(hi) * (1.0 / 4294967296.0));
+}
+__device__ __forceinline__ double unit_complement(uint32_t hi, uint32_t lo) {
+    return __builtin_fma(static_cast<double>(lo >> 11), -1.0 / 9007199254740992.0,
+                         __builtin_fma(static_cast<double>(hi), -1.0 / 4294967296.0, 1.0));
 }
 
 template <class T>
@@ -114,7 +118,7 @@ __global__ void __launch_bounds__(kBlock) normal_kernel(T *out, int64_t n, int64
         const Word4 b = philox_block(offset + static_cast<uint64_t>(i), seed);
         // Box-Muller in f64: each block gives two normals, the cosine first. Outputs narrower than f64 take
         // the short polynomials of normal_math.hpp.
-        const double u1 = 1.0 - unit_f64(b.v[0], b.v[1]), u2 = unit_f64(b.v[2], b.v[3]);
+        const double u1 = unit_complement(b.v[0], b.v[1]), u2 = unit_f64(b.v[2], b.v[3]);
         double r, c, s;
         if constexpr (std::is_same_v<T, double>) {
             const double theta = 2.0 * 3.14159265358979323846 * u2;
@@ -195,7 +199,7 @@ __device__ __forceinline__ uint32_t rank_in_tile(uint32_t mine, uint32_t &total)
 
 // A workgroup takes kTilesPerGroup tiles one after the other, so that the scan between the two passes
 // has few entries (the workspace has room for one per tile; the first `groups` of each half are used).
-constexpr int kTilesPerGroup = 16;
+constexpr int kTilesPerGroup = 64;
 
 // Counts the accepted words of each group and, on the way, writes word j as element j: right as it
 // stands when the batch rejects nothing, which is all but certain for a small range (a word is rejected
@@ -222,28 +226,33 @@ __global__ void __launch_bounds__(kBlock) int_count_kernel(uint64_t *counts, int
     if (threadIdx.x == 0) counts[blockIdx.x] = total;
 }
 
-// One workgroup: offsets[t] = the sum of counts[0..t), total = the sum of all.
+// One workgroup: offsets[t] = the sum of counts[0..t), total = the sum of all. A lane takes `per` adjacent
+// counts; the lanes' sums are scanned with shuffles inside a wave and through LDS across the waves.
 constexpr int kScanThreads = 1024;
 __global__ void __launch_bounds__(kScanThreads) int_scan_kernel(const uint64_t *counts, uint64_t *offsets, uint64_t *total,
                                                                 int64_t tiles) {
-    __shared__ uint64_t part[kScanThreads];
+    __shared__ uint64_t wave_sum[kScanThreads / 64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int64_t per = (tiles + kScanThreads - 1) / kScanThreads;
     const int64_t first = per * threadIdx.x, last = first + per < tiles ? first + per : tiles;
     uint64_t sum = 0;
     for (int64_t t = first; t < last; ++t) sum += counts[t];
-    part[threadIdx.x] = sum;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        uint64_t running = 0;
-        for (int k = 0; k < kScanThreads; ++k) {
-            const uint64_t s = part[k];
-            part[k] = running;
-            running += s;
-        }
-        *total = running;
+    uint64_t x = sum;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const uint64_t lo = static_cast<uint32_t>(__shfl_up(static_cast<int>(x), d, 64));
+        const uint64_t hi = static_cast<uint32_t>(__shfl_up(static_cast<int>(x >> 32), d, 64));
+        if (lane >= d) x += (hi << 32) | lo;
     }
+    if (lane == 63) wave_sum[wave] = x;
     __syncthreads();
-    uint64_t running = part[threadIdx.x];
+    uint64_t running = x - sum, all = 0;
+#pragma unroll
+    for (int w = 0; w < kScanThreads / 64; ++w) {
+        running += w < wave ? wave_sum[w] : 0;
+        all += wave_sum[w];
+    }
+    if (threadIdx.x == 0) *total = all;
     for (int64_t t = first; t < last; ++t) {
         offsets[t] = running;
         running += counts[t];
@@ -276,9 +285,12 @@ __global__ void __launch_bounds__(kBlock) int_write_kernel(int64_t *out, int64_t
     }
 }
 
-inline unsigned grid_of(int64_t threads) {
+// With a cap below the need a thread takes several blocks. The normal samples want that: the constants of
+// their arithmetic and the key schedule are then set up once per thread (190 -> 170 us for 67 million f32
+// samples). The kernels that mostly write are faster with a workgroup per tile.
+constexpr int64_t kNormalGrid = 16384;
+inline unsigned grid_of(int64_t threads, int64_t cap = int64_t{1} << 22) {
     const int64_t want = (threads + kBlock - 1) / kBlock;
-    const int64_t cap = int64_t{1} << 22;
     return static_cast<unsigned>(want < 1 ? 1 : (want < cap ? want : cap));
 }
 
@@ -329,7 +341,7 @@ hmr_status hmr_random_normal(hmr_context_t ctx, const hmr_tensor_desc *out, uint
             return hmr::with_float_type(out->dtype, [&](auto t) {
                 using T = typename decltype(t)::type;
                 const int64_t blocks = (n + 1) / 2;
-                hipLaunchKernelGGL((hmr::normal_kernel<T>), dim3(hmr::grid_of(blocks)), dim3(hmr::kBlock), 0, stream,
+                hipLaunchKernelGGL((hmr::normal_kernel<T>), dim3(hmr::grid_of(blocks, hmr::kNormalGrid)), dim3(hmr::kBlock), 0, stream,
                                    reinterpret_cast<T *>(first), n, blocks, seed, offset, mean, std);
             });
         });
