@@ -391,7 +391,9 @@ hmr_status hmr_index_positions(hmr_context_t ctx, const hmr_tensor_desc *out,
 /* ref :382-389  cpu::index_overwrite (misc.rs:104-126): slice i of src along dim is copied to slice
  * positions[i] of out, the last of repeated positions winning. `positions` is a 1-D tensor of valid
  * positions; out and src are described as for hmr_index_add. The workspace has
- * hmr_index_overwrite_workspace bytes for out's size along dim (a word per position). */
+ * hmr_index_overwrite_workspace bytes for out's size along dim: an 8-byte word per position of that
+ * dimension, whatever the number of slices written. Every call clears all of it first, so a put of a
+ * few rows into a dimension of 2^28 positions still asks for 2 GiB and moves 4 GiB. */
 hmr_status hmr_index_overwrite_workspace(int64_t size, int64_t *bytes);
 hmr_status hmr_index_overwrite(hmr_context_t ctx, const hmr_tensor_desc *out,
                                const hmr_tensor_desc *src, const hmr_tensor_desc *positions,
