@@ -369,6 +369,60 @@ def test_transposed_outer_dimensions_in_every_depth():
             assert_bitwise(pga.neg() if dtype != DT.I64 else pga.abs(), pa.neg() if dtype != DT.I64 else pa.abs(), f"unary of {what}")
 
 
+def test_transposed_operands_through_tiles_of_two_dimensions():
+    """Views whose contiguous dimension is not the output's (a transposition or permutation made contiguous, or
+    combined with operands that run with the output): sizes on, below and across the tile edges (64 elements, 128
+    for 1- and 2-byte types), every element width, one and two inputs in either position, both inputs turned,
+    broadcast partners, conversions between widths, views with an offset and a pitch, up to six dimensions."""
+    def both(dtype, shape, seed):
+        t = tensor(values(dtype, int(np.prod(shape)), seed), dtype, shape)
+        return t, t.to(GPU)
+
+    for dtype in (DT.U8, DT.Bool, DT.BF16, DT.F16, DT.F32, DT.I32, DT.I64, DT.F64):
+        wide = dtype in (DT.U8, DT.Bool, DT.BF16, DT.F16)
+        sizes = [(64, 64), (70, 33), (129, 65), (257, 100)] if not wide else [(128, 128), (140, 65), (257, 130), (64, 300)]
+        for rows, cols in sizes:
+            (a, ga), (b, gb) = both(dtype, [rows, cols], 91), both(dtype, [cols, rows], 92)
+            at, gat = a.transpose(0, 1), ga.transpose(0, 1)  # [cols, rows], contiguous along dimension 0
+            what = f"{dtype} [{rows},{cols}] transposed"
+            assert_bitwise(gat.contiguous(), at.contiguous(), f"copy of {what}")
+            if dtype == DT.Bool:
+                assert_bitwise(gat.logical_not(), at.logical_not(), f"not of {what}")
+                continue
+            assert_bitwise(gat.add(gb), at.add(b), f"{what} + contiguous")
+            assert_bitwise(gb.sub(gat), b.sub(at), f"contiguous - {what}")
+            (c, gc) = both(dtype, [rows, cols], 93)
+            assert_bitwise(gat.mul(gc.transpose(0, 1)).contiguous(), at.mul(c.transpose(0, 1)).contiguous(), f"{what} * the same view")
+            (bias, gbias), (col, gcol) = both(dtype, [rows], 94), both(dtype, [cols, 1], 95)
+            assert_bitwise(gat.add(gbias), at.add(bias), f"{what} + bias")
+            assert_bitwise(gat.add(gcol), at.add(col), f"{what} + column")
+            assert_bitwise(gat.abs(), at.abs(), f"abs of {what}")
+    # Conversions: the input and the output differ in width.
+    for src, dst in ((DT.F32, DT.BF16), (DT.BF16, DT.F32), (DT.I64, DT.I32), (DT.U8, DT.F32), (DT.F32, DT.F64), (DT.F16, DT.I64)):
+        (a, ga) = both(src, [150, 131], 96)
+        assert_bitwise(ga.transpose(0, 1).to(dst), a.transpose(0, 1).to(dst), f"{src} transposed -> {dst}")
+        (b, gb) = both(dst, [131, 150], 97)
+        if src in FLOATS and dst in FLOATS:
+            assert_bitwise(ga.transpose(0, 1).add(gb), a.transpose(0, 1).add(b), f"{src} transposed + {dst}")
+    # A view with an offset and a pitch on both sides, and permutations of three to six dimensions.
+    for dtype in (DT.BF16, DT.F32, DT.I64):
+        (a, ga) = both(dtype, [200, 190], 98)
+        v, gv = a.narrow(0, 7, 150).narrow(1, 3, 170).transpose(0, 1), ga.narrow(0, 7, 150).narrow(1, 3, 170).transpose(0, 1)
+        assert_bitwise(gv.contiguous(), v.contiguous(), f"{dtype} offset view transposed")
+        (b, gb) = both(dtype, [190, 200], 99)
+        w, gw = b.narrow(0, 5, 170).narrow(1, 11, 150), gb.narrow(0, 5, 170).narrow(1, 11, 150)
+        assert_bitwise(gv.add(gw), v.add(w), f"{dtype} offset view transposed + offset view")
+        for shape, perm in (([5, 70, 140], [2, 0, 1]), ([5, 70, 140], [1, 2, 0]), ([5, 70, 140], [2, 1, 0]),
+                            ([3, 66, 2, 130], [0, 3, 2, 1]), ([2, 129, 3, 2, 70], [4, 2, 0, 3, 1]),
+                            ([2, 2, 65, 2, 3, 131], [5, 0, 3, 1, 4, 2])):
+            (a, ga) = both(dtype, shape, 100)
+            pa, pga = a.permute(perm), ga.permute(perm)
+            assert_bitwise(pga.contiguous(), pa.contiguous(), f"{dtype} {shape} permuted {perm}")
+            (b, gb) = both(dtype, list(pa.shape), 101)
+            assert_bitwise(pga.add(gb), pa.add(b), f"{dtype} {shape} permuted {perm} + contiguous")
+            assert_bitwise(gb.sub(pga), b.sub(pa), f"{dtype} contiguous - {shape} permuted {perm}")
+
+
 def test_uniform_operands_in_every_position():
     """An operand broadcast from one element, in each position (ref: rocm_elementwise.rs:864-937)."""
     for dtype in (DT.F32, DT.BF16, DT.I32):
