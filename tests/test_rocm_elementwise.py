@@ -380,7 +380,10 @@ def test_transposed_operands_through_tiles_of_two_dimensions():
 
     for dtype in (DT.U8, DT.Bool, DT.BF16, DT.F16, DT.F32, DT.I32, DT.I64, DT.F64):
         wide = dtype in (DT.U8, DT.Bool, DT.BF16, DT.F16)
-        sizes = [(64, 64), (70, 33), (129, 65), (257, 100)] if not wide else [(128, 128), (140, 65), (257, 130), (64, 300)]
+        # The last two of each list are whole tiles of the 16-byte form (64 x 64 elements of 8 bytes, 128 x 128 of
+        # 4, 256 x 128 of 2, 256 x 256 of 1).
+        sizes = ([(64, 64), (70, 33), (129, 65), (257, 100), (128, 256), (384, 128)] if not wide else
+                 [(128, 128), (140, 65), (257, 130), (64, 300), (256, 512), (768, 256)])
         for rows, cols in sizes:
             (a, ga), (b, gb) = both(dtype, [rows, cols], 91), both(dtype, [cols, rows], 92)
             at, gat = a.transpose(0, 1), ga.transpose(0, 1)  # [cols, rows], contiguous along dimension 0
@@ -412,7 +415,14 @@ def test_transposed_operands_through_tiles_of_two_dimensions():
         (b, gb) = both(dtype, [190, 200], 99)
         w, gw = b.narrow(0, 5, 170).narrow(1, 11, 150), gb.narrow(0, 5, 170).narrow(1, 11, 150)
         assert_bitwise(gv.add(gw), v.add(w), f"{dtype} offset view transposed + offset view")
+        # Whole tiles inside a wider buffer, at offsets that keep 16-byte alignment and at ones that do not.
+        (a, ga) = both(dtype, [300, 424], 102)
+        for r0, c0 in ((8, 16), (3, 16), (8, 5)):
+            v, gv = a.narrow(0, r0, 256).narrow(1, c0, 384).transpose(0, 1), ga.narrow(0, r0, 256).narrow(1, c0, 384).transpose(0, 1)
+            assert_bitwise(gv.contiguous(), v.contiguous(), f"{dtype} whole tiles at ({r0}, {c0}) transposed")
+            assert_bitwise(gv.neg(), v.neg(), f"{dtype} neg of whole tiles at ({r0}, {c0}) transposed")
         for shape, perm in (([5, 70, 140], [2, 0, 1]), ([5, 70, 140], [1, 2, 0]), ([5, 70, 140], [2, 1, 0]),
+                            ([3, 128, 256], [2, 0, 1]), ([3, 128, 256], [1, 2, 0]), ([2, 256, 3, 128], [2, 0, 3, 1]),
                             ([3, 66, 2, 130], [0, 3, 2, 1]), ([2, 129, 3, 2, 70], [4, 2, 0, 3, 1]),
                             ([2, 2, 65, 2, 3, 131], [5, 0, 3, 1, 4, 2])):
             (a, ga) = both(dtype, shape, 100)
