@@ -347,12 +347,12 @@ def per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP
     # of the two dimensions goes through LDS), and every other column (one element per lane).
     sqm = residual.reshape([8192, 8192])
     sqt = sqm.transpose(0, 1)
-    add(None, "transpose f32 [8192,8192] -> contiguous (tiles through LDS)", 8 * N, lambda: sqt.contiguous(), 10)
-    add(None, "transposed + contiguous f32 [8192,8192] (tiles through LDS)", 12 * N, lambda: sqt.add(sqm), 10)
+    add(None, "transpose f32 [8192,8192] -> contiguous (tiles through LDS, 16-byte accesses)", 8 * N, lambda: sqt.contiguous(), 10)
+    add(None, "transposed + contiguous f32 [8192,8192] (tiles through LDS, 16-byte accesses)", 12 * N, lambda: sqt.add(sqm), 10)
     sqb = x.reshape([8192, 8192]).transpose(0, 1)
-    add(None, "transpose bf16 [8192,8192] -> contiguous (tiles through LDS)", 4 * N, lambda: sqb.contiguous(), 10)
+    add(None, "transpose bf16 [8192,8192] -> contiguous (tiles through LDS, 16-byte accesses)", 4 * N, lambda: sqb.contiguous(), 10)
     cube = residual.reshape([64, 1024, 1024]).permute([2, 0, 1])
-    add(None, "permute(2,0,1) f32 [64,1024,1024] -> contiguous (tiles through LDS)", 8 * N, lambda: cube.contiguous(), 10)
+    add(None, "permute(2,0,1) f32 [64,1024,1024] -> contiguous (tiles through LDS, 16-byte accesses)", 8 * N, lambda: cube.contiguous(), 10)
     halfcols = sqm.slice(1, 0, 8192, 2)
     add(None, "every other column f32 [8192,4096] -> contiguous (general kernel, an element per lane)", 4 * N,
         lambda: halfcols.contiguous(), 10)
