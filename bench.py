@@ -325,7 +325,7 @@ def per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP
     cols = tensor((words(0x5EED0601, 16384 * 512) % np.uint64(4096)).astype(np.int32), DT.I32, [16384, 512], GPU)
     add(None, "gather f32 [16384,4096] dim 1 by i32 [16384,512]", (4 + 4 + 4) * 16384 * 512, lambda: mat.gather(1, cols), 10)
     vals = mat.narrow(1, 0, 512)
-    add(None, "scatter_add f32 [16384,512] into [16384,4096] dim 1 (copy, check, sort, ordered sums)",
+    add(None, "scatter_add f32 [16384,512] into [16384,4096] dim 1 (copy, check, ordered sums line by line in LDS)",
         8 * N + (4 + 4 + 8) * 16384 * 512, lambda: mat.scatter_add(1, cols, vals), 3)
     # A boolean mask over the f32 matrix, 60 % true: the coordinates (count, scan, write; two i64 per true element),
     # then the selected elements (positions, one element per pick).
