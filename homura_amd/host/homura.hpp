@@ -269,6 +269,23 @@ class Tensor {
     Tensor clamp_max(const Operand &max) const { return minimum(max); }
     Tensor masked_fill(const Tensor &mask, const Operand &value) const;
 
+    // In-place operations: the result of the out-of-place operation is checked against `self` (same shape, a
+    // dtype that can be cast to its own, elements that are distinct memory locations) and copied into it
+    // (ref: src/ops/binary.rs:225-242, 340-366, 419-429, 479-515, src/ops/mod.rs:308-392).
+    const Tensor &binary_(BinaryOp op, const Operand &other) const;
+    const Tensor &add_(const Operand &o) const { return binary_(BinaryOp::Add, o); }
+    const Tensor &sub_(const Operand &o) const { return binary_(BinaryOp::Sub, o); }
+    const Tensor &mul_(const Operand &o) const { return binary_(BinaryOp::Mul, o); }
+    const Tensor &div_(const Operand &o) const { return binary_(BinaryOp::Div, o); }
+    const Tensor &pow_(const Operand &o) const { return binary_(BinaryOp::Pow, o); }
+    const Tensor &clamp_(const Operand &min, const Operand &max) const;
+    const Tensor &masked_fill_(const Tensor &mask, const Operand &value) const;
+    // Copies `src` into self, broadcasting it and converting its dtype; `src` may be on another device and may
+    // overlap self (ref: src/ops/binary.rs:504-515, 594-641).
+    const Tensor &copy_(const Tensor &src) const;
+    const Tensor &fill_(Scalar value) const;  // ref: src/ops/binary.rs:532-560, 606-622
+    const Tensor &zero_() const { return fill_(Scalar::of_int(0)); }
+
     // Reductions (ref: src/ops/reduce.rs).
     Tensor sum() const;
     Tensor sum_dim(const std::vector<int64_t> &dims, bool keepdim) const;

@@ -1,7 +1,9 @@
 // The ops front end: argument checks, type promotion, broadcasting, output allocation and the
 // call into the backend. See homura.hpp for the map to the reference's files.
+#include <algorithm>
 #include <cmath>
 #include <cstring>
+#include <optional>
 
 #include "homura.hpp"
 
@@ -407,6 +409,106 @@ Tensor Tensor::masked_fill(const Tensor &mask, const Operand &value) const {
                     std::to_string(t.num_dims()) + " dimension(s).");
     }
     return select_op(mask, Operand(t.to(dtype())), Operand(*this), dtype());
+}
+
+// ---- in-place operations (ref: src/ops/mod.rs:308-392, src/ops/binary.rs:594-692) -----------------------
+
+namespace {
+
+// Whether distinct indices of the layout might be one storage element: dimensions longer than 1 sorted by
+// stride, each stride must exceed what the smaller ones reach (ref: src/tensor/mod.rs:258-287).
+bool may_overlap_internally(const Layout &l) {
+    std::vector<std::pair<int64_t, int64_t>> dims;
+    for (size_t d = 0; d < l.shape.size(); ++d) {
+        if (l.shape[d] == 0) return false;
+        if (l.shape[d] > 1) dims.emplace_back(l.strides[d], l.shape[d]);
+    }
+    std::sort(dims.begin(), dims.end());
+    int64_t reach = 0;
+    for (const auto &[stride, n] : dims) {
+        if (stride <= reach) return true;
+        reach += (n - 1) * stride;
+    }
+    return false;
+}
+
+// The element offsets [first, end) a layout can touch; nothing for a layout without elements
+// (ref: src/tensor/mod.rs:187-197).
+std::optional<std::pair<int64_t, int64_t>> span_of(const Layout &l) {
+    int64_t last = l.offset;
+    for (size_t d = 0; d < l.shape.size(); ++d) {
+        if (l.shape[d] == 0) return std::nullopt;
+        last += (l.shape[d] - 1) * l.strides[d];
+    }
+    return std::make_pair(l.offset, last + 1);
+}
+
+// Whether two views may refer to the same memory without being the same view (ref: src/tensor/mod.rs:295-310).
+bool partially_overlaps(const TensorData &a, const TensorData &b) {
+    if (a.storage != b.storage) return false;
+    const auto sa = span_of(a.layout), sb = span_of(b.layout);
+    if (!sa || !sb) return false;
+    const int64_t ea = static_cast<int64_t>(size_in_bytes(a.dtype)), eb = static_cast<int64_t>(size_in_bytes(b.dtype));
+    const bool disjoint = sa->second * ea <= sb->first * eb || sb->second * eb <= sa->first * ea;
+    const bool same = a.dtype == b.dtype && a.layout.offset == b.layout.offset && a.layout.shape == b.layout.shape &&
+                      a.layout.strides == b.layout.strides;
+    return !disjoint && !same;
+}
+
+// ref: src/ops/binary.rs:665-692
+void check_writable(const TensorData &dst) {
+    if (may_overlap_internally(dst.layout)) {
+        throw Error("unsupported operation: more than one element of the written-to tensor may refer to a single memory "
+                    "location. Please deep_clone() the tensor before performing the operation.");
+    }
+}
+
+// The end of an in-place operation: `result` was computed out of place on self's device
+// (ref: src/ops/mod.rs:317-392).
+void finish_in_place(const Tensor &self, const Tensor &result) {
+    if (self.shape() != result.shape()) {
+        throw Error("output with shape " + shape_str(self.shape()) + " doesn't match the broadcast shape " + shape_str(result.shape()));
+    }
+    if (!can_cast(result.dtype(), self.dtype())) {
+        throw Error(std::string("result type ") + name_of(result.dtype()) + " can't be cast to the desired output type " +
+                    name_of(self.dtype()));
+    }
+    check_writable(self.data());
+    backend::copy(self.data(), result.data());
+}
+
+}  // namespace
+
+const Tensor &Tensor::binary_(BinaryOp op, const Operand &other) const {
+    finish_in_place(*this, binary(op, other));
+    return *this;
+}
+
+const Tensor &Tensor::clamp_(const Operand &min, const Operand &max) const {
+    finish_in_place(*this, clamp(min, max));
+    return *this;
+}
+
+const Tensor &Tensor::masked_fill_(const Tensor &mask, const Operand &value) const {
+    finish_in_place(*this, masked_fill(mask, value));
+    return *this;
+}
+
+const Tensor &Tensor::copy_(const Tensor &src) const {
+    check_writable(d_);
+    src.data().layout.expand_to(d_.layout.shape);  // checks that src broadcasts to self
+    // The source on self's device: moved (and converted) if it is elsewhere, copied if it partially overlaps self.
+    Tensor s = src;
+    if (src.device() != device()) s = src.to(dtype()).to(device());
+    else if (partially_overlaps(d_, src.data())) s = Tensor(clone_data(src.data()));
+    backend::copy(d_, s.data());
+    return *this;
+}
+
+const Tensor &Tensor::fill_(Scalar value) const {
+    check_writable(d_);
+    backend::fill(d_, fill_value(value, d_.dtype));
+    return *this;
 }
 
 // ---- reductions (ref: src/ops/reduce.rs:175-405) --------------------------------------------------------

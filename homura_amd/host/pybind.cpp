@@ -224,6 +224,23 @@ PYBIND11_MODULE(_host, m) {
     T.def("masked_fill", [](const Tensor &t, const Tensor &mask, const py::handle &v) {
         return t.masked_fill(mask, to_operand(v));
     });
+    // In-place operations return the tensor they wrote.
+    const std::pair<const char *, BinaryOp> in_place_ops[] = {{"add_", BinaryOp::Add}, {"sub_", BinaryOp::Sub},
+                                                              {"mul_", BinaryOp::Mul}, {"div_", BinaryOp::Div},
+                                                              {"pow_", BinaryOp::Pow}};
+    for (auto &b : in_place_ops) {
+        BinaryOp op = b.second;
+        T.def(b.first, [op](const Tensor &t, const py::handle &o) { return t.binary_(op, to_operand(o)); });
+    }
+    T.def("clamp_", [](const Tensor &t, const py::handle &lo, const py::handle &hi) {
+        return t.clamp_(to_operand(lo), to_operand(hi));
+    });
+    T.def("masked_fill_", [](const Tensor &t, const Tensor &mask, const py::handle &v) {
+        return t.masked_fill_(mask, to_operand(v));
+    });
+    T.def("copy_", [](const Tensor &t, const Tensor &src) { return t.copy_(src); });
+    T.def("fill_", [](const Tensor &t, const py::handle &v) { return t.fill_(std::get<Scalar>(to_operand(v))); });
+    T.def("zero_", [](const Tensor &t) { return t.zero_(); });
 
     T.def("sum", &Tensor::sum);
     T.def("sum_dim", [](const Tensor &t, const py::handle &d, bool k) { return t.sum_dim(to_dims(d), k); });

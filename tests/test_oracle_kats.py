@@ -539,3 +539,53 @@ def test_addr_known_answers_and_coefficient_rules():
     big, two = tensor(np.array([3.0e38], dtype=np.float32), DT.F32), tensor(np.array([2.0], dtype=np.float32), DT.F32)
     got = array(h.full([1, 1], 0.0, DT.F32, "cpu").addr(big, two, 1, 1e-30))
     assert got.tolist() == [[np.float32(1e-30) * np.float32(3.0e38) * np.float32(2.0)]] and np.isfinite(got).all()
+
+
+def test_in_place_operations_check_the_target_and_write_through_views():
+    """add_ / mul_ / sub_ / clamp_ / masked_fill_ / copy_ / fill_ compute out of place and copy into the target
+    (ref: src/ops/mod.rs:308-392, src/ops/binary.rs:225-242, 504-515, 594-692): known answers through views, the
+    messages for a shape that would grow, a dtype that cannot be cast and a target whose elements share memory,
+    and a copy onto an overlapping part of itself (ref: tests/rocm_copy.rs:180-183)."""
+    base = tensor(np.arange(12, dtype=np.float32), DT.F32, [3, 4])
+    col = base.narrow(1, 1, 2)                    # a strided view: the write lands in the base
+    col.add_(tensor(np.array([10.0, 20.0], dtype=np.float32), DT.F32, [2])).mul_(2.0)
+    assert array(base).tolist() == [[0, 22, 44, 3], [4, 30, 52, 7], [8, 38, 60, 11]]
+    base.transpose(0, 1).sub_(1)
+    assert array(base).tolist() == [[-1, 21, 43, 2], [3, 29, 51, 6], [7, 37, 59, 10]]
+    base.clamp_(0, 40)
+    assert array(base).tolist() == [[0, 21, 40, 2], [3, 29, 40, 6], [7, 37, 40, 10]]
+    mask = tensor(np.array([1, 0, 0, 1], dtype=np.uint8), DT.Bool, [4])
+    base.masked_fill_(mask, -5.0)
+    assert array(base).tolist() == [[-5, 21, 40, -5], [-5, 29, 40, -5], [-5, 37, 40, -5]]
+    # An integer target takes an integer result, and refuses a float one.
+    ints = tensor(np.arange(6, dtype=np.int32), DT.I32, [6])
+    ints.add_(tensor(np.ones(6, dtype=np.int64), DT.I64, [6])).mul_(3)
+    assert array(ints).tolist() == [3, 6, 9, 12, 15, 18]
+    for call, message in (
+            (lambda: ints.mul_(0.5), "result type f32 can't be cast to the desired output type i32"),
+            (lambda: ints.div_(2), "result type f32 can't be cast to the desired output type i32"),
+            (lambda: tensor(np.zeros(4, dtype=np.float32), DT.F32, [4]).add_(base),
+             "output with shape [4] doesn't match the broadcast shape [3, 4]"),
+            (lambda: tensor(np.zeros(3, dtype=np.float32), DT.F32, [3]).expand([2, 3]).add_(1.0),
+             "unsupported operation: more than one element of the written-to tensor may refer to a single memory "
+             "location. Please deep_clone() the tensor before performing the operation."),
+            (lambda: tensor(np.zeros(3, dtype=np.float32), DT.F32, [3]).expand([2, 3]).fill_(1.0),
+             "unsupported operation: more than one element of the written-to tensor may refer to a single memory "
+             "location. Please deep_clone() the tensor before performing the operation.")):
+        with pytest.raises(Exception) as e:
+            call()
+        assert message in str(e.value), str(e.value)
+    assert array(ints).tolist() == [3, 6, 9, 12, 15, 18]  # a refused operation wrote nothing
+    # copy_: a transposed target, a broadcast source of another dtype (ref: tests/rocm_copy.rs:160-170).
+    target = tensor(np.zeros(15, dtype=np.int8), DT.I8, [5, 3]).transpose(0, 1)
+    target.copy_(tensor(np.array([1.9, -2.9, 300.0, 0.0, -0.5], dtype=np.float32), DT.F32, [1, 5]))
+    assert array(target).tolist() == [[1, -2, 44, 0, 0]] * 3
+    with pytest.raises(Exception):
+        target.copy_(tensor(np.zeros(4, dtype=np.float32), DT.F32, [4]))
+    x = tensor(np.arange(6, dtype=np.int64), DT.I64, [6])
+    x.narrow(0, 1, 5).copy_(x.narrow(0, 0, 5))
+    assert array(x).tolist() == [0, 0, 1, 2, 3, 4]
+    x.fill_(7).narrow(0, 2, 2).zero_()
+    assert array(x).tolist() == [7, 7, 0, 0, 7, 7]
+    with pytest.raises(Exception):
+        tensor(np.zeros(2, dtype=np.uint8), DT.U8, [2]).fill_(300)

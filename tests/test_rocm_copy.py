@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 
 from tests import oracle
-from tests.support import DT, DTYPES, GPU, NP, array, assert_same, h, large_layouts, layouts, tensor, words
+from tests.support import DT, DTYPES, GPU, NP, array, assert_same, bits, h, large_layouts, layouts, tensor, values, words
 
 pytestmark = pytest.mark.gpu
 h.register_cpu_backend(oracle.backend_address())
@@ -117,3 +117,70 @@ def test_fill_writes_exactly_its_span_at_every_offset_and_length():
             buf.free()
     finally:
         ctx.close()
+
+
+def test_moves_between_the_cpu_and_the_gpu():
+    """ref: tests/rocm_copy.rs:126-157"""
+    for k, dtype in enumerate(DTYPES):
+        for pair in layouts(dtype, 100 + k):
+            what = f"{dtype}, {pair.name}"
+            up = pair.cpu.to(GPU)
+            assert_same(up, pair.cpu, what)
+            assert up.is_contiguous(), what
+            down = pair.gpu.to("cpu")
+            assert str(down.device) == "cpu" and np.array_equal(bits(down), bits(pair.cpu)), what
+            assert np.array_equal(bits(up.to("cpu")), bits(pair.cpu)), what
+            for to in (DT.F16, DT.I32, DT.Bool, DT.F64):
+                expected = pair.cpu.to(to)
+                assert_same(pair.cpu.to(to).to(GPU), expected, f"{what} -> {to}")
+                down = pair.gpu.to(to).to("cpu")
+                assert str(down.device) == "cpu" and np.array_equal(bits(down), bits(expected)), f"{what} -> {to} on the cpu"
+
+
+def test_copy_into_strided_targets():
+    """A transposed target, a broadcast source of another dtype, on the same device and across devices; a copy onto
+    an overlapping part of itself goes through a copy (ref: tests/rocm_copy.rs:160-184)."""
+    for k, src_dtype in enumerate(DTYPES):
+        for to in (DT.F32, DT.I8, DT.BF16, src_dtype):
+            src = tensor(values(src_dtype, 5, 300 + k), src_dtype, [5])
+            zeros = np.zeros(15, dtype=NP[to])
+            cpu = tensor(zeros, to, [5, 3]).transpose(0, 1)
+            gpu = tensor(zeros, to, [5, 3], GPU).transpose(0, 1)
+            cpu.copy_(src.reshape([1, 5]))
+            gpu.copy_(src.to(GPU).reshape([1, 5]))
+            what = f"{src_dtype} -> {to}"
+            assert_same(gpu, cpu, what)
+            gpu = tensor(zeros, to, [5, 3], GPU).transpose(0, 1)
+            gpu.copy_(src.reshape([1, 5]))
+            assert_same(gpu, cpu, f"{what}, cpu source")
+            back = tensor(zeros, to, [5, 3]).transpose(0, 1)
+            back.copy_(src.to(GPU).reshape([1, 5]))
+            assert np.array_equal(bits(back), bits(cpu)), f"{what}, gpu source"
+    x = tensor(np.arange(6, dtype=np.int64), DT.I64, [6], GPU)
+    x.narrow(0, 1, 5).copy_(x.narrow(0, 0, 5))
+    assert array(x).tolist() == [0, 0, 1, 2, 3, 4]
+    # A large strided target: every other row of a matrix takes rows of another dtype.
+    rows = tensor(values(DT.F32, 512 * 384, 7), DT.F32, [512, 384])
+    for to in (DT.F32, DT.BF16):
+        zeros = np.zeros(1024 * 384, dtype=NP[to])
+        cpu, gpu = tensor(zeros, to, [1024, 384]), tensor(zeros, to, [1024, 384], GPU)
+        cpu.slice(0, 1, None, 2).copy_(rows)
+        gpu.slice(0, 1, None, 2).copy_(rows.to(GPU))
+        assert_same(gpu, cpu, f"every other row <- f32 as {to}")
+        cpu.transpose(0, 1).narrow(0, 5, 300).fill_(2.5)
+        gpu.transpose(0, 1).narrow(0, 5, 300).fill_(2.5)
+        assert_same(gpu, cpu, f"fill_ of a transposed part, {to}")
+
+
+def test_strided_gpu_tensors_read_back_directly():
+    """ref: tests/rocm_copy.rs:265-283"""
+    cpu = tensor(np.arange(12, dtype=np.float32), DT.F32, [3, 4])
+    gpu = cpu.to(GPU)
+    ct, gt = cpu.transpose(0, 1), gpu.transpose(0, 1)
+    assert not gt.is_contiguous()
+    assert array(gt).tolist() == array(ct).tolist()
+    assert array(gpu.select(1, 2).select(0, 1)).item() == 6.0
+    half = gpu.to(DT.F16).transpose(0, 1).narrow(0, 1, 2)
+    assert np.array_equal(bits(half), bits(cpu.to(DT.F16).transpose(0, 1).narrow(0, 1, 2)))
+    b = h.full([2, 3], True, DT.Bool, GPU).expand([4, 2, 3]).transpose(0, 2)
+    assert array(b).reshape(-1).tolist() == [1] * 24

@@ -433,6 +433,37 @@ def test_transposed_operands_through_tiles_of_two_dimensions():
             assert_bitwise(gb.sub(pga), b.sub(pa), f"{dtype} contiguous - {shape} permuted {perm}")
 
 
+def test_in_place_ops_are_bitwise():
+    """ref: tests/rocm_elementwise.rs:720-737 (each layout views a base of its own, so writing into it changes nothing
+    else; writes into a broadcast view are refused on both devices)"""
+    for dtype in (DT.I32, DT.F16, DT.F32, DT.F64):
+        qs = layouts(dtype, 61)
+        for p, q in zip(layouts(dtype, 60), qs):
+            if 0 in p.cpu.strides:
+                for t in (p.cpu, p.gpu):
+                    with pytest.raises(Exception) as e:
+                        t.add_(1)
+                    assert "more than one element of the written-to tensor" in str(e.value)
+                continue
+            p.cpu.add_(q.cpu).mul_(p.cpu).sub_(1)
+            p.gpu.add_(q.gpu).mul_(p.gpu).sub_(1)
+            assert_bitwise(p.gpu, p.cpu, f"in place {dtype} {p.name}")
+            p.cpu.clamp_(-1, 1)
+            p.gpu.clamp_(-1, 1)
+            assert_bitwise(p.gpu, p.cpu, f"clamp_ {dtype} {p.name}")
+            mask = p.cpu.greater(0)
+            p.cpu.masked_fill_(mask, 3)
+            p.gpu.masked_fill_(mask.to(GPU), 3)
+            assert_bitwise(p.gpu, p.cpu, f"masked_fill_ {dtype} {p.name}")
+    # A result that the target cannot hold is refused before anything is written.
+    ints = tensor(values(DT.I32, 100, 62), DT.I32, [100])
+    gints = ints.to(GPU)
+    with pytest.raises(Exception) as e:
+        gints.mul_(0.5)
+    assert "result type f32 can't be cast to the desired output type i32" in str(e.value)
+    assert_bitwise(gints, ints, "a refused in-place product")
+
+
 def test_uniform_operands_in_every_position():
     """An operand broadcast from one element, in each position (ref: rocm_elementwise.rs:864-937)."""
     for dtype in (DT.F32, DT.BF16, DT.I32):
