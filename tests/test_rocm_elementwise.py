@@ -284,6 +284,60 @@ def test_type_promotion_matches_the_cpu_front_end():
                 assert_bitwise(getattr(a.to(GPU), name)(s), cpu, f"{name} {dtype} scalar {s!r}")
 
 
+def test_scalar_operands_are_bitwise():
+    """F16 and BF16 products and quotients keep the scalar in f32, the other operations round it to the dtype
+    (ref: tests/rocm_elementwise.rs:318-346)."""
+    scalars = [2.5, 1.0 / 3.0, 1e-5, 70000.0, -0.0, math.inf, math.nan, 1e300]
+    for dtype in DTYPES:
+        for p in layouts(dtype, 9):
+            for s in scalars:
+                if dtype in FLOATS or (math.isfinite(s) and s == int(s)):
+                    for name in ("mul", "div", "add", "maximum", "less"):
+                        assert_bitwise(getattr(p.gpu, name)(s), getattr(p.cpu, name)(s), f"{name} {dtype} {p.name} with {s}")
+
+
+def test_every_binary_op_with_a_scalar_is_bitwise():
+    """The scalar reaches the kernel as a constant of the dtype, except in F16 and BF16 products and quotients.
+    Integers beyond the dtype wrap, the last integer rounds differently to f32 directly and through f64, float
+    scalars promote integer and bool tensors; a call that one device refuses must be refused by the other with the
+    same message (ref: tests/rocm_elementwise.rs:358-470)."""
+    scalars = [0, 3, -1, 300, -129, (1 << 63) - 1, -(1 << 63), (1 << 62) + (1 << 38) + 1, 2.5, 1.0 / 3.0, -0.0, math.nan,
+               -math.inf, 1e300, True, False]
+    names = ["add", "sub", "mul", "div", "pow", "maximum", "minimum", "greater", "greater_equal", "less", "less_equal",
+             "equal", "not_equal", "logical_and", "logical_or", "radd", "rsub", "rmul", "rdiv"]
+    checked = 0
+    for dtype in DTYPES:
+        for p in layouts(dtype, 21):
+            for s in scalars:
+                for name in names:
+                    what = f"{name} {dtype} {p.name} with {s!r}"
+                    cpu = gpu = cpu_error = gpu_error = None
+                    try:
+                        cpu = getattr(p.cpu, name)(s)
+                    except h.HomuraError as e:
+                        cpu_error = str(e)
+                    try:
+                        gpu = getattr(p.gpu, name)(s)
+                    except h.HomuraError as e:
+                        gpu_error = str(e)
+                    assert cpu_error == gpu_error, f"{what}: {gpu_error!r} on the GPU, {cpu_error!r} on the CPU"
+                    if cpu is None:
+                        continue
+                    if name == "pow" and cpu.dtype in FLOATS:
+                        # Float powers come from the device library: against the GPU's tensor-tensor kernel, with the
+                        # scalar as a tensor of the computation type.
+                        base = p.gpu.to(cpu.dtype)
+                        kind = np.bool_ if isinstance(s, bool) else (np.int64 if isinstance(s, int) else np.float64)
+                        source = {np.bool_: DT.Bool, np.int64: DT.I64, np.float64: DT.F64}[kind]
+                        e = tensor(np.array([s], dtype=np.uint8 if kind is np.bool_ else kind), source, [1])
+                        e = e.to(cpu.dtype).to(GPU).reshape([]).expand(base.shape)
+                        assert_bitwise(gpu, base.pow(e), what)
+                    else:
+                        assert_bitwise(gpu, cpu, what)
+                    checked += 1
+    assert checked > 20000, checked
+
+
 def test_half_scalar_products_keep_the_scalar_in_f32():
     """ref: tests/tensor_api.rs:686-701: 7*(1/3) etc. for f16 and bf16."""
     third = 1.0 / 3.0
