@@ -69,6 +69,22 @@ Scalar fill_value(Scalar value, DType dtype) {
     throw Error(std::string("value cannot be converted to type ") + name_of(dtype) + " without overflow");
 }
 
+// The value of a one-element tensor as a scalar of its kind; on a GPU the read waits for it
+// (ref: src/ops/mod.rs:261-268).
+Scalar scalar_value(const Tensor &t) {
+    if (t.dtype() == DType::Bool) {
+        return Scalar::of_bool(t.to_bytes()[0] != 0);
+    }
+    if (is_floating_point(t.dtype())) {
+        double v;
+        std::memcpy(&v, t.to(DType::F64).to_bytes().data(), sizeof v);
+        return Scalar::of_float(v);
+    }
+    int64_t v;
+    std::memcpy(&v, t.to(DType::I64).to_bytes().data(), sizeof v);
+    return Scalar::of_int(v);
+}
+
 // ---- Resolved operands (ref: src/ops/binary.rs:12-61) -----------------------------------------------
 
 struct Resolved {
@@ -408,6 +424,9 @@ Tensor Tensor::masked_fill(const Tensor &mask, const Operand &value) const {
         throw Error("masked_fill only supports a 0-dimensional value tensor, but got tensor with " +
                     std::to_string(t.num_dims()) + " dimension(s).");
     }
+    // The value must fit the dtype like a scalar one; a value of the same dtype always fits and is not read
+    // (ref: src/ops/binary.rs:466-472).
+    if (t.dtype() != dtype()) fill_value(scalar_value(t), dtype());
     return select_op(mask, Operand(t.to(dtype())), Operand(*this), dtype());
 }
 

@@ -375,6 +375,70 @@ def test_where_and_masked_fill_move_exact_bits():
     assert_bitwise(scores.to(GPU).masked_fill(mask.to(GPU), -math.inf), scores.masked_fill(mask, -math.inf), "causal mask")
 
 
+def test_where_and_masked_fill_with_scalars_are_bitwise():
+    """A scalar branch reaches the kernel as a constant of the result's dtype, in either position, both, and as
+    masked_fill's value, which keeps the dtype of self. Integers beyond the dtype wrap (where) or are refused
+    (masked_fill), on both devices alike (ref: tests/rocm_elementwise.rs:538-617)."""
+    scalars = [0, -1, 300, (1 << 63) - 1, -(1 << 63), (1 << 62) + (1 << 38) + 1, 2.5, 1.0 / 3.0, -0.0, math.nan, -math.inf,
+               1e300, True]
+    ops = [("where(c, x, s)", lambda c, x, s: h.where_(c, x, s)), ("where(c, s, x)", lambda c, x, s: h.where_(c, s, x)),
+           ("where(c, s, 7)", lambda c, x, s: h.where_(c, s, 7)), ("where(c, -0.5, s)", lambda c, x, s: h.where_(c, -0.5, s)),
+           ("masked_fill", lambda c, x, s: x.masked_fill(c, s))]
+
+    def same(c, x, s, what):
+        for name, f in ops:
+            cpu = gpu = cpu_error = gpu_error = None
+            try:
+                cpu = f(c.cpu, x.cpu, s)
+            except h.HomuraError as e:
+                cpu_error = str(e)
+            try:
+                gpu = f(c.gpu, x.gpu, s)
+            except h.HomuraError as e:
+                gpu_error = str(e)
+            assert cpu_error == gpu_error, f"{name} {what}: {gpu_error!r} on the GPU, {cpu_error!r} on the CPU"
+            if cpu is not None:
+                assert_bitwise(gpu, cpu, f"{name} {what}")
+                yield 1
+
+    checked = 0
+    for dtype in DTYPES:
+        for p, c in zip(layouts(dtype, 40), layouts(DT.Bool, 41)):
+            for s in scalars:
+                checked += sum(same(c, p, s, f"{dtype} {p.name} with {s!r}"))
+    assert checked > 5000, checked
+    # Every offset and tail of the contiguous paths, and past one round of the launch grid.
+    from tests.support import Pair
+    for dtype in (DT.U8, DT.F16, DT.F64):
+        a, m = tensor(values(dtype, 16, 42), dtype, [16]), tensor(values(DT.Bool, 16, 43), DT.Bool, [16])
+        ag, mg = a.to(GPU), m.to(GPU)
+        for offset in range(5):
+            for length in range(10):
+                x = Pair("", a.narrow(0, offset, length), ag.narrow(0, offset, length))
+                c = Pair("", m.narrow(0, offset, length), mg.narrow(0, offset, length))
+                assert sum(same(c, x, 5, f"{dtype} offset {offset} length {length}")) == len(ops)
+    for dtype in (DT.F16, DT.BF16):
+        n = (1 << 24) + 1000
+        cm = tensor(values(DT.Bool, n, 44), DT.Bool, [n])
+        c = Pair("", cm, cm.to(GPU))
+        for p in large_layouts(dtype, 45):
+            assert sum(same(c, p, 0.1, f"{dtype} {p.name}")) == len(ops)
+
+
+def test_masked_fill_values_are_checked_on_the_gpu_as_on_the_cpu():
+    """ref: tests/rocm_elementwise.rs:629-649"""
+    x = tensor(np.array([1, 2, 3], dtype=np.int8), DT.I8, [3])
+    mask = tensor(np.array([1, 0, 1], dtype=np.uint8), DT.Bool, [3])
+    value = tensor(np.array([300], dtype=np.int64), DT.I64, [])
+    for cpu_call, gpu_call in ((lambda: x.masked_fill(mask, 300), lambda: x.to(GPU).masked_fill(mask.to(GPU), 300)),
+                               (lambda: x.masked_fill(mask, value), lambda: x.to(GPU).masked_fill(mask.to(GPU), value.to(GPU)))):
+        with pytest.raises(h.HomuraError) as c:
+            cpu_call()
+        with pytest.raises(h.HomuraError) as g:
+            gpu_call()
+        assert str(c.value) and str(g.value) == str(c.value)
+
+
 def test_tails_and_alignments():
     """Every start offset and length around the vector widths, so that the aligned 128-bit path, the
     ragged last tile and the unaligned fallback all run (ref: rocm_elementwise.rs:801-824)."""
