@@ -244,13 +244,23 @@ def test_ieee_binary_ops_comparisons_and_logic_are_bitwise():
 
 
 def test_float_pow_stays_within_one_ulp():
+    """Positive bases with any exponent, the dtype's special values on both sides, and bases of either sign with
+    integer exponents (ref: tests/rocm_elementwise.rs:478-513, whose bound is the looser 2 u m + 1 ulp)."""
     for dtype in FLOATS:
-        base = float_tensor(np.abs(uniform(31, 4096, 0.0, 20.0)), dtype)
-        expo = float_tensor(uniform(32, 4096, -4.0, 4.0), dtype)
-        cpu = base.pow(expo)
-        gpu = base.to(GPU).pow(expo.to(GPU))
-        d, m = check_within(gpu, cpu, extra=0.0, max_ulp=1 if dtype != DT.F64 else 2, what=f"pow {dtype}")
-        print(f"ulp pow {dtype}: max {m} ulp, {d} differ")
+        pairs = [(float_tensor(np.abs(uniform(31, 4096, 0.0, 20.0)), dtype), float_tensor(uniform(32, 4096, -4.0, 4.0), dtype)),
+                 (tensor(values(dtype, 1031, 14), dtype, [1031]), tensor(values(dtype, 1031, 17), dtype, [1031])),
+                 (float_tensor(uniform(16, 1031, -10.0, 10.0), dtype), float_tensor(uniform(19, 1031, -4.0, 4.0), dtype).to(DT.I64).to(dtype))]
+        for k, (base, expo) in enumerate(pairs):
+            cpu = base.pow(expo)
+            gpu = base.to(GPU).pow(expo.to(GPU))
+            d, m = check_within(gpu, cpu, extra=0.0, max_ulp=1 if dtype != DT.F64 else 2, what=f"pow {dtype}, pair {k}")
+            print(f"ulp pow {dtype} pair {k}: max {m} ulp, {d} differ")
+    for dtype in INTS:
+        base = tensor(values(dtype, 200, 13), dtype, [200])
+        # Exponents from -3 to 70, so that the loop and the negative rules both run.
+        expo = tensor((np.arange(200) % 74 - 3).astype(np.int64), DT.I64, [200]).to(dtype)
+        assert_bitwise(base.to(GPU).pow(expo.to(GPU)), base.pow(expo), f"pow {dtype}")
+        assert_bitwise(base.to(GPU).pow(3), base.pow(3), f"pow {dtype} by 3")
 
 
 def test_type_promotion_matches_the_cpu_front_end():
