@@ -319,6 +319,27 @@ PLAN_SHAPES = [
 ]
 
 
+def test_ties_and_nans_pick_the_cpus_position():
+    """Equal maxima, zeros of both signs, NaNs of both signs before an infinity, a row of -inf and a constant row,
+    along either dimension and over everything (ref: tests/rocm_reduce.rs:214-243)."""
+    inf, nan = math.inf, math.nan
+    rows = np.array([[1.0, 3.0, 3.0, 2.0, 3.0], [0.0, -0.0, 0.0, -0.0, -1.0], [-0.0, 0.0, -0.0, 0.0, 1.0],
+                     [1.0, nan, 5.0, -nan, inf], [-inf] * 5, [2.0] * 5])
+    for dtype in FLOATS:
+        x = tensor(rows, DT.F64, [6, 5]).to(dtype)
+        g = x.to(GPU)
+        for d in (0, 1):
+            for (gv, gi), (cv, ci) in ((g.max_dim(d, False), x.max_dim(d, False)), (g.min_dim(d, False), x.min_dim(d, False))):
+                assert_bitwise(gv, cv, f"{dtype} dim {d} values")
+                assert_bitwise(gi, ci, f"{dtype} dim {d} indices")
+            assert_bitwise(g.argmax_dim(d, False), x.argmax_dim(d, False), f"{dtype} argmax dim {d}")
+            assert_bitwise(g.argmin_dim(d, True), x.argmin_dim(d, True), f"{dtype} argmin dim {d}")
+        assert_bitwise(g.max(), x.max(), f"{dtype} max")
+        assert_bitwise(g.min(), x.min(), f"{dtype} min")
+        assert_bitwise(g.argmin(), x.argmin(), f"{dtype} argmin")
+        assert_bitwise(g.argmax(), x.argmax(), f"{dtype} argmax")
+
+
 def test_every_plan_folds_each_element_once():
     """Integer sums of random words change with any missing or repeated element; max_dim over values
     with many ties must return the first position across lanes and slices
