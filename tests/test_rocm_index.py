@@ -343,3 +343,36 @@ def test_a_sort_whose_histogram_table_needs_several_rounds_of_the_totals_scan():
     got = array(x.to(GPU).scatter_add(0, picks.to(GPU), src.to(GPU)))
     wrong = np.flatnonzero(got.view(np.uint64) != want.view(np.uint64))
     assert wrong.size == 0, f"first difference at target {wrong[0]}: {got[wrong[0]]} != {want[wrong[0]]}"
+
+
+def test_sorts_too_large_to_size_fail_before_any_kernel():
+    """Indices and sources of 2^58 elements (views of one element with zero strides): the size of the sort's
+    workspace is refused before anything is queued, and the tensor the call was made on is unchanged
+    (ref: tests/rocm_index.rs:461-477; the reference words it "the workspace is too large", this library names
+    its limit of 2^31 - 1 positions)."""
+    n = 1 << 58
+    x = tensor(np.arange(4, dtype=np.float32), DT.F32, [4], GPU)
+    index = tensor(np.array([1], dtype=np.int64), DT.I64, [1], GPU).expand([n])
+    src = tensor(np.ones(1, dtype=np.float32), DT.F32, [1], GPU).expand([n])
+    for call, message in ((lambda: x.index_add(0, index, src), "index_add: more than 2^31 - 1 positions"),
+                          (lambda: x.scatter_add(0, index, src), "scatter_add: more than 2^31 - 1 positions")):
+        with pytest.raises(h.HomuraError) as e:
+            call()
+        assert message in str(e.value), str(e.value)
+    assert array(x).tolist() == [0.0, 1.0, 2.0, 3.0]
+
+
+def test_zero_dimensional_gpu_indices_select():
+    """A zero-dimensional integer tensor on the GPU selects like an integer (its value is read back); out of range,
+    the CPU's message (ref: tests/rocm_index.rs:577-589)."""
+    x = tensor(np.arange(12, dtype=np.float32), DT.F32, [3, 4])
+    g = x.to(GPU)
+    for i in (2, -1):
+        zero_dim = tensor(np.array([i], dtype=np.int64), DT.I64, [])
+        assert_same(g.index_tensors([zero_dim.to(GPU)]), x.index_tensors([zero_dim]), f"x[{i}]")
+    bad = tensor(np.array([3], dtype=np.int64), DT.I64, [])
+    with pytest.raises(h.HomuraError) as c:
+        x.index_tensors([bad])
+    with pytest.raises(h.HomuraError) as e:
+        g.index_tensors([bad.to(GPU)])
+    assert str(e.value) == str(c.value)
