@@ -516,6 +516,102 @@ Tensor Tensor::unsqueeze(int64_t dim) const {
     return Tensor(TensorData{d_.storage, l, d_.dtype});
 }
 
+// ref: src/tensor/view.rs (view_layout): a reshape that must not copy.
+Tensor Tensor::view(const std::vector<int64_t> &spec) const {
+    const Layout &l = d_.layout;
+    Shape shape = infer_size(spec, l.num_elements());
+    auto st = compute_view_strides(l.shape, l.strides, shape);
+    if (!st) {
+        throw Error("view size is not compatible with input tensor's size and stride (at least one dimension spans "
+                    "across two contiguous subspaces). Use .reshape(...) instead.");
+    }
+    return Tensor(TensorData{d_.storage, Layout{shape, *st, l.offset}, d_.dtype});
+}
+
+Tensor Tensor::expand_as(const Tensor &other) const {
+    return expand(std::vector<int64_t>(other.shape().begin(), other.shape().end()));
+}
+
+namespace {
+Layout without_dims(const Layout &l, const std::vector<bool> &remove) {
+    Layout out{{}, {}, l.offset};
+    for (size_t d = 0; d < l.shape.size(); ++d) {
+        if (remove[d]) continue;
+        out.shape.push_back(l.shape[d]);
+        out.strides.push_back(l.strides[d]);
+    }
+    return out;
+}
+}  // namespace
+
+// Removes all dimensions of size 1.
+Tensor Tensor::squeeze() const {
+    const Layout &l = d_.layout;
+    std::vector<bool> remove(l.shape.size());
+    for (size_t d = 0; d < l.shape.size(); ++d) remove[d] = l.shape[d] == 1;
+    return Tensor(TensorData{d_.storage, without_dims(l, remove), d_.dtype});
+}
+
+// Removes the given dimensions where they have size 1; an empty list removes none.
+Tensor Tensor::squeeze_dim(const std::vector<int64_t> &dims) const {
+    const Layout &l = d_.layout;
+    std::vector<bool> remove(l.shape.size(), false);
+    if (!dims.empty()) {
+        std::vector<bool> mask = dims_mask(dims, l.shape.size());
+        for (size_t d = 0; d < l.shape.size(); ++d) remove[d] = mask[d] && l.shape[d] == 1;
+    }
+    return Tensor(TensorData{d_.storage, without_dims(l, remove), d_.dtype});
+}
+
+// All windows of `size` elements, `step` apart, along `dim`, as a new last dimension.
+Tensor Tensor::unfold(int64_t dim, int64_t size, int64_t step) const {
+    const Layout &l = d_.layout;
+    const size_t nd = l.shape.size();
+    const size_t d = normalize_dim(dim, nd);
+    const int64_t max = nd == 0 ? 1 : l.shape[d];
+    if (size < 0 || size > max) {
+        throw Error("maximum size for tensor at dimension " + std::to_string(d) + " is " + std::to_string(max) +
+                    " but size is " + std::to_string(size));
+    }
+    if (step <= 0) throw Error("step is " + std::to_string(step) + " but must be > 0");
+    Layout out = l;
+    out.shape.push_back(size);
+    out.strides.push_back(nd == 0 ? 1 : l.strides[d]);
+    if (nd > 0) {
+        out.shape[d] = (l.shape[d] - size) / step + 1;
+        // With a single window the stride is never used, and a huge step may not fit.
+        int64_t stride;
+        out.strides[d] = __builtin_mul_overflow(l.strides[d], step, &stride) ? l.strides[d] : stride;
+    }
+    return Tensor(TensorData{d_.storage, out, d_.dtype});
+}
+
+// A view with an explicit shape, strides and storage offset (in elements); it must lie inside the storage
+// (ref: src/tensor/mod.rs:199-218).
+Tensor Tensor::as_strided(const Shape &size, const Strides &stride, int64_t storage_offset) const {
+    if (size.size() != stride.size()) throw Error("mismatch in length of strides and shape");
+    bool empty = false, fits = storage_offset >= 0;
+    int64_t end = storage_offset;
+    for (size_t d = 0; d < size.size() && fits; ++d) {
+        if (size[d] < 0 || stride[d] < 0) throw Error("as_strided: sizes and strides must not be negative");
+        if (size[d] == 0) empty = true;
+        int64_t reach;
+        if (size[d] > 0) fits = !__builtin_mul_overflow(size[d] - 1, stride[d], &reach) && !__builtin_add_overflow(end, reach, &end);
+    }
+    const int64_t item = static_cast<int64_t>(size_in_bytes(d_.dtype));
+    int64_t needed = 0;
+    if (!empty && fits) fits = !__builtin_add_overflow(end, int64_t{1}, &end) && !__builtin_mul_overflow(end, item, &needed);
+    if (empty) needed = 0;
+    const int64_t have = static_cast<int64_t>(d_.storage->nbytes());
+    if (!fits || needed > have) {
+        throw Error("setStorage: sizes " + shape_str(size) + ", strides " + shape_str(stride) + ", storage offset " +
+                    std::to_string(storage_offset) + ", and itemsize " + std::to_string(item) + " requiring a storage size of " +
+                    (fits ? std::to_string(needed) : std::string("more than usize::MAX")) +
+                    " are out of bounds for storage of size " + std::to_string(have));
+    }
+    return Tensor(TensorData{d_.storage, Layout{size, stride, storage_offset}, d_.dtype});
+}
+
 Tensor Tensor::narrow(int64_t dim, int64_t start, int64_t length) const {
     Layout l = d_.layout;
     if (l.shape.empty()) throw Error("narrow() cannot be applied to a 0-dim tensor.");

@@ -222,6 +222,13 @@ class Tensor {
     Tensor select(int64_t dim, int64_t index) const;
     Tensor slice(int64_t dim, std::optional<int64_t> start, std::optional<int64_t> end, int64_t step) const;
     Tensor flatten(int64_t start_dim, int64_t end_dim) const;
+    // ref: src/tensor/view.rs (view, expand_as, squeeze, squeeze_dim, unfold, as_strided)
+    Tensor view(const std::vector<int64_t> &spec) const;
+    Tensor expand_as(const Tensor &other) const;
+    Tensor squeeze() const;
+    Tensor squeeze_dim(const std::vector<int64_t> &dims) const;
+    Tensor unfold(int64_t dim, int64_t size, int64_t step) const;
+    Tensor as_strided(const Shape &size, const Strides &stride, int64_t storage_offset) const;
 
     // Unary (ref: src/ops/unary.rs).
     Tensor unary(UnaryOp op) const;

@@ -277,6 +277,12 @@ PYBIND11_MODULE(_host, m) {
     T.def("gather", &Tensor::gather);
     T.def("index_add", &Tensor::index_add);
     T.def("scatter_add", &Tensor::scatter_add);
+    T.def("view", &Tensor::view);
+    T.def("expand_as", &Tensor::expand_as);
+    T.def("squeeze", &Tensor::squeeze);
+    T.def("squeeze_dim", [](const Tensor &t, const py::handle &d) { return t.squeeze_dim(to_dims(d)); });
+    T.def("unfold", &Tensor::unfold);
+    T.def("as_strided", &Tensor::as_strided);
     T.def("slice", &Tensor::slice, py::arg("dim"), py::arg("start") = py::none(), py::arg("end") = py::none(), py::arg("step") = 1);
     T.def("index_tensors", &Tensor::index_tensors, py::call_guard<py::gil_scoped_release>());
     T.def("index_put_tensors", &Tensor::index_put_tensors);

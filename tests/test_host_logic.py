@@ -172,3 +172,63 @@ def test_scalar_bits():
     assert sb(2, DT.Bool) == 1
     assert sb(1.0 / 3.0, DT.BF16) == 0x3EAB
     assert sb(-2.5, DT.I32) == 0xFFFFFFFE                      # truncation toward zero, then wrap
+
+
+def test_the_remaining_views_follow_numpy_and_keep_the_references_messages():
+    """view, expand_as, squeeze, squeeze_dim, unfold, as_strided (ref: src/tensor/view.rs): shapes, strides and offsets
+    against numpy's views of the same buffer (sliding_window_view for unfold, as_strided itself), and the messages
+    for a view that would need a copy, a window longer than the dimension and a view outside its storage."""
+    from numpy.lib.stride_tricks import as_strided, sliding_window_view
+    from tests import oracle
+    from tests.support import array, tensor
+    h.register_cpu_backend(oracle.backend_address())
+    a = np.arange(2 * 1 * 3 * 1 * 4, dtype=np.int32).reshape(2, 1, 3, 1, 4)
+    t = tensor(a, DT.I32, list(a.shape))
+
+    def same(view, expected):
+        assert view.shape == list(expected.shape), (view.shape, expected.shape)
+        assert np.array_equal(array(view), expected)
+
+    same(t.squeeze(), a.squeeze())
+    same(t.squeeze_dim([1]), a.squeeze(1))
+    same(t.squeeze_dim([0]), a)                      # not of size 1: left alone
+    same(t.squeeze_dim([1, -2]), a.squeeze((1, 3)))
+    same(t.squeeze_dim([]), a)                       # an empty list removes none
+    same(t.squeeze().transpose(0, 1).squeeze(), a.squeeze().transpose(1, 0, 2))
+    same(t.view([2, 3, 4]), a.reshape(2, 3, 4))
+    same(t.view([-1, 4]), a.reshape(-1, 4))
+    same(t.squeeze().transpose(1, 2).view([2, 4, 3, 1]), a.squeeze().transpose(0, 2, 1).reshape(2, 4, 3, 1))
+    with pytest.raises(h.HomuraError) as e:
+        t.squeeze().transpose(1, 2).view([2, 12])
+    assert "view size is not compatible with input tensor's size and stride" in str(e.value)
+    row = tensor(np.arange(4, dtype=np.int32), DT.I32, [4])
+    same(row.expand_as(t), np.broadcast_to(np.arange(4, dtype=np.int32), a.shape))
+    # unfold: every window of `size` elements, `step` apart, as a new last dimension.
+    m = np.arange(30, dtype=np.int32).reshape(5, 6)
+    tm = tensor(m, DT.I32, [5, 6])
+    for dim, size, step in ((1, 3, 1), (1, 2, 2), (0, 2, 3), (-1, 6, 1), (0, 5, 7), (1, 0, 2)):
+        windows = sliding_window_view(m, size, axis=dim % 2)[(slice(None, None, step),) if dim % 2 == 0 else (slice(None), slice(None, None, step))]
+        same(tm.unfold(dim, size, step), windows)
+    same(tensor(np.array([7], dtype=np.int32), DT.I32, []).unfold(0, 1, 1), np.array([7], dtype=np.int32))
+    for call, message in ((lambda: tm.unfold(1, 7, 1), "maximum size for tensor at dimension 1 is 6 but size is 7"),
+                          (lambda: tm.unfold(0, 2, 0), "step is 0 but must be > 0")):
+        with pytest.raises(h.HomuraError) as e:
+            call()
+        assert message in str(e.value)
+    # as_strided: overlapping windows and a diagonal; outside the storage it is refused with PyTorch's message.
+    same(tm.as_strided([4, 3], [6, 1], 2), as_strided(m.reshape(-1)[2:], (4, 3), (24, 4)))
+    same(tm.as_strided([5], [7], 0), m.diagonal())
+    same(tm.as_strided([3, 3], [1, 1], 4), as_strided(m.reshape(-1)[4:], (3, 3), (4, 4)))
+    same(tm.as_strided([0, 9], [100, 100], 1000), np.zeros((0, 9), dtype=np.int32))
+    with pytest.raises(h.HomuraError) as e:
+        tm.as_strided([4, 3], [8, 1], 5)
+    assert str(e.value) == ("setStorage: sizes [4, 3], strides [8, 1], storage offset 5, and itemsize 4 requiring a storage "
+                            "size of 128 are out of bounds for storage of size 120")
+    with pytest.raises(h.HomuraError) as e:
+        tm.as_strided([4, 3], [8], 0)
+    assert "mismatch in length of strides and shape" in str(e.value)
+    # Writing through a view whose elements overlap is refused; reading it is not.
+    overlapping = tm.as_strided([3, 3], [1, 1], 4)
+    with pytest.raises(h.HomuraError):
+        overlapping.add_(1)
+    assert array(overlapping.add(1)).tolist() == (as_strided(m.reshape(-1)[4:], (3, 3), (4, 4)) + 1).tolist()

@@ -592,6 +592,24 @@ def test_in_place_ops_are_bitwise():
     assert_bitwise(gints, ints, "a refused in-place product")
 
 
+def test_overlapping_window_views_are_read_like_on_the_cpu():
+    """Inputs whose elements share memory (unfold's sliding windows, as_strided) are legal operands: unary, binary and
+    reduction kernels read them through their strides (ref: src/tensor/view.rs, unfold / as_strided)."""
+    for dtype in (DT.F32, DT.BF16, DT.I64):
+        base = tensor(values(dtype, 40 * 37, 111), dtype, [40, 37])
+        g = base.to(GPU)
+        for view in (lambda t: t.unfold(1, 5, 2), lambda t: t.unfold(0, 8, 3), lambda t: t.unfold(1, 37, 1),
+                     lambda t: t.as_strided([30, 16], [37, 1], 3), lambda t: t.as_strided([9, 9, 4], [1, 2, 37], 0),
+                     lambda t: t.squeeze().view([37, 40]).transpose(0, 1).unfold(0, 2, 2)):
+            c, v = view(base), view(g)
+            assert v.shape == c.shape and v.strides == c.strides
+            assert_bitwise(v.contiguous(), c.contiguous(), f"{dtype} {c.shape} {c.strides} copied")
+            assert_bitwise(v.add(v), c.add(c), f"{dtype} {c.shape} {c.strides} doubled")
+            assert_bitwise(v.abs(), c.abs(), f"{dtype} {c.shape} abs")
+            if dtype == DT.I64:
+                assert_bitwise(v.sum_dim([-1], False), c.sum_dim([-1], False), f"{dtype} {c.shape} window sums")
+
+
 def test_uniform_operands_in_every_position():
     """An operand broadcast from one element, in each position (ref: rocm_elementwise.rs:864-937)."""
     for dtype in (DT.F32, DT.BF16, DT.I32):
