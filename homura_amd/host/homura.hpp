@@ -338,6 +338,10 @@ class Tensor {
     Tensor addcmul(const Tensor &tensor1, const Tensor &tensor2, Scalar value) const;
     Tensor addcdiv(const Tensor &tensor1, const Tensor &tensor2, Scalar value) const;
     Tensor lerp(const Tensor &end, const Operand &weight) const;
+    // ref: src/ops/composite.rs (addcmul_, addcdiv_, lerp_)
+    const Tensor &addcmul_(const Tensor &tensor1, const Tensor &tensor2, Scalar value) const;
+    const Tensor &addcdiv_(const Tensor &tensor1, const Tensor &tensor2, Scalar value) const;
+    const Tensor &lerp_(const Tensor &end, const Operand &weight) const;
     // beta * self + alpha * outer(vec1, vec2), one kernel (ref: src/ops/composite.rs:346-384).
     Tensor addr(const Tensor &vec1, const Tensor &vec2, Scalar beta, Scalar alpha) const;
 

@@ -632,6 +632,19 @@ Tensor Tensor::addcdiv(const Tensor &tensor1, const Tensor &tensor2, Scalar valu
     return add(tensor1.mul(value).div(tensor2));
 }
 
+const Tensor &Tensor::addcmul_(const Tensor &tensor1, const Tensor &tensor2, Scalar value) const {
+    finish_in_place(*this, addcmul(tensor1, tensor2, value));
+    return *this;
+}
+const Tensor &Tensor::addcdiv_(const Tensor &tensor1, const Tensor &tensor2, Scalar value) const {
+    finish_in_place(*this, addcdiv(tensor1, tensor2, value));
+    return *this;
+}
+const Tensor &Tensor::lerp_(const Tensor &end, const Operand &weight) const {
+    finish_in_place(*this, lerp(end, weight));
+    return *this;
+}
+
 Tensor Tensor::lerp(const Tensor &end, const Operand &weight) const {
     Tensor diff = end.sub(*this);
     if (std::holds_alternative<Scalar>(weight)) {

@@ -239,6 +239,13 @@ PYBIND11_MODULE(_host, m) {
         return t.masked_fill_(mask, to_operand(v));
     });
     T.def("copy_", [](const Tensor &t, const Tensor &src) { return t.copy_(src); });
+    T.def("addcmul_", [](const Tensor &t, const Tensor &a, const Tensor &b, const py::handle &v) {
+        return t.addcmul_(a, b, std::get<Scalar>(to_operand(v)));
+    });
+    T.def("addcdiv_", [](const Tensor &t, const Tensor &a, const Tensor &b, const py::handle &v) {
+        return t.addcdiv_(a, b, std::get<Scalar>(to_operand(v)));
+    });
+    T.def("lerp_", [](const Tensor &t, const Tensor &end, const py::handle &w) { return t.lerp_(end, to_operand(w)); });
     T.def("fill_", [](const Tensor &t, const py::handle &v) { return t.fill_(std::get<Scalar>(to_operand(v))); });
     T.def("zero_", [](const Tensor &t) { return t.zero_(); });
 

@@ -589,3 +589,10 @@ def test_in_place_operations_check_the_target_and_write_through_views():
     assert array(x).tolist() == [7, 7, 0, 0, 7, 7]
     with pytest.raises(Exception):
         tensor(np.zeros(2, dtype=np.uint8), DT.U8, [2]).fill_(300)
+    # The composites' in-place forms (ref: src/ops/composite.rs, addcmul_ / addcdiv_ / lerp_).
+    f = lambda v: tensor(np.array(v, dtype=np.float32), DT.F32, [len(v)])
+    y = f([1.0, 2.0, 3.0])
+    y.addcmul_(f([2.0, 2.0, 2.0]), f([1.0, 0.5, 4.0]), 0.5).addcdiv_(f([1.0, 1.0, 1.0]), f([4.0, 2.0, 1.0]), 2.0)
+    assert array(y).tolist() == [2.5, 3.5, 9.0]
+    y.lerp_(f([4.5, 3.5, 1.0]), 0.5)
+    assert array(y).tolist() == [3.5, 3.5, 5.0]

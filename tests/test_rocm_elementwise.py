@@ -583,6 +583,10 @@ def test_in_place_ops_are_bitwise():
             p.cpu.masked_fill_(mask, 3)
             p.gpu.masked_fill_(mask.to(GPU), 3)
             assert_bitwise(p.gpu, p.cpu, f"masked_fill_ {dtype} {p.name}")
+            if dtype in FLOATS:
+                p.cpu.addcmul_(q.cpu, q.cpu, 0.25).lerp_(q.cpu, 0.3).addcdiv_(q.cpu, p.cpu.abs().add(1), -2)
+                p.gpu.addcmul_(q.gpu, q.gpu, 0.25).lerp_(q.gpu, 0.3).addcdiv_(q.gpu, p.gpu.abs().add(1), -2)
+                assert_bitwise(p.gpu, p.cpu, f"addcmul_ / lerp_ / addcdiv_ {dtype} {p.name}")
     # A result that the target cannot hold is refused before anything is written.
     ints = tensor(values(DT.I32, 100, 62), DT.I32, [100])
     gints = ints.to(GPU)
