@@ -1146,6 +1146,20 @@ void launch_map(const MapCall &c, hipStream_t stream) {
             launch_tiled<F>(c, b, stream);
             return;
         }
+        // An output that runs along another dimension than the last one (a write into a transposed or permuted
+        // view): elements are independent, so the dimensions may be taken in any order; with that dimension
+        // last the call is a transposition like any other.
+        for (int d = 0; d + 1 < c.ndim; ++d) {
+            if (c.stride[0][d] != 1) continue;
+            MapCall t = c;
+            std::swap(t.size[d], t.size[c.ndim - 1]);
+            for (int k = 0; k < c.nops; ++k) std::swap(t.stride[k][d], t.stride[k][c.ndim - 1]);
+            if (tiled_applies<F>(t, b)) {
+                launch_tiled<F>(t, b, stream);
+                return;
+            }
+            break;
+        }
     }
     unsigned grid = grid_for(c.n, kBlock);
     if (variant == 2) {

@@ -543,6 +543,23 @@ def test_transposed_operands_through_tiles_of_two_dimensions():
         (b, gb) = both(dtype, [190, 200], 99)
         w, gw = b.narrow(0, 5, 170).narrow(1, 11, 150), gb.narrow(0, 5, 170).narrow(1, 11, 150)
         assert_bitwise(gv.add(gw), v.add(w), f"{dtype} offset view transposed + offset view")
+        # Writes into a transposed or permuted view: the output is the operand that runs along another dimension.
+        for rows, cols in ((70, 33), (128, 256), (257, 130), (384, 128)):
+            (d, gd), (src, gsrc) = both(dtype, [rows, cols], 103), both(dtype, [cols, rows], 104)
+            d.transpose(0, 1).copy_(src)
+            gd.transpose(0, 1).copy_(gsrc)
+            assert_bitwise(gd, d, f"{dtype} [{rows},{cols}] written through its transpose")
+            d.transpose(0, 1).add_(src).mul_(src)
+            gd.transpose(0, 1).add_(gsrc).mul_(gsrc)
+            assert_bitwise(gd, d, f"{dtype} [{rows},{cols}] updated through its transpose")
+            other = DT.F32 if dtype != DT.F32 else DT.BF16
+            d.transpose(0, 1).copy_(src.to(other))
+            gd.transpose(0, 1).copy_(gsrc.to(other))
+            assert_bitwise(gd, d, f"{dtype} [{rows},{cols}] written through its transpose from {other}")
+        (d, gd), (src, gsrc) = both(dtype, [4, 128, 256], 105), both(dtype, [256, 4, 128], 106)
+        d.permute([2, 0, 1]).copy_(src)
+        gd.permute([2, 0, 1]).copy_(gsrc)
+        assert_bitwise(gd, d, f"{dtype} written through permute(2,0,1)")
         # Whole tiles inside a wider buffer, at offsets that keep 16-byte alignment and at ones that do not.
         (a, ga) = both(dtype, [300, 424], 102)
         for r0, c0 in ((8, 16), (3, 16), (8, 5)):
