@@ -1126,6 +1126,13 @@ void launch_map(const MapCall &c, hipStream_t stream) {
                     hipLaunchKernelGGL((map_rows_kernel<F, kFlat, 2>), dim3(grid), dim3(kBlock), 0, stream, a);
                     return;
                 }
+                if constexpr (F::N >= 3) {
+                    // Two broadcast inputs in front of a streamed one (addr with its input: v1, v2, input).
+                    if (reused == 3) {
+                        hipLaunchKernelGGL((map_rows_kernel<F, kFlat, 3>), dim3(grid), dim3(kBlock), 0, stream, a);
+                        return;
+                    }
+                }
             }
             // An output of twice the memory-side cache or more gains nothing from passing through it.
             if constexpr (T::V * T::so == 16) {
