@@ -77,9 +77,12 @@ __device__ __forceinline__ void store_span(T *out, int64_t first, int64_t n, con
     }
 }
 
-template <class T>
+// PLAIN (narrow outputs only): `scale` is (to - from) * 2^-bits, exactly, so that bits * scale is the CPU's
+// u * (to - from) with u = bits * 2^-bits (scaling by a power of two commutes with the rounding), and the host
+// has checked that the largest sample rounds below `to`, so nothing needs mapping back to `from`.
+template <class T, bool PLAIN = false>
 __global__ void __launch_bounds__(kBlock) uniform_kernel(T *out, int64_t n, int64_t blocks, uint64_t seed, uint64_t offset,
-                                                         double from, double to) {
+                                                         double from, double to, double scale) {
     constexpr int PER = std::is_same_v<T, double> ? 2 : 4;  // F64 takes two words per value
     const T low = Conv<T>::from_f64(from);
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; i < blocks;
@@ -89,7 +92,11 @@ __global__ void __launch_bounds__(kBlock) uniform_kernel(T *out, int64_t n, int6
 #pragma unroll
         for (int j = 0; j < PER; ++j) {
             double u;
-            if constexpr (PER == 2) {
+            if constexpr (PLAIN && PER == 4) {
+                const double p = static_cast<double>(b.v[j] >> (32 - Digits<T>::value)) * scale;
+                v[j] = Conv<T>::from_f64(from + p);
+                continue;
+            } else if constexpr (PER == 2) {
                 u = unit_f64(b.v[2 * j], b.v[2 * j + 1]);
             } else {
                 constexpr int bits = Digits<T>::value;
@@ -323,8 +330,19 @@ hmr_status hmr_random_uniform(hmr_context_t ctx, const hmr_tensor_desc *out, uin
                 using T = typename decltype(t)::type;
                 const int64_t per = std::is_same_v<T, double> ? 2 : 4;
                 const int64_t blocks = (n + per - 1) / per;
+                if constexpr (!std::is_same_v<T, double>) {
+                    constexpr int bits = hmr::Digits<T>::value;
+                    const double span = to - from, scale = std::ldexp(span, -bits);
+                    const double largest = from + static_cast<double>((uint32_t{1} << bits) - 1) * scale;
+                    const bool below = hmr::Conv<T>::to_f64(hmr::Conv<T>::from_f64(largest)) < to;
+                    if (std::isfinite(span) && std::ldexp(scale, bits) == span && (below || !(from < to))) {
+                        hipLaunchKernelGGL((hmr::uniform_kernel<T, true>), dim3(hmr::grid_of(blocks)), dim3(hmr::kBlock), 0, stream,
+                                           reinterpret_cast<T *>(first), n, blocks, seed, offset, from, to, scale);
+                        return;
+                    }
+                }
                 hipLaunchKernelGGL((hmr::uniform_kernel<T>), dim3(hmr::grid_of(blocks)), dim3(hmr::kBlock), 0, stream,
-                                   reinterpret_cast<T *>(first), n, blocks, seed, offset, from, to);
+                                   reinterpret_cast<T *>(first), n, blocks, seed, offset, from, to, 0.0);
             });
         });
     });
