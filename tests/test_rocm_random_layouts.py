@@ -1,0 +1,155 @@
+"""Randomly composed views through every kernel family on the GPU against the CPU oracle, bit for bit.
+
+The layout tables of the other tests are fixed lists; the kernels, though, pick their variant from sizes, strides,
+alignment and offsets (flat rows, rows with outer dimensions, tiles of two dimensions in both forms, lines, the general
+kernel), and the edges between the variants are where a wrong choice would hide. Every case here is drawn from a seeded
+generator, so a failure names the seed and the case and repeats: a base tensor with a random shape, a random chain of
+view operations (permute, transpose, narrow, stepped slices, select, unsqueeze + expand, unfold), the same chain on the
+CPU and on the GPU, and an operation whose result must have the CPU's bits (copy and conversion, unary and binary
+arithmetic with a partner that is contiguous, broadcast or viewed the same way, comparison, where, integer sums and
+extremes with their positions along every dimension, writes through the view)."""
+import numpy as np
+import pytest
+
+from tests import oracle
+from tests.support import DT, GPU, NP, assert_bitwise, h, tensor, values
+
+pytestmark = pytest.mark.gpu
+h.register_cpu_backend(oracle.backend_address())
+
+# Sizes that sit on, below and above the tile edges of the kernels (8, 16, 64, 128, 256) and a few odd ones.
+SIZES = [1, 2, 3, 4, 5, 7, 8, 9, 16, 17, 31, 32, 33, 63, 64, 65, 96, 127, 128, 129, 130, 200, 256, 257, 384]
+
+
+def random_shape(rng, limit):
+    ndim = int(rng.integers(1, 5))
+    while True:
+        shape = [int(rng.choice(SIZES)) for _ in range(ndim)]
+        if int(np.prod(shape)) <= limit:
+            return shape
+
+
+def random_chain(rng, shape):
+    """A list of (method, arguments) applicable in order to a tensor of `shape`, and the shape it ends with."""
+    chain, shape = [], list(shape)
+    for _ in range(int(rng.integers(0, 4))):
+        nd = len(shape)
+        kind = rng.choice(["permute", "transpose", "narrow", "slice", "select", "expand", "unfold"])
+        if kind == "permute" and nd >= 2:
+            perm = [int(p) for p in rng.permutation(nd)]
+            chain.append(("permute", (perm,)))
+            shape = [shape[p] for p in perm]
+        elif kind == "transpose" and nd >= 2:
+            a, b = (int(x) for x in rng.choice(nd, 2, replace=False))
+            chain.append(("transpose", (a, b)))
+            shape[a], shape[b] = shape[b], shape[a]
+        elif kind == "narrow" and nd >= 1:
+            d = int(rng.integers(0, nd))
+            if shape[d] >= 2:
+                start = int(rng.integers(0, shape[d] - 1))
+                length = int(rng.integers(1, shape[d] - start + 1))
+                chain.append(("narrow", (d, start, length)))
+                shape[d] = length
+        elif kind == "slice" and nd >= 1:
+            d = int(rng.integers(0, nd))
+            if shape[d] >= 3:
+                start, step = int(rng.integers(0, 2)), int(rng.integers(2, 4))
+                chain.append(("slice", (d, start, None, step)))
+                shape[d] = len(range(start, shape[d], step))
+        elif kind == "select" and nd >= 2:
+            d = int(rng.integers(0, nd))
+            chain.append(("select", (d, int(rng.integers(0, shape[d])))))
+            del shape[d]
+        elif kind == "expand" and nd <= 3:
+            d = int(rng.integers(0, nd + 1))
+            times = int(rng.choice([2, 3, 8, 64]))
+            chain.append(("unsqueeze", (d,)))
+            shape.insert(d, times)
+            chain.append(("expand", (list(shape),)))
+        elif kind == "unfold" and nd >= 1 and nd <= 3:
+            d = int(rng.integers(0, nd))
+            if shape[d] >= 4:
+                size, step = int(rng.integers(2, 5)), int(rng.integers(1, 4))
+                chain.append(("unfold", (d, size, step)))
+                shape[d] = (shape[d] - size) // step + 1
+                shape.append(size)
+    return chain, shape
+
+
+def apply(t, chain):
+    for method, args in chain:
+        t = getattr(t, method)(*args)
+    return t
+
+
+def pair(dtype, shape, seed):
+    t = tensor(values(dtype, int(np.prod(shape)), seed), dtype, shape)
+    return t, t.to(GPU)
+
+
+def overlapping(t):
+    """Whether two indices of the view may be one element (expanded or unfolded): such a view cannot be written."""
+    reach = 0
+    for stride, size in sorted((s, n) for s, n in zip(t.strides, t.shape) if n > 1):
+        if stride <= reach:
+            return True
+        reach += (size - 1) * stride
+    return False
+
+
+@pytest.mark.parametrize("seed", range(32))
+def test_random_views_through_every_kernel_family(seed):
+    rng = np.random.default_rng(0x5EED0000 + seed)
+    dtypes = [DT.F32, DT.BF16, DT.I64, DT.U8, DT.F16, DT.I32, DT.F64, DT.Bool]
+    for case in range(150):
+        dtype = dtypes[int(rng.integers(0, len(dtypes)))]
+        base_shape = random_shape(rng, 120000)
+        chain, shape = random_chain(rng, base_shape)
+        what = f"seed {seed} case {case}: {dtype} {base_shape} {chain}"
+        (c, g) = pair(dtype, base_shape, 1000 * seed + case)
+        vc, vg = apply(c, chain), apply(g, chain)
+        assert vg.shape == vc.shape and vg.strides == vc.strides and vg.offset == vc.offset, what
+        assert_bitwise(vg.contiguous(), vc.contiguous(), f"{what}: copy")
+        other = dtypes[int(rng.integers(0, len(dtypes)))]
+        assert_bitwise(vg.to(other), vc.to(other), f"{what}: to {other}")
+        # A partner: contiguous of the view's shape, viewed the same way, or broadcast along some dimensions.
+        choice = int(rng.integers(0, 3))
+        if choice == 0 or not shape:
+            pc, pg = pair(dtype, shape, 77 + case)
+        elif choice == 1:
+            bc, bg = pair(dtype, base_shape, 78 + case)
+            pc, pg = apply(bc, chain), apply(bg, chain)
+        else:
+            small = [n if rng.integers(0, 2) else 1 for n in shape]
+            pc, pg = pair(dtype, small, 79 + case)
+        if dtype == DT.Bool:
+            assert_bitwise(vg.logical_and(pg), vc.logical_and(pc), f"{what}: and")
+            assert_bitwise(vg.logical_not(), vc.logical_not(), f"{what}: not")
+        else:
+            assert_bitwise(vg.add(pg), vc.add(pc), f"{what}: + partner {choice}")
+            assert_bitwise(pg.sub(vg), pc.sub(vc), f"{what}: partner {choice} -")
+            assert_bitwise(vg.mul(3), vc.mul(3), f"{what}: * 3")
+            assert_bitwise(vg.abs(), vc.abs(), f"{what}: abs")
+            assert_bitwise(vg.greater(pg), vc.greater(pc), f"{what}: >")
+            mask_c = vc.greater(pc)
+            assert_bitwise(h.where_(mask_c.to(GPU), vg, pg), h.where_(mask_c, vc, pc), f"{what}: where")
+        if dtype in (DT.I64, DT.I32, DT.U8) and shape:
+            d = int(rng.integers(0, len(shape)))
+            assert_bitwise(vg.sum_dim([d], False), vc.sum_dim([d], False), f"{what}: sum along {d}")
+            if shape[d] > 0:
+                (gv, gi), (cv, ci) = vg.max_dim(d, False), vc.max_dim(d, False)
+                assert_bitwise(gv, cv, f"{what}: max along {d}")
+                assert_bitwise(gi, ci, f"{what}: positions of the max along {d}")
+        if dtype in (DT.F32, DT.BF16) and shape and shape[-1] > 0:
+            (gv, gi), (cv, ci) = vg.min_dim(-1, True), vc.min_dim(-1, True)
+            assert_bitwise(gv, cv, f"{what}: min along the last dimension")
+            assert_bitwise(gi, ci, f"{what}: positions of the min")
+        # Writing through the view (when its elements are distinct): the whole base must agree afterwards.
+        if not overlapping(vc) and dtype != DT.Bool:
+            sc, sg = pair(dtype, shape, 80 + case)
+            vc.copy_(sc)
+            vg.copy_(sg)
+            assert_bitwise(g, c, f"{what}: written through the view")
+            vc.add_(pc)
+            vg.add_(pg)
+            assert_bitwise(g, c, f"{what}: updated through the view")
