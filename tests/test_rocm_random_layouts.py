@@ -21,10 +21,14 @@ h.register_cpu_backend(oracle.backend_address())
 SIZES = [1, 2, 3, 4, 5, 7, 8, 9, 16, 17, 31, 32, 33, 63, 64, 65, 96, 127, 128, 129, 130, 200, 256, 257, 384]
 
 
-def random_shape(rng, limit):
+# For a few cases of several million elements: more than one workgroup per row, tile, line and slice.
+LARGE_SIZES = [2, 3, 8, 64, 128, 256, 257, 384, 512, 1000, 1024, 2048]
+
+
+def random_shape(rng, limit, sizes=SIZES):
     ndim = int(rng.integers(1, 5))
     while True:
-        shape = [int(rng.choice(SIZES)) for _ in range(ndim)]
+        shape = [int(rng.choice(sizes)) for _ in range(ndim)]
         if int(np.prod(shape)) <= limit:
             return shape
 
@@ -97,13 +101,14 @@ def overlapping(t):
     return False
 
 
-@pytest.mark.parametrize("seed", range(32))
+@pytest.mark.parametrize("seed", list(range(32)) + [100, 101, 102, 103])
 def test_random_views_through_every_kernel_family(seed):
     rng = np.random.default_rng(0x5EED0000 + seed)
     dtypes = [DT.F32, DT.BF16, DT.I64, DT.U8, DT.F16, DT.I32, DT.F64, DT.Bool]
-    for case in range(150):
+    large = seed >= 100
+    for case in range(20 if large else 150):
         dtype = dtypes[int(rng.integers(0, len(dtypes)))]
-        base_shape = random_shape(rng, 120000)
+        base_shape = random_shape(rng, 3000000, LARGE_SIZES) if large else random_shape(rng, 120000)
         chain, shape = random_chain(rng, base_shape)
         what = f"seed {seed} case {case}: {dtype} {base_shape} {chain}"
         (c, g) = pair(dtype, base_shape, 1000 * seed + case)
