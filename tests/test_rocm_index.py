@@ -376,3 +376,32 @@ def test_zero_dimensional_gpu_indices_select():
     with pytest.raises(h.HomuraError) as e:
         g.index_tensors([bad.to(GPU)])
     assert str(e.value) == str(c.value)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_gathers_and_scatter_adds_around_the_line_kernels_limits(seed):
+    """gather and scatter_add along a random dimension of random shapes whose line counts, line lengths and numbers of
+    positions straddle what the per-line kernels accept (128 lines, 64 to 2048 positions, 64 KiB of line), with
+    contiguous and permuted operands, I32 and I64 positions, repeated targets in every density: the CPU's bits."""
+    rng = np.random.default_rng(0x1D0000 + seed)
+    for case in range(12):
+        dtype = [DT.F32, DT.BF16, DT.I64, DT.F64, DT.U8][int(rng.integers(0, 5))]
+        lines = int(rng.choice([1, 7, 127, 128, 129, 300]))
+        length = int(rng.choice([5, 63, 64, 100, 1000, 2048, 4096, 20000]))
+        count = int(rng.choice([1, 63, 64, 65, 500, 2047, 2048, 2049]))
+        if lines * max(length, count) > 3000000:
+            lines = 128
+        dim = int(rng.integers(0, 2))
+        shape = [lines, length] if dim == 1 else [length, lines]
+        ishape = [lines, count] if dim == 1 else [count, lines]
+        what = f"seed {seed} case {case}: {dtype} {shape} dim {dim}, {count} positions a line"
+        x = tensor(values(dtype, lines * length, 500 + case), dtype, shape)
+        if rng.integers(0, 3) == 0:   # the other dimension contiguous
+            x = x.transpose(0, 1).contiguous().transpose(0, 1)
+        spread = int(rng.choice([length, max(1, length // 50), 1 + length // 3]))   # few targets: long runs of repeats
+        picks = (words(600 + 31 * seed + case, lines * count) % np.uint64(spread)).astype(np.int64)
+        index = ints(picks, ishape, DT.I32 if rng.integers(0, 2) else DT.I64)
+        g = x.to(GPU)
+        assert_same(g.gather(dim, index.to(GPU)), x.gather(dim, index), f"gather {what}")
+        src = tensor(values(dtype, lines * count, 700 + case), dtype, ishape)
+        assert_bitwise(g.scatter_add(dim, index.to(GPU), src.to(GPU)), x.scatter_add(dim, index, src), f"scatter_add {what}")
