@@ -596,3 +596,70 @@ def test_in_place_operations_check_the_target_and_write_through_views():
     assert array(y).tolist() == [2.5, 3.5, 9.0]
     y.lerp_(f([4.5, 3.5, 1.0]), 0.5)
     assert array(y).tolist() == [3.5, 3.5, 5.0]
+
+
+def test_the_references_known_answers_for_in_place_operations_and_overlapping_copies():
+    """ref: tests/m0_boundaries.rs (as_strided_offset_bounds_and_independent_copy, overlap_copy_transpose_and_broadcast,
+    rejected_writes_leave_destination_unchanged, composite_in_place_operations_preserve_aliases_and_values) and
+    tests/tensor_api.rs (in_place_on_itself_and_overlapping_copy, in_place_casts_and_broadcasts and the four
+    should_panic cases after them)."""
+    i64 = lambda v, shape=None: tensor(np.array(v, dtype=np.int64), DT.I64, shape if shape is not None else [len(v)])
+    f32 = lambda v, shape=None: tensor(np.array(v, dtype=np.float32), DT.F32, shape if shape is not None else [len(v)])
+    x = i64(np.arange(10))
+    y = x.as_strided([2, 3], [4, 1], 1)
+    assert array(y).reshape(-1).tolist() == [1, 2, 3, 5, 6, 7]
+    y.copy_(i64([20, 30, 40]))
+    assert array(x).tolist() == [0, 20, 30, 40, 4, 20, 30, 40, 8, 9]
+    for bad in (lambda: x.as_strided([2, 3], [4, 1], 5), lambda: x.as_strided([2, 3], [1], 0)):
+        with pytest.raises(h.HomuraError):
+            bad()
+    x = i64(np.arange(9)).view([3, 3])
+    x.copy_(x.transpose(0, 1))
+    assert array(x).reshape(-1).tolist() == [0, 3, 6, 1, 4, 7, 2, 5, 8]
+    x.copy_(x.narrow(0, 0, 1))
+    assert array(x).reshape(-1).tolist() == [0, 3, 6, 0, 3, 6, 0, 3, 6]
+    y = i64(np.arange(6))
+    y.narrow(0, 0, 5).copy_(y.narrow(0, 1, 5))
+    assert array(y).tolist() == [1, 2, 3, 4, 5, 5]
+    x = i64([1, 2, 3])
+    for bad in (lambda: x.add_(f32(np.zeros(6), [2, 3])), lambda: x.copy_(i64([1, 2])), lambda: x.add_(0.5)):
+        with pytest.raises(h.HomuraError):
+            bad()
+    assert array(x).tolist() == [1, 2, 3]
+    assert array(i64([2, 3]).mul(4)).tolist() == [8, 12]
+    # tensor_api.rs
+    x = f32([1.0, 2.0, 3.0])
+    x.add_(x)
+    assert array(x).tolist() == [2.0, 4.0, 6.0]
+    x.mul_(x.narrow(0, 0, 1))
+    assert array(x).tolist() == [4.0, 8.0, 12.0]
+    y = i64(np.arange(6))
+    y.narrow(0, 1, 5).copy_(y.narrow(0, 0, 5))
+    assert array(y).tolist() == [0, 0, 1, 2, 3, 4]
+    half = tensor(np.zeros(6, dtype=np.uint16), DT.F16, [2, 3])
+    half.add_(f32([1.0, 2.0, 3.0]))
+    assert half.dtype == DT.F16 and to_f64(array(half), DT.F16).reshape(-1).tolist() == [1.0, 2.0, 3.0, 1.0, 2.0, 3.0]
+    i = i64([1, 2, 3])
+    i.mul_(2)
+    assert array(i).tolist() == [2, 4, 6]
+    i.copy_(f32([1.9, -1.9, 0.5]))
+    assert array(i).tolist() == [1, -1, 0]
+    for bad, message in ((lambda: i64([1, 2]).add_(1.5), "result type f32 can't be cast to the desired output type i64"),
+                         (lambda: i64([1, 2]).div_(2), "result type f32 can't be cast to the desired output type i64"),
+                         (lambda: f32(np.zeros(3)).add_(f32(np.zeros(6), [2, 3])),
+                          "output with shape [3] doesn't match the broadcast shape [2, 3]"),
+                         (lambda: f32(np.zeros(3), [1, 3]).expand([4, 3]).fill_(1.0),
+                          "more than one element of the written-to tensor")):
+        with pytest.raises(h.HomuraError) as e:
+            bad()
+        assert message in str(e.value), str(e.value)
+    # m0_boundaries.rs: the composites, through an alias of the same storage.
+    x = f32([2.0, 4.0])
+    alias = x.view([2])
+    a, b = f32([3.0, 6.0]), f32([2.0, 2.0])
+    x.addcmul_(a, b, 1).addcdiv_(a, b, 2)
+    assert array(alias).tolist() == [11.0, 22.0]
+    x.lerp_(f32([0.0, 0.0]), 0.5).pow_(2).sub_(0.25).mul_(2).div_(4)
+    assert array(alias).tolist() == [15.0, 60.375]
+    x.clamp_(0, 20).masked_fill_(tensor(np.array([1, 0], dtype=np.uint8), DT.Bool, [2]), -1)
+    assert array(alias).tolist() == [-1.0, 20.0]
