@@ -663,3 +663,50 @@ def test_the_references_known_answers_for_in_place_operations_and_overlapping_co
     assert array(alias).tolist() == [15.0, 60.375]
     x.clamp_(0, 20).masked_fill_(tensor(np.array([1, 0], dtype=np.uint8), DT.Bool, [2]), -1)
     assert array(alias).tolist() == [-1.0, 20.0]
+
+
+def test_more_known_answers_of_the_references_boundary_tests():
+    """ref: tests/m0_boundaries.rs (noncontiguous_offset_kernels, scalar_reductions_views_and_softmax,
+    view_strides_and_contiguous_alias_contract, the triangles of shape_operators_on_noncontiguous_inputs, the view and
+    elementwise parts of empty_creation_views_and_broadcasting); what needs matmul, concat or stack is out of scope."""
+    i64 = lambda v, shape=None: tensor(np.array(v, dtype=np.int64), DT.I64, shape if shape is not None else [len(v)])
+    flat = lambda t: array(t).reshape(-1).tolist()
+    x = i64(np.arange(24)).view([2, 3, 4]).narrow(2, 1, 2).permute([1, 0, 2])
+    assert flat(x) == [1, 2, 13, 14, 5, 6, 17, 18, 9, 10, 21, 22]
+    assert flat(x.sum_dim([0, 2], False)) == [33, 105]
+    assert flat(x.max_dim(2, False)[0]) == [2, 14, 6, 18, 10, 22]
+    assert flat(x.pow(2)) == [1, 4, 169, 196, 25, 36, 289, 324, 81, 100, 441, 484]
+    assert x.to(DT.F16).is_contiguous()
+    t = tensor(np.array([3.0], dtype=np.float32), DT.F32, [])
+    for dim in (0, -1):
+        assert t.sum_dim([dim], True).shape == []
+        v, i = t.max_dim(dim, True)
+        assert array(v).item() == 3.0 and array(i).item() == 0
+        assert array(t.softmax(dim)).item() == 1.0 and array(t.log_softmax(dim)).item() == 0.0
+        assert t.transpose(dim, dim).shape == []
+    assert t.unsqueeze(-1).squeeze().shape == []
+    assert array(t.var(0)).item() == 0.0 and math.isnan(array(t.var(1)).item())
+    assert t.flatten(0, -1).shape == [1]
+    source = i64(np.arange(12)).view([3, 4])
+    strided = source.slice(1, 0, 4, 2)
+    assert strided.strides == [4, 2] and strided.view([6]).strides == [2]
+    strided.view([6]).fill_(9)
+    assert flat(source) == [9, 1, 9, 3, 9, 5, 9, 7, 9, 9, 9, 11]
+    copied = source.transpose(0, 1).contiguous()
+    copied.fill_(-1)
+    assert array(source.select(0, 0).select(0, 0)).item() == 9
+    expanded = i64([7]).expand([3, 4])
+    assert flat(expanded) == [7] * 12
+    with pytest.raises(h.HomuraError):
+        expanded.copy_(i64(np.ones(12), [3, 4]))
+    tt = i64(np.arange(6)).view([2, 3]).transpose(0, 1)
+    assert flat(tt.triu(1)) == [0, 3, 0, 0, 0, 0] and flat(tt.tril(-1)) == [0, 0, 1, 0, 2, 5]
+    with pytest.raises(h.HomuraError):
+        tt.flip([0, -2])
+    for dtype in (DT.Bool, DT.U8, DT.I64, DT.F16, DT.BF16, DT.F32, DT.F64):
+        e = tensor(np.zeros(0, dtype=NP[dtype]), dtype, [2, 0, 3])
+        assert e.num_elements() == 0 and e.is_contiguous()
+        assert e.to(dtype).shape == [2, 0, 3] and e.transpose(0, 2).reshape([0, 6]).shape == [0, 6]
+        assert e.add(tensor(np.ones(3, dtype=NP[dtype]), dtype, [1, 3])).shape == [2, 0, 3]
+        assert e.flip([0, 2]).shape == [2, 0, 3]
+    assert tensor(np.zeros(0, dtype=np.float32), DT.F32, [0]).view([-1, 3]).shape == [0, 3]
