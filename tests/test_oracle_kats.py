@@ -599,12 +599,16 @@ def test_in_place_operations_check_the_target_and_write_through_views():
 
 
 def test_the_references_known_answers_for_in_place_operations_and_overlapping_copies():
+    in_place_known_answers("cpu")
+
+
+def in_place_known_answers(device):
     """ref: tests/m0_boundaries.rs (as_strided_offset_bounds_and_independent_copy, overlap_copy_transpose_and_broadcast,
     rejected_writes_leave_destination_unchanged, composite_in_place_operations_preserve_aliases_and_values) and
     tests/tensor_api.rs (in_place_on_itself_and_overlapping_copy, in_place_casts_and_broadcasts and the four
-    should_panic cases after them)."""
-    i64 = lambda v, shape=None: tensor(np.array(v, dtype=np.int64), DT.I64, shape if shape is not None else [len(v)])
-    f32 = lambda v, shape=None: tensor(np.array(v, dtype=np.float32), DT.F32, shape if shape is not None else [len(v)])
+    should_panic cases after them). Also run on the GPU (tests/test_rocm_elementwise.py)."""
+    i64 = lambda v, shape=None: tensor(np.array(v, dtype=np.int64), DT.I64, shape if shape is not None else [len(v)], device)
+    f32 = lambda v, shape=None: tensor(np.array(v, dtype=np.float32), DT.F32, shape if shape is not None else [len(v)], device)
     x = i64(np.arange(10))
     y = x.as_strided([2, 3], [4, 1], 1)
     assert array(y).reshape(-1).tolist() == [1, 2, 3, 5, 6, 7]
@@ -636,7 +640,7 @@ def test_the_references_known_answers_for_in_place_operations_and_overlapping_co
     y = i64(np.arange(6))
     y.narrow(0, 1, 5).copy_(y.narrow(0, 0, 5))
     assert array(y).tolist() == [0, 0, 1, 2, 3, 4]
-    half = tensor(np.zeros(6, dtype=np.uint16), DT.F16, [2, 3])
+    half = tensor(np.zeros(6, dtype=np.uint16), DT.F16, [2, 3], device)
     half.add_(f32([1.0, 2.0, 3.0]))
     assert half.dtype == DT.F16 and to_f64(array(half), DT.F16).reshape(-1).tolist() == [1.0, 2.0, 3.0, 1.0, 2.0, 3.0]
     i = i64([1, 2, 3])
@@ -661,15 +665,20 @@ def test_the_references_known_answers_for_in_place_operations_and_overlapping_co
     assert array(alias).tolist() == [11.0, 22.0]
     x.lerp_(f32([0.0, 0.0]), 0.5).pow_(2).sub_(0.25).mul_(2).div_(4)
     assert array(alias).tolist() == [15.0, 60.375]
-    x.clamp_(0, 20).masked_fill_(tensor(np.array([1, 0], dtype=np.uint8), DT.Bool, [2]), -1)
+    x.clamp_(0, 20).masked_fill_(tensor(np.array([1, 0], dtype=np.uint8), DT.Bool, [2], device), -1)
     assert array(alias).tolist() == [-1.0, 20.0]
 
 
 def test_more_known_answers_of_the_references_boundary_tests():
+    boundary_known_answers("cpu")
+
+
+def boundary_known_answers(device):
     """ref: tests/m0_boundaries.rs (noncontiguous_offset_kernels, scalar_reductions_views_and_softmax,
     view_strides_and_contiguous_alias_contract, the triangles of shape_operators_on_noncontiguous_inputs, the view and
-    elementwise parts of empty_creation_views_and_broadcasting); what needs matmul, concat or stack is out of scope."""
-    i64 = lambda v, shape=None: tensor(np.array(v, dtype=np.int64), DT.I64, shape if shape is not None else [len(v)])
+    elementwise parts of empty_creation_views_and_broadcasting); what needs matmul, concat or stack is out of scope.
+    Also run on the GPU (tests/test_rocm_elementwise.py)."""
+    i64 = lambda v, shape=None: tensor(np.array(v, dtype=np.int64), DT.I64, shape if shape is not None else [len(v)], device)
     flat = lambda t: array(t).reshape(-1).tolist()
     x = i64(np.arange(24)).view([2, 3, 4]).narrow(2, 1, 2).permute([1, 0, 2])
     assert flat(x) == [1, 2, 13, 14, 5, 6, 17, 18, 9, 10, 21, 22]
@@ -677,7 +686,7 @@ def test_more_known_answers_of_the_references_boundary_tests():
     assert flat(x.max_dim(2, False)[0]) == [2, 14, 6, 18, 10, 22]
     assert flat(x.pow(2)) == [1, 4, 169, 196, 25, 36, 289, 324, 81, 100, 441, 484]
     assert x.to(DT.F16).is_contiguous()
-    t = tensor(np.array([3.0], dtype=np.float32), DT.F32, [])
+    t = tensor(np.array([3.0], dtype=np.float32), DT.F32, [], device)
     for dim in (0, -1):
         assert t.sum_dim([dim], True).shape == []
         v, i = t.max_dim(dim, True)
@@ -704,9 +713,9 @@ def test_more_known_answers_of_the_references_boundary_tests():
     with pytest.raises(h.HomuraError):
         tt.flip([0, -2])
     for dtype in (DT.Bool, DT.U8, DT.I64, DT.F16, DT.BF16, DT.F32, DT.F64):
-        e = tensor(np.zeros(0, dtype=NP[dtype]), dtype, [2, 0, 3])
+        e = tensor(np.zeros(0, dtype=NP[dtype]), dtype, [2, 0, 3], device)
         assert e.num_elements() == 0 and e.is_contiguous()
         assert e.to(dtype).shape == [2, 0, 3] and e.transpose(0, 2).reshape([0, 6]).shape == [0, 6]
-        assert e.add(tensor(np.ones(3, dtype=NP[dtype]), dtype, [1, 3])).shape == [2, 0, 3]
+        assert e.add(tensor(np.ones(3, dtype=NP[dtype]), dtype, [1, 3], device)).shape == [2, 0, 3]
         assert e.flip([0, 2]).shape == [2, 0, 3]
-    assert tensor(np.zeros(0, dtype=np.float32), DT.F32, [0]).view([-1, 3]).shape == [0, 3]
+    assert tensor(np.zeros(0, dtype=np.float32), DT.F32, [0], device).view([-1, 3]).shape == [0, 3]

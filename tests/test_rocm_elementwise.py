@@ -631,6 +631,14 @@ def test_overlapping_window_views_are_read_like_on_the_cpu():
                 assert_bitwise(v.sum_dim([-1], False), c.sum_dim([-1], False), f"{dtype} {c.shape} window sums")
 
 
+def test_the_references_known_answers_on_the_gpu():
+    """The known answers of the reference's boundary and API tests for in-place operations, overlapping copies,
+    as_strided, non-contiguous views, scalar reductions and empty tensors, with every tensor on the GPU."""
+    from tests.test_oracle_kats import boundary_known_answers, in_place_known_answers
+    in_place_known_answers(GPU)
+    boundary_known_answers(GPU)
+
+
 def test_uniform_operands_in_every_position():
     """An operand broadcast from one element, in each position (ref: rocm_elementwise.rs:864-937)."""
     for dtype in (DT.F32, DT.BF16, DT.I32):
