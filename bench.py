@@ -354,7 +354,7 @@ def per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP
     cube = residual.reshape([64, 1024, 1024]).permute([2, 0, 1])
     add(None, "permute(2,0,1) f32 [64,1024,1024] -> contiguous (tiles through LDS, 16-byte accesses)", 8 * N, lambda: cube.contiguous(), 10)
     halfcols = sqm.slice(1, 0, 8192, 2)
-    add(None, "every other column f32 [8192,4096] -> contiguous (general kernel, an element per lane)", 4 * N,
+    add(None, "every other column f32 [8192,4096] -> contiguous (general kernel, four elements per lane in flight)", 4 * N,
         lambda: halfcols.contiguous(), 10)
     del sqm, sqt, sqb, cube, halfcols
     sq = residual.reshape([16, 2048, 2048])
