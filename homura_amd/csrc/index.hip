@@ -52,13 +52,16 @@ __global__ void __launch_bounds__(kBlock) check_kernel(const void *index, int is
     if ((threadIdx.x & 63) == 0 && first != ~0ull) atomicMin(slot, first);
 }
 
-// The same for an index that is one aligned contiguous run: 16 bytes per lane and load, four loads in flight
-// (an element per lane reads 33 MB of positions in 22 us; this form in a third of that).
+// The same for an index that is one contiguous run: 16 bytes per lane and load, four loads in flight (an
+// element per lane reads 33 MB of positions in 22 us; this form in a third of that). `head` elements (fewer
+// than a tile) come before the first 16-byte boundary; they and the ragged end go to the first workgroup's lanes.
 template <class I>
-__global__ void __launch_bounds__(kBlock) check_flat_kernel(const I *index, int64_t n, int64_t low, int64_t high, int has_exempt,
-                                                            int64_t exempt, unsigned long long *slot) {
+__global__ void __launch_bounds__(kBlock) check_flat_kernel(const I *start, int head, int64_t total, int64_t low, int64_t high,
+                                                            int has_exempt, int64_t exempt, unsigned long long *slot) {
     constexpr int V = 16 / static_cast<int>(sizeof(I)), U = 4;
     unsigned long long first = ~0ull;
+    const I *index = start + head;  // aligned; position p of the run is index[p - head]
+    const int64_t n = total - head;
     const int64_t tiles = n / V;
     for (int64_t t0 = static_cast<int64_t>(blockIdx.x) * (U * kBlock) + threadIdx.x; t0 < tiles;
          t0 += static_cast<int64_t>(gridDim.x) * (U * kBlock)) {
@@ -75,16 +78,21 @@ __global__ void __launch_bounds__(kBlock) check_flat_kernel(const I *index, int6
             for (int i = V - 1; i >= 0; --i) {  // backwards: the smallest position of the tile ends up in `first`
                 const int64_t x = static_cast<int64_t>(v[u][i]);
                 const bool bad = t < tiles && !(x >= low && x < high) && !(has_exempt && x == exempt);
-                const unsigned long long p = static_cast<unsigned long long>(t * V + i);
+                const unsigned long long p = static_cast<unsigned long long>(t * V + i + head);
                 if (bad && p < first) first = p;
             }
         }
     }
-    // The ragged end (fewer than V elements), by the first lanes of the first workgroup.
-    if (blockIdx.x == 0 && threadIdx.x < static_cast<unsigned>(n - tiles * V)) {
-        const int64_t p = tiles * V + threadIdx.x;
-        const int64_t x = static_cast<int64_t>(index[p]);
-        if (!(x >= low && x < high) && !(has_exempt && x == exempt) && static_cast<unsigned long long>(p) < first) first = p;
+    // The head and the ragged end (fewer than V elements each), by the first lanes of the first workgroup.
+    if (blockIdx.x == 0) {
+        const int64_t tail = n - tiles * V;
+        int64_t p = -1;
+        if (threadIdx.x < static_cast<unsigned>(head)) p = threadIdx.x;
+        else if (threadIdx.x - head < tail) p = head + tiles * V + (threadIdx.x - head);
+        if (p >= 0) {
+            const int64_t x = static_cast<int64_t>(start[p]);
+            if (!(x >= low && x < high) && !(has_exempt && x == exempt) && static_cast<unsigned long long>(p) < first) first = p;
+        }
     }
 #pragma unroll
     for (int m = 32; m >= 1; m >>= 1) {
@@ -596,8 +604,12 @@ hmr_status hmr_index_check(hmr_context_t ctx, const hmr_tensor_desc *index, int6
             }
             hipLaunchKernelGGL(hmr::check_init_kernel, dim3(1), dim3(1), 0, stream, slot);
             if (n > 0) {
-                // One aligned contiguous run (after merging: a size-1 dimension's stride does not count)?
-                bool flat = reinterpret_cast<uintptr_t>(base) % 16 == 0;
+                // One contiguous run (after merging: a size-1 dimension's stride does not count)? Its elements
+                // before the first 16-byte boundary are the head.
+                const int elem = is64 ? 8 : 4;
+                const int64_t to_boundary = static_cast<int64_t>((16 - reinterpret_cast<uintptr_t>(base) % 16) % 16) / elem;
+                const int head = static_cast<int>(to_boundary < n ? to_boundary : n);
+                bool flat = reinterpret_cast<uintptr_t>(base) % elem == 0;
                 int64_t run = 1;
                 for (int k = index->ndim - 1; flat && k >= 0; --k) {
                     flat = index->sizes[k] == 1 || index->strides[k] == run;
@@ -608,11 +620,11 @@ hmr_status hmr_index_check(hmr_context_t ctx, const hmr_tensor_desc *index, int6
                     const unsigned grid = hmr::grid_of((n + per_block - 1) / per_block * hmr::kBlock);
                     if (is64) {
                         hipLaunchKernelGGL((hmr::check_flat_kernel<int64_t>), dim3(grid), dim3(hmr::kBlock), 0, stream,
-                                           static_cast<const int64_t *>(base), n, low, high, has_exempt, exempt,
+                                           static_cast<const int64_t *>(base), head, n, low, high, has_exempt, exempt,
                                            reinterpret_cast<unsigned long long *>(slot));
                     } else {
                         hipLaunchKernelGGL((hmr::check_flat_kernel<int32_t>), dim3(grid), dim3(hmr::kBlock), 0, stream,
-                                           static_cast<const int32_t *>(base), n, low, high, has_exempt, exempt,
+                                           static_cast<const int32_t *>(base), head, n, low, high, has_exempt, exempt,
                                            reinterpret_cast<unsigned long long *>(slot));
                     }
                 } else {

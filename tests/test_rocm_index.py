@@ -405,3 +405,30 @@ def test_random_gathers_and_scatter_adds_around_the_line_kernels_limits(seed):
         assert_same(g.gather(dim, index.to(GPU)), x.gather(dim, index), f"gather {what}")
         src = tensor(values(dtype, lines * count, 700 + case), dtype, ishape)
         assert_bitwise(g.scatter_add(dim, index.to(GPU), src.to(GPU)), x.scatter_add(dim, index, src), f"scatter_add {what}")
+
+
+def test_a_contiguous_index_off_the_16_byte_boundary_is_checked_like_any_other():
+    """An index that is one contiguous run starting 1 to 3 elements into its buffer (its head lies before the first
+    16-byte boundary, its end may be ragged): the first position out of range is reported wherever it lies, with the
+    CPU's message, and a valid index selects the CPU's rows."""
+    x = tensor(values(DT.F32, 50 * 3, 9), DT.F32, [50, 3])
+    g = x.to(GPU)
+    for dtype in (DT.I32, DT.I64):
+        for offset in (1, 2, 3):
+            for n in (70001, 65537 + offset):
+                picks = random_positions(n + offset, 50, 10 * offset + n % 7)
+                for bad_at in (None, 0, 1, 2, n // 2, n - 2, n - 1):
+                    v = picks.copy()
+                    if bad_at is not None:
+                        v[offset + bad_at] = 50 + bad_at % 5
+                        v[min(offset + bad_at + 3, n + offset - 1)] = -7 if bad_at % 2 else 99   # a later one must not win
+                    index = ints(v, [n + offset], dtype).narrow(0, offset, n)
+                    what = f"{dtype} offset {offset} n {n} bad at {bad_at}"
+                    if bad_at is None:
+                        assert_same(g.index_select(0, index.to(GPU)), x.index_select(0, index), what)
+                        continue
+                    with pytest.raises(h.HomuraError) as c:
+                        x.index_select(0, index)
+                    with pytest.raises(h.HomuraError) as e:
+                        g.index_select(0, index.to(GPU))
+                    assert str(e.value) == str(c.value), what
