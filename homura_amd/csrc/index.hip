@@ -187,19 +187,42 @@ __global__ void check_value_kernel(const void *index, int is64, Dims d, uint64_t
 template <class W>
 __global__ void __launch_bounds__(kBlock) pick_kernel(W *out, const W *src, const void *index, int is64, Dims d, int64_t n,
                                                       int64_t wrap) {
-    for (int64_t p = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; p < n; p += static_cast<int64_t>(gridDim.x) * kBlock) {
-        int64_t rest = p, oo = 0, so = 0, io = 0;
-        for (int k = 0; k < d.ndim; ++k) {
-            const int64_t q = rest / d.size[k];
-            const int64_t c = rest - q * d.size[k];
-            rest = q;
-            oo += c * d.stride[0][k];
-            io += c * d.stride[2][k];
-            if (k != d.at) so += c * d.stride[1][k];
+    // Four picks per lane, a workgroup apart: their positions are read first, then their elements, then they are
+    // stored (one pick per lane leaves a wave with one dependent pair of loads in flight). The outermost
+    // dimension needs no division.
+    constexpr int U = 4;
+    for (int64_t base = static_cast<int64_t>(blockIdx.x) * (U * kBlock); base < n; base += static_cast<int64_t>(gridDim.x) * (U * kBlock)) {
+        int64_t oo[U], so[U], j[U];
+        bool valid[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int64_t wanted = base + static_cast<int64_t>(u) * kBlock + threadIdx.x;
+            valid[u] = wanted < n;
+            int64_t rest = valid[u] ? wanted : n - 1, io = 0;
+            oo[u] = so[u] = 0;
+            for (int k = 0; k < d.ndim; ++k) {
+                int64_t c = rest;
+                if (k + 1 < d.ndim) {
+                    const int64_t q = rest / d.size[k];
+                    c = rest - q * d.size[k];
+                    rest = q;
+                }
+                oo[u] += c * d.stride[0][k];
+                io += c * d.stride[2][k];
+                if (k != d.at) so[u] += c * d.stride[1][k];
+            }
+            j[u] = read_index(index, is64, io);
         }
-        int64_t j = read_index(index, is64, io);
-        if (j < 0) j += wrap;
-        out[oo] = src[so + j * d.stride[1][d.at]];
+        W v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (j[u] < 0) j[u] += wrap;
+            v[u] = src[so[u] + j[u] * d.stride[1][d.at]];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (valid[u]) out[oo[u]] = v[u];
+        }
     }
 }
 
@@ -721,7 +744,7 @@ hmr_status hmr_index_select(hmr_context_t ctx, const hmr_tensor_desc *out, const
                     hipLaunchKernelGGL((hmr::select_rows_kernel<W>), dim3(static_cast<unsigned>((a.n_tiles + per_block - 1) / per_block)),
                                        dim3(hmr::kBlock), 0, stream, a);
                 } else {
-                    hipLaunchKernelGGL((hmr::pick_kernel<W>), dim3(hmr::grid_of(n)), dim3(hmr::kBlock), 0, stream,
+                    hipLaunchKernelGGL((hmr::pick_kernel<W>), dim3(hmr::grid_of((n + 3) / 4)), dim3(hmr::kBlock), 0, stream,
                                        reinterpret_cast<W *>(hmr::first_of(*out)), reinterpret_cast<const W *>(hmr::first_of(*src)),
                                        static_cast<const void *>(hmr::first_of(*index)), is64, d, n, wrap);
                 }
@@ -769,7 +792,7 @@ hmr_status hmr_gather(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_t
                     else run(hmr::IntTag<65536>{});
                     return;
                 }
-                hipLaunchKernelGGL((hmr::pick_kernel<W>), dim3(hmr::grid_of(n)), dim3(hmr::kBlock), 0, stream,
+                hipLaunchKernelGGL((hmr::pick_kernel<W>), dim3(hmr::grid_of((n + 3) / 4)), dim3(hmr::kBlock), 0, stream,
                                    reinterpret_cast<W *>(hmr::first_of(*out)), reinterpret_cast<const W *>(hmr::first_of(*src)),
                                    static_cast<const void *>(hmr::first_of(*index)), index->dtype == HMR_I64 ? 1 : 0, d, n, int64_t{0});
             });
