@@ -19,18 +19,36 @@ namespace {
 // stride[0] out, [1] the coordinates.
 __global__ void __launch_bounds__(kBlock) positions_kernel(int64_t *out, const void *coord, int is64, Dims d, int64_t n, int64_t size,
                                                            int64_t stride, int first) {
-    for (int64_t p = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; p < n; p += static_cast<int64_t>(gridDim.x) * kBlock) {
-        int64_t rest = p, oo = 0, co = 0;
-        for (int k = 0; k < d.ndim; ++k) {
-            const int64_t q = rest / d.size[k];
-            const int64_t c = rest - q * d.size[k];
-            rest = q;
-            oo += c * d.stride[0][k];
-            co += c * d.stride[1][k];
+    // Four positions per lane, a workgroup apart, every load before the first store; the outermost dimension
+    // needs no division.
+    constexpr int U = 4;
+    for (int64_t base = static_cast<int64_t>(blockIdx.x) * (U * kBlock); base < n; base += static_cast<int64_t>(gridDim.x) * (U * kBlock)) {
+        int64_t oo[U], v[U], before[U];
+        bool valid[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int64_t wanted = base + static_cast<int64_t>(u) * kBlock + threadIdx.x;
+            valid[u] = wanted < n;
+            int64_t rest = valid[u] ? wanted : n - 1, co = 0;
+            oo[u] = 0;
+            for (int k = 0; k < d.ndim; ++k) {
+                int64_t c = rest;
+                if (k + 1 < d.ndim) {
+                    const int64_t q = rest / d.size[k];
+                    c = rest - q * d.size[k];
+                    rest = q;
+                }
+                oo[u] += c * d.stride[0][k];
+                co += c * d.stride[1][k];
+            }
+            v[u] = read_index(coord, is64, co);
+            before[u] = first ? 0 : out[oo[u]];
         }
-        int64_t v = read_index(coord, is64, co);
-        if (v < 0) v += size;
-        out[oo] = (first ? 0 : out[oo]) + v * stride;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (v[u] < 0) v[u] += size;
+            if (valid[u]) out[oo[u]] = before[u] + v[u] * stride;
+        }
     }
 }
 
@@ -289,7 +307,7 @@ hmr_status hmr_index_positions(hmr_context_t ctx, const hmr_tensor_desc *out, co
         const hmr_tensor_desc *const ops[3] = {out, coord, nullptr};
         const hmr::Dims d = hmr::dims_of(*out, ops, -1);
         return hmr::queue_on(ctx, "index_positions", [&](hipStream_t stream) {
-            hipLaunchKernelGGL(hmr::positions_kernel, dim3(hmr::grid_of(n)), dim3(hmr::kBlock), 0, stream,
+            hipLaunchKernelGGL(hmr::positions_kernel, dim3(hmr::grid_of((n + 3) / 4)), dim3(hmr::kBlock), 0, stream,
                                reinterpret_cast<int64_t *>(hmr::first_of(*out)), static_cast<const void *>(hmr::first_of(*coord)),
                                coord->dtype == HMR_I64 ? 1 : 0, d, n, size, stride, first);
             return true;
