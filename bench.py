@@ -12,8 +12,8 @@ The same JSON line carries
   cpu_baseline  the CPU oracle (a port of homura's single-threaded CPU backend) timed on one host
                 core on the same workload;
   ops           achieved GB/s and fraction of the 8 TB/s HBM peak for every op of every BASELINE
-                config (--ops none to skip; cfg = index into BASELINE.json's configs), algorithmic bytes as in
-                BASELINE.md section 3.
+                config (--ops none to skip; cfg = index into BASELINE.json's configs); algorithmic bytes:
+                every input read once and the output written once, broadcast operands at their own size.
 
 usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--ops all|none]
 """
@@ -115,7 +115,8 @@ def main():
         dst.free()
         ctx.close()
 
-    chain_bytes = (4 * N + 2 * H) + (4 * N + 2 * B * S) + 10 * N  # BASELINE.md section 3, promotion fused
+    # x + bias: 2N + 2N + the bias; t * scale: 2N + 2N + the scales; t + residual with the promotion fused: 2N + 4N + 4N.
+    chain_bytes = (4 * N + 2 * H) + (4 * N + 2 * B * S) + 10 * N
     # Untimed: bring the GPU out of its idle clocks before anything is measured (a fresh process starts at
     # low clocks and the first few milliseconds of kernels run up to 15 % slow). The W warm-up steps follow.
     for _ in range(200):
