@@ -2,7 +2,7 @@
 //
 // Replaces the reference's three generic kernels (ref: csrc/elementwise.hip:412-551 and
 // csrc/kernel.hpp:83-103, which index every element of every broadcast with int64 div/mod).
-// Two kernels, picked on the host from the operands' merged dimensions:
+// Four kernels, picked on the host from the operands' merged dimensions:
 //
 //  map_rows_kernel   every operand walks its innermost dimension with stride 1 or 0. A lane owns
 //                    V consecutive elements of a row, V = 16 bytes of the widest operand, so the
@@ -13,9 +13,14 @@
 //                    at all. Stride-0 operands (bias rows, per-row scales, scalars) are read once
 //                    per lane-tile and replicated in registers. Each lane runs U tiles per pass,
 //                    loads first, stores after, to keep >= 64 bytes per operand in flight.
-//  map_any_kernel    anything else (transposed, every-other, overflowing 32 bits ...): one
-//                    element per lane per step, 32-bit multiply-shift indexing when every offset
-//                    fits, int64 otherwise.
+//  map_tiled_kernel, map_tiled16_kernel
+//                    an input (or the output) contiguous along another dimension than the rest: a
+//                    transposition. A tile of the two dimensions goes through LDS so that both sides
+//                    move whole runs; the 16-byte form serves whole aligned tiles of equal-width
+//                    operands, the other one everything else that is long enough to fill a tile.
+//  map_any_kernel    anything else (every-other views, misaligned, overflowing 32 bits ...): an
+//                    element at a time, four of them per lane in flight, 32-bit multiply-shift
+//                    indexing when every offset fits, int64 otherwise.
 //
 // A functor F describes one op:
 //   static constexpr int N;           number of inputs (1..3)
