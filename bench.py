@@ -242,8 +242,13 @@ def per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP
     del sets
     # configs[1]: the three steps.
     t1 = x.add(bias)
-    add(1, "x_bf16 + bias_bf16[4096] (inner broadcast)", 4 * N + 2 * 4096, lambda: x.add(bias))
-    add(1, "t_bf16 * scale_bf16[8,2048,1] (row broadcast)", 4 * N + 2 * 8 * 2048, lambda: t1.mul(scale))
+    add(1, "x_bf16 + bias_bf16[4096] (inner broadcast; same buffers, 268 MB working set)", 4 * N + 2 * 4096, lambda: x.add(bias))
+    add(1, "t_bf16 * scale_bf16[8,2048,1] (row broadcast; same buffers)", 4 * N + 2 * 8 * 2048, lambda: t1.mul(scale))
+    # The same two steps with three input buffers in rotation: nothing of a call's input is left in the cache.
+    xs = [x, x.mul(1.0), x.mul(1.0)]
+    add(1, "x_bf16 + bias_bf16[4096] (HBM-resident, rotating buffers)", 4 * N + 2 * 4096, [lambda t=t: t.add(bias) for t in xs])
+    add(1, "t_bf16 * scale_bf16[8,2048,1] (HBM-resident, rotating buffers)", 4 * N + 2 * 8 * 2048, [lambda t=t: t.mul(scale) for t in xs])
+    del xs
     add(1, "t_bf16 + residual_f32 -> f32 (promotion fused)", 10 * N, lambda: t2.add(residual))
     h.set_fused_promotion(False)
     add(1, "t_bf16 + residual_f32 -> f32 (reference style: cast kernel + add, 2 launches)", 18 * N,
@@ -268,8 +273,16 @@ def per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP
     del xbs
     # configs[3]: permuted bf16 unary; int64 ops.
     p = tensor(from_f64(normal(0x5EED0400, N, 0.0, 2.0), DT.BF16), DT.BF16, [8, 2048, 32, 128], GPU).permute([0, 2, 1, 3])
-    add(3, "silu bf16 [8,2048,32,128].permute(0,2,1,3) -> contiguous", 4 * N, lambda: p.silu())
-    add(3, "gelu(erf) bf16, same view", 4 * N, lambda: p.gelu())
+    add(3, "silu bf16 [8,2048,32,128].permute(0,2,1,3) -> contiguous (same buffers, 268 MB working set)", 4 * N, lambda: p.silu())
+    add(3, "gelu(erf) bf16, same view (same buffers)", 4 * N, lambda: p.gelu())
+    ps = [p, p.contiguous().permute([0, 2, 1, 3]).contiguous().permute([0, 2, 1, 3]),
+          p.contiguous().permute([0, 2, 1, 3]).contiguous().permute([0, 2, 1, 3])]
+    assert ps[1].strides == p.strides
+    add(3, "silu bf16, same view (HBM-resident, rotating buffers)", 4 * N, [lambda t=t: t.silu() for t in ps])
+    add(3, "gelu(erf) bf16, same view (HBM-resident, rotating buffers)", 4 * N, [lambda t=t: t.gelu() for t in ps])
+    pc = p.contiguous()
+    add(3, "silu bf16 on the contiguous copy of the same data (same buffers), for comparison", 4 * N, lambda: pc.silu())
+    del ps, pc
     del p
     w1 = words(0x5EED0401, N)
     w2 = words(0x5EED0402, N)
