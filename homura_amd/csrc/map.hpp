@@ -975,22 +975,30 @@ RowsArgs<F::N + 1> rows_args(const MapCall &c, int variant) {
             for (int k = 0; k < NOPS; ++k) outer[n].stride[k] = c.is_const[k] ? 0 : c.stride[k][src];
         }
         // A transposed pair (a permuted view copied or mapped into a contiguous tensor): the output runs along
-        // dimension 0, an input along dimension 1. Walking 8 steps of dimension 0, then dimension 1, then the rest
-        // of dimension 0 gives a workgroup's 64 rows runs of 8 rows in the output and in that input alike,
-        // instead of 64 rows in one and single rows in the other.
-        constexpr int kTile = 8;  // measured on a [8, 2048, 32, 128] view: 2 to 64 rows tried, 8 is fastest
-        if (n >= 2 && n < kFastDims - 1 && outer[0].size % kTile == 0 && outer[0].size > kTile && outer[1].size >= kTile) {
-            bool transposed = false;
+        // dimension 0, an input along dimension 1. Walking a few steps of dimension 0, then dimension 1, then the
+        // rest of dimension 0 gives a workgroup's rows runs of that many rows in the output and a few rows in
+        // that input, instead of 64 rows in one and single rows in the other. The run is 4 KB of output: measured
+        // on [8, 32, S, D] views of 134 MB with rows of 128 bytes to 2 KB, runs of 4 KB are the fastest or within
+        // 1 % of it for every row width, and take the same time wherever the buffers lie (runs of 2 KB are as fast
+        // for some placements of the output and 3 to 13 % slower for others; 8 KB and more are slower everywhere).
+        bool transposed = false;
+        if (n >= 2 && n < kFastDims - 1 && outer[1].size >= 8) {
             for (int k = 1; k < NOPS && !transposed; ++k) {
                 transposed = !c.is_const[k] && outer[1].stride[k] != 0 && outer[1].stride[k] < outer[0].stride[k] &&
                              outer[0].stride[0] < outer[1].stride[0];
             }
-            if (transposed) {
+        }
+        if (transposed) {
+            const int64_t row_bytes = c.size[last] * static_cast<int64_t>(sizeof(typename F::Out));
+            int64_t run = 4096 / row_bytes;
+            run = run < 4 ? 4 : run > 64 ? 64 : run;
+            while (run >= 4 && (outer[0].size % run != 0 || outer[0].size <= run)) run /= 2;
+            if (run >= 4) {
                 for (int d = n; d > 2; --d) outer[d] = outer[d - 1];
                 outer[2] = outer[0];
-                outer[2].size = outer[0].size / kTile;
-                for (int k = 0; k < NOPS; ++k) outer[2].stride[k] = outer[0].stride[k] * kTile;
-                outer[0].size = kTile;
+                outer[2].size = outer[0].size / run;
+                for (int k = 0; k < NOPS; ++k) outer[2].stride[k] = outer[0].stride[k] * run;
+                outer[0].size = run;
                 ++n;
             }
         }
