@@ -4,6 +4,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <map>
+#include <set>
 #include <mutex>
 #include <utility>
 #include <vector>
@@ -31,7 +32,7 @@ struct DeviceState {
     hmr_context_t ctx = nullptr;
     std::recursive_mutex exec;  // makes one op's kernel submissions atomic
     std::mutex alloc;
-    std::multimap<size_t, void *> cache;  // freed blocks by size, reused in stream order
+    std::set<std::pair<size_t, uintptr_t>> cache;  // freed blocks by size, then address; reused in stream order
 };
 
 std::mutex g_registry;
@@ -67,9 +68,11 @@ void *device_alloc(int index, size_t block) {
     DeviceState &st = device_state(index);
     {
         std::lock_guard<std::mutex> lock(st.alloc);
-        auto it = st.cache.find(block);
-        if (it != st.cache.end()) {
-            void *p = it->second;
+        // Of the cached blocks of this size the one at the lowest address, as the reference's best fit picks
+        // (ref: src/backend/caching.rs:5-6): a loop that frees its result and asks again gets the same block.
+        auto it = st.cache.lower_bound({block, 0});
+        if (it != st.cache.end() && it->first == block) {
+            void *p = reinterpret_cast<void *>(it->second);
             st.cache.erase(it);
             return p;
         }
@@ -82,7 +85,7 @@ void *device_alloc(int index, size_t block) {
             std::lock_guard<std::recursive_mutex> run(st.exec);
             expect(hmr_context_synchronize(st.ctx));
             std::lock_guard<std::mutex> lock(st.alloc);
-            for (auto &kv : st.cache) expect(hmr_free(index, kv.second));
+            for (auto &kv : st.cache) expect(hmr_free(index, reinterpret_cast<void *>(kv.second)));
             st.cache.clear();
         }
         s = hmr_malloc(index, block, &p);
@@ -94,7 +97,7 @@ void *device_alloc(int index, size_t block) {
 void device_release(int index, size_t block, void *p) {
     DeviceState &st = device_state(index);
     std::lock_guard<std::mutex> lock(st.alloc);
-    st.cache.emplace(block, p);
+    st.cache.emplace(block, reinterpret_cast<uintptr_t>(p));
 }
 
 const hcb_backend *g_cpu = nullptr;
@@ -278,7 +281,7 @@ void empty_cache() {
         std::lock_guard<std::recursive_mutex> run(st->exec);
         expect(hmr_context_synchronize(st->ctx));
         std::lock_guard<std::mutex> a(st->alloc);
-        for (auto &b : st->cache) expect(hmr_free(index, b.second));
+        for (auto &b : st->cache) expect(hmr_free(index, reinterpret_cast<void *>(b.second)));
         st->cache.clear();
     }
 }
