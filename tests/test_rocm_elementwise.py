@@ -209,6 +209,32 @@ def test_large_half_tensors_take_the_table_and_get_the_direct_kernels_bits(dtype
     ctx.close()
 
 
+@pytest.mark.parametrize("shape, view", [
+    ([6, 96, 24, 128], ("permute", [0, 2, 1, 3])),     # sizes that are no powers of two: three low dimensions
+    ([4, 512, 32, 64], ("permute", [0, 2, 1, 3])),     # rows of 128 bytes, runs of 32
+    ([2, 64, 32, 512], ("permute", [0, 2, 1, 3])),     # rows of 1 KB, runs of 4
+    ([64, 256, 128], ("permute", [1, 0, 2])),          # no batch dimension
+    ([8, 2048, 1024], ("narrow", 2, 256, 512)),        # rows of a wider buffer, one outer dimension low, one high
+    ([3, 1000, 520], ("narrow", 2, 8, 504)),           # passes that do not keep step: every chunk walks
+    ([5, 72, 24, 128], ("permute", [0, 2, 1, 3])),     # a ragged last pass
+    ([2, 2048, 32, 128], ("permute", [0, 2, 1, 3])),   # more passes than workgroups
+], ids=lambda v: str(v).replace(" ", ""))
+def test_the_table_kernels_walks_over_outer_dimensions(shape, view):
+    """The lookup kernel finds a lane's offsets once when its passes keep step with the outer dimensions and per
+    chunk otherwise; both must read and write the elements the view names. The data is every pattern, repeated."""
+    n = int(np.prod(shape))
+    assert n >= 1 << 20
+    patterns = np.arange(65536, dtype=np.uint16)
+    data = np.resize(patterns * np.uint16(40503) + np.uint16(7), n)   # a permutation of the patterns, repeated
+    small = tensor(patterns, DT.BF16).to(GPU)
+    base = tensor(data, DT.BF16, shape).to(GPU)
+    v = getattr(base, view[0])(*view[1:])
+    for name in ("silu", "erf"):
+        direct = array(getattr(small, name)()).reshape(-1)
+        got = array(getattr(v, name)())
+        np.testing.assert_array_equal(got, direct[array(v)], err_msg=f"{name} {shape} {view}")
+
+
 BINARY_FLOAT = ["add", "sub", "mul", "div", "maximum", "minimum"]
 BINARY_INT = ["add", "sub", "mul", "maximum", "minimum", "pow", "bitwise_and"]
 BINARY_BOOL = ["add", "mul", "maximum", "minimum", "bitwise_and"]
