@@ -236,7 +236,7 @@ def per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP
         a = tensor(uniform(0x5EED0100 + 2 * i, n1, -1.0, 1.0).astype(np.float32), DT.F32, [4096, 4096], GPU)
         b = tensor(uniform(0x5EED0101 + 2 * i, n1, -1.0, 1.0).astype(np.float32), DT.F32, [4096, 4096], GPU)
         sets.append((a, b))
-    add(0, "add f32 [4096,4096] (HBM-resident, rotating buffers)", 12 * n1, [lambda a=a, b=b: a.add(b) for a, b in sets], 40)
+    add(0, "add f32 [4096,4096] (inputs from HBM: four pairs in rotation; the result reuses one block)", 12 * n1, [lambda a=a, b=b: a.add(b) for a, b in sets], 40)
     a0, b0 = sets[0]
     add(0, "add f32 [4096,4096] (same buffers, Infinity-Cache-resident)", 12 * n1, lambda: a0.add(b0), 40)
     del sets
@@ -246,8 +246,13 @@ def per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP
     add(1, "t_bf16 * scale_bf16[8,2048,1] (row broadcast; same buffers)", 4 * N + 2 * 8 * 2048, lambda: t1.mul(scale))
     # The same two steps with three input buffers in rotation: nothing of a call's input is left in the cache.
     xs = [x, x.mul(1.0), x.mul(1.0)]
-    add(1, "x_bf16 + bias_bf16[4096] (HBM-resident, rotating buffers)", 4 * N + 2 * 4096, [lambda t=t: t.add(bias) for t in xs])
-    add(1, "t_bf16 * scale_bf16[8,2048,1] (HBM-resident, rotating buffers)", 4 * N + 2 * 8 * 2048, [lambda t=t: t.mul(scale) for t in xs])
+    add(1, "x_bf16 + bias_bf16[4096] (input from HBM: three buffers in rotation; the result reuses one block)", 4 * N + 2 * 4096, [lambda t=t: t.add(bias) for t in xs])
+    add(1, "t_bf16 * scale_bf16[8,2048,1] (input from HBM: three buffers in rotation; the result reuses one block)", 4 * N + 2 * 8 * 2048, [lambda t=t: t.mul(scale) for t in xs])
+    # And with the results kept in three slots, so that a call's result block is not the previous call's either.
+    kept = [None] * len(xs)
+    add(1, "x_bf16 + bias_bf16[4096] (input and result from HBM: three of each in rotation)", 4 * N + 2 * 4096,
+        [lambda i=i: kept.__setitem__(i, xs[i].add(bias)) for i in range(len(xs))])
+    del kept
     del xs
     add(1, "t_bf16 + residual_f32 -> f32 (promotion fused)", 10 * N, lambda: t2.add(residual))
     h.set_fused_promotion(False)
@@ -269,7 +274,7 @@ def per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP
     add(2, "sum over all elements f32", 4 * N + 4, lambda: xf.sum())
     # 134 MB would fit the 256 MB Infinity Cache: three copies in rotation, so that every call reads from HBM.
     xbs = [xf.to(DT.BF16) for _ in range(3)]
-    add(2, "sum dim=-1 bf16 (HBM-resident, rotating buffers)", 2 * N + 2 * R, [lambda t=t: t.sum_dim(-1, False) for t in xbs])
+    add(2, "sum dim=-1 bf16 (input from HBM: three buffers in rotation; the result reuses one block)", 2 * N + 2 * R, [lambda t=t: t.sum_dim(-1, False) for t in xbs])
     del xbs
     # configs[3]: permuted bf16 unary; int64 ops.
     p = tensor(from_f64(normal(0x5EED0400, N, 0.0, 2.0), DT.BF16), DT.BF16, [8, 2048, 32, 128], GPU).permute([0, 2, 1, 3])
@@ -278,8 +283,12 @@ def per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP
     ps = [p, p.contiguous().permute([0, 2, 1, 3]).contiguous().permute([0, 2, 1, 3]),
           p.contiguous().permute([0, 2, 1, 3]).contiguous().permute([0, 2, 1, 3])]
     assert ps[1].strides == p.strides
-    add(3, "silu bf16, same view (HBM-resident, rotating buffers)", 4 * N, [lambda t=t: t.silu() for t in ps])
-    add(3, "gelu(erf) bf16, same view (HBM-resident, rotating buffers)", 4 * N, [lambda t=t: t.gelu() for t in ps])
+    add(3, "silu bf16, same view (input from HBM: three buffers in rotation; the result reuses one block)", 4 * N, [lambda t=t: t.silu() for t in ps])
+    add(3, "gelu(erf) bf16, same view (input from HBM: three buffers in rotation; the result reuses one block)", 4 * N, [lambda t=t: t.gelu() for t in ps])
+    kept = [None] * len(ps)
+    add(3, "silu bf16, same view (input and result from HBM: three of each in rotation)", 4 * N,
+        [lambda i=i: kept.__setitem__(i, ps[i].silu()) for i in range(len(ps))])
+    del kept
     pc = p.contiguous()
     add(3, "silu bf16 on the contiguous copy of the same data (same buffers), for comparison", 4 * N, lambda: pc.silu())
     del ps, pc

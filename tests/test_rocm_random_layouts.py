@@ -158,3 +158,59 @@ def test_random_views_through_every_kernel_family(seed):
             vc.add_(pc)
             vg.add_(pg)
             assert_bitwise(g, c, f"{what}: updated through the view")
+
+
+@pytest.mark.parametrize("seed", list(range(12)) + [200, 201])
+def test_random_views_through_float_reductions_and_softmax(seed):
+    """The reduction and softmax plans pick their kernels from the merged kept and reduced dimensions of the view
+    (rows, columns, slices cut across workgroups, the general walk): the same random chains of views as above, float
+    data, and the classes of tests/test_rocm_reduce.py as the bar (sums and means within 2 n eps of the sum of
+    magnitudes, variances within 4 n eps v, softmax within its row's class; extremes and their positions bit for bit)."""
+    from tests.support import FLOATS
+    from tests.test_rocm_reduce import EPS, check_softmax, check_sum, f64, finite, folded
+    from tests.support import check_within
+
+    rng = np.random.default_rng(0x5EED1000 + seed)
+    large = seed >= 200
+    for case in range(12 if large else 60):
+        dtype = FLOATS[int(rng.integers(0, len(FLOATS)))]
+        base_shape = random_shape(rng, 3000000, LARGE_SIZES) if large else random_shape(rng, 60000)
+        chain, shape = random_chain(rng, base_shape)
+        if not shape:
+            continue
+        what = f"seed {seed} case {case}: {dtype} {base_shape} {chain}"
+        n = int(np.prod(base_shape))
+        c = finite(dtype, n, 12 if dtype == DT.F16 else 30, 5000 * seed + case).reshape(base_shape)
+        g = c.to(GPU)
+        vc, vg = apply(c, chain), apply(g, chain)
+        wide = vc.to(DT.F64)
+        nd = len(shape)
+        dims = sorted(int(d) for d in rng.choice(nd, int(rng.integers(1, nd + 1)), replace=False))
+        keep = bool(rng.integers(0, 2))
+        want = vc.sum_dim(dims, keep)
+        count = folded(vc, want)
+        abs_sum = wide.abs().sum_dim(dims, keep)
+        check_sum(vg.sum_dim(dims, keep), want, abs_sum, count, False, f"{what}: sum over {dims}")
+        check_sum(vg.mean_dim(dims, keep), vc.mean_dim(dims, keep), abs_sum, count, True, f"{what}: mean over {dims}")
+        correction = int(rng.integers(0, 2))
+        v = f64(wide.var_dim(dims, correction, keep))
+        # The class of the reduce tests, 4 n eps v, plus what the rounding of the mean alone can move a variance by,
+        # (n eps)^2 times the mean square: nothing next to the class unless the reduced elements are all but equal
+        # (an expanded dimension reduced: v is 0 exactly and the CPU's own result is that rounding).
+        mean_square = f64(wide.mul(wide).mean_dim(dims, keep))
+        with np.errstate(all="ignore"):
+            delta = np.nan_to_num(4.0 * count * EPS * v + 4.0 * (count * EPS) ** 2 * mean_square, nan=0.0, posinf=0.0)
+        check_within(vg.var_dim(dims, correction, keep), vc.var_dim(dims, correction, keep), extra=delta,
+                     what=f"{what}: var over {dims} correction {correction}")
+        d = int(rng.integers(0, nd))
+        (gv, gi), (cv, ci) = vg.max_dim(d, keep), vc.max_dim(d, keep)
+        assert_bitwise(gv, cv, f"{what}: max along {d}")
+        assert_bitwise(gi, ci, f"{what}: positions of the max along {d}")
+        # Softmax on data of a few binades, as the reduce tests use (larger spreads make every row one-hot).
+        sc = finite(dtype, n, 3, 7000 * seed + case).reshape(base_shape)
+        sg = sc.to(GPU)
+        svc, svg = apply(sc, chain), apply(sg, chain)
+        log = bool(rng.integers(0, 2))
+        want = svc.log_softmax(d) if log else svc.softmax(d)
+        got = svg.log_softmax(d) if log else svg.softmax(d)
+        check_softmax(got, want, svc.to(DT.F64), d, log, f"{what}: {'log_' if log else ''}softmax along {d}")

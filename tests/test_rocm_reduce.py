@@ -261,6 +261,30 @@ def test_softmax_and_log_softmax_stay_within_their_class():
             check_softmax(xt.to(GPU).softmax(0), xt.softmax(0), xt.to(DT.F64), 0, False, f"{dtype} strided rows of {n}")
 
 
+def test_log_softmax_of_rows_that_one_element_dominates():
+    """log_softmax of the largest element is -log(1 + s), s the sum of the other exponentials: for a small s the
+    result is about -s, and the class asks for one ulp of THAT (ref: tests/rocm_reduce.rs:216-220), so s must keep
+    its own relative accuracy and not that of 1 + s. Rows of every plan, one element 6 to 30 above the rest, the
+    largest in several positions; softmax of the same rows rides along."""
+    for dtype in FLOATS:
+        for n in (8, 16, 64, 100, 513, 2048, 4096, 32000, 70000):
+            for lift in (6.0, 10.0, 15.5, 22.0, 30.0):
+                rows = 6
+                base = to_f64(array(finite(dtype, rows * n, 1, 900 + n)), dtype).reshape(rows, n)
+                for r in range(rows):
+                    base[r, (r * 7919) % n] = lift + 0.25 * r
+                if n >= 64:
+                    base[rows - 1, n - 1] = base[rows - 1].max()    # the maximum twice in the last row
+                x = tensor(from_f64(base.reshape(-1), dtype), dtype, [rows, n])
+                for log in (True, False):
+                    c = x.log_softmax(1) if log else x.softmax(1)
+                    g = x.to(GPU).log_softmax(1) if log else x.to(GPU).softmax(1)
+                    check_softmax(g, c, x.to(DT.F64), 1, log, f"{dtype} rows of {n}, one element {lift} above, log {log}")
+            # ... and strided (along dimension 0 of the transpose): the walking kernel.
+            xt = x.transpose(0, 1)
+            check_softmax(xt.to(GPU).log_softmax(0), xt.log_softmax(0), xt.to(DT.F64), 0, True, f"{dtype} strided rows of {n}")
+
+
 def test_softmax_extreme_rows_match_the_cpu():
     """ref: tests/rocm_reduce.rs:615-653; plus the KAT of ref: tests/m0_boundaries.rs:468-480."""
     inf, nan = math.inf, math.nan
