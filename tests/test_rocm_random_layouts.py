@@ -214,3 +214,70 @@ def test_random_views_through_float_reductions_and_softmax(seed):
         want = svc.log_softmax(d) if log else svc.softmax(d)
         got = svg.log_softmax(d) if log else svg.softmax(d)
         check_softmax(got, want, svc.to(DT.F64), d, log, f"{what}: {'log_' if log else ''}softmax along {d}")
+
+
+def positions(rng, count, below, dtype, shape):
+    picks = rng.integers(0, below, count).astype(np.int64 if dtype == DT.I64 else np.int32)
+    return tensor(picks, dtype, shape)
+
+
+@pytest.mark.parametrize("seed", list(range(16)) + [300, 301])
+def test_random_views_through_the_families_next_to_the_path(seed):
+    """flip, triu / tril, the fused optimizer steps, addr, exclusive_cumprod, masked_fill and the index family
+    (index_select, gather, scatter_add, index_add) take their operands as views too, and each picks its kernel from
+    the layout it finds (tiles of rows, lines staged in LDS, the element-wise walk): the same random chains of views,
+    and the CPU's bits."""
+    from tests.support import FLOATS
+
+    rng = np.random.default_rng(0x5EED2000 + seed)
+    every = [DT.F32, DT.BF16, DT.I64, DT.U8, DT.F16, DT.I32, DT.F64, DT.Bool, DT.I8, DT.I16]
+    large = seed >= 300
+    for case in range(10 if large else 80):
+        dtype = every[int(rng.integers(0, len(every)))]
+        base_shape = random_shape(rng, 2000000, LARGE_SIZES) if large else random_shape(rng, 50000)
+        chain, shape = random_chain(rng, base_shape)
+        if not shape:
+            continue
+        what = f"seed {seed} case {case}: {dtype} {base_shape} {chain}"
+        (c, g) = pair(dtype, base_shape, 3000 * seed + case)
+        vc, vg = apply(c, chain), apply(g, chain)
+        nd = len(shape)
+        d = int(rng.integers(0, nd))
+        dims = sorted(int(x) for x in rng.choice(nd, int(rng.integers(1, nd + 1)), replace=False))
+        assert_bitwise(vg.flip(dims), vc.flip(dims), f"{what}: flip {dims}")
+        if nd >= 2:
+            k = int(rng.integers(-3, 4))
+            assert_bitwise(vg.triu(k), vc.triu(k), f"{what}: triu {k}")
+            assert_bitwise(vg.tril(k), vc.tril(k), f"{what}: tril {k}")
+        pc, pg = pair(dtype, shape, 81 + case)
+        mask_c = pc.greater(vc) if dtype != DT.Bool else pc
+        fill = True if dtype == DT.Bool else 3
+        assert_bitwise(vg.masked_fill(mask_c.to(GPU), fill), vc.masked_fill(mask_c, fill), f"{what}: masked_fill")
+        # The index family along d.
+        itype = DT.I64 if rng.integers(0, 2) else DT.I32
+        count = int(rng.integers(1, 2 * shape[d] + 2))
+        idx = positions(rng, count, shape[d], itype, [count])
+        assert_bitwise(vg.index_select(d, idx.to(GPU)), vc.index_select(d, idx), f"{what}: index_select along {d}")
+        sshape = list(shape)
+        sshape[d] = count
+        sc, sg = pair(dtype, sshape, 82 + case)
+        assert_bitwise(vg.index_add(d, idx.to(GPU), sg), vc.index_add(d, idx, sc), f"{what}: index_add along {d}")
+        ishape = [max(1, n - int(rng.integers(0, 2))) for n in shape]
+        ishape[d] = count
+        picks = positions(rng, int(np.prod(ishape)), shape[d], itype, ishape)
+        assert_bitwise(vg.gather(d, picks.to(GPU)), vc.gather(d, picks), f"{what}: gather along {d}")
+        assert_bitwise(vg.scatter_add(d, picks.to(GPU), sg), vc.scatter_add(d, picks, sc), f"{what}: scatter_add along {d}")
+        if dtype in FLOATS:
+            qc, qg = pair(dtype, shape, 83 + case)
+            v = float(rng.choice([0.3, -0.7, 1.0 / 3.0, 2.0]))
+            assert_bitwise(h.scaled_add(vg, pg, v), h.scaled_add(vc, pc, v), f"{what}: scaled_add {v}")
+            assert_bitwise(h.lerp_step(vg, pg, v), h.lerp_step(vc, pc, v), f"{what}: lerp step {v}")
+            assert_bitwise(h.addcmul_step(vg, pg, qg, v), h.addcmul_step(vc, pc, qc, v), f"{what}: addcmul step {v}")
+            assert_bitwise(h.addcdiv_step(pg, qg, vg, v), h.addcdiv_step(pc, qc, vc, v), f"{what}: addcdiv step {v}")
+            reverse = bool(rng.integers(0, 2))
+            assert_bitwise(h.exclusive_cumprod(vg, d, reverse), h.exclusive_cumprod(vc, d, reverse),
+                           f"{what}: exclusive_cumprod along {d} reverse {reverse}")
+        if nd == 2 and dtype != DT.Bool:
+            (ac, ag), (bc, bg) = pair(dtype, [shape[0]], 84 + case), pair(dtype, [shape[1]], 85 + case)
+            beta, alpha = (0.5, -1.5) if dtype in FLOATS else (2, -3)
+            assert_bitwise(vg.addr(ag, bg, beta, alpha), vc.addr(ac, bc, beta, alpha), f"{what}: addr")
