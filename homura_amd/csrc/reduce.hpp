@@ -221,8 +221,9 @@ struct DeviationFold {
 // (column reductions). A lane keeps sums of (x - K) and (x - K)^2 about its first element K, which
 // is as stable as the two-pass form unless K lies many standard deviations from the mean; lanes,
 // waves and slices then merge (count, mean, M2) triples with Chan's update, all in f64. The
-// result differs from the CPU's two-pass f64 value by rounding only (a few f64 ulps), far below
-// one ulp of any output dtype.
+// result differs from the CPU's two-pass f64 value by rounding only (a few f64 ulps, a few times n of
+// them when K is an outlier of its column), far below one ulp of an f16, bf16 or f32 output; f64
+// columns take the two-pass form.
 struct Moments {
     double n, mean, m2;
 };
@@ -558,7 +559,7 @@ struct ColState<MomentsFold<T>> {
         const double n = static_cast<double>(count);
         const double mean_shift = s1 * count_reciprocal(n);
         const double m2 = s2 - s1 * mean_shift;
-        return Moments{n, k + mean_shift, m2 > 0.0 ? m2 : 0.0};
+        return Moments{n, k + mean_shift, m2 < 0.0 ? 0.0 : m2};  // a NaN stays one
     }
 };
 

@@ -27,10 +27,6 @@ static int var_row_tiles(const ReducePlan &plan, int elem) {
     return per <= 4 ? 4 : (per <= 8 ? 8 : (per <= 16 ? 16 : 0));
 }
 
-bool var_is_single_pass(const ReducePlan &plan) {
-    return plan.kind == ReduceKind::Cols || (plan.kind == ReduceKind::Rows && plan.splits == 1);
-}
-
 bool launch_var_single_pass(int dtype, const ReducePlan &plan, void *partials, void *out, double divisor,
                             bool take_sqrt, hipStream_t stream) {
     if (plan.args.nred == 0) return false;
@@ -39,6 +35,10 @@ bool launch_var_single_pass(int dtype, const ReducePlan &plan, void *partials, v
         using T = typename decltype(t)::type;
         VarSink<T> sink{static_cast<T *>(out), divisor, take_sqrt};
         if (plan.kind == ReduceKind::Cols) {
+            // The shifted one-pass sums lose about a factor n when a column's first element lies far from its
+            // mean. In f64 arithmetic that is nothing next to an ulp of an f16, bf16 or f32 result; an f64
+            // result is held to 4 n eps of the variance itself, so f64 columns take the two passes.
+            if constexpr (std::is_same_v<T, double>) return;
             launch_reduce(plan, partials, MomentsFold<T>{}, sink, stream);
             done = true;
             return;

@@ -120,7 +120,6 @@ bool launch_extreme_reduce(bool is_max, int dtype, const ReducePlan &plan, void 
 // pass over memory); false when the two-pass form below has to run.
 bool launch_var_single_pass(int dtype, const ReducePlan &plan, void *partials, void *out, double divisor,
                             bool take_sqrt, hipStream_t stream);
-bool var_is_single_pass(const ReducePlan &plan);
 // The two passes of the variance: means (f64) then squared deviations.
 bool launch_mean_pass(int dtype, const ReducePlan &plan, void *partials, double *means, hipStream_t stream);
 bool launch_deviation_pass(int dtype, const ReducePlan &plan, void *partials, const double *means, void *out,

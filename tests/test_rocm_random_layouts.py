@@ -160,6 +160,23 @@ def test_random_views_through_every_kernel_family(seed):
             assert_bitwise(g, c, f"{what}: updated through the view")
 
 
+def sprinkle(rng, t, dtype, shape):
+    """A few NaNs, infinities of both signs and zeros at random places of t: some lines get one, most stay clean."""
+    from tests.support import from_f64, to_f64
+
+    flat = to_f64(_storage(t), dtype).copy()
+    count = max(1, flat.size // 200)
+    where = rng.integers(0, flat.size, count)
+    flat[where] = rng.choice([np.nan, np.inf, -np.inf, 0.0, -0.0], count)
+    return tensor(from_f64(flat, dtype), dtype, shape)
+
+
+def _storage(t):
+    from tests.support import array
+
+    return array(t).reshape(-1).copy()
+
+
 @pytest.mark.parametrize("seed", list(range(12)) + [200, 201])
 def test_random_views_through_float_reductions_and_softmax(seed):
     """The reduction and softmax plans pick their kernels from the merged kept and reduced dimensions of the view
@@ -181,6 +198,9 @@ def test_random_views_through_float_reductions_and_softmax(seed):
         what = f"seed {seed} case {case}: {dtype} {base_shape} {chain}"
         n = int(np.prod(base_shape))
         c = finite(dtype, n, 12 if dtype == DT.F16 else 30, 5000 * seed + case).reshape(base_shape)
+        sprinkled = case % 3 == 2
+        if sprinkled:
+            c = sprinkle(rng, c, dtype, base_shape)
         g = c.to(GPU)
         vc, vg = apply(c, chain), apply(g, chain)
         wide = vc.to(DT.F64)
@@ -208,6 +228,8 @@ def test_random_views_through_float_reductions_and_softmax(seed):
         assert_bitwise(gi, ci, f"{what}: positions of the max along {d}")
         # Softmax on data of a few binades, as the reduce tests use (larger spreads make every row one-hot).
         sc = finite(dtype, n, 3, 7000 * seed + case).reshape(base_shape)
+        if sprinkled:
+            sc = sprinkle(rng, sc, dtype, base_shape)
         sg = sc.to(GPU)
         svc, svg = apply(sc, chain), apply(sg, chain)
         log = bool(rng.integers(0, 2))

@@ -285,6 +285,49 @@ def test_log_softmax_of_rows_that_one_element_dominates():
             check_softmax(xt.to(GPU).log_softmax(0), xt.log_softmax(0), xt.to(DT.F64), 0, True, f"{dtype} strided rows of {n}")
 
 
+def test_variances_down_columns_with_special_values():
+    """A column that holds a NaN or an infinity has the variance NaN, whichever row holds it and whatever the
+    others are; its neighbours are not touched. Shapes of every column plan (one slice, slices cut across
+    workgroups), var and std, both corrections."""
+    for dtype in FLOATS:
+        for rows, cols in ((8, 1152), (64, 4096), (1000, 520), (4096, 256), (3, 8)):
+            base = to_f64(array(finite(dtype, rows * cols, 4, 800 + rows)), dtype).reshape(rows, cols)
+            specials = [np.nan, np.inf, -np.inf]
+            for k, col in enumerate(range(0, cols, max(1, cols // 23))):
+                row = (0, rows - 1, rows // 2, (7 * k) % rows)[k % 4]
+                base[row, col] = specials[k % 3]
+                if k % 5 == 4:
+                    base[:, col] = np.inf          # every row the same infinity
+            x = tensor(from_f64(base.reshape(-1), dtype), dtype, [rows, cols])
+            g = x.to(GPU)
+            for correction in (0, 1):
+                c = x.var_dim(0, correction, False)
+                v64 = f64(x.to(DT.F64).var_dim(0, correction, False))
+                with np.errstate(all="ignore"):
+                    delta = np.nan_to_num(4.0 * rows * EPS * v64, nan=0.0, posinf=0.0)
+                check_within(g.var_dim(0, correction, False), c, extra=delta, what=f"{dtype} var [{rows}, {cols}] down columns")
+                assert np.isnan(f64(c)).sum() >= min(20, cols // 2)
+                with np.errstate(all="ignore"):
+                    sd = np.where(v64 > 0, np.minimum(delta / np.sqrt(np.where(v64 > 0, v64, 1.0)), np.sqrt(delta)), np.sqrt(delta))
+                check_within(g.std_dim(0, correction, False), x.std_dim(0, correction, False), extra=np.nan_to_num(sd),
+                             what=f"{dtype} std [{rows}, {cols}] down columns")
+
+
+def test_variances_down_columns_whose_first_row_is_an_outlier():
+    """The class 4 n eps v holds when a column's first element lies far from the column's mean (sums about the
+    first element would lose about a factor n there), in f64 as in the narrower dtypes."""
+    for dtype in FLOATS:
+        for rows, cols in ((63, 508), (512, 1024), (4096, 256)):
+            base = to_f64(array(finite(dtype, rows * cols, 1, 850 + rows)), dtype).reshape(rows, cols)
+            base[0, :] *= 2.0 ** (9 if dtype == DT.F16 else 30)
+            base[1:, ::3] += 100.0                       # and a mean far from zero in every third column
+            x = tensor(from_f64(base.reshape(-1), dtype), dtype, [rows, cols])
+            v64 = f64(x.to(DT.F64).var_dim(0, 1, False))
+            delta = 4.0 * rows * EPS * v64
+            check_within(x.to(GPU).var_dim(0, 1, False), x.var_dim(0, 1, False), extra=delta,
+                         what=f"{dtype} var [{rows}, {cols}] down columns, first row an outlier")
+
+
 def test_softmax_extreme_rows_match_the_cpu():
     """ref: tests/rocm_reduce.rs:615-653; plus the KAT of ref: tests/m0_boundaries.rs:468-480."""
     inf, nan = math.inf, math.nan
