@@ -3,7 +3,9 @@
 // to the computation type (f32 for F16/BF16/F32, f64 for F64), compute, and round once; integer
 // ops wrap.
 //
-// Transcendental accuracy. The CPU calls the host libm in the computation type. Here:
+// Transcendental accuracy. The CPU calls the host libm in the computation type. Here exp of an f32
+// value is the host library's expf restated (expf_like_libm.hpp: the same bits for every input), and
+// for the other functions:
 //   F32 tensors   evaluate the function in f64 and round to f32. That is the correctly rounded
 //                 f32 value except within ~2^-29 of a rounding boundary, which is also what a good
 //                 libm returns, so results agree to the last bit nearly everywhere and to 1 ulp
@@ -18,6 +20,7 @@
 #pragma once
 
 #include "elem.hpp"
+#include "expf_like_libm.hpp"
 #include "map.hpp"
 
 namespace hmr {
@@ -37,8 +40,6 @@ struct Eval<double> {
     using E = double;
 };
 
-__device__ __forceinline__ float m_exp(float x) { return expf(x); }
-__device__ __forceinline__ double m_exp(double x) { return exp(x); }
 __device__ __forceinline__ float m_log(float x) { return logf(x); }
 __device__ __forceinline__ double m_log(double x) { return log(x); }
 __device__ __forceinline__ float m_log1p(float x) { return log1pf(x); }
@@ -63,13 +64,21 @@ __device__ __forceinline__ double m_abs(double x) { return fabs(x); }
         using E = typename Eval<T>::E;                                 \
         return static_cast<typename Comp<T>::C>(FN(static_cast<E>(x))); \
     }
-HMR_EVAL1(e_exp, m_exp)
 HMR_EVAL1(e_log, m_log)
 HMR_EVAL1(e_log1p, m_log1p)
 HMR_EVAL1(e_sin, m_sin)
 HMR_EVAL1(e_cos, m_cos)
 HMR_EVAL1(e_tanh, m_tanh)
 #undef HMR_EVAL1
+
+// exp in the computation type: for f32 (F16, BF16 and F32 tensors) the host library's own expf, bit for
+// bit (expf_like_libm.hpp), because sigmoid, silu and log_sigmoid divide by or take the logarithm of
+// 1 + e and turn one ulp of e into up to four of their result; for f64 the device library's exp.
+template <class T>
+__device__ __forceinline__ typename Comp<T>::C e_exp(typename Comp<T>::C x) {
+    if constexpr (std::is_same_v<typename Comp<T>::C, float>) return expf_like_libm<true>(x);
+    else return exp(x);
+}
 
 template <class T>
 __device__ __forceinline__ typename Comp<T>::C e_pow(typename Comp<T>::C x, typename Comp<T>::C y) {

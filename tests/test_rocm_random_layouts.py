@@ -138,6 +138,29 @@ def test_random_views_through_every_kernel_family(seed):
             assert_bitwise(vg.greater(pg), vc.greater(pc), f"{what}: >")
             mask_c = vc.greater(pc)
             assert_bitwise(h.where_(mask_c.to(GPU), vg, pg), h.where_(mask_c, vc, pc), f"{what}: where")
+        # One more binary op, one exact unary op and (floats) one transcendental, drawn from the whole lists.
+        from tests.test_rocm_elementwise import COMPARE, IEEE_UNARY, ONE_ULP, ops_for
+        from tests.support import FLOATS, check_within
+
+        name = str(rng.choice(ops_for(dtype) + COMPARE + ["logical_and", "logical_or"]))
+        assert_bitwise(getattr(vg, name)(pg), getattr(vc, name)(pc), f"{what}: {name} with partner {choice}")
+        name = str(rng.choice([u for u in IEEE_UNARY if not (dtype == DT.Bool and u in ("neg", "abs", "relu"))]))
+        assert_bitwise(getattr(vg, name)(), getattr(vc, name)(), f"{what}: {name}")
+        if dtype in (DT.F32, DT.BF16, DT.F16):
+            name = str(rng.choice(sorted(ONE_ULP)))
+            check_within(getattr(vg, name)(), getattr(vc, name)(), extra=0.0, max_ulp=1, what=f"{what}: {name}")
+        # A partner of another dtype: the result type and the converted operands must be the CPU's.
+        if shape:
+            qc, qg = pair(other, shape, 90 + case)
+            name = str(rng.choice(["add", "mul", "sub", "maximum", "greater", "equal"]))
+            try:
+                want = getattr(vc, name)(qc)
+            except Exception as refusal:            # e.g. bool - bool: the GPU must refuse in the same words
+                with pytest.raises(type(refusal)) as got:
+                    getattr(vg, name)(qg)
+                assert str(got.value) == str(refusal), f"{what}: {name} with a {other} partner"
+            else:
+                assert_bitwise(getattr(vg, name)(qg), want, f"{what}: {name} with a {other} partner")
         if dtype in (DT.I64, DT.I32, DT.U8) and shape:
             d = int(rng.integers(0, len(shape)))
             assert_bitwise(vg.sum_dim([d], False), vc.sum_dim([d], False), f"{what}: sum along {d}")
