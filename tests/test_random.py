@@ -355,3 +355,53 @@ def test_sampling_through_the_c_abi_at_odd_offsets_and_its_errors():
         assert out.download(np.int64, 2 * blocks)[:len(kept)].tolist() == kept
     finally:
         ctx.close()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", range(4))
+def test_random_sizes_and_ranges_follow_the_cpu(seed):
+    """Sizes, ranges and dtypes drawn from a seeded generator (the lists above are fixed): uniform and integer
+    samples have the CPU's bits, normal samples stay within their bound, and the generator has advanced by the same
+    number of blocks after every call."""
+    rng = np.random.default_rng(0x5EED3000 + seed)
+    for case in range(40):
+        n = int(np.exp(rng.uniform(0.0, np.log(300000.0))))
+        shape = [n] if rng.integers(0, 2) else [int(rng.integers(1, 8)), max(1, n // 7)]
+        count = int(np.prod(shape))
+        s = int(rng.integers(0, 1 << 40))
+        kind = int(rng.integers(0, 3))
+        if kind == 0:
+            dtype = FLOATS[int(rng.integers(0, len(FLOATS)))]
+            lo = float(rng.choice([0.0, -1.0, 1.0, -3.5, 1e-3, 100.0])) * float(rng.choice([1.0, 16.0, 1e-2]))
+            hi = lo + float(rng.choice([1.0, 0.125, 2.0 ** -6, 37.0, 1000.0]))
+            what = f"seed {seed} case {case}: uniform {dtype} {shape} [{lo}, {hi})"
+            g, c = both(s, lambda d: h.uniform(shape, lo, hi, dtype, d))
+            assert_bitwise(g, c, what)
+        elif kind == 1:
+            dtype = [DT.I64, DT.I32, DT.I16, DT.U8, DT.F32, DT.F64][int(rng.integers(0, 6))]
+            span = int(rng.choice([2, 3, 7, 11, 100, 255]))
+            low = 0 if dtype == DT.U8 else int(rng.choice([0, -5, -100, 17]))
+            if dtype == DT.I64 and rng.integers(0, 3) == 0:
+                low, span = int(rng.choice([I64_MIN, -(1 << 62), 0])), int(rng.choice([(1 << 62) + 12345, (1 << 63) - 1, 1 << 40]))
+            high = min(low + span, I64_MAX) if dtype == DT.I64 else min(low + span, 255 if dtype == DT.U8 else low + span)
+            what = f"seed {seed} case {case}: randint {dtype} {shape} [{low}, {high})"
+            g, c = both(s, lambda d: h.randint(low, high, shape, dtype, d))
+            assert_bitwise(g, c, what)
+        else:
+            dtype = FLOATS[int(rng.integers(0, len(FLOATS)))]
+            mean, std = float(rng.choice([0.0, 3.0, -250.0, 1e-2])), float(rng.choice([1.0, 0.5, 10.0, 1e-3]))
+            what = f"seed {seed} case {case}: normal {dtype} {shape} ({mean}, {std})"
+            g, c = both(s, lambda d: h.normal(shape, mean, std, dtype, d))
+            check_within(g.reshape([count]), c.reshape([count]), extra=NORMAL_K * NORMAL_U * normal_sizes(s, count, mean, std), what=what)
+
+        def after(d, kind=kind, dtype=dtype):
+            if kind == 0:
+                h.uniform(shape, lo, hi, dtype, d)
+            elif kind == 1:
+                h.randint(low, high, shape, dtype, d)
+            else:
+                h.normal(shape, mean, std, dtype, d)
+            return h.rand([3], DT.F64, "cpu").to(GPU)
+
+        g, c = both(s, after)
+        assert_bitwise(g, c.to("cpu"), what + ": the generator afterwards")
