@@ -431,3 +431,95 @@ def test_masked_reads_and_empty_cache_from_two_threads_do_not_deadlock():
     worker.join(timeout=60)
     assert not worker.is_alive(), "x[mask] and empty_cache wait for each other"
     assert not failures, failures
+
+
+def random_indices(rng, shape):
+    """A list of None / integer arrays / bool masks for a tensor of `shape`, as numpy arrays: integer tensors of one
+    broadcast shape with repeats and negatives, or one mask over one or two dimensions with scalar indices beside."""
+    nd = len(shape)
+    out = []
+    if rng.integers(0, 3) == 0 and nd >= 1:
+        # one mask, placed at a random dimension
+        span = int(rng.integers(1, min(2, nd) + 1))
+        at = int(rng.integers(0, nd - span + 1))
+        density = float(rng.choice([0.0, 0.05, 0.5, 0.95, 1.0]))
+        m = rng.random(shape[at:at + span]) < density
+        d = 0
+        while d < nd:
+            if d == at:
+                out.append(m)
+                d += span
+            else:
+                pick = rng.integers(0, 3) == 0
+                out.append(np.array(int(rng.integers(-shape[d], shape[d]))) if pick else None)
+                d += 1
+    else:
+        bshape = [int(rng.choice([1, 2, 3, 17, 300])) for _ in range(int(rng.integers(0, 3)))]
+        some = False
+        for d in range(nd):
+            if rng.integers(0, 2) == 0 and not (d == nd - 1 and not some):
+                out.append(None)
+                continue
+            some = True
+            ishape = [n if rng.integers(0, 4) else 1 for n in bshape]
+            out.append(rng.integers(-shape[d], shape[d], ishape).astype(np.int64))
+    while out and out[-1] is None:
+        out.pop()
+    return out
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", range(10))
+def test_random_index_expressions_match_the_cpu(seed):
+    """Index expressions drawn from a seeded generator over tensors of random shapes and layouts: reading, writing
+    (the last of repeated positions wins) and accumulating (added in the CPU's order), with the indices on the GPU."""
+    rng = np.random.default_rng(0x5EED4000 + seed)
+    every = [DT.F32, DT.BF16, DT.I64, DT.U8, DT.F64, DT.Bool, DT.F16, DT.I32]
+    sizes = [1, 2, 3, 5, 8, 17, 64, 130]
+    for case in range(60):
+        dtype = every[int(rng.integers(0, len(every)))]
+        shape = [int(rng.choice(sizes)) for _ in range(int(rng.integers(1, 5)))]
+        if int(np.prod(shape)) > 200000:
+            continue
+        indices = random_indices(rng, shape)
+        if not any(i is not None for i in indices):
+            continue
+        layouts = operand_layouts(dtype, shape, 9000 * seed + case)
+        sname, cpu, gpu = layouts[int(rng.integers(0, len(layouts)))]
+        what = f"seed {seed} case {case}: {dtype} {shape} {sname} " + str([None if i is None else (str(i.dtype), i.shape) for i in indices])
+        itype = DT.I64 if rng.integers(0, 2) else DT.I32
+        ci = [as_index(i, "cpu", itype) for i in indices]
+        gi = [as_index(i, GPU, itype) for i in indices]
+        want = cpu.index_tensors(ci)
+        assert_same(gpu.index_tensors(gi), want, f"{what}: read")
+        n = int(np.prod(want.shape))
+        v = tensor(values(dtype, n, 9500 + case), dtype, list(want.shape))
+        assert_same(gpu.index_put_tensors(gi, v.to(GPU), False), cpu.index_put_tensors(ci, v, False), f"{what}: index_put")
+        assert_bitwise(gpu.index_put_tensors(gi, v.to(GPU), True), cpu.index_put_tensors(ci, v, True), f"{what}: accumulate")
+        if n > 0 and len(want.shape) >= 1:
+            # a value that broadcasts: the result's last dimension alone
+            tail = tensor(values(dtype, want.shape[-1], 9600 + case), dtype, [want.shape[-1]])
+            assert_same(gpu.index_put_tensors(gi, tail.to(GPU), False), cpu.index_put_tensors(ci, tail, False), f"{what}: broadcast value")
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_random_index_expressions_follow_numpy(seed):
+    """The same generator on the CPU against numpy's advanced indexing: reading, and assignment where no position
+    repeats (numpy leaves the winner of repeated positions open, the reference does not)."""
+    rng = np.random.default_rng(0x5EED4000 + seed)
+    sizes = [1, 2, 3, 5, 8, 17, 64, 130]
+    for case in range(60):
+        dtype = [DT.F32, DT.I64, DT.U8, DT.F64][int(rng.integers(0, 4))]
+        shape = [int(rng.choice(sizes)) for _ in range(int(rng.integers(1, 5)))]
+        if int(np.prod(shape)) > 200000:
+            continue
+        indices = random_indices(rng, shape)
+        if not any(i is not None for i in indices):
+            continue
+        x = values(dtype, int(np.prod(shape)), 9000 * seed + case).reshape(shape)
+        t = tensor(x, dtype, shape)
+        key = tuple(slice(None) if i is None else i for i in indices)
+        want = x[key]
+        got = t.index_tensors([as_index(i, "cpu") for i in indices])
+        what = f"seed {seed} case {case}: {dtype} {shape} " + str([None if i is None else (str(i.dtype), i.shape) for i in indices])
+        assert same(array(got), want), what
