@@ -264,7 +264,10 @@ struct MomentsFold {
         const double n = a.n + b.n;
         const double delta = b.mean - a.mean;
         const double wb = b.n * count_reciprocal(n);
-        return Acc{n, a.mean + delta * wb, a.m2 + b.m2 + delta * delta * (a.n * wb)};
+        // An infinite mean on either side makes the merged mean infinite, and the deviation of an infinite
+        // element from it is inf - inf: the CPU's sum of squares is NaN there, while delta^2 alone would say inf.
+        const double poison = delta - delta;  // 0, or NaN when delta is not finite
+        return Acc{n, a.mean + delta * wb, a.m2 + b.m2 + delta * delta * (a.n * wb) + poison};
     }
 };
 
@@ -548,7 +551,7 @@ struct ColState<MomentsFold<T>> {
     __device__ __forceinline__ void first(const Op &, T x, int32_t, NoCtx) {
         k = Conv<T>::to_f64(x);
         s1 = 0.0;
-        s2 = 0.0;
+        s2 = k - k;  // 0, or NaN when the element is an infinity or a NaN: its deviation from itself, as the CPU has it
     }
     __device__ __forceinline__ void next(const Op &, T x, int32_t, NoCtx) {
         const double d = Conv<T>::to_f64(x) - k;

@@ -290,7 +290,7 @@ def test_variances_down_columns_with_special_values():
     others are; its neighbours are not touched. Shapes of every column plan (one slice, slices cut across
     workgroups), var and std, both corrections."""
     for dtype in FLOATS:
-        for rows, cols in ((8, 1152), (64, 4096), (1000, 520), (4096, 256), (3, 8)):
+        for rows, cols in ((8, 1152), (64, 4096), (1000, 520), (4096, 256), (3, 8), (2, 4096), (1, 520)):
             base = to_f64(array(finite(dtype, rows * cols, 4, 800 + rows)), dtype).reshape(rows, cols)
             specials = [np.nan, np.inf, -np.inf]
             for k, col in enumerate(range(0, cols, max(1, cols // 23))):
@@ -307,6 +307,11 @@ def test_variances_down_columns_with_special_values():
                     delta = np.nan_to_num(4.0 * rows * EPS * v64, nan=0.0, posinf=0.0)
                 check_within(g.var_dim(0, correction, False), c, extra=delta, what=f"{dtype} var [{rows}, {cols}] down columns")
                 assert np.isnan(f64(c)).sum() >= min(20, cols // 2)
+                if rows == 2:   # the same two rows as a middle dimension: [cols / 128, 2, 128] over dimension 1
+                    x3, g3 = x.transpose(0, 1).reshape([cols // 128, 128, 2]).transpose(1, 2), None
+                    x3 = x3.contiguous()
+                    check_within(x3.to(GPU).var_dim(1, correction, False), x3.var_dim(1, correction, False), extra=0.0,
+                                 max_ulp=1, what=f"{dtype} var [{cols // 128}, 2, 128] over the middle dimension")
                 with np.errstate(all="ignore"):
                     sd = np.where(v64 > 0, np.minimum(delta / np.sqrt(np.where(v64 > 0, v64, 1.0)), np.sqrt(delta)), np.sqrt(delta))
                 check_within(g.std_dim(0, correction, False), x.std_dim(0, correction, False), extra=np.nan_to_num(sd),
