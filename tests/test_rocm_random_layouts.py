@@ -249,6 +249,19 @@ def test_random_views_through_float_reductions_and_softmax(seed):
         (gv, gi), (cv, ci) = vg.max_dim(d, keep), vc.max_dim(d, keep)
         assert_bitwise(gv, cv, f"{what}: max along {d}")
         assert_bitwise(gi, ci, f"{what}: positions of the max along {d}")
+        if case % 3 == 1:
+            # Ties, signed zeros and NaNs from a five-letter alphabet: the CPU keeps the first of equal values and the
+            # first NaN, and the GPU's value and position must be that one (ref: src/backend/cpu/reduce.rs:75-86).
+            from tests.support import from_f64
+            letters = rng.choice([-1.0, 0.0, -0.0, 1.0, np.nan], n, p=[0.3, 0.2, 0.2, 0.28, 0.02])
+            tc = tensor(from_f64(letters, dtype), dtype, base_shape)
+            tvc, tvg = apply(tc, chain), apply(tc.to(GPU), chain)
+            for best in ("max_dim", "min_dim"):
+                (gv, gi), (cv, ci) = getattr(tvg, best)(d, keep), getattr(tvc, best)(d, keep)
+                assert_bitwise(gv, cv, f"{what}: {best} of tied values along {d}")
+                assert_bitwise(gi, ci, f"{what}: positions of {best} of tied values along {d}")
+            assert_bitwise(tvg.argmax(), tvc.argmax(), f"{what}: argmax of tied values")
+            assert_bitwise(tvg.min(), tvc.min(), f"{what}: min of tied values")
         # Softmax on data of a few binades, as the reduce tests use (larger spreads make every row one-hot).
         sc = finite(dtype, n, 3, 7000 * seed + case).reshape(base_shape)
         if sprinkled:
