@@ -325,21 +325,25 @@ __global__ void __launch_bounds__(G > kBlock ? G : kBlock) softmax_regs_kernel(S
                     E e[V];
 #pragma unroll
                     for (int i = 0; i < V; ++i) e[i] = M::ex(x[i], mx);
+                    float part = ((e[0] + e[1]) + (e[2] + e[3])) + ((e[4] + e[5]) + (e[6] + e[7]));
                     if constexpr (LOG) {
                         // log_softmax of a row that one element dominates is -log(1 + s) ~ -s with s the sum of
                         // the other terms, and s must keep its own relative accuracy: next to a 1 in an f32 sum
                         // it would keep 2^-24 absolute. The terms that are exactly 1 (the maximum and anything
-                        // that rounds to it) are counted instead of added; the count joins the f64 sum.
-                        float ones = 0.0f;
+                        // that rounds to it) are counted instead of added; the count joins the f64 sum. Only a
+                        // chunk whose terms reach 1 together can hold one: the few that do are summed again.
+                        if (part >= 1.0f) {
+                            float ones = 0.0f;
 #pragma unroll
-                        for (int i = 0; i < V; ++i) {
-                            const bool one = e[i] == 1.0f;
-                            ones += one ? 1.0f : 0.0f;
-                            e[i] = one ? 0.0f : e[i];
+                            for (int i = 0; i < V; ++i) {
+                                const bool one = e[i] == 1.0f;
+                                ones += one ? 1.0f : 0.0f;
+                                e[i] = one ? 0.0f : e[i];
+                            }
+                            part = ((e[0] + e[1]) + (e[2] + e[3])) + ((e[4] + e[5]) + (e[6] + e[7]));
+                            sum += static_cast<double>(ones);
                         }
-                        sum += static_cast<double>(ones);
                     }
-                    float part = ((e[0] + e[1]) + (e[2] + e[3])) + ((e[4] + e[5]) + (e[6] + e[7]));
                     sum += static_cast<double>(part);
                 }
             }
