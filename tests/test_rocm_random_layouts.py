@@ -152,7 +152,7 @@ def test_random_views_through_every_kernel_family(seed):
         # A partner of another dtype: the result type and the converted operands must be the CPU's.
         if shape:
             qc, qg = pair(other, shape, 90 + case)
-            name = str(rng.choice(["add", "mul", "sub", "maximum", "greater", "equal"]))
+            name = str(rng.choice(["add", "mul", "sub", "maximum", "greater", "equal", "div"]))   # div of integers is true division
             try:
                 want = getattr(vc, name)(qc)
             except Exception as refusal:            # e.g. bool - bool: the GPU must refuse in the same words
