@@ -80,9 +80,25 @@ __device__ __forceinline__ typename Comp<T>::C e_exp(typename Comp<T>::C x) {
     else return exp(x);
 }
 
+// A NaN whose quiet bit is clear. Conversions and arithmetic quiet it, so it has to be looked for in the bits.
+__device__ __forceinline__ bool is_signaling(float x) {
+    const uint32_t b = __float_as_uint(x);
+    return (b & 0x7fc00000u) == 0x7f800000u && (b & 0x003fffffu) != 0;
+}
+__device__ __forceinline__ bool is_signaling(double x) {
+    const uint64_t b = static_cast<uint64_t>(__double_as_longlong(x));
+    return (b & 0x7ff8000000000000ull) == 0x7ff0000000000000ull && (b & 0x0007ffffffffffffull) != 0;
+}
+
+// pow(x, 0) and pow(1, y) are 1 for every x and y, a quiet NaN included, but the host library answers a
+// signaling NaN with a NaN (IEEE 754's pow: invalid operation); the device library says 1 for both kinds.
 template <class T>
 __device__ __forceinline__ typename Comp<T>::C e_pow(typename Comp<T>::C x, typename Comp<T>::C y) {
     using E = typename Eval<T>::E;
+    // Halves: the CPU's widening to f32 quiets a NaN before pow sees it, and bf16's widening here is a shift.
+    if constexpr (sizeof(T) >= 4) {
+        if (is_signaling(x) || is_signaling(y)) return x + y;
+    }
     return static_cast<typename Comp<T>::C>(m_pow(static_cast<E>(x), static_cast<E>(y)));
 }
 

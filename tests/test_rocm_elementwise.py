@@ -171,6 +171,27 @@ def test_half_unary_ops_over_every_input(name, dtype):
     print(f"exhaustive {name} {dtype}: {differ} of 65536 differ, max {worst} ulp")
 
 
+def test_pow_of_signaling_nans_is_a_nan_as_on_the_cpu():
+    """pow(x, 0) and pow(1, y) are 1 even for a quiet NaN, but the host library answers a signaling NaN with a NaN
+    (and so does the CPU backend, which calls it); every float dtype, tensor and scalar exponents."""
+    patterns = {DT.F64: (np.array([0x7ff0000000000001, 0x7ff4000000000000, 0xfff0000000000123, 0x7ff8000000000000, 0xfff8000000000001,
+                                   0x3ff0000000000000, 0x4000000000000000], dtype=np.uint64).view(np.float64)),
+                DT.F32: (np.array([0x7f800001, 0x7fa00000, 0xff800123, 0x7fc00000, 0xffc00001, 0x3f800000, 0x40000000],
+                                  dtype=np.uint32).view(np.float32)),
+                DT.BF16: np.array([0x7f81, 0x7fa0, 0xff83, 0x7fc0, 0xffc1, 0x3f80, 0x4000], dtype=np.uint16),
+                DT.F16: np.array([0x7c01, 0x7d00, 0xfc23, 0x7e00, 0xfe01, 0x3c00, 0x4000], dtype=np.uint16)}
+    for dtype, raw in patterns.items():
+        x = tensor(raw, dtype)
+        zero = tensor(from_f64(np.zeros(raw.size), dtype), dtype)
+        one = tensor(from_f64(np.ones(raw.size), dtype), dtype)
+        for what, f in (("x ** 0 (tensor)", lambda t, z, o: t.pow(z)), ("x ** 0.0 (scalar)", lambda t, z, o: t.pow(0.0)),
+                        ("x ** -0.0 (scalar)", lambda t, z, o: t.pow(-0.0)), ("1 ** y", lambda t, z, o: o.pow(t)),
+                        ("x ** x", lambda t, z, o: t.pow(t))):
+            cpu = f(x, zero, one)
+            gpu = f(x.to(GPU), zero.to(GPU), one.to(GPU))
+            check_within(gpu, cpu, extra=0.0, max_ulp=1, what=f"{dtype} {what}")
+
+
 def test_exp_sigmoid_and_silu_have_the_cpus_bits():
     """exp of an f32 value is the host library's expf restated, and sigmoid and silu are f32 arithmetic on it in the
     CPU's order: the same bits as the CPU for every 16-bit input and for millions of f32 inputs of every range

@@ -161,6 +161,20 @@ def test_random_views_through_every_kernel_family(seed):
                 assert str(got.value) == str(refusal), f"{what}: {name} with a {other} partner"
             else:
                 assert_bitwise(getattr(vg, name)(qg), want, f"{what}: {name} with a {other} partner")
+        # A scalar operand: the scalar's kind and the tensor's dtype decide the result type (ref: src/ops/binary.rs).
+        scalar = [3, -2, 2.5, 0.1, 1e20, -0.0, 255, 65536, True, float("inf")][int(rng.integers(0, 10))]
+        name = str(rng.choice(["add", "mul", "sub", "div", "maximum", "greater", "equal", "pow"]))
+        try:
+            want = getattr(vc, name)(scalar)
+        except Exception as refusal:
+            with pytest.raises(type(refusal)) as got:
+                getattr(vg, name)(scalar)
+            assert str(got.value) == str(refusal), f"{what}: {name} {scalar!r}"
+        else:
+            if name == "pow" and want.dtype in FLOATS:
+                check_within(getattr(vg, name)(scalar), want, extra=0.0, max_ulp=1, what=f"{what}: pow {scalar!r}")
+            else:
+                assert_bitwise(getattr(vg, name)(scalar), want, f"{what}: {name} {scalar!r}")
         if dtype in (DT.I64, DT.I32, DT.U8) and shape:
             d = int(rng.integers(0, len(shape)))
             assert_bitwise(vg.sum_dim([d], False), vc.sum_dim([d], False), f"{what}: sum along {d}")
