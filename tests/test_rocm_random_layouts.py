@@ -325,6 +325,29 @@ def test_random_views_through_the_families_next_to_the_path(seed):
         mask_c = pc.greater(vc) if dtype != DT.Bool else pc
         fill = True if dtype == DT.Bool else 3
         assert_bitwise(vg.masked_fill(mask_c.to(GPU), fill), vc.masked_fill(mask_c, fill), f"{what}: masked_fill")
+        # clamp with scalar bounds, full and fill_ with scalars of every kind: the same result or the same refusal.
+        def same(f_gpu, f_cpu, label):
+            try:
+                want = f_cpu()
+            except Exception as refusal:
+                with pytest.raises(type(refusal)) as got:
+                    f_gpu()
+                assert str(got.value) == str(refusal), f"{what}: {label}"
+            else:
+                assert_bitwise(f_gpu(), want, f"{what}: {label}")
+
+        if dtype != DT.Bool:
+            lo, hi = (float(x) for x in rng.choice([-100.0, -1.0, 0.0, 0.5, 3.0, 100.0], 2))
+            if dtype not in FLOATS:
+                lo, hi = int(lo), int(hi)
+            same(lambda: vg.clamp(lo, hi), lambda: vc.clamp(lo, hi), f"clamp({lo}, {hi})")
+            same(lambda: vg.clamp_min(lo), lambda: vc.clamp_min(lo), f"clamp_min({lo})")
+            same(lambda: vg.clamp_max(hi), lambda: vc.clamp_max(hi), f"clamp_max({hi})")
+        scalar = [0, 1, -1, 3, 255, 256, -129, 70000, 2.5, -0.0, 1e20, 1e-50, float("inf"), float("nan"), True][int(rng.integers(0, 15))]
+        same(lambda: h.full(list(shape), scalar, dtype, GPU), lambda: h.full(list(shape), scalar, dtype, "cpu"), f"full {scalar!r}")
+        if not overlapping(vc):
+            fc, fg = pair(dtype, base_shape, 3000 * seed + case)
+            same(lambda: (apply(fg, chain).fill_(scalar), fg)[1], lambda: (apply(fc, chain).fill_(scalar), fc)[1], f"fill_ {scalar!r} through the view")
         # The index family along d.
         itype = DT.I64 if rng.integers(0, 2) else DT.I32
         count = int(rng.integers(1, 2 * shape[d] + 2))
