@@ -376,3 +376,50 @@ def test_random_views_through_the_families_next_to_the_path(seed):
             (ac, ag), (bc, bg) = pair(dtype, [shape[0]], 84 + case), pair(dtype, [shape[1]], 85 + case)
             beta, alpha = (0.5, -1.5) if dtype in FLOATS else (2, -3)
             assert_bitwise(vg.addr(ag, bg, beta, alpha), vc.addr(ac, bc, beta, alpha), f"{what}: addr")
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_views_of_large_tensors_agree_with_the_cpu_on_windows(seed):
+    """Hundreds of megabytes: the sizes at which the kernels change their cache hints and their store forms. The
+    operands are sampled on the GPU, the operation runs on the whole view, and windows of the result (a few rows of
+    its first dimension) are compared with the CPU's result on the same windows of the operands: an element-wise
+    operation on a window is the window of the operation."""
+    rng = np.random.default_rng(0x5EED5000 + seed)
+    bases = {DT.I64: [[8, 2048, 4096], [4, 4096, 32, 128]], DT.F32: [[12, 2048, 4096], [96, 1024, 1024]],
+             DT.BF16: [[8192, 32000], [16, 2048, 32, 128], [8, 2048, 4096]], DT.U8: [[16384, 32768], [8, 4096, 128, 128]]}
+    dtype = list(bases)[seed % 4]
+    base_shape = bases[dtype][int(rng.integers(0, len(bases[dtype])))]
+    while True:
+        chain, shape = random_chain(rng, base_shape)
+        if all(m not in ("expand", "unfold", "select") for m, _ in chain) and int(np.prod(shape)) >= int(np.prod(base_shape)) // 4:
+            break
+    what = f"seed {seed}: {dtype} {base_shape} {chain}"
+    h.manual_seed(1234 + seed)
+    if dtype in (DT.F32, DT.BF16):
+        a, b = h.uniform(base_shape, -4.0, 4.0, dtype, GPU), h.uniform(base_shape, -4.0, 4.0, dtype, GPU)
+    else:
+        a, b = h.randint(0, 200, base_shape, dtype, GPU), h.randint(0, 200, base_shape, dtype, GPU)
+    va, vb = apply(a, chain), apply(b, chain)
+    ops = [("add", lambda x, y: x.add(y)), ("greater", lambda x, y: x.greater(y)), ("copy", lambda x, y: x.contiguous()),
+           ("mul by 3", lambda x, y: x.mul(3)), ("where", lambda x, y: h.where_(x.greater(y), x, y))]
+    if dtype == DT.BF16:
+        ops += [("silu", lambda x, y: x.silu()), ("add an f32 partner", lambda x, y: x.add(y.to(DT.F32)))]
+    if dtype == DT.I64:
+        ops += [("bitwise_and", lambda x, y: x.bitwise_and(y))]
+    rows = shape[0]
+    for name, f in ops:
+        whole = f(va, vb)
+        for _ in range(3):
+            k = max(1, min(rows, (1 << 21) // max(1, int(np.prod(shape[1:])))))
+            start = int(rng.integers(0, rows - k + 1))
+            wa, wb = va.narrow(0, start, k).contiguous().to("cpu"), vb.narrow(0, start, k).contiguous().to("cpu")
+            assert_bitwise(whole.narrow(0, start, k).contiguous(), f(wa, wb), f"{what}: {name}, rows {start}..{start + k}")
+        del whole
+    if dtype in (DT.I64, DT.U8) and len(shape) >= 2:
+        whole = va.sum_dim([len(shape) - 1], False)
+        k = max(1, min(rows, (1 << 21) // max(1, int(np.prod(shape[1:])))))
+        start = int(rng.integers(0, rows - k + 1))
+        wa = va.narrow(0, start, k).contiguous().to("cpu")
+        assert_bitwise(whole.narrow(0, start, k).contiguous(), wa.sum_dim([len(shape) - 1], False), f"{what}: sum along the last dimension")
+    del a, b, va, vb
+    h.empty_cache()
