@@ -421,5 +421,32 @@ def test_random_views_of_large_tensors_agree_with_the_cpu_on_windows(seed):
         start = int(rng.integers(0, rows - k + 1))
         wa = va.narrow(0, start, k).contiguous().to("cpu")
         assert_bitwise(whole.narrow(0, start, k).contiguous(), wa.sum_dim([len(shape) - 1], False), f"{what}: sum along the last dimension")
+    if dtype in (DT.F32, DT.BF16) and len(shape) >= 2:
+        from tests.test_rocm_reduce import check_softmax, check_sum, folded
+        last = len(shape) - 1
+        k = max(1, min(rows, (1 << 21) // max(1, int(np.prod(shape[1:])))))
+        start = int(rng.integers(0, rows - k + 1))
+        wa = va.narrow(0, start, k).contiguous().to("cpu")
+        wide = wa.to(DT.F64)
+        for log in (False, True):
+            whole = va.log_softmax(last) if log else va.softmax(last)
+            want = wa.log_softmax(last) if log else wa.softmax(last)
+            check_softmax(whole.narrow(0, start, k).contiguous(), want, wide, last, log, f"{what}: softmax along the last dimension, log {log}")
+            del whole
+        whole = va.sum_dim([last], False)
+        want = wa.sum_dim([last], False)
+        check_sum(whole.narrow(0, start, k).contiguous(), want, wide.abs().sum_dim([last], False), folded(wa, want), False,
+                  f"{what}: sum along the last dimension")
+        whole = va.var_dim([last], 1, False)
+        v64 = np.nan_to_num(to_f64_of(wide.var_dim([last], 1, False)))
+        from tests.support import check_within
+        from tests.test_rocm_reduce import EPS
+        check_within(whole.narrow(0, start, k).contiguous(), wa.var_dim([last], 1, False), extra=4.0 * shape[last] * EPS * v64,
+                     what=f"{what}: var along the last dimension")
     del a, b, va, vb
     h.empty_cache()
+
+
+def to_f64_of(t):
+    from tests.support import array, to_f64
+    return to_f64(array(t).reshape(-1), t.dtype)
