@@ -9,7 +9,7 @@
 // correctly rounded one, which is why this is a restatement and not a call of an accurate exp. The host
 // library is built twice, with and without fused multiply-adds, and picks by the CPU it runs on (every
 // x86-64 core this library runs beside has FMA); FUSED restates the first build. Compared with the host's
-// expf over all 2^32 inputs (tests/expf_check.cpp) the fused form differs for none, the other for two; the
+// expf over all 2^32 inputs (tests/libm_check.cpp) the fused form differs for none, the other for two; the
 // same comparison pins every constant and the table.
 //
 // Plain C++ apart from the fused multiply-add builtin, so a host program compiles it.

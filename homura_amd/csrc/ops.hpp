@@ -3,9 +3,10 @@
 // to the computation type (f32 for F16/BF16/F32, f64 for F64), compute, and round once; integer
 // ops wrap.
 //
-// Transcendental accuracy. The CPU calls the host libm in the computation type. Here exp of an f32
-// value is the host library's expf restated (expf_like_libm.hpp: the same bits for every input), and
-// for the other functions:
+// Transcendental accuracy. The CPU calls the host libm in the computation type. Here exp, tanh and
+// log1p of an f32 value are the host library's expf, tanhf and log1pf restated (expf_like_libm.hpp,
+// f32_like_libm.hpp: the same bits for every input), so exp, sigmoid, silu, tanh, gelu_tanh and
+// log_sigmoid have the CPU's bits, and for the other functions:
 //   F32 tensors   evaluate the function in f64 and round to f32. That is the correctly rounded
 //                 f32 value except within ~2^-29 of a rounding boundary, which is also what a good
 //                 libm returns, so results agree to the last bit nearly everywhere and to 1 ulp
@@ -21,6 +22,7 @@
 
 #include "elem.hpp"
 #include "expf_like_libm.hpp"
+#include "f32_like_libm.hpp"
 #include "map.hpp"
 
 namespace hmr {
@@ -42,14 +44,10 @@ struct Eval<double> {
 
 __device__ __forceinline__ float m_log(float x) { return logf(x); }
 __device__ __forceinline__ double m_log(double x) { return log(x); }
-__device__ __forceinline__ float m_log1p(float x) { return log1pf(x); }
-__device__ __forceinline__ double m_log1p(double x) { return log1p(x); }
 __device__ __forceinline__ float m_sin(float x) { return sinf(x); }
 __device__ __forceinline__ double m_sin(double x) { return sin(x); }
 __device__ __forceinline__ float m_cos(float x) { return cosf(x); }
 __device__ __forceinline__ double m_cos(double x) { return cos(x); }
-__device__ __forceinline__ float m_tanh(float x) { return tanhf(x); }
-__device__ __forceinline__ double m_tanh(double x) { return tanh(x); }
 __device__ __forceinline__ float m_pow(float x, float y) { return powf(x, y); }
 __device__ __forceinline__ double m_pow(double x, double y) { return pow(x, y); }
 __device__ __forceinline__ float m_sqrt(float x) { return sqrtf(x); }  // correctly rounded
@@ -65,10 +63,8 @@ __device__ __forceinline__ double m_abs(double x) { return fabs(x); }
         return static_cast<typename Comp<T>::C>(FN(static_cast<E>(x))); \
     }
 HMR_EVAL1(e_log, m_log)
-HMR_EVAL1(e_log1p, m_log1p)
 HMR_EVAL1(e_sin, m_sin)
 HMR_EVAL1(e_cos, m_cos)
-HMR_EVAL1(e_tanh, m_tanh)
 #undef HMR_EVAL1
 
 // exp in the computation type: for f32 (F16, BF16 and F32 tensors) the host library's own expf, bit for
@@ -78,6 +74,18 @@ template <class T>
 __device__ __forceinline__ typename Comp<T>::C e_exp(typename Comp<T>::C x) {
     if constexpr (std::is_same_v<typename Comp<T>::C, float>) return expf_like_libm<true>(x);
     else return exp(x);
+}
+// tanh and log1p likewise (f32_like_libm.hpp): gelu_tanh's 1 + tanh cancels next to its zero, and log_sigmoid is
+// a difference of which the log1p is one part.
+template <class T>
+__device__ __forceinline__ typename Comp<T>::C e_tanh(typename Comp<T>::C x) {
+    if constexpr (std::is_same_v<typename Comp<T>::C, float>) return tanhf_like_libm(x);
+    else return tanh(x);
+}
+template <class T>
+__device__ __forceinline__ typename Comp<T>::C e_log1p(typename Comp<T>::C x) {
+    if constexpr (std::is_same_v<typename Comp<T>::C, float>) return log1pf_like_libm(x);
+    else return log1p(x);
 }
 
 // A NaN whose quiet bit is clear. Conversions and arithmetic quiet it, so it has to be looked for in the bits.

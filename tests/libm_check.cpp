@@ -1,0 +1,78 @@
+// Compares the restated f32 library functions of homura_amd/csrc (expf_like_libm.hpp, f32_like_libm.hpp) with the
+// host C library's over bit patterns of f32: `libm_check <function> <stride> [fused]` with function one of expf,
+// expm1f, tanhf, log1pf walks every stride-th pattern (1: all 2^32) on all hardware threads and prints the number of
+// inputs whose results differ in any bit (a NaN for a NaN counts as equal). `fused` (expf only, default 1) picks
+// the form with fused multiply-adds.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <thread>
+#include <vector>
+
+#include "expf_like_libm.hpp"
+#include "f32_like_libm.hpp"
+
+template <class Host, class Port>
+static uint64_t count(uint64_t begin, uint64_t end, uint64_t stride, uint32_t *first, Host host, Port port) {
+    uint64_t bad = 0;
+    for (uint64_t b = begin; b < end; b += stride) {
+        const uint32_t bits = static_cast<uint32_t>(b);
+        float x;
+        memcpy(&x, &bits, 4);
+        volatile float xv = x;  // keep the compiler from folding the library call
+        const float want = host(xv), got = port(x);
+        uint32_t w, g;
+        memcpy(&w, &want, 4);
+        memcpy(&g, &got, 4);
+        if (w != g && !(want != want && got != got)) {
+            if (bad == 0) *first = bits;
+            ++bad;
+        }
+    }
+    return bad;
+}
+
+int main(int argc, char **argv) {
+    if (argc < 3) {
+        std::fprintf(stderr, "usage: libm_check expf|expm1f|tanhf|log1pf <stride> [fused]\n");
+        return 2;
+    }
+    const std::string name = argv[1];
+    const uint64_t stride = strtoull(argv[2], nullptr, 10);
+    const bool fused = argc > 3 ? atoi(argv[3]) != 0 : true;
+    const unsigned workers = std::max(1u, std::thread::hardware_concurrency());
+    std::vector<uint64_t> bad(workers, 0);
+    std::vector<uint32_t> first(workers, 0);
+    std::vector<std::thread> pool;
+    const uint64_t total = uint64_t{1} << 32, span = (total / workers / stride + 1) * stride;
+    for (unsigned w = 0; w < workers; ++w) {
+        pool.emplace_back([&, w] {
+            const uint64_t begin = w * span, end = std::min(total, begin + span);
+            auto run = [&](auto host, auto port) { bad[w] = count(begin, end, stride, &first[w], host, port); };
+            if (name == "expf" && fused) run([](float x) { return expf(x); }, [](float x) { return hmr::expf_like_libm<true>(x); });
+            else if (name == "expf") run([](float x) { return expf(x); }, [](float x) { return hmr::expf_like_libm<false>(x); });
+            else if (name == "expm1f") run([](float x) { return expm1f(x); }, [](float x) { return hmr::expm1f_like_libm(x); });
+            else if (name == "tanhf") run([](float x) { return tanhf(x); }, [](float x) { return hmr::tanhf_like_libm(x); });
+            else if (name == "log1pf") run([](float x) { return log1pf(x); }, [](float x) { return hmr::log1pf_like_libm(x); });
+            else bad[w] = ~uint64_t{0};
+        });
+    }
+    for (auto &t : pool) t.join();
+    uint64_t sum = 0;
+    uint32_t example = 0;
+    for (unsigned w = 0; w < workers; ++w) {
+        if (bad[w] == ~uint64_t{0}) {
+            std::fprintf(stderr, "unknown function %s\n", name.c_str());
+            return 2;
+        }
+        if (bad[w] && !sum) example = first[w];
+        sum += bad[w];
+    }
+    std::printf("%llu differ", static_cast<unsigned long long>(sum));
+    if (sum) std::printf(" (first at bits 0x%08x)", example);
+    std::printf("\n");
+    return 0;
+}

@@ -87,11 +87,9 @@ def magnitude(name, x, y):
         return np.abs(y)
 
 
-# Ops whose f32 / half results must sit within ONE ulp of the output dtype of the oracle's, with no
-# further allowance. The others (tanh, log_sigmoid, gelu_tanh) go through glibc functions whose own
-# error exceeds half an ulp, so they are held to the reference's bound k*u*m + ulp instead (measured: 2 ulp for
-# tanh and log_sigmoid, up to 178 ulp of a tiny result where gelu_tanh's 1 + tanh cancels), and to one ulp
-# against the CPU's formula with correctly rounded functions in the test after this one.
+# Ops whose f32 / half results must sit within ONE ulp of the output dtype of the oracle's, with no further
+# allowance, in this test; the others are held to the reference's bound k*u*m + ulp here and to the CPU's very bits
+# in test_ops_built_on_exp_tanh_and_log1p_have_the_cpus_bits, as are exp, sigmoid and silu.
 ONE_ULP = {"exp", "log", "sin", "cos", "erf", "sigmoid", "silu", "gelu"}
 
 
@@ -115,49 +113,6 @@ def test_transcendental_unary_ops_stay_within_the_bounds(name, k, tails):
             worst = max(worst, m)
             total += cpu.num_elements()
         print(f"ulp {name:<12} {dtype}: max {worst} ulp, {differ} of {total} elements differ")
-
-
-def follows_the_formula(name, x):
-    """The CPU's f32 formula for an op (ref: src/backend/cpu/mod.rs:378-403) step by step in float32, with every
-    library function replaced by its correctly rounded value (float64 evaluation, one rounding): what the
-    device computes."""
-    f = np.float32
-    x = x.astype(np.float32)
-    fn = lambda g, v: g(v.astype(np.float64)).astype(np.float32)
-    # exp is the exception: the device restates the host library's expf (the same bits for every input), so the
-    # formula takes the CPU's own.
-    host_exp = lambda v: array(tensor(v.astype(np.float32), DT.F32).exp()).reshape(v.shape)
-    with np.errstate(all="ignore"):
-        if name == "tanh":
-            return fn(np.tanh, x)
-        if name == "log_sigmoid":
-            lower = np.where(np.isnan(x) | (x < 0), x, f(0))
-            return lower - fn(np.log1p, host_exp(-np.abs(x)))
-        k, c = f(math.sqrt(2.0 / math.pi)), f(0.044715)
-        return f(0.5) * x * (f(1) + fn(np.tanh, k * (x + c * x * x * x)))
-
-
-@pytest.mark.parametrize("name", ["tanh", "log_sigmoid", "gelu_tanh"])
-def test_f32_ops_outside_the_one_ulp_class_are_the_cpus_formula_with_correctly_rounded_functions(name):
-    """tanh, log_sigmoid and gelu_tanh in F32 are judged against the oracle with the reference's bound k*u*m + ulp
-    (above), because the oracle's glibc tanhf / log1pf / expf are themselves up to 2 ulp off and `1 + tanh(..)`
-    magnifies that where it cancels. What the device computes is pinned here instead: the CPU's formula in f32
-    with each library function correctly rounded - against that it is within one ulp everywhere (the device's
-    f64 functions and numpy's may round a float32 tie differently), and the distance to the oracle is printed."""
-    tails = dict((t[0], t[2]) for t in TRANSCENDENTAL)[name]
-    worst = worst_oracle = 0
-    for what, x in domains(DT.F32, tails, 11):
-        gpu = getattr(x.to(GPU), name)()
-        xs = array(x.contiguous()).reshape(-1)
-        want = tensor(follows_the_formula(name, xs), DT.F32, list(x.shape))
-        _, m = check_within(gpu, want, extra=0.0, max_ulp=1, what=f"{name} f32 {what} against the formula")
-        worst = max(worst, m)
-        g, c = bits(gpu).astype(np.int64), bits(getattr(x, name)()).astype(np.int64)
-        order = lambda b: np.where(b & 0x80000000, 0x80000000 - b, b)
-        finite = np.isfinite(array(gpu).reshape(-1)) & np.isfinite(array(getattr(x, name)()).reshape(-1))
-        if finite.any():
-            worst_oracle = max(worst_oracle, int(np.abs(order(g[finite]) - order(c[finite])).max()))
-    print(f"ulp {name} F32: at most {worst} ulp from the formula with correctly rounded functions, {worst_oracle} ulp from the oracle")
 
 
 @pytest.mark.parametrize("dtype", [DT.BF16, DT.F16], ids=["bf16", "f16"])
@@ -192,12 +147,14 @@ def test_pow_of_signaling_nans_is_a_nan_as_on_the_cpu():
             check_within(gpu, cpu, extra=0.0, max_ulp=1, what=f"{dtype} {what}")
 
 
-def test_exp_sigmoid_and_silu_have_the_cpus_bits():
-    """exp of an f32 value is the host library's expf restated, and sigmoid and silu are f32 arithmetic on it in the
-    CPU's order: the same bits as the CPU for every 16-bit input and for millions of f32 inputs of every range
-    (with a correctly rounded exp instead, 1 in 18 000 sigmoids was two to four ulps from the CPU's)."""
+def test_ops_built_on_exp_tanh_and_log1p_have_the_cpus_bits():
+    """exp, tanh and log1p of an f32 value are the host library's expf, tanhf and log1pf restated, and sigmoid, silu,
+    gelu_tanh and log_sigmoid are f32 arithmetic on them in the CPU's order: the same bits as the CPU for every
+    16-bit input and for millions of f32 inputs of every range. (With correctly rounded functions instead, 1 in
+    18 000 sigmoids was two to four ulps from the CPU's, tanh and log_sigmoid up to 2 ulp, and gelu_tanh up to 178
+    next to its zero, where 1 + tanh cancels.)"""
     rng = np.random.default_rng(0xE5F)
-    for name in ("exp", "sigmoid", "silu"):
+    for name in ("exp", "sigmoid", "silu", "tanh", "gelu_tanh", "log_sigmoid"):
         for dtype in (DT.BF16, DT.F16):
             x = tensor(np.arange(65536, dtype=np.uint16), dtype)
             assert_bitwise(getattr(x.to(GPU), name)(), getattr(x, name)(), f"{name} {dtype}, every pattern")
