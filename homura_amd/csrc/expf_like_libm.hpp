@@ -12,6 +12,10 @@
 // expf over all 2^32 inputs (tests/libm_check.cpp) the fused form differs for none, the other for two; the
 // same comparison pins every constant and the table.
 //
+// The scheme, its table and its coefficients are those of Arm's optimized-routines (math/expf.c, math/exp2f_data.c;
+// MIT licence, Copyright (c) 2017-2018 Arm Limited), from which glibc took its expf; the table is recomputed here
+// (2^(i/32) correctly rounded, by integer arithmetic) rather than copied.
+//
 // Plain C++ apart from the fused multiply-add builtin, so a host program compiles it.
 #pragma once
 #include <cstdint>

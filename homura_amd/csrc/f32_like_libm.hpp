@@ -12,6 +12,10 @@
 // Every step is an IEEE f32 operation (this library compiles without contraction and with correctly rounded
 // division), so the same source gives the same bits on the host: tests/libm_check.cpp compares each function
 // with the host library's over all 2^32 inputs, and none differs.
+//
+// The algorithms and constants are fdlibm's, whose notice reads: "Copyright (C) 1993 by Sun Microsystems, Inc. All
+// rights reserved. Developed at SunPro, a Sun Microsystems, Inc. business. Permission to use, copy, modify, and
+// distribute this software is freely granted, provided that this notice is preserved."
 #pragma once
 #include <cstdint>
 #include <cstring>
