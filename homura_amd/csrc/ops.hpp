@@ -3,19 +3,15 @@
 // to the computation type (f32 for F16/BF16/F32, f64 for F64), compute, and round once; integer
 // ops wrap.
 //
-// Transcendental accuracy. The CPU calls the host libm in the computation type. Here exp, tanh and
-// log1p of an f32 value are the host library's expf, tanhf and log1pf restated (expf_like_libm.hpp,
-// f32_like_libm.hpp: the same bits for every input), so exp, sigmoid, silu, tanh, gelu_tanh and
-// log_sigmoid have the CPU's bits, and for the other functions:
-//   F32 tensors   evaluate the function in f64 and round to f32. That is the correctly rounded
-//                 f32 value except within ~2^-29 of a rounding boundary, which is also what a good
-//                 libm returns, so results agree to the last bit nearly everywhere and to 1 ulp
-//                 otherwise.
-//   F16/BF16      evaluate in f32; an f32-ulp difference can only flip the final rounding to the
-//                 16-bit type by one ulp. GELU is the exception: 1 + erf(z) cancels for z << 0, so
-//                 erf is always evaluated in f64 and rounded to f32 exactly as the CPU does
-//                 (ref: src/backend/cpu/num.rs:30-33).
-//   F64           the device library's f64 functions.
+// Transcendental accuracy. The CPU calls the host libm in the computation type. For f32 values (F16,
+// BF16 and F32 tensors) exp, log, sin, cos, tanh and log1p are the host library's expf, logf, sinf,
+// cosf, tanhf and log1pf restated (expf_like_libm.hpp, f32_like_libm.hpp,
+// sinf_cosf_logf_like_libm.hpp: the same bits for every one of the 2^32 inputs), so every unary op
+// built on them has the CPU's bits; erf is the CPU's own f64 algorithm (ref: src/backend/cpu/num.rs:
+// 30-33, 189-219), always evaluated in f64 and rounded to f32 as the CPU does, because GELU's
+// 1 + erf(z) cancels for z << 0. What is left to the device library: pow of f32 values, evaluated in
+// f64 and rounded once (the correctly rounded value except within ~2^-29 of a rounding boundary, a good
+// libm's answer, one ulp from it otherwise), and every function of F64 tensors.
 // The surrounding arithmetic (1/(1+e), 0.5*x*(1+t), ...) is done in the computation type in the
 // CPU's order, so it contributes no difference of its own.
 #pragma once
@@ -23,6 +19,7 @@
 #include "elem.hpp"
 #include "expf_like_libm.hpp"
 #include "f32_like_libm.hpp"
+#include "sinf_cosf_logf_like_libm.hpp"
 #include "map.hpp"
 
 namespace hmr {
@@ -42,12 +39,6 @@ struct Eval<double> {
     using E = double;
 };
 
-__device__ __forceinline__ float m_log(float x) { return logf(x); }
-__device__ __forceinline__ double m_log(double x) { return log(x); }
-__device__ __forceinline__ float m_sin(float x) { return sinf(x); }
-__device__ __forceinline__ double m_sin(double x) { return sin(x); }
-__device__ __forceinline__ float m_cos(float x) { return cosf(x); }
-__device__ __forceinline__ double m_cos(double x) { return cos(x); }
 __device__ __forceinline__ float m_pow(float x, float y) { return powf(x, y); }
 __device__ __forceinline__ double m_pow(double x, double y) { return pow(x, y); }
 __device__ __forceinline__ float m_sqrt(float x) { return sqrtf(x); }  // correctly rounded
@@ -55,17 +46,6 @@ __device__ __forceinline__ double m_sqrt(double x) { return sqrt(x); }
 __device__ __forceinline__ float m_abs(float x) { return fabsf(x); }
 __device__ __forceinline__ double m_abs(double x) { return fabs(x); }
 
-// fn evaluated for a value of computation type C that belongs to storage type T.
-#define HMR_EVAL1(NAME, FN)                                            \
-    template <class T>                                                 \
-    __device__ __forceinline__ typename Comp<T>::C NAME(typename Comp<T>::C x) { \
-        using E = typename Eval<T>::E;                                 \
-        return static_cast<typename Comp<T>::C>(FN(static_cast<E>(x))); \
-    }
-HMR_EVAL1(e_log, m_log)
-HMR_EVAL1(e_sin, m_sin)
-HMR_EVAL1(e_cos, m_cos)
-#undef HMR_EVAL1
 
 // exp in the computation type: for f32 (F16, BF16 and F32 tensors) the host library's own expf, bit for
 // bit (expf_like_libm.hpp), because sigmoid, silu and log_sigmoid divide by or take the logarithm of
@@ -81,6 +61,22 @@ template <class T>
 __device__ __forceinline__ typename Comp<T>::C e_tanh(typename Comp<T>::C x) {
     if constexpr (std::is_same_v<typename Comp<T>::C, float>) return tanhf_like_libm(x);
     else return tanh(x);
+}
+// log, sin and cos likewise (sinf_cosf_logf_like_libm.hpp).
+template <class T>
+__device__ __forceinline__ typename Comp<T>::C e_log(typename Comp<T>::C x) {
+    if constexpr (std::is_same_v<typename Comp<T>::C, float>) return logf_like_libm<true>(x);
+    else return log(x);
+}
+template <class T>
+__device__ __forceinline__ typename Comp<T>::C e_sin(typename Comp<T>::C x) {
+    if constexpr (std::is_same_v<typename Comp<T>::C, float>) return sincosf_like_libm<true, false>(x);
+    else return sin(x);
+}
+template <class T>
+__device__ __forceinline__ typename Comp<T>::C e_cos(typename Comp<T>::C x) {
+    if constexpr (std::is_same_v<typename Comp<T>::C, float>) return sincosf_like_libm<true, true>(x);
+    else return cos(x);
 }
 template <class T>
 __device__ __forceinline__ typename Comp<T>::C e_log1p(typename Comp<T>::C x) {

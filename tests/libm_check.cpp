@@ -1,8 +1,8 @@
 // Compares the restated f32 library functions of homura_amd/csrc (expf_like_libm.hpp, f32_like_libm.hpp) with the
 // host C library's over bit patterns of f32: `libm_check <function> <stride> [fused]` with function one of expf,
-// expm1f, tanhf, log1pf walks every stride-th pattern (1: all 2^32) on all hardware threads and prints the number of
-// inputs whose results differ in any bit (a NaN for a NaN counts as equal). `fused` (expf only, default 1) picks
-// the form with fused multiply-adds.
+// expm1f, tanhf, log1pf, sinf, cosf, logf walks every stride-th pattern (1: all 2^32) on all hardware threads and prints the number of
+// inputs whose results differ in any bit (a NaN for a NaN counts as equal). `fused` (expf, sinf, cosf, logf; default 1)
+// picks the form with fused multiply-adds.
 #include <hip/hip_runtime.h>
 
 #include <cmath>
@@ -14,6 +14,7 @@
 
 #include "expf_like_libm.hpp"
 #include "f32_like_libm.hpp"
+#include "sinf_cosf_logf_like_libm.hpp"
 
 template <class Host, class Port>
 static uint64_t count(uint64_t begin, uint64_t end, uint64_t stride, uint32_t *first, Host host, Port port) {
@@ -37,7 +38,7 @@ static uint64_t count(uint64_t begin, uint64_t end, uint64_t stride, uint32_t *f
 
 int main(int argc, char **argv) {
     if (argc < 3) {
-        std::fprintf(stderr, "usage: libm_check expf|expm1f|tanhf|log1pf <stride> [fused]\n");
+        std::fprintf(stderr, "usage: libm_check expf|expm1f|tanhf|log1pf|sinf|cosf|logf <stride> [fused]\n");
         return 2;
     }
     const std::string name = argv[1];
@@ -57,6 +58,12 @@ int main(int argc, char **argv) {
             else if (name == "expm1f") run([](float x) { return expm1f(x); }, [](float x) { return hmr::expm1f_like_libm(x); });
             else if (name == "tanhf") run([](float x) { return tanhf(x); }, [](float x) { return hmr::tanhf_like_libm(x); });
             else if (name == "log1pf") run([](float x) { return log1pf(x); }, [](float x) { return hmr::log1pf_like_libm(x); });
+            else if (name == "sinf" && fused) run([](float x) { return sinf(x); }, [](float x) { return hmr::sincosf_like_libm<true, false>(x); });
+            else if (name == "sinf") run([](float x) { return sinf(x); }, [](float x) { return hmr::sincosf_like_libm<false, false>(x); });
+            else if (name == "cosf" && fused) run([](float x) { return cosf(x); }, [](float x) { return hmr::sincosf_like_libm<true, true>(x); });
+            else if (name == "cosf") run([](float x) { return cosf(x); }, [](float x) { return hmr::sincosf_like_libm<false, true>(x); });
+            else if (name == "logf" && fused) run([](float x) { return logf(x); }, [](float x) { return hmr::logf_like_libm<true>(x); });
+            else if (name == "logf") run([](float x) { return logf(x); }, [](float x) { return hmr::logf_like_libm<false>(x); });
             else bad[w] = ~uint64_t{0};
         });
     }

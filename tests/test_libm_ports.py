@@ -1,10 +1,12 @@
 """The restated f32 library functions (homura_amd/csrc/expf_like_libm.hpp, f32_like_libm.hpp) against the host C
 library's, on the CPU.
 
-The GPU's exp, expm1, tanh and log1p for f32 values restate the algorithms of the host's expf, expm1f, tanhf and
-log1pf so that exp, sigmoid, silu, tanh, gelu_tanh and log_sigmoid get the CPU's bits. tests/libm_check.cpp compiles
+The GPU's exp, log, sin, cos, expm1, tanh and log1p for f32 values restate the algorithms of the host's expf, logf,
+sinf, cosf, expm1f, tanhf and log1pf so that exp, log, sin, cos, sigmoid, silu, tanh, gelu_tanh and log_sigmoid get
+the CPU's bits. tests/libm_check.cpp compiles
 the same headers for the host and compares each function with the library's, bit for bit. Over all 2^32 inputs none
-of the four differs (expf in the fused form, which is what the library builds; its unfused form differs for two);
+of the seven differs (expf, sinf, cosf and logf in the fused form, which is what the library builds; unfused, expf
+differs for 2 inputs, sinf for 12, cosf for 22);
 that walk takes half a minute of eight cores a function (`libm_check tanhf 1`), so the suite walks every 61st
 pattern: 70 million inputs a function, every binade and both tails."""
 import os
@@ -24,12 +26,13 @@ def checker(tmp_path_factory):
     return exe
 
 
-@pytest.mark.parametrize("function", ["expf", "expm1f", "tanhf", "log1pf"])
+@pytest.mark.parametrize("function", ["expf", "expm1f", "tanhf", "log1pf", "sinf", "cosf", "logf"])
 def test_the_restated_function_has_the_host_librarys_bits(checker, function):
     out = subprocess.run([checker, function, "61"], check=True, capture_output=True, text=True).stdout
     assert out.strip() == "0 differ", out
 
 
-def test_the_unfused_expf_differs_for_two_inputs_at_most(checker):
-    out = subprocess.run([checker, "expf", "61", "0"], check=True, capture_output=True, text=True).stdout
-    assert int(out.split()[0]) <= 2, out
+@pytest.mark.parametrize("function, most", [("expf", 2), ("sinf", 12), ("cosf", 22), ("logf", 0)])
+def test_the_unfused_forms_differ_for_a_handful_of_inputs_at_most(checker, function, most):
+    out = subprocess.run([checker, function, "61", "0"], check=True, capture_output=True, text=True).stdout
+    assert int(out.split()[0]) <= most, out

@@ -89,7 +89,7 @@ def magnitude(name, x, y):
 
 # Ops whose f32 / half results must sit within ONE ulp of the output dtype of the oracle's, with no further
 # allowance, in this test; the others are held to the reference's bound k*u*m + ulp here and to the CPU's very bits
-# in test_ops_built_on_exp_tanh_and_log1p_have_the_cpus_bits, as are exp, sigmoid and silu.
+# in test_ops_built_on_the_restated_library_functions_have_the_cpus_bits, as are all of these but pow.
 ONE_ULP = {"exp", "log", "sin", "cos", "erf", "sigmoid", "silu", "gelu"}
 
 
@@ -147,18 +147,19 @@ def test_pow_of_signaling_nans_is_a_nan_as_on_the_cpu():
             check_within(gpu, cpu, extra=0.0, max_ulp=1, what=f"{dtype} {what}")
 
 
-def test_ops_built_on_exp_tanh_and_log1p_have_the_cpus_bits():
-    """exp, tanh and log1p of an f32 value are the host library's expf, tanhf and log1pf restated, and sigmoid, silu,
-    gelu_tanh and log_sigmoid are f32 arithmetic on them in the CPU's order: the same bits as the CPU for every
-    16-bit input and for millions of f32 inputs of every range. (With correctly rounded functions instead, 1 in
-    18 000 sigmoids was two to four ulps from the CPU's, tanh and log_sigmoid up to 2 ulp, and gelu_tanh up to 178
-    next to its zero, where 1 + tanh cancels.)"""
+def test_ops_built_on_the_restated_library_functions_have_the_cpus_bits():
+    """exp, log, sin, cos, tanh and log1p of an f32 value are the host library's expf, logf, sinf, cosf, tanhf and
+    log1pf restated, and sigmoid, silu, gelu_tanh and log_sigmoid are f32 arithmetic on them in the CPU's order; erf
+    and gelu are the CPU's own algorithm: the same bits as the CPU for every 16-bit input and for millions of f32
+    inputs of every range. (With correctly rounded functions instead, 1 in 18 000 sigmoids was two to four ulps from
+    the CPU's, tanh and log_sigmoid up to 2 ulp, gelu_tanh up to 178 next to its zero, where 1 + tanh cancels, and
+    about one log, sin or cos in a hundred one ulp.)"""
     rng = np.random.default_rng(0xE5F)
-    for name in ("exp", "sigmoid", "silu", "tanh", "gelu_tanh", "log_sigmoid"):
+    for name in ("exp", "log", "sin", "cos", "sigmoid", "silu", "tanh", "gelu_tanh", "log_sigmoid", "erf", "gelu"):
         for dtype in (DT.BF16, DT.F16):
             x = tensor(np.arange(65536, dtype=np.uint16), dtype)
             assert_bitwise(getattr(x.to(GPU), name)(), getattr(x, name)(), f"{name} {dtype}, every pattern")
-        for lo, hi in ((-2.0, 2.0), (-20.0, 20.0), (-110.0, 95.0)):
+        for lo, hi in ((-2.0, 2.0), (-20.0, 20.0), (-110.0, 95.0), (-1e5, 1e5), (0.0, 1e-30), (1e30, 3e38)):
             x = tensor(rng.uniform(lo, hi, 1 << 21).astype(np.float32), DT.F32)
             assert_bitwise(getattr(x.to(GPU), name)(), getattr(x, name)(), f"{name} f32 in [{lo}, {hi}]")
         x = tensor(values(DT.F32, 1 << 20, 77), DT.F32)       # special values and random bit patterns

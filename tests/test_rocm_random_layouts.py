@@ -178,8 +178,8 @@ def test_random_views_through_every_kernel_family(seed):
         name = str(rng.choice([u for u in IEEE_UNARY if not (dtype == DT.Bool and u in ("neg", "abs", "relu"))]))
         assert_bitwise(getattr(vg, name)(), getattr(vc, name)(), f"{what}: {name}")
         if dtype in (DT.F32, DT.BF16, DT.F16):
-            # The ops built on the restated expf, tanhf and log1pf have the CPU's bits; the others stay within an ulp.
-            exact = ["exp", "sigmoid", "silu", "tanh", "gelu_tanh", "log_sigmoid"]
+            # The ops built on the restated library functions have the CPU's bits.
+            exact = ["exp", "log", "sin", "cos", "erf", "sigmoid", "silu", "gelu", "tanh", "gelu_tanh", "log_sigmoid"]
             name = str(rng.choice(sorted(set(ONE_ULP) | set(exact))))
             if name in exact:
                 assert_bitwise(getattr(vg, name)(), getattr(vc, name)(), f"{what}: {name}")
