@@ -34,9 +34,8 @@ __host__ __device__ __forceinline__ double expf_mad(double a, double b, double c
 }
 
 // FUSED: the polynomial's multiply-adds are single roundings, as in the host library's build for CPUs with FMA.
-template <bool FUSED>
-__host__ __device__ __forceinline__ float expf_like_libm(float x) {
-    // table[i] = bits(2^(i/32)) - (i << 47): adding k << 47 to entry k % 32 yields the bits of 2^(k/32).
+// bits(2^(i/32)) - (i << 47) for i in 0..31: adding k << 47 to entry k % 32 yields the bits of 2^(k/32).
+__host__ __device__ __forceinline__ uint64_t libm_exp2_entry(uint64_t i) {
     static constexpr uint64_t table[32] = {
         0x3ff0000000000000ull, 0x3fefd9b0d3158574ull, 0x3fefb5586cf9890full, 0x3fef9301d0125b51ull,
         0x3fef72b83c7d517bull, 0x3fef54873168b9aaull, 0x3fef387a6e756238ull, 0x3fef1e9df51fdee1ull,
@@ -46,6 +45,11 @@ __host__ __device__ __forceinline__ float expf_like_libm(float x) {
         0x3feeace5422aa0dbull, 0x3feeb737b0cdc5e5ull, 0x3feec49182a3f090ull, 0x3feed503b23e255dull,
         0x3feee89f995ad3adull, 0x3feeff76f2fb5e47ull, 0x3fef199bdd85529cull, 0x3fef3720dcef9069ull,
         0x3fef5818dcfba487ull, 0x3fef7c97337b9b5full, 0x3fefa4afa2a490daull, 0x3fefd0765b6e4540ull};
+    return table[i];
+}
+
+template <bool FUSED>
+__host__ __device__ __forceinline__ float expf_like_libm(float x) {
     uint32_t bits;
     memcpy(&bits, &x, 4);
     const uint32_t top = (bits >> 20) & 0x7ff;  // exponent and the top three fraction bits of |x|
@@ -68,7 +72,7 @@ __host__ __device__ __forceinline__ float expf_like_libm(float x) {
     // With FMA the product in z is not rounded before kd is taken off it: the one place where the two builds of
     // the host library differ in their results (for 2 of the 2^32 inputs).
     const double r = FUSED ? __builtin_fma(kInvLn2N, static_cast<double>(x), -kd) : z - kd;
-    const uint64_t t = table[ki % 32] + (ki << 47);
+    const uint64_t t = libm_exp2_entry(ki % 32) + (ki << 47);
     double s;
     memcpy(&s, &t, 8);
     const double p = expf_mad<FUSED>(kC0, r, kC1);

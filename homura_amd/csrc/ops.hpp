@@ -9,9 +9,9 @@
 // sinf_cosf_logf_like_libm.hpp: the same bits for every one of the 2^32 inputs), so every unary op
 // built on them has the CPU's bits; erf is the CPU's own f64 algorithm (ref: src/backend/cpu/num.rs:
 // 30-33, 189-219), always evaluated in f64 and rounded to f32 as the CPU does, because GELU's
-// 1 + erf(z) cancels for z << 0. What is left to the device library: pow of f32 values, evaluated in
-// f64 and rounded once (the correctly rounded value except within ~2^-29 of a rounding boundary, a good
-// libm's answer, one ulp from it otherwise), and every function of F64 tensors.
+// 1 + erf(z) cancels for z << 0. pow of f32 values is the host library's powf restated as well
+// (powf_like_libm.hpp; two arguments, so pinned by sweeps and billions of random pairs rather than by
+// every input). What is left to the device library: every function of F64 tensors.
 // The surrounding arithmetic (1/(1+e), 0.5*x*(1+t), ...) is done in the computation type in the
 // CPU's order, so it contributes no difference of its own.
 #pragma once
@@ -20,27 +20,13 @@
 #include "expf_like_libm.hpp"
 #include "f32_like_libm.hpp"
 #include "sinf_cosf_logf_like_libm.hpp"
+#include "powf_like_libm.hpp"
 #include "map.hpp"
 
 namespace hmr {
 
 // ---- math in the evaluation type ---------------------------------------------------------------
 
-template <class T>
-struct Eval {  // halves and their f32 computation type: evaluate in f32
-    using E = float;
-};
-template <>
-struct Eval<float> {
-    using E = double;
-};
-template <>
-struct Eval<double> {
-    using E = double;
-};
-
-__device__ __forceinline__ float m_pow(float x, float y) { return powf(x, y); }
-__device__ __forceinline__ double m_pow(double x, double y) { return pow(x, y); }
 __device__ __forceinline__ float m_sqrt(float x) { return sqrtf(x); }  // correctly rounded
 __device__ __forceinline__ double m_sqrt(double x) { return sqrt(x); }
 __device__ __forceinline__ float m_abs(float x) { return fabsf(x); }
@@ -85,25 +71,27 @@ __device__ __forceinline__ typename Comp<T>::C e_log1p(typename Comp<T>::C x) {
 }
 
 // A NaN whose quiet bit is clear. Conversions and arithmetic quiet it, so it has to be looked for in the bits.
-__device__ __forceinline__ bool is_signaling(float x) {
-    const uint32_t b = __float_as_uint(x);
-    return (b & 0x7fc00000u) == 0x7f800000u && (b & 0x003fffffu) != 0;
-}
 __device__ __forceinline__ bool is_signaling(double x) {
     const uint64_t b = static_cast<uint64_t>(__double_as_longlong(x));
     return (b & 0x7ff8000000000000ull) == 0x7ff0000000000000ull && (b & 0x0007ffffffffffffull) != 0;
 }
 
-// pow(x, 0) and pow(1, y) are 1 for every x and y, a quiet NaN included, but the host library answers a
-// signaling NaN with a NaN (IEEE 754's pow: invalid operation); the device library says 1 for both kinds.
+// pow in the computation type: for f32 the host library's powf restated (powf_like_libm.hpp), which also tells a
+// signaling NaN from a quiet one (x ** 0 and 1 ** y are 1 for a quiet NaN and NaN for a signaling one). The CPU
+// widens a 16-bit NaN to a quiet f32 NaN before powf sees it, and bf16's widening here is a shift: quiet those.
+// For f64 the device library's pow, which says 1 for both kinds of NaN, behind the same check.
 template <class T>
 __device__ __forceinline__ typename Comp<T>::C e_pow(typename Comp<T>::C x, typename Comp<T>::C y) {
-    using E = typename Eval<T>::E;
-    // Halves: the CPU's widening to f32 quiets a NaN before pow sees it, and bf16's widening here is a shift.
-    if constexpr (sizeof(T) >= 4) {
+    if constexpr (std::is_same_v<typename Comp<T>::C, float>) {
+        if constexpr (sizeof(T) == 2) {
+            x = x != x ? __uint_as_float(__float_as_uint(x) | 0x00400000u) : x;
+            y = y != y ? __uint_as_float(__float_as_uint(y) | 0x00400000u) : y;
+        }
+        return powf_like_libm<true>(x, y);
+    } else {
         if (is_signaling(x) || is_signaling(y)) return x + y;
+        return pow(x, y);
     }
-    return static_cast<typename Comp<T>::C>(m_pow(static_cast<E>(x), static_cast<E>(y)));
 }
 
 // erf of a computation-type value: always through f64 (see the header comment).

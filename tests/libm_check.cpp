@@ -1,7 +1,8 @@
 // Compares the restated f32 library functions of homura_amd/csrc (expf_like_libm.hpp, f32_like_libm.hpp) with the
 // host C library's over bit patterns of f32: `libm_check <function> <stride> [fused]` with function one of expf,
 // expm1f, tanhf, log1pf, sinf, cosf, logf walks every stride-th pattern (1: all 2^32) on all hardware threads and prints the number of
-// inputs whose results differ in any bit (a NaN for a NaN counts as equal). `fused` (expf, sinf, cosf, logf; default 1)
+// inputs whose results differ in any bit (a NaN for a NaN counts as equal); powf has two arguments and a mode of its
+// own (below). `fused` (expf, sinf, cosf, logf; default 1)
 // picks the form with fused multiply-adds.
 #include <hip/hip_runtime.h>
 
@@ -9,12 +10,14 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <string>
 #include <thread>
 #include <vector>
 
 #include "expf_like_libm.hpp"
 #include "f32_like_libm.hpp"
 #include "sinf_cosf_logf_like_libm.hpp"
+#include "powf_like_libm.hpp"
 
 template <class Host, class Port>
 static uint64_t count(uint64_t begin, uint64_t end, uint64_t stride, uint32_t *first, Host host, Port port) {
@@ -36,7 +39,60 @@ static uint64_t count(uint64_t begin, uint64_t end, uint64_t stride, uint32_t *f
     return bad;
 }
 
+// powf: `libm_check powf <stride> [fused]` walks every stride-th base for each of 26 exponents, then
+// 250 000 000 / stride * 8 random pairs (half of them with exponents that are multiples of 1/64).
+template <bool FUSED>
+static uint64_t powf_differences(uint64_t stride) {
+    const float exponents[] = {0.5f, 2.0f, 3.0f, -1.0f, 1.0f / 3.0f, 0.1f, 2.5f, -0.5f, 7.0f, 1e-3f, 100.0f, -3.0f, 1.0f,
+                               0.0f, -0.0f, INFINITY, -INFINITY, NAN, 1e-30f, 1e30f, 4.0f, 5.0f, 0.75f, -2.0f, 33.333f, 1.5f};
+    const unsigned workers = std::max(1u, std::thread::hardware_concurrency());
+    std::vector<uint64_t> bad(workers, 0);
+    std::vector<std::thread> pool;
+    auto differ = [](float x, float y) {
+        volatile float xv = x, yv = y;
+        const float want = powf(xv, yv), got = hmr::powf_like_libm<FUSED>(x, y);
+        uint32_t w, g;
+        memcpy(&w, &want, 4);
+        memcpy(&g, &got, 4);
+        return w != g && !(want != want && got != got);
+    };
+    for (unsigned w = 0; w < workers; ++w) {
+        pool.emplace_back([&, w] {
+            const uint64_t total = uint64_t{1} << 32, span = (total / workers / stride + 1) * stride;
+            for (float y : exponents) {
+                for (uint64_t b = w * span; b < std::min(total, (w + 1) * span); b += stride) {
+                    const uint32_t bits = static_cast<uint32_t>(b);
+                    float x;
+                    memcpy(&x, &bits, 4);
+                    bad[w] += differ(x, y);
+                }
+            }
+            uint64_t state = 0x9E3779B97F4A7C15ull * (w + 1);
+            for (uint64_t i = 0; i < 250000000ull / stride; ++i) {
+                state = state * 6364136223846793005ull + 1442695040888963407ull;
+                const uint64_t r = state ^ (state >> 29);
+                const uint32_t xb = static_cast<uint32_t>(r), yb = static_cast<uint32_t>(r >> 32);
+                float x, y;
+                memcpy(&x, &xb, 4);
+                memcpy(&y, &yb, 4);
+                if (i & 1) y = static_cast<float>(static_cast<int>(yb % 2001u) - 1000) / 64.0f;
+                bad[w] += differ(x, y);
+            }
+        });
+    }
+    for (auto &t : pool) t.join();
+    uint64_t sum = 0;
+    for (uint64_t b : bad) sum += b;
+    return sum;
+}
+
 int main(int argc, char **argv) {
+    if (argc >= 3 && std::string(argv[1]) == "powf") {
+        const uint64_t stride = strtoull(argv[2], nullptr, 10);
+        const bool fused = argc > 3 ? atoi(argv[3]) != 0 : true;
+        std::printf("%llu differ\n", static_cast<unsigned long long>(fused ? powf_differences<true>(stride) : powf_differences<false>(stride)));
+        return 0;
+    }
     if (argc < 3) {
         std::fprintf(stderr, "usage: libm_check expf|expm1f|tanhf|log1pf|sinf|cosf|logf <stride> [fused]\n");
         return 2;

@@ -126,6 +126,33 @@ def test_half_unary_ops_over_every_input(name, dtype):
     print(f"exhaustive {name} {dtype}: {differ} of 65536 differ, max {worst} ulp")
 
 
+def test_pow_has_the_cpus_bits_on_f32_and_the_halves():
+    """pow of f32 values is the host library's powf restated: random pairs of every kind (arbitrary bits, moderate
+    bases with exponents that are multiples of 1/8, negative bases with integer exponents, subnormal bases, results
+    that overflow and vanish), scalar exponents, and every 16-bit pattern as base and as exponent."""
+    rng = np.random.default_rng(0x90F)
+    n = 1 << 21
+    pairs = [("random bits", rng.integers(0, 1 << 32, n, dtype=np.uint64).astype(np.uint32).view(np.float32),
+              rng.integers(0, 1 << 32, n, dtype=np.uint64).astype(np.uint32).view(np.float32)),
+             ("moderate", rng.uniform(-50.0, 50.0, n).astype(np.float32), (rng.integers(-80, 81, n) / 8.0).astype(np.float32)),
+             ("near one", (1.0 + rng.uniform(-1e-3, 1e-3, n)).astype(np.float32), rng.uniform(-1e5, 1e5, n).astype(np.float32)),
+             ("subnormal bases", (rng.uniform(0.0, 1.0, n) * 1e-38).astype(np.float32), rng.uniform(-3.0, 3.0, n).astype(np.float32)),
+             ("large", rng.uniform(0.0, 3e38, n).astype(np.float32), rng.uniform(-2.0, 2.0, n).astype(np.float32))]
+    for what, x, y in pairs:
+        cx, cy = tensor(x, DT.F32), tensor(y, DT.F32)
+        assert_bitwise(cx.to(GPU).pow(cy.to(GPU)), cx.pow(cy), f"pow f32, {what}")
+    x = tensor(rng.uniform(-30.0, 30.0, n).astype(np.float32), DT.F32)
+    for e in (2.0, 3.0, 0.5, -1.0, -0.5, 1.0 / 3.0, 2.5, 7.0, 0.0, 1.0, -2.0, 100.0):
+        assert_bitwise(x.to(GPU).pow(e), x.pow(e), f"pow f32 by the scalar {e}")
+    for dtype in (DT.BF16, DT.F16):
+        every = tensor(np.arange(65536, dtype=np.uint16), dtype)
+        for e in (2.0, 0.5, -1.0, 3.0, 0.0, 1.5):
+            assert_bitwise(every.to(GPU).pow(e), every.pow(e), f"pow {dtype}, every base, by the scalar {e}")
+        for b in (2.0, 0.5, -2.0, 10.0, 1.0):
+            base = tensor(from_f64(np.full(65536, b), dtype), dtype)
+            assert_bitwise(base.to(GPU).pow(every.to(GPU)), base.pow(every), f"pow {dtype}, {b} to every exponent")
+
+
 def test_pow_of_signaling_nans_is_a_nan_as_on_the_cpu():
     """pow(x, 0) and pow(1, y) are 1 even for a quiet NaN, but the host library answers a signaling NaN with a NaN
     (and so does the CPU backend, which calls it); every float dtype, tensor and scalar exponents."""
