@@ -199,7 +199,7 @@ TABLE_OPS = ["exp", "log", "sqrt", "rsqrt", "reciprocal", "sin", "cos", "erf", "
 
 @pytest.mark.parametrize("dtype", [DT.BF16, DT.F16], ids=["bf16", "f16"])
 def test_large_half_tensors_take_the_table_and_get_the_direct_kernels_bits(dtype):
-    """From 2^20 elements on, 16-bit unary operations are looked up in a table of all 65 536 results. Every
+    """From 2^15 elements on, 16-bit unary operations are looked up in a table of all 65 536 results. Every
     pattern, in a contiguous tensor with a ragged end, in rows of a wider buffer, through a permuted view
     and in place (out == src through the C ABI): the same bits as the direct kernel on the patterns alone."""
     import ctypes
