@@ -33,99 +33,83 @@ __host__ __device__ inline float libm_float(uint32_t b) {
     return x;
 }
 
-__host__ __device__ inline float expm1f_like_libm(float x) {
+// expm1f. The library's source branches on k; here the cases are computed side by side and selected, each with the
+// library's own operations: lanes of a wave would take different branches anyway, and without them the compiler
+// can interleave the independent elements a lane holds (these are chains of some two hundred dependent operations).
+__host__ __device__ inline float expm1f_like_libm(float x0) {
     const float one = 1.0f, tiny = 1.0e-30f, huge = 1.0e+30f;
     const float o_threshold = 8.8721679688e+01f, ln2_hi = 6.9313812256e-01f, ln2_lo = 9.0580006145e-06f, invln2 = 1.4426950216e+00f;
     const float Q1 = -3.3333335072e-02f, Q2 = 1.5873016091e-03f, Q3 = -7.9365076090e-05f, Q4 = 4.0082177293e-06f, Q5 = -2.0109921195e-07f;
-    float y, hi, lo, c = 0.0f, t, e, hxs, hfx, r1;
-    int32_t k;
-    uint32_t hx = libm_bits(x);
-    const uint32_t xsb = hx & 0x80000000u;
-    hx &= 0x7fffffffu;
+    const uint32_t bits = libm_bits(x0), hx = bits & 0x7fffffffu;
+    const bool neg = (bits >> 31) != 0;
+    // argument reduction
+    const bool reduce = hx > 0x3eb17218u, unit = hx < 0x3F851592u;
+    const int32_t kg = static_cast<int32_t>(invln2 * x0 + (neg ? -0.5f : 0.5f));
+    const int32_t k = reduce ? (unit ? (neg ? -1 : 1) : kg) : 0;
+    const float t0 = static_cast<float>(k);
+    const float hi = x0 - t0 * ln2_hi, lo = t0 * ln2_lo;
+    const float xr = hi - lo;
+    const float x = reduce ? xr : x0;
+    const float c = reduce ? (hi - xr) - lo : 0.0f;
+    // primary range
+    const float hfx = 0.5f * x, hxs = x * hfx;
+    const float r1 = one + hxs * (Q1 + hxs * (Q2 + hxs * (Q3 + hxs * (Q4 + hxs * Q5))));
+    const float t = 3.0f - r1 * hfx;
+    const float e0 = hxs * ((r1 - t) / (6.0f - x * t));
+    const float res_k0 = x - (x * e0 - hxs);
+    float e = (x * (e0 - c) - c);
+    e -= hxs;
+    const float res_m1 = 0.5f * (x - e) - 0.5f;
+    const float res_p1 = x < -0.25f ? -2.0f * (e - (x + 0.5f)) : one + 2.0f * (x - e);
+    const uint32_t kshift = static_cast<uint32_t>(k) << 23;
+    const float ya = one - (e - x);
+    const float res_far = libm_float(libm_bits(ya) + kshift) - one;
+    const uint32_t ks = static_cast<uint32_t>(k) & 31u;  // shifts below are only used for 0 <= k < 23
+    const float tb = libm_float(0x3f800000u - (0x1000000u >> ks));
+    const float res_lo = libm_float(libm_bits(tb - (e - x)) + kshift);
+    const float tc = libm_float(static_cast<uint32_t>(0x7f - k) << 23);
+    float yc = x - (e + tc);
+    yc += one;
+    const float res_hi = libm_float(libm_bits(yc) + kshift);
+    float r = k == 0 ? res_k0 : k == -1 ? res_m1 : k == 1 ? res_p1 : (k <= -2 || k > 56) ? res_far : k < 23 ? res_lo : res_hi;
+    // |x| < 2^-25
+    const float tt = huge + x0;
+    r = (!reduce && hx < 0x33000000u) ? x0 - (tt - (huge + x0)) : r;
+    // huge and non-finite arguments
     if (hx >= 0x4195b844u) {
         if (hx >= 0x42b17218u) {
-            if (hx > 0x7f800000u) return x + x;
-            if (hx == 0x7f800000u) return xsb == 0 ? x : -1.0f;
-            if (x > o_threshold) return huge * huge;
+            if (hx > 0x7f800000u) return x0 + x0;
+            if (hx == 0x7f800000u) return neg ? -1.0f : x0;
+            if (x0 > o_threshold) return huge * huge;
         }
-        if (xsb != 0) return tiny - one;
+        if (neg) return tiny - one;
     }
-    if (hx > 0x3eb17218u) {
-        if (hx < 0x3F851592u) {
-            if (xsb == 0) { hi = x - ln2_hi; lo = ln2_lo; k = 1; }
-            else { hi = x + ln2_hi; lo = -ln2_lo; k = -1; }
-        } else {
-            k = static_cast<int32_t>(invln2 * x + (xsb == 0 ? 0.5f : -0.5f));
-            t = static_cast<float>(k);
-            hi = x - t * ln2_hi;
-            lo = t * ln2_lo;
-        }
-        x = hi - lo;
-        c = (hi - x) - lo;
-    } else if (hx < 0x33000000u) {
-        t = huge + x;
-        return x - (t - (huge + x));
-    } else {
-        k = 0;
-    }
-    hfx = 0.5f * x;
-    hxs = x * hfx;
-    r1 = one + hxs * (Q1 + hxs * (Q2 + hxs * (Q3 + hxs * (Q4 + hxs * Q5))));
-    t = 3.0f - r1 * hfx;
-    e = hxs * ((r1 - t) / (6.0f - x * t));
-    if (k == 0) return x - (x * e - hxs);
-    e = (x * (e - c) - c);
-    e -= hxs;
-    if (k == -1) return 0.5f * (x - e) - 0.5f;
-    if (k == 1) {
-        if (x < -0.25f) return -2.0f * (e - (x + 0.5f));
-        return one + 2.0f * (x - e);
-    }
-    if (k <= -2 || k > 56) {
-        y = one - (e - x);
-        y = libm_float(libm_bits(y) + (static_cast<uint32_t>(k) << 23));
-        return y - one;
-    }
-    if (k < 23) {
-        t = libm_float(0x3f800000u - (0x1000000u >> k));
-        y = t - (e - x);
-        y = libm_float(libm_bits(y) + (static_cast<uint32_t>(k) << 23));
-    } else {
-        t = libm_float(static_cast<uint32_t>(0x7f - k) << 23);
-        y = x - (e + t);
-        y += one;
-        y = libm_float(libm_bits(y) + (static_cast<uint32_t>(k) << 23));
-    }
-    return y;
+    return r;
 }
-
 __host__ __device__ inline float tanhf_like_libm(float x) {
     const float one = 1.0f, two = 2.0f, tiny = 1.0e-30f;
-    float t, z;
     const uint32_t jx = libm_bits(x), ix = jx & 0x7fffffffu;
     const bool neg = (jx >> 31) != 0;
+    const float ax = libm_float(ix);
+    const bool big = ix >= 0x3f800000u;
+    const float t = expm1f_like_libm(big ? two * ax : -two * ax);
+    const float q = (big ? two : t) / (t + two);
+    float z = big ? one - q : -q;
+    z = ix < 0x41b00000u ? z : one - tiny;
+    float r = neg ? -z : z;
+    r = ix < 0x24000000u ? x * (one + x) : r;
+    r = ix == 0 ? x : r;
     if (ix >= 0x7f800000u) return neg ? one / x - one : one / x + one;
-    if (ix < 0x41b00000u) {
-        if (ix == 0) return x;
-        if (ix < 0x24000000u) return x * (one + x);
-        const float ax = libm_float(ix);
-        if (ix >= 0x3f800000u) { t = expm1f_like_libm(two * ax); z = one - two / (t + two); }
-        else { t = expm1f_like_libm(-two * ax); z = -t / (t + two); }
-    } else {
-        z = one - tiny;
-    }
-    return neg ? -z : z;
+    return r;
 }
 
+// log1pf, its cases side by side like expm1f's (the rare ones, which return early, first).
 __host__ __device__ inline float log1pf_like_libm(float x) {
     const float ln2_hi = 6.9313812256e-01f, ln2_lo = 9.0580006145e-06f, two25 = 3.355443200e+07f, zero = 0.0f;
     const float Lp1 = 6.6666668653e-01f, Lp2 = 4.0000000596e-01f, Lp3 = 2.8571429849e-01f, Lp4 = 2.2222198546e-01f,
                 Lp5 = 1.8183572590e-01f, Lp6 = 1.5313838422e-01f, Lp7 = 1.4798198640e-01f;
-    float hfsq, f = 0.0f, c = 0.0f, s, z, R, u;
-    int32_t k, hx, hu = 0, ax;
-    hx = static_cast<int32_t>(libm_bits(x));
-    ax = hx & 0x7fffffff;
-    k = 1;
+    const int32_t hx = static_cast<int32_t>(libm_bits(x)), ax = hx & 0x7fffffff;
+    // the rare cases first
     if (hx < 0x3ed413d7) {
         if (ax >= 0x3f800000) {
             if (x == -1.0f) return -two25 / zero;
@@ -135,48 +119,38 @@ __host__ __device__ inline float log1pf_like_libm(float x) {
             if (ax < 0x24800000) return x;
             return x - x * x * 0.5f;
         }
-        if (hx > 0 || hx <= static_cast<int32_t>(0xbe95f61fu)) { k = 0; f = x; hu = 1; }
     }
     if (hx >= 0x7f800000) return x + x;
-    if (k != 0) {
-        if (hx < 0x5a000000) {
-            u = 1.0f + x;
-            hu = static_cast<int32_t>(libm_bits(u));
-            k = (hu >> 23) - 127;
-            c = (k > 0) ? 1.0f - (u - x) : x - (u - 1.0f);
-            c /= u;
-        } else {
-            u = x;
-            hu = static_cast<int32_t>(libm_bits(u));
-            k = (hu >> 23) - 127;
-            c = 0;
-        }
-        hu &= 0x007fffff;
-        if (hu < 0x3504f7) {
-            u = libm_float(static_cast<uint32_t>(hu) | 0x3f800000u);
-        } else {
-            k += 1;
-            u = libm_float(static_cast<uint32_t>(hu) | 0x3f000000u);
-            hu = (0x00800000 - hu) >> 2;
-        }
-        f = u - 1.0f;
-    }
-    hfsq = 0.5f * f * f;
-    if (hu == 0) {
-        if (f == zero) {
-            if (k == 0) return zero;
-            c += k * ln2_lo;
-            return k * ln2_hi + c;
-        }
-        R = hfsq * (1.0f - 0.66666666666666666f * f);
-        if (k == 0) return f - R;
-        return k * ln2_hi - ((R - (k * ln2_lo + c)) - f);
-    }
-    s = f / (2.0f + f);
-    z = s * s;
-    R = z * (Lp1 + z * (Lp2 + z * (Lp3 + z * (Lp4 + z * (Lp5 + z * (Lp6 + z * Lp7))))));
-    if (k == 0) return f - (hfsq - s * (hfsq + R));
-    return k * ln2_hi - ((hfsq - (s * (hfsq + R) + (k * ln2_lo + c))) - f);
+    // -0.2929 < x < 0.41422: no scaling
+    const bool direct = hx < 0x3ed413d7 && (hx > 0 || hx <= static_cast<int32_t>(0xbe95f61fu));
+    // otherwise 1 + x = 2^k u with a correction c for the rounding of 1 + x
+    const bool small = hx < 0x5a000000;
+    const float u0 = small ? 1.0f + x : x;
+    int32_t hu = static_cast<int32_t>(libm_bits(u0));
+    int32_t k = (hu >> 23) - 127;
+    float c = small ? ((k > 0) ? 1.0f - (u0 - x) : x - (u0 - 1.0f)) / u0 : 0.0f;
+    hu &= 0x007fffff;
+    const bool low = hu < 0x3504f7;
+    const float u = libm_float(static_cast<uint32_t>(hu) | (low ? 0x3f800000u : 0x3f000000u));
+    k = low ? k : k + 1;
+    hu = low ? hu : (0x00800000 - hu) >> 2;
+    float f = u - 1.0f;
+    // the direct case overrides
+    f = direct ? x : f;
+    k = direct ? 0 : k;
+    hu = direct ? 1 : hu;
+    c = direct ? 0.0f : c;
+    const float fk = static_cast<float>(k);
+    const float hfsq = 0.5f * f * f;
+    // |f| < 2^-20
+    const float Rs = hfsq * (1.0f - 0.66666666666666666f * f);
+    const float near_zero = k == 0 ? zero : fk * ln2_hi + (c + fk * ln2_lo);
+    const float near = k == 0 ? f - Rs : fk * ln2_hi - ((Rs - (fk * ln2_lo + c)) - f);
+    // the general case
+    const float s = f / (2.0f + f), z = s * s;
+    const float R = z * (Lp1 + z * (Lp2 + z * (Lp3 + z * (Lp4 + z * (Lp5 + z * (Lp6 + z * Lp7))))));
+    const float general = k == 0 ? f - (hfsq - s * (hfsq + R)) : fk * ln2_hi - ((hfsq - (s * (hfsq + R) + (fk * ln2_lo + c))) - f);
+    return hu == 0 ? (f == zero ? near_zero : near) : general;
 }
 
 }  // namespace hmr
