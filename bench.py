@@ -388,7 +388,7 @@ def per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP
     shape = [8, 2048, 4096]
     add(None, "rand f32 [8,2048,4096] (Philox on the device, write only)", 4 * N, lambda: h.rand(shape, DT.F32, GPU))
     add(None, "rand bf16 [8,2048,4096]", 2 * N, lambda: h.rand(shape, DT.BF16, GPU))
-    add(None, "randn f32 [8,2048,4096] (Box-Muller, short f64 polynomials)", 4 * N, lambda: h.randn(shape, DT.F32, GPU), 10)
+    add(None, "randn f32 [8,2048,4096] (Box-Muller, f64 polynomials)", 4 * N, lambda: h.randn(shape, DT.F32, GPU), 10)
     add(None, "randint [0, 1024) i64 [8,2048,4096] (no rejection)", 8 * N, lambda: h.randint(0, 1024, shape, DT.I64, GPU), 10)
     add(None, "randint [-5, 6) i64 [8,2048,4096] (rejection: count + write as if none, scan, rewrite only if any + a read-back)", 8 * N,
         lambda: h.randint(-5, 6, shape, DT.I64, GPU), 5)

@@ -87,9 +87,9 @@ int main() {
         if (i % 8 == 0) one(std::ldexp(1.0 - a * 0.5, -static_cast<int>(gen() % 53)), std::floor(b * 8.0) / 8.0 + b * 1e-9);
     }
     std::printf("log %.3g sqrt %.3g turn %.3g\n", worst_log, worst_root, worst_turn);
-    const double limit = std::ldexp(1.0, -36);
+    const double limit = std::ldexp(1.0, -49);
     if (worst_log > limit || worst_root > limit || worst_turn > limit) {
-        std::printf("over 2^-36\n");
+        std::printf("over 2^-49\n");
         return 1;
     }
     std::printf("normal math ok\n");

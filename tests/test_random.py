@@ -305,6 +305,19 @@ def test_normal_samples_stay_within_the_bound(dtype):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [DT.F32, DT.BF16, DT.F16])
+def test_normal_samples_hold_the_bound_where_mean_and_deviation_cancel(dtype):
+    """A sample is mean + std z: where the two cancel the result is small, its ulp with it, and the bound is left
+    with its first term, 6 * 2^-53 * M: an f64 evaluation's accuracy. Millions of samples of distributions whose
+    mean lies a fraction of a deviation from zero, so that thousands of them land next to zero."""
+    for seed, (mean, std) in enumerate(((3.0, 10.0), (-250.0, 1000.0), (1.0, 1.0), (0.001, 0.01))):
+        n = 1 << 22
+        g, c = both(40 + seed, lambda d: h.normal([n], mean, std, dtype, d))
+        m = normal_sizes(40 + seed, n, mean, std)
+        check_within(g, c, extra=NORMAL_K * NORMAL_U * m, what=f"normal {dtype} ({mean}, {std}) [{n}]")
+
+
+@pytest.mark.gpu
 def test_seeded_sampling_on_gpu():
     seeded_sampling(GPU)
 
