@@ -34,8 +34,8 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the bf16 + f32 -> f32 add kernel at configs[1], from rocprofv3 --pmc FETCH_SIZE
 # and --pmc WRITE_SIZE (two runs), each scaled by the reading of a plain copy of known size:
-# (196 642.0 x 1.99963 = 393 212, + 262 144.0 x 1.0) KiB; profiles/map_rows_add_bf16_f32_configs1_chain.md.
-ADD_KERNEL_TRAFFIC_BYTES = 671084544
+# (196 642.0 x 1.99963 = 393 211, + 262 144.0 x 1.0) KiB; profiles/map_rows_add_bf16_f32_configs1_chain.md.
+ADD_KERNEL_TRAFFIC_BYTES = 671083520
 METRIC = "achieved HBM GB/s & % of MI355X peak per op; speedup vs host-CPU reference"
 
 
