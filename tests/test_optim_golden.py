@@ -13,7 +13,7 @@ import numpy as np
 import pytest
 
 from tests import oracle
-from tests.support import DT, GPU, array, bits, h, load_golden, tensor
+from tests.support import DT, GPU, array, assert_bitwise, bits, from_f64, h, load_golden, normal, tensor
 
 h.register_cpu_backend(oracle.backend_address())
 
@@ -221,3 +221,56 @@ def test_coefficients_that_overflow_are_rejected_on_cpu_oracle():
 @pytest.mark.gpu
 def test_coefficients_that_overflow_are_rejected_on_gpu():
     rejected(GPU)
+
+
+def random_runs(seed, device_pair):
+    """Three steps of SGD and of Adam / AdamW with options drawn from a seeded generator, on both devices: the
+    parameter and the state after every step."""
+    cpu, gpu = device_pair
+    rng = np.random.default_rng(0x5EED6000 + seed)
+    for case in range(12):
+        dtype = [DT.F32, DT.BF16, DT.F16, DT.F64][int(rng.integers(0, 4))]
+        shape = [int(rng.choice([1, 3, 17, 64, 1000, 4099]))] if rng.integers(0, 2) else [int(rng.choice([2, 5, 33])), int(rng.choice([7, 128, 513]))]
+        n = int(np.prod(shape))
+        p0 = from_f64(normal(100 * seed + case, n), dtype)
+        grads = [from_f64(normal(100 * seed + case + 1 + s, n, 0.0, 0.3), dtype) for s in range(3)]
+        lr = float(rng.choice([1e-3, 0.05, 0.5]))
+        wd = float(rng.choice([0.0, 1e-2, 0.1]))
+        maximize = bool(rng.integers(0, 2))
+        if rng.integers(0, 2):
+            momentum = float(rng.choice([0.0, 0.9, 0.5]))
+            dampening = float(rng.choice([0.0, 0.1])) if momentum else 0.0
+            nesterov = bool(momentum and dampening == 0.0 and rng.integers(0, 2))
+            what = f"seed {seed} case {case}: sgd {dtype} {shape} lr {lr} wd {wd} momentum {momentum} dampening {dampening} nesterov {nesterov} maximize {maximize}"
+            states = {d: None for d in (cpu, gpu)}
+            params = {d: tensor(p0, dtype, shape, d) for d in (cpu, gpu)}
+            for s in range(3):
+                for d in (cpu, gpu):
+                    params[d], states[d] = h.sgd_step(params[d], tensor(grads[s], dtype, shape, d), states[d], lr=lr, momentum=momentum,
+                                                      dampening=dampening, weight_decay=wd, nesterov=nesterov, maximize=maximize)
+                assert_bitwise(params[gpu], params[cpu], f"{what}: parameter after step {s}")
+                if states[cpu] is not None:
+                    assert_bitwise(states[gpu], states[cpu], f"{what}: momentum buffer after step {s}")
+        else:
+            decoupled, amsgrad = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+            beta1, beta2 = float(rng.choice([0.9, 0.5])), float(rng.choice([0.999, 0.9]))
+            eps = float(rng.choice([1e-8, 1e-4]))
+            what = f"seed {seed} case {case}: adam {dtype} {shape} lr {lr} wd {wd} betas {beta1}, {beta2} eps {eps} amsgrad {amsgrad} decoupled {decoupled} maximize {maximize}"
+            states = {d: None for d in (cpu, gpu)}
+            params = {d: tensor(p0, dtype, shape, d) for d in (cpu, gpu)}
+            for s in range(3):
+                for d in (cpu, gpu):
+                    params[d], states[d] = h.adam_step(params[d], tensor(grads[s], dtype, shape, d), states[d], lr=lr, beta1=beta1, beta2=beta2,
+                                                       eps=eps, weight_decay=wd, amsgrad=amsgrad, maximize=maximize,
+                                                       decoupled_weight_decay=decoupled)
+                assert_bitwise(params[gpu], params[cpu], f"{what}: parameter after step {s}")
+                assert states[gpu][0] == states[cpu][0]
+                for k in (1, 2, 3):
+                    if states[cpu][k] is not None:
+                        assert_bitwise(states[gpu][k], states[cpu][k], f"{what}: state {k} after step {s}")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", range(6))
+def test_random_optimizer_runs_match_the_cpu(seed):
+    random_runs(seed, ("cpu", GPU))
