@@ -137,14 +137,63 @@ def test_gradients_of_larger_tensors_match_the_cpu(dtype):
         "prod_dim with zeros": lambda d: h.grad_prod(g_rows.to(d), small.to(d), small.to(d).prod_dim(1, False), 1, False),
         "sum_to_size": lambda d: h.grad_sum_to_size(g_rows.to(d).reshape([rows, 1]), x.shape),
     }
-    tol = TOL[dtype]
     for name, f in pairs.items():
-        gpu, cpu = f(GPU), f("cpu")
-        assert gpu.device == GPU and gpu.dtype == dtype and gpu.shape == cpu.shape, name
-        a, e = to_f64(array(gpu.contiguous()), dtype).reshape(-1), to_f64(array(cpu.contiguous()), dtype).reshape(-1)
-        nan = np.isnan(a) | np.isnan(e)
-        assert (np.isnan(a) == np.isnan(e)).all(), name
-        with np.errstate(all="ignore"):
-            scale = np.abs(e) + (np.abs(e).max() if name.startswith(("softmax", "log_softmax", "var", "std")) else 0.0)
-            bad = ~nan & ~(np.abs(a - e) <= tol * scale + 1e-300) & ~(a == e)
-        assert not bad.any(), f"{name} {dtype}: element {np.nonzero(bad)[0][0]}: gpu {a[bad][0]!r}, cpu {e[bad][0]!r}"
+        close_to_the_cpu(f(GPU), f("cpu"), dtype, name)
+
+
+def close_to_the_cpu(gpu, cpu, dtype, name):
+    """Every element within the fixture's tolerance for the dtype (relative to the element, for the compositions
+    that subtract also to the largest element), NaNs in the same places."""
+    tol = TOL[dtype]
+    assert gpu.device == GPU and gpu.dtype == dtype and gpu.shape == cpu.shape, name
+    a, e = to_f64(array(gpu.contiguous()), dtype).reshape(-1), to_f64(array(cpu.contiguous()), dtype).reshape(-1)
+    nan = np.isnan(a) | np.isnan(e)
+    assert (np.isnan(a) == np.isnan(e)).all(), name
+    if a.size == 0:
+        return
+    with np.errstate(all="ignore"):
+        scale = np.abs(e) + (np.nanmax(np.abs(e)) if name.startswith(("softmax", "log_softmax", "var", "std")) else 0.0)
+        bad = ~nan & ~(np.abs(a - e) <= tol * scale + 1e-300) & ~(a == e)
+    assert not bad.any(), f"{name} {dtype}: element {np.nonzero(bad)[0][0]}: gpu {a[bad][0]!r}, cpu {e[bad][0]!r}"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", range(6))
+def test_gradients_over_random_shapes_and_dimensions_match_the_cpu(seed):
+    """The same compositions with shapes, dimensions, keepdim and corrections drawn from a seeded generator."""
+    from tests.support import from_f64, normal
+    rng = np.random.default_rng(0x5EED7000 + seed)
+    for case in range(25):
+        dtype = [DT.BF16, DT.F32, DT.F64, DT.F16][int(rng.integers(0, 4))]
+        shape = [int(rng.choice([1, 2, 3, 7, 16, 65, 300])) for _ in range(int(rng.integers(1, 4)))]
+        n, nd = int(np.prod(shape)), len(shape)
+        x = tensor(from_f64(normal(50 * seed + case, n), dtype), dtype).reshape(shape)
+        dims = sorted(int(d) for d in rng.choice(nd, int(rng.integers(1, nd + 1)), replace=False))
+        keep = bool(rng.integers(0, 2))
+        d = int(rng.integers(0, nd))
+        correction = int(rng.integers(0, 3))
+        reduced = x.sum_dim(dims, keep)
+        g_red = tensor(from_f64(normal(51 * seed + case, reduced.num_elements()), dtype), dtype).reshape(reduced.shape)
+        g_full = tensor(from_f64(normal(52 * seed + case, n), dtype), dtype).reshape(shape)
+        one = x.max_dim(d, keep)[0]
+        g_one = tensor(from_f64(normal(53 * seed + case, one.num_elements()), dtype), dtype).reshape(one.shape)
+        what = f"seed {seed} case {case}: {dtype} {shape} dims {dims} keep {keep} along {d} correction {correction}"
+        pairs = {
+            "sum": lambda v: h.grad_sum(g_red.to(v), shape, dims, keep),
+            "mean": lambda v: h.grad_mean(g_red.to(v), shape, dims, keep),
+            "var": lambda v: h.grad_var_std(g_red.to(v), x.to(v), None, dims, correction, keep),
+            "std": lambda v: h.grad_var_std(g_red.to(v), x.to(v), x.to(v).std_dim(dims, correction, keep), dims, correction, keep),
+            "softmax": lambda v: h.grad_softmax(g_full.to(v), x.to(v).softmax(d), d, False),
+            "log_softmax": lambda v: h.grad_softmax(g_full.to(v), x.to(v).log_softmax(d), d, True),
+            "max_dim": lambda v: h.grad_extremum_dim(g_one.to(v), x.to(v).max_dim(d, keep)[1], shape, d, keep),
+            "prod_dim": lambda v: h.grad_prod(g_one.to(v), x.to(v), x.to(v).prod_dim(d, keep), d, keep),
+        }
+        for name, f in pairs.items():
+            try:
+                cpu = f("cpu")
+            except Exception as refusal:
+                with pytest.raises(type(refusal)) as got:
+                    f(GPU)
+                assert str(got.value) == str(refusal), f"{what}: {name}"
+                continue
+            close_to_the_cpu(f(GPU), cpu, dtype, f"{name} ({what})")
