@@ -11,7 +11,8 @@
 // 30-33, 189-219), always evaluated in f64 and rounded to f32 as the CPU does, because GELU's
 // 1 + erf(z) cancels for z << 0. pow of f32 values is the host library's powf restated as well
 // (powf_like_libm.hpp; two arguments, so pinned by sweeps and billions of random pairs rather than by
-// every input). What is left to the device library: every function of F64 tensors.
+// every input). F64 tensors: tanh (and with it gelu_tanh) is the host library's f64 tanh restated
+// (f64_like_libm.hpp, pinned by sampling); the other functions are the device library's.
 // The surrounding arithmetic (1/(1+e), 0.5*x*(1+t), ...) is done in the computation type in the
 // CPU's order, so it contributes no difference of its own.
 #pragma once
@@ -19,6 +20,7 @@
 #include "elem.hpp"
 #include "expf_like_libm.hpp"
 #include "f32_like_libm.hpp"
+#include "f64_like_libm.hpp"
 #include "sinf_cosf_logf_like_libm.hpp"
 #include "powf_like_libm.hpp"
 #include "map.hpp"
@@ -46,7 +48,7 @@ __device__ __forceinline__ typename Comp<T>::C e_exp(typename Comp<T>::C x) {
 template <class T>
 __device__ __forceinline__ typename Comp<T>::C e_tanh(typename Comp<T>::C x) {
     if constexpr (std::is_same_v<typename Comp<T>::C, float>) return tanhf_like_libm(x);
-    else return tanh(x);
+    else return tanh_like_libm(x);  // f64_like_libm.hpp: the host library's, pinned by 480 million sampled inputs
 }
 // log, sin and cos likewise (sinf_cosf_logf_like_libm.hpp).
 template <class T>

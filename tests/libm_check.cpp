@@ -2,7 +2,7 @@
 // host C library's over bit patterns of f32: `libm_check <function> <stride> [fused]` with function one of expf,
 // expm1f, tanhf, log1pf, sinf, cosf, logf walks every stride-th pattern (1: all 2^32) on all hardware threads and prints the number of
 // inputs whose results differ in any bit (a NaN for a NaN counts as equal); powf has two arguments and a mode of its
-// own (below). `fused` (expf, sinf, cosf, logf; default 1)
+// own, the f64 functions tanh and expm1 are sampled (both below). `fused` (expf, sinf, cosf, logf; default 1)
 // picks the form with fused multiply-adds.
 #include <hip/hip_runtime.h>
 
@@ -18,6 +18,7 @@
 #include "f32_like_libm.hpp"
 #include "sinf_cosf_logf_like_libm.hpp"
 #include "powf_like_libm.hpp"
+#include "f64_like_libm.hpp"
 
 template <class Host, class Port>
 static uint64_t count(uint64_t begin, uint64_t end, uint64_t stride, uint32_t *first, Host host, Port port) {
@@ -86,7 +87,47 @@ static uint64_t powf_differences(uint64_t stride) {
     return sum;
 }
 
+// The f64 functions: `libm_check tanh|expm1 <stride>` draws 480 000 000 / stride inputs (arbitrary bits, (-25, 25),
+// (-2, 2) and every binade down to 2^-70, a quarter each).
+static uint64_t f64_differences(bool tanh_not_expm1, uint64_t stride) {
+    const unsigned workers = std::max(1u, std::thread::hardware_concurrency());
+    std::vector<uint64_t> bad(workers, 0);
+    std::vector<std::thread> pool;
+    for (unsigned w = 0; w < workers; ++w) {
+        pool.emplace_back([&, w] {
+            uint64_t state = 0xD1B54A32D192ED03ull * (w + 1);
+            for (uint64_t i = 0; i < 480000000ull / stride / workers; ++i) {
+                state = state * 6364136223846793005ull + 1442695040888963407ull;
+                const uint64_t r = state ^ (state >> 31);
+                const double unit = static_cast<double>(r >> 11) / 9007199254740992.0;
+                double x;
+                switch (i & 3) {
+                    case 0: memcpy(&x, &r, 8); break;
+                    case 1: x = (unit - 0.5) * 50.0; break;
+                    case 2: x = (unit - 0.5) * 4.0; break;
+                    default: x = std::ldexp(unit + 0.5, -static_cast<int>(r % 70)) * ((r & 1024) ? 1 : -1); break;
+                }
+                volatile double xv = x;
+                const double want = tanh_not_expm1 ? tanh(xv) : expm1(xv);
+                const double got = tanh_not_expm1 ? hmr::tanh_like_libm(x) : hmr::expm1_like_libm(x);
+                uint64_t a, b;
+                memcpy(&a, &want, 8);
+                memcpy(&b, &got, 8);
+                bad[w] += a != b && !(want != want && got != got);
+            }
+        });
+    }
+    for (auto &t : pool) t.join();
+    uint64_t sum = 0;
+    for (uint64_t b : bad) sum += b;
+    return sum;
+}
+
 int main(int argc, char **argv) {
+    if (argc >= 3 && (std::string(argv[1]) == "tanh" || std::string(argv[1]) == "expm1")) {
+        std::printf("%llu differ\n", static_cast<unsigned long long>(f64_differences(std::string(argv[1]) == "tanh", strtoull(argv[2], nullptr, 10))));
+        return 0;
+    }
     if (argc >= 3 && std::string(argv[1]) == "powf") {
         const uint64_t stride = strtoull(argv[2], nullptr, 10);
         const bool fused = argc > 3 ? atoi(argv[3]) != 0 : true;

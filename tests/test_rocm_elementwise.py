@@ -126,6 +126,20 @@ def test_half_unary_ops_over_every_input(name, dtype):
     print(f"exhaustive {name} {dtype}: {differ} of 65536 differ, max {worst} ulp")
 
 
+def test_f64_tanh_and_gelu_tanh_have_the_cpus_bits():
+    """tanh of an f64 value is the host library's tanh restated (fdlibm's, with expm1): the CPU's bits for millions
+    of inputs of every range and for the special values."""
+    rng = np.random.default_rng(0x7A9)
+    n = 1 << 21
+    inputs = [rng.uniform(-2.0, 2.0, n), rng.uniform(-25.0, 25.0, n), rng.uniform(-1e-3, 1e-3, n),
+              np.ldexp(rng.uniform(0.5, 1.0, n), -rng.integers(0, 80, n)) * rng.choice([-1.0, 1.0], n),
+              values(DT.F64, n, 78)]
+    for x in inputs:
+        t = tensor(np.asarray(x, dtype=np.float64), DT.F64)
+        for name in ("tanh", "gelu_tanh"):
+            assert_bitwise(getattr(t.to(GPU), name)(), getattr(t, name)(), f"{name} f64")
+
+
 def test_pow_has_the_cpus_bits_on_f32_and_the_halves():
     """pow of f32 values is the host library's powf restated: random pairs of every kind (arbitrary bits, moderate
     bases with exponents that are multiples of 1/8, negative bases with integer exponents, subnormal bases, results
