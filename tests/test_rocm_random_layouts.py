@@ -35,12 +35,19 @@ LARGE_SIZES = [2, 3, 8, 64, 128, 256, 257, 384, 512, 1000, 1024, 2048]
 TINY_SIZES = [0, 0, 1, 1, 2, 3, 4, 5, 8, 17]
 
 
+# Five to eight dimensions of a few elements each, for the seeds from 600 on: more dimensions than the row kernels
+# walk, so the general kernels and the plans for many kept and reduced dimensions.
+DEEP_SIZES = [1, 2, 2, 3, 3, 4, 5, 7]
+
+
 def sizes_of(seed):
+    if 600 <= seed < 700:
+        return DEEP_SIZES
     return TINY_SIZES if 400 <= seed < 500 else (LARGE_SIZES if seed >= 100 else SIZES)
 
 
 def random_shape(rng, limit, sizes=SIZES):
-    ndim = int(rng.integers(1, 5))
+    ndim = int(rng.integers(5, 9)) if sizes is DEEP_SIZES else int(rng.integers(1, 5))
     while True:
         shape = [int(rng.choice(sizes)) for _ in range(ndim)]
         if int(np.prod(shape)) <= limit:
@@ -133,7 +140,7 @@ def overlapping(t):
     return False
 
 
-@pytest.mark.parametrize("seed", list(range(32)) + [100, 101, 102, 103, 400, 401, 402])
+@pytest.mark.parametrize("seed", list(range(32)) + [100, 101, 102, 103, 400, 401, 402, 600, 601, 602])
 def test_random_views_through_every_kernel_family(seed):
     rng = np.random.default_rng(0x5EED0000 + seed)
     dtypes = [DT.F32, DT.BF16, DT.I64, DT.U8, DT.F16, DT.I32, DT.F64, DT.Bool]
@@ -247,7 +254,7 @@ def sprinkle(rng, t, dtype, shape):
     return tensor(from_f64(flat, dtype), dtype, shape)
 
 
-@pytest.mark.parametrize("seed", list(range(12)) + [200, 201, 400, 401, 402])
+@pytest.mark.parametrize("seed", list(range(12)) + [200, 201, 400, 401, 402, 600, 601, 602])
 def test_random_views_through_float_reductions_and_softmax(seed):
     """The reduction and softmax plans pick their kernels from the merged kept and reduced dimensions of the view
     (rows, columns, slices cut across workgroups, the general walk): the same random chains of views as above, float
@@ -332,7 +339,7 @@ def positions(rng, count, below, dtype, shape):
     return tensor(picks, dtype, shape)
 
 
-@pytest.mark.parametrize("seed", list(range(16)) + [300, 301, 400, 401, 402])
+@pytest.mark.parametrize("seed", list(range(16)) + [300, 301, 400, 401, 402, 600, 601, 602])
 def test_random_views_through_the_families_next_to_the_path(seed):
     """flip, triu / tril, the fused optimizer steps, addr, exclusive_cumprod, masked_fill and the index family
     (index_select, gather, scatter_add, index_add) take their operands as views too, and each picks its kernel from
