@@ -36,6 +36,8 @@ HBM_PEAK_GBS = 8000.0
 # and --pmc WRITE_SIZE (two runs), each scaled by the reading of a plain copy of known size:
 # (196 642.0 x 1.99963 = 393 211, + 262 144.0 x 1.0) KiB; profiles/map_rows_add_bf16_f32_configs1_chain.md.
 ADD_KERNEL_TRAFFIC_BYTES = 671083520
+TRAFFIC_SOURCE = ("profiles/map_rows_add_bf16_f32_configs1_chain.md: a constant from that profile's FETCH_SIZE / "
+                  "WRITE_SIZE readings, not a reading of this run")
 METRIC = "achieved HBM GB/s & % of MI355X peak per op; speedup vs host-CPU reference"
 
 
@@ -154,6 +156,7 @@ def main():
     achieved = add_bytes / (ms_add * 1e-3) / 1e9
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": ADD_KERNEL_TRAFFIC_BYTES,
+                "traffic_source": TRAFFIC_SOURCE,
                 "kernel": "map_rows_kernel<FloatBinary<ADD, f32, bf16, f32>> (bf16 + f32 -> f32)",
                 "algorithmic_bytes_per_launch": add_bytes, "us_per_launch": round(ms_add * 1e3, 2)}
 
@@ -161,6 +164,21 @@ def main():
     ops = []
     if args.ops == "all":
         ops = per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP, x, bias, scale, residual, t2)
+
+    # Per config, the op furthest below the roofline among the rows whose inputs and results come from HBM (the
+    # rows "for comparison" left out): carried inside `config`, which the driver's record keeps whole.
+    per_config = {}
+    for key in range(5):
+        judged = [r for r in ops if r["cfg"] == key and r.get("mode") == "hbm" and "for comparison" not in r["op"]]
+        if not judged:
+            continue
+        lowest = min(judged, key=lambda r: r["frac"])
+        per_config[str(key)] = {"rows": len(judged), "lowest_frac": lowest["frac"], "op": lowest["op"].split(" [")[0],
+                                "us": lowest["us"], "highest_frac": max(r["frac"] for r in judged)}
+    cold = next((r for r in ops if r["cfg"] == 1 and r.get("mode") == "hbm" and "residual" in r["op"]), None)
+    if cold is not None:
+        roofline["frac_from_cold_hbm"] = cold["frac"]
+        roofline["us_from_cold_hbm"] = cold["us"]
 
     # ---- CPU baseline: the oracle on one host core, same workload ------------------------------------------
     cpu = None
@@ -196,19 +214,33 @@ def main():
                    "graph_replay": None if graph_ms is None else {
                        "ms_per_step": round(graph_ms, 4), "gbs": round(chain_bytes / (graph_ms * 1e-3) / 1e9, 1),
                        "what": "the same three launches captured into one HIP graph and replayed (not `value`)"},
-                   "seeds": "SplitMix64 0x5EED0001..4"},
+                   "seeds": "SplitMix64 0x5EED0001..4",
+                   "per_config": per_config or None,
+                   "per_config_what": "per BASELINE config, over its rows measured with inputs AND results rotating "
+                                      "through HBM: the lowest fraction of the 8 TB/s peak, its op and time, and the "
+                                      "highest fraction"},
         "roofline": roofline, "cpu_baseline": cpu, "ops": ops,
     }
     print(json.dumps(line))
 
 
 def per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP, x, bias, scale, residual, t2):
-    """[{cfg, op, bytes, us, gbs, frac}] for the ops of BASELINE.json configs[0..4] (cfg = index)."""
-    rows = []
+    """[{cfg, op, mode, bytes, us, gbs, frac}] for the ops of BASELINE.json configs[0..4] (cfg = index) and for the
+    callers built next to the path (cfg null).
 
-    def add(cfg, op, nbytes, fns, iters=50):
-        """fns: one callable, or several over disjoint buffers that are cycled so that a working set
-        smaller than the 256 MB Infinity Cache is read from HBM every time."""
+    mode "hbm": several sets of inputs AND as many result slots in rotation, sized so that the results in rotation
+    and the inputs in rotation each exceed the 256 MB memory-side cache: every byte a call reads comes from HBM and
+    every byte it writes goes there. These rows are each config's figures. mode "cache": the same buffers every
+    call (the result block is the one the previous call wrote), shown beside them: what the same kernel reaches
+    while the memory-side cache absorbs part of the traffic."""
+    rows = []
+    MALL = 256 << 20
+
+    def clone(t):
+        return h.full(t.shape, 0, t.dtype, GPU).copy_(t)
+
+    def add(cfg, op, nbytes, fns, iters=50, mode=None):
+        """fns: one callable, or several over disjoint buffers that are cycled."""
         fns = fns if isinstance(fns, list) else [fns]
         k = [0]
 
@@ -225,89 +257,87 @@ def per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP
             h.synchronize(GPU)
         ms = timed(call, iters, 3)
         gbs = nbytes / (ms * 1e-3) / 1e9
-        rows.append({"cfg": cfg, "op": op, "bytes": nbytes, "us": round(ms * 1e3, 2), "gbs": round(gbs, 1),
+        rows.append({"cfg": cfg, "op": op, "mode": mode, "bytes": nbytes, "us": round(ms * 1e3, 2), "gbs": round(gbs, 1),
                      "frac": round(gbs / HBM_PEAK_GBS, 4)})
 
+    def hbm(cfg, op, nbytes, inputs, fn, in_bytes, out_bytes, iters=50, cache=False):
+        """The op over copies of `inputs` (a tuple of tensors) in rotation, results kept in as many slots; as many
+        sets as it takes for the inputs and the results in rotation to exceed the memory-side cache 1.25 times
+        each (at least three)."""
+        need = lambda b: -(-(MALL * 5 // 4) // b) if b >= (1 << 20) else 0
+        sets = max(3, need(in_bytes), need(out_bytes))
+        copies = [inputs] + [tuple(clone(t) for t in inputs) for _ in range(sets - 1)]
+        kept = [None] * sets
+        add(cfg, f"{op} [{sets} input sets and {sets} results in rotation]", nbytes,
+            [lambda i=i: kept.__setitem__(i, fn(*copies[i])) for i in range(sets)], iters, "hbm")
+        del kept
+        if cache:
+            add(cfg, f"{op} [same buffers]", nbytes, lambda: fn(*inputs), iters, "cache")
+
+    def copy_row(cfg, op, nbytes, source, view_of):
+        """One hmr_copy per call, from three sources into three destinations in rotation."""
+        sources = [source, clone(source), clone(source)]
+        targets = [h.full(view_of(t).shape, 0, t.dtype, GPU) for t in sources]
+        add(cfg, f"{op} [3 sources and 3 destinations in rotation]", nbytes,
+            [lambda i=i: targets[i].copy_(view_of(sources[i])) for i in range(3)], 50, "hbm")
+
     N = x.num_elements()
-    # configs[0]: f32 add [4096, 4096], four disjoint buffer sets (805 MB in rotation).
+    # configs[0]: f32 add [4096, 4096].
     n1 = 4096 * 4096
-    sets = []
-    for i in range(4):
-        a = tensor(uniform(0x5EED0100 + 2 * i, n1, -1.0, 1.0).astype(np.float32), DT.F32, [4096, 4096], GPU)
-        b = tensor(uniform(0x5EED0101 + 2 * i, n1, -1.0, 1.0).astype(np.float32), DT.F32, [4096, 4096], GPU)
-        sets.append((a, b))
-    add(0, "add f32 [4096,4096] (inputs from HBM: four pairs in rotation; the result reuses one block)", 12 * n1, [lambda a=a, b=b: a.add(b) for a, b in sets], 40)
-    a0, b0 = sets[0]
-    add(0, "add f32 [4096,4096] (same buffers, Infinity-Cache-resident)", 12 * n1, lambda: a0.add(b0), 40)
-    del sets
+    a0 = tensor(uniform(0x5EED0100, n1, -1.0, 1.0).astype(np.float32), DT.F32, [4096, 4096], GPU)
+    b0 = tensor(uniform(0x5EED0101, n1, -1.0, 1.0).astype(np.float32), DT.F32, [4096, 4096], GPU)
+    hbm(0, "add f32 [4096,4096]", 12 * n1, (a0, b0), lambda a, b: a.add(b), 8 * n1, 4 * n1, 40, cache=True)
+    del a0, b0
     # configs[1]: the three steps.
-    t1 = x.add(bias)
-    add(1, "x_bf16 + bias_bf16[4096] (inner broadcast; same buffers, 268 MB working set)", 4 * N + 2 * 4096, lambda: x.add(bias))
-    add(1, "t_bf16 * scale_bf16[8,2048,1] (row broadcast; same buffers)", 4 * N + 2 * 8 * 2048, lambda: t1.mul(scale))
-    # The same two steps with three input buffers in rotation: nothing of a call's input is left in the cache.
-    xs = [x, x.mul(1.0), x.mul(1.0)]
-    add(1, "x_bf16 + bias_bf16[4096] (input from HBM: three buffers in rotation; the result reuses one block)", 4 * N + 2 * 4096, [lambda t=t: t.add(bias) for t in xs])
-    add(1, "t_bf16 * scale_bf16[8,2048,1] (input from HBM: three buffers in rotation; the result reuses one block)", 4 * N + 2 * 8 * 2048, [lambda t=t: t.mul(scale) for t in xs])
-    # And with the results kept in three slots, so that a call's result block is not the previous call's either.
-    kept = [None] * len(xs)
-    add(1, "x_bf16 + bias_bf16[4096] (input and result from HBM: three of each in rotation)", 4 * N + 2 * 4096,
-        [lambda i=i: kept.__setitem__(i, xs[i].add(bias)) for i in range(len(xs))])
-    del kept
-    del xs
-    add(1, "t_bf16 + residual_f32 -> f32 (promotion fused)", 10 * N, lambda: t2.add(residual))
+    hbm(1, "x_bf16 + bias_bf16[4096] (inner broadcast)", 4 * N + 2 * 4096, (x,), lambda t: t.add(bias), 2 * N, 2 * N, cache=True)
+    hbm(1, "t_bf16 * scale_bf16[8,2048,1] (row broadcast)", 4 * N + 2 * 8 * 2048, (x,), lambda t: t.mul(scale), 2 * N, 2 * N, cache=True)
+    hbm(1, "t_bf16 + residual_f32 -> f32 (promotion fused)", 10 * N, (t2, residual), lambda t, r: t.add(r), 6 * N, 4 * N, 30, cache=True)
+    # The plain copy of the same bytes under the same rotation: what a 134 MB -> 134 MB stream reaches on this part.
+    copy_row(1, "hmr_copy bf16 [8,2048,4096] (for comparison: the same bytes as x + bias, no arithmetic)", 4 * N, x, lambda t: t)
     h.set_fused_promotion(False)
-    add(1, "t_bf16 + residual_f32 -> f32 (reference style: cast kernel + add, 2 launches)", 18 * N,
-        lambda: t2.add(residual))
+    add(1, "t_bf16 + residual_f32 -> f32 (reference style: cast kernel + add, 2 launches) [same buffers]", 18 * N,
+        lambda: t2.add(residual), 30, "cache")
     h.set_fused_promotion(True)
-    del t1
     # configs[2]: reductions of f32 [16384, 4096] and of its bf16 copy.
     R, C = 16384, 4096
     xf = residual.reshape([R, C])
-    add(2, "sum dim=-1 f32", 4 * N + 4 * R, lambda: xf.sum_dim(-1, False))
-    add(2, "mean dim=-1 f32", 4 * N + 4 * R, lambda: xf.mean_dim(-1, False))
-    add(2, "amax dim=-1 f32 (max_dim: values + i64 indices)", 4 * N + 12 * R, lambda: xf.max_dim(-1, False))
-    add(2, "var(unbiased) dim=-1 f32", 4 * N + 4 * R, lambda: xf.var_dim(-1, 1, False))
-    add(2, "sum dim=0 f32", 4 * N + 4 * C, lambda: xf.sum_dim(0, False))
-    add(2, "mean dim=0 f32", 4 * N + 4 * C, lambda: xf.mean_dim(0, False))
-    add(2, "amax dim=0 f32 (max_dim: values + i64 indices)", 4 * N + 12 * C, lambda: xf.max_dim(0, False))
-    add(2, "var(unbiased) dim=0 f32", 4 * N + 4 * C, lambda: xf.var_dim(0, 1, False))
-    add(2, "sum over all elements f32", 4 * N + 4, lambda: xf.sum())
-    # 134 MB would fit the 256 MB Infinity Cache: three copies in rotation, so that every call reads from HBM.
-    xbs = [xf.to(DT.BF16) for _ in range(3)]
-    add(2, "sum dim=-1 bf16 (input from HBM: three buffers in rotation; the result reuses one block)", 2 * N + 2 * R, [lambda t=t: t.sum_dim(-1, False) for t in xbs])
-    del xbs
-    # configs[3]: permuted bf16 unary; int64 ops.
-    p = tensor(from_f64(normal(0x5EED0400, N, 0.0, 2.0), DT.BF16), DT.BF16, [8, 2048, 32, 128], GPU).permute([0, 2, 1, 3])
-    add(3, "silu bf16 [8,2048,32,128].permute(0,2,1,3) -> contiguous (same buffers, 268 MB working set)", 4 * N, lambda: p.silu())
-    add(3, "gelu(erf) bf16, same view (same buffers)", 4 * N, lambda: p.gelu())
-    ps = [p, p.contiguous().permute([0, 2, 1, 3]).contiguous().permute([0, 2, 1, 3]),
-          p.contiguous().permute([0, 2, 1, 3]).contiguous().permute([0, 2, 1, 3])]
-    assert ps[1].strides == p.strides
-    add(3, "silu bf16, same view (input from HBM: three buffers in rotation; the result reuses one block)", 4 * N, [lambda t=t: t.silu() for t in ps])
-    add(3, "gelu(erf) bf16, same view (input from HBM: three buffers in rotation; the result reuses one block)", 4 * N, [lambda t=t: t.gelu() for t in ps])
-    kept = [None] * len(ps)
-    add(3, "silu bf16, same view (input and result from HBM: three of each in rotation)", 4 * N,
-        [lambda i=i: kept.__setitem__(i, ps[i].silu()) for i in range(len(ps))])
-    del kept
-    pc = p.contiguous()
-    add(3, "silu bf16 on the contiguous copy of the same data (same buffers), for comparison", 4 * N, lambda: pc.silu())
-    del ps, pc
+    for name, nbytes, fn in (
+            ("sum dim=-1 f32", 4 * N + 4 * R, lambda t: t.sum_dim(-1, False)),
+            ("mean dim=-1 f32", 4 * N + 4 * R, lambda t: t.mean_dim(-1, False)),
+            ("amax dim=-1 f32 (max_dim: values + i64 indices)", 4 * N + 12 * R, lambda t: t.max_dim(-1, False)),
+            ("var(unbiased) dim=-1 f32", 4 * N + 4 * R, lambda t: t.var_dim(-1, 1, False)),
+            ("sum dim=0 f32", 4 * N + 4 * C, lambda t: t.sum_dim(0, False)),
+            ("mean dim=0 f32", 4 * N + 4 * C, lambda t: t.mean_dim(0, False)),
+            ("amax dim=0 f32 (max_dim: values + i64 indices)", 4 * N + 12 * C, lambda t: t.max_dim(0, False)),
+            ("var(unbiased) dim=0 f32", 4 * N + 4 * C, lambda t: t.var_dim(0, 1, False)),
+            ("sum over all elements f32", 4 * N + 4, lambda t: t.sum())):
+        hbm(2, name, nbytes, (xf,), fn, 4 * N, 0, 40)
+    xb = xf.to(DT.BF16)
+    hbm(2, "sum dim=-1 bf16", 2 * N + 2 * R, (xb,), lambda t: t.sum_dim(-1, False), 2 * N, 0, 40)
+    del xb
+    # configs[3]: permuted bf16 unary; int64 tensors.
+    p = tensor(from_f64(normal(0x5EED0400, N, 0.0, 2.0), DT.BF16), DT.BF16, [8, 2048, 32, 128], GPU)
+    view = lambda t: t.permute([0, 2, 1, 3])
+    hbm(3, "silu bf16 [8,2048,32,128].permute(0,2,1,3) -> contiguous", 4 * N, (p,), lambda t: view(t).silu(), 2 * N, 2 * N, cache=True)
+    hbm(3, "gelu(erf) bf16, same view", 4 * N, (p,), lambda t: view(t).gelu(), 2 * N, 2 * N, cache=True)
+    copy_row(3, "hmr_copy bf16 of the same view -> contiguous (for comparison: the same bytes, no lookup)", 4 * N, p, view)
+    hbm(3, "silu bf16 on a contiguous tensor of the same size (for comparison)", 4 * N, (p,), lambda t: t.silu(), 2 * N, 2 * N)
     del p
     w1 = words(0x5EED0401, N)
     w2 = words(0x5EED0402, N)
     ia = tensor(((w1 % np.uint64(2001)).astype(np.int64) - 1000), DT.I64, [8, 2048, 4096], GPU)
     ib = tensor(((w2 % np.uint64(2001)).astype(np.int64) - 1000), DT.I64, [8, 2048, 4096], GPU)
     del w1, w2
-    add(3, "bitwise_and i64", 24 * N, lambda: ia.bitwise_and(ib))
-    add(3, "greater i64 -> bool", 17 * N, lambda: ia.greater(ib))
+    hbm(3, "bitwise_and i64", 24 * N, (ia, ib), lambda a, b: a.bitwise_and(b), 16 * N, 8 * N, 20)
+    hbm(3, "greater i64 -> bool", 17 * N, (ia, ib), lambda a, b: a.greater(b), 16 * N, N, 20)
     mask = ia.greater(ib)
-    add(3, "where(mask, a, b) i64", 25 * N, lambda: h.where_(mask, ia, ib))
+    hbm(3, "where(mask, a, b) i64", 25 * N, (mask, ia, ib), lambda m, a, b: h.where_(m, a, b), 17 * N, 8 * N, 20)
     del ia, ib, mask
     # configs[4] case 1: bf16 logits [4096, 32000].
     n5a = 4096 * 32000
     logits = tensor(from_f64(normal(0x5EED0500, n5a, 0.0, 3.0), DT.BF16), DT.BF16, [4096, 32000], GPU)
-    add(4, "softmax bf16 [4096,32000]", 4 * n5a, lambda: logits.softmax(-1))
-    add(4, "log_softmax bf16 [4096,32000]", 4 * n5a, lambda: logits.log_softmax(-1))
+    hbm(4, "softmax bf16 [4096,32000]", 4 * n5a, (logits,), lambda t: t.softmax(-1), 2 * n5a, 2 * n5a, 30)
+    hbm(4, "log_softmax bf16 [4096,32000]", 4 * n5a, (logits,), lambda t: t.log_softmax(-1), 2 * n5a, 2 * n5a, 30)
     del logits
     # configs[4] case 2: causal f32 scores [32, 2048, 2048].
     n5b = 32 * 2048 * 2048
@@ -315,8 +345,8 @@ def per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP
     s[:, np.triu_indices(2048, 1)[0], np.triu_indices(2048, 1)[1]] = -np.inf
     scores = tensor(s, DT.F32, [32, 2048, 2048], GPU)
     del s
-    add(4, "softmax f32 [32,2048,2048] causal", 8 * n5b, lambda: scores.softmax(-1))
-    add(4, "log_softmax f32 [32,2048,2048] causal", 8 * n5b, lambda: scores.log_softmax(-1))
+    hbm(4, "softmax f32 [32,2048,2048] causal", 8 * n5b, (scores,), lambda t: t.softmax(-1), 4 * n5b, 4 * n5b, 20)
+    hbm(4, "log_softmax f32 [32,2048,2048] causal", 8 * n5b, (scores,), lambda t: t.log_softmax(-1), 4 * n5b, 4 * n5b, 20)
     # The callers next to the path (cfg null: not a BASELINE config): the optimizers' single-rounding steps on
     # 67 108 864 parameters, a whole SGD / Adam update (bytes = the sum over its kernels), triangles of the causal
     # scores and flips.

@@ -22,11 +22,9 @@ struct hmr_context {
     hipStream_t stream = nullptr;
     int compute_units = 256;  // multiProcessorCount of the device (256 on MI355X), for grid sizing
     // Result tables of the 16-bit unary operations (one 128 KiB table per operation and dtype, every
-    // input pattern -> its output pattern). The block is allocated at the first use and lives as long
-    // as the context; a table is filled, on `stream`, by the first call that needs it.
-    std::mutex table_lock;
+    // input pattern -> its output pattern): allocated and filled by hmr_context_create, read-only afterwards,
+    // freed with the context.
     void *tables = nullptr;
-    uint64_t tables_filled = 0;  // bit per table
     // Device address, on this context's GPU, of the library's static block for partial results
     // (hmr_reduce_static). Each GPU holds its own copy of the block at its own address.
     void *reduce_scratch = nullptr;
@@ -53,6 +51,10 @@ hmr_status hip_failure(hipError_t error, const char *what) noexcept;
 // Looks up where the static block of hmr_reduce_static lives on the current device and keeps the address
 // in the context. Called once per context, with its device current (defined beside the block, reduce.hip).
 hmr_status bind_reduce_scratch(hmr_context &ctx);
+
+// Allocates the tables of the 16-bit unary operations on the context's GPU, fills them on its stream and waits
+// for the fills. Called once per context, after its stream exists (defined beside the operations, ew_unary.hip).
+hmr_status build_unary_tables(hmr_context &ctx);
 
 // ---- one entry point's stay in the library ---------------------------------------------------------------
 

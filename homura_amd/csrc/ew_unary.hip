@@ -11,23 +11,7 @@ constexpr int kFirstTableOp = HMR_UNARY_EXP, kLastTableOp = HMR_UNARY_GELU_TANH;
 constexpr int kTableOps = kLastTableOp - kFirstTableOp + 1;
 constexpr int kTableSlots = 2 * kTableOps;  // f16, bf16
 
-bool is_table_op(int op, int dtype) {
-    return (dtype == HMR_F16 || dtype == HMR_BF16) && op >= kFirstTableOp && op <= kLastTableOp;
-}
 int table_slot(int op, int dtype) { return (dtype == HMR_BF16 ? kTableOps : 0) + (op - kFirstTableOp); }
-
-// Allocates the context's block of tables at the first use.
-hmr_status ensure_tables(hmr_context_t ctx) {
-    std::lock_guard<std::mutex> lock(ctx->table_lock);
-    if (ctx->tables != nullptr) return HMR_OK;
-    Visit v;
-    if (hmr_status s = v.use_device(ctx->device)) return s;
-    void *p = nullptr;
-    if (hmr_status s = v.hip(hipMalloc(&p, kTableSlots * kTableBytes), "hipMalloc(&p, kTableSlots * kTableBytes)")) return s;
-    ctx->tables = p;
-    ctx->tables_filled = 0;
-    return HMR_OK;
-}
 
 using FloatOps = std::integer_sequence<int, HMR_UNARY_NEG, HMR_UNARY_ABS, HMR_UNARY_SIGN, HMR_UNARY_RELU,
                                        HMR_UNARY_EXP, HMR_UNARY_LOG, HMR_UNARY_SQRT, HMR_UNARY_RSQRT,
@@ -64,17 +48,7 @@ bool pick_unary(hmr_context_t ctx, int op, int out_dtype, int dtype, const MapCa
             if constexpr (sizeof(T) == 2 && decltype(o)::value >= kFirstTableOp && decltype(o)::value <= kLastTableOp) {
                 if (ctx->tables != nullptr && table_applies<F>(call)) {
                     const int slot = table_slot(op, dtype);
-                    uint16_t *table = reinterpret_cast<uint16_t *>(static_cast<char *>(ctx->tables) + slot * kTableBytes);
-                    {
-                        // The fill is queued, under the lock, on the context's one stream: ahead of every
-                        // lookup of this table that any thread queues afterwards.
-                        std::lock_guard<std::mutex> lock(ctx->table_lock);
-                        if (!(ctx->tables_filled >> slot & 1u)) {
-                            launch_table_fill<F>(table, stream);
-                            ctx->tables_filled |= uint64_t{1} << slot;
-                        }
-                    }
-                    launch_table<F>(call, table, stream);
+                    launch_table<F>(call, reinterpret_cast<uint16_t *>(static_cast<char *>(ctx->tables) + slot * kTableBytes), stream);
                     return;
                 }
             }
@@ -85,6 +59,42 @@ bool pick_unary(hmr_context_t ctx, int op, int out_dtype, int dtype, const MapCa
 }
 
 }  // namespace
+
+// Every table of the context, allocated and filled before hmr_context_create returns, so that hmr_unary never
+// allocates and never queues anything but the operation itself (a caller may be capturing the stream into a
+// graph, where a fill would be recorded instead of run). 28 tables of 128 KiB; a fill runs the operation's own
+// functor over the 65 536 patterns.
+hmr_status build_unary_tables(hmr_context &ctx) {
+    Visit v;
+    if (hmr_status s = v.use_device(ctx.device)) return s;
+    void *block = nullptr;
+    if (hmr_status s = v.hip(hipMalloc(&block, kTableSlots * kTableBytes), "hipMalloc(&tables, kTableSlots * kTableBytes)")) return s;
+    (void)hipGetLastError();
+    const auto fill = [&](auto t) {
+        using T = typename decltype(t)::type;
+        const int dtype = std::is_same_v<T, bf16_t> ? HMR_BF16 : HMR_F16;
+        for (int op = kFirstTableOp; op <= kLastTableOp; ++op) {
+            with_code(op, FloatOps{}, [&](auto o) {
+                if constexpr (decltype(o)::value >= kFirstTableOp && decltype(o)::value <= kLastTableOp) {
+                    using F = UnaryFloat<decltype(o)::value, T>;
+                    launch_table_fill<F>(reinterpret_cast<uint16_t *>(static_cast<char *>(block) + table_slot(op, dtype) * kTableBytes),
+                                         ctx.stream);
+                }
+            });
+        }
+    };
+    fill(TypeTag<f16_t>{});
+    fill(TypeTag<bf16_t>{});
+    hipError_t ran = hipGetLastError();
+    if (ran == hipSuccess) ran = hipStreamSynchronize(ctx.stream);
+    if (ran != hipSuccess) {
+        (void)hipFree(block);
+        return v.hip(ran, "filling the tables of the 16-bit unary operations");
+    }
+    ctx.tables = block;
+    return HMR_OK;
+}
+
 }  // namespace hmr
 
 extern "C" hmr_status hmr_unary(hmr_context_t ctx, int32_t op, const hmr_tensor_desc *out,
@@ -95,12 +105,6 @@ extern "C" hmr_status hmr_unary(hmr_context_t ctx, int32_t op, const hmr_tensor_
             ctx, "unary", 2, descs, nullptr,
             [&](const hmr::MapCall &call, hipStream_t stream) {
                 return hmr::pick_unary(ctx, op, out->dtype, src->dtype, call, stream);
-            },
-            [&](const hmr::MapCall &call) {
-                if (out->dtype == src->dtype && hmr::is_table_op(op, src->dtype) && call.n >= hmr::kTableMinElements) {
-                    return hmr::ensure_tables(ctx);
-                }
-                return HMR_OK;
             });
     });
 }

@@ -41,6 +41,16 @@
 namespace hmr {
 
 constexpr int kBlock = 256;      // 4 waves of 64
+#ifndef HMR_ROWS_BLOCK
+#define HMR_ROWS_BLOCK 64
+#endif
+#ifndef HMR_ROWS_U
+#define HMR_ROWS_U 2
+#endif
+#ifndef HMR_BIG_NT
+#define HMR_BIG_NT 1
+#endif
+constexpr int kRowsBlock = HMR_ROWS_BLOCK;  // lanes of a workgroup of the rows kernel
 constexpr int kFastDims = 6;     // merged dimensions the 32-bit kernels take
 constexpr int kMaxOperands = 4;  // output + 3 inputs
 // The vector kernels mark their 128-bit accesses nontemporal (see load_tile). The hint has to be
@@ -114,7 +124,8 @@ struct RowsArgs {
     uint64_t cbits[NOPS];
     uint32_t const_mask;   // bit k: operand k is a constant
     uint32_t bcast_mask;   // bit k: operand k has inner stride 0
-    uint32_t gather;       // nonzero: 2-byte output tiles of eight lanes leave as one 16-byte store (2: nontemporal)
+    uint32_t gather;       // nonzero: 2-byte output tiles of eight lanes leave as one 16-byte store
+    uint32_t out32;        // nonzero: every byte offset into the output fits 32 bits
     int64_t n;             // elements
     uint32_t inner;        // size of the innermost dimension
     int32_t nouter;        // outer dimensions (0 for contiguous)
@@ -171,6 +182,35 @@ __device__ __forceinline__ void load_tile(const char *p, T (&r)[V]) {
     }
 }
 
+// Where a kernel's 16-byte stores go. They write through the compute die's L2 (scope bits sc0 sc1 on the store):
+// an L2 that keeps the dirty lines of a stream writes them back in bursts that the loads wait behind (measured on
+// MI355X, a 134 MB -> 134 MB stream whose buffers come from HBM: plain stores 46 us, nontemporal ones 43.7,
+// write-through ones 41.7; an f32 add of 3 x 67 MB 31.7 / 31.5 / 29.4 us), and the memory-side cache still keeps the
+// result for the next kernel (the same stream reading what the previous launch wrote: 39.3 / 43.5 / 37.2 us). The
+// scope bits are reachable through the buffer form of the store only, whose offset has 32 bits: an output that
+// spans more (`narrow` false) takes nontemporal global stores.
+struct OutStores {
+    __amdgpu_buffer_rsrc_t rsrc;
+    char *base;
+    bool narrow;
+    __device__ __forceinline__ OutStores(char *out, bool fits32)
+        : rsrc(__builtin_amdgcn_make_buffer_rsrc(out, 0, -1, 0x00020000)), base(out), narrow(fits32) {}
+    // Stores `w` at byte offset `at` of the output.
+    __device__ __forceinline__ void put16(int64_t at, u32x4 w) const {
+        constexpr int kSc0Sc1 = 17;
+        if (narrow) __builtin_amdgcn_raw_buffer_store_b128(w, rsrc, static_cast<int>(static_cast<uint32_t>(at)), 0, kSc0Sc1);
+        else __builtin_nontemporal_store(w, reinterpret_cast<u32x4 *>(base + at));
+    }
+};
+// The largest span of an output that `OutStores` addresses with 32 bits.
+constexpr int64_t kNarrowSpanBytes = (int64_t{1} << 32) - 64;
+
+template <int MODE>
+__device__ __forceinline__ void store16(u32x4 *q, u32x4 w) {
+    if constexpr (MODE == 1) __builtin_nontemporal_store(w, q);
+    else *q = w;
+}
+
 template <class T, int V, bool NT = false>
 __device__ __forceinline__ void store_tile(char *p, const T (&r)[V]) {
     constexpr int bytes = V * static_cast<int>(sizeof(T));
@@ -180,8 +220,7 @@ __device__ __forceinline__ void store_tile(char *p, const T (&r)[V]) {
             u32x4 w;
             __builtin_memcpy(&w, reinterpret_cast<const char *>(r) + 16 * i, 16);
             u32x4 *q = reinterpret_cast<u32x4 *>(p) + i;
-            if constexpr (NT) __builtin_nontemporal_store(w, q);
-            else *q = w;
+            store16<NT ? 1 : 0>(q, w);
         }
     } else if constexpr (bytes == 8) {
         uint2 w;
@@ -207,8 +246,7 @@ __device__ __forceinline__ void store_tile(char *p, const T (&r)[V]) {
 //   pair      lanes 2k:  own bytes + those of lane 2k+1        (quad_perm [1,0,3,2])
 //   next_pair lanes 4k:  the pair of lane 4k+2                 (quad_perm [2,3,0,1])
 //   far       lanes 8k:  pair and next_pair of lane 8k+4       (row_shl:4)
-template <bool NT>
-__device__ __forceinline__ void store_eight_lanes(char *p, uint16_t own) {
+__device__ __forceinline__ void store_eight_lanes(const OutStores &out, int64_t at, uint16_t own) {
     constexpr int kSwapPairs = 1 | (0 << 2) | (3 << 4) | (2 << 6), kSwapHalves = 2 | (3 << 2) | (0 << 4) | (1 << 6);
     constexpr int kRowShl4 = 0x104;
     const int x = static_cast<int>(own);
@@ -219,9 +257,7 @@ __device__ __forceinline__ void store_eight_lanes(char *p, uint16_t own) {
     if ((threadIdx.x & 7u) == 0) {
         u32x4 w = {static_cast<uint32_t>(pair), static_cast<uint32_t>(next_pair), static_cast<uint32_t>(far0),
                    static_cast<uint32_t>(far1)};
-        u32x4 *q = reinterpret_cast<u32x4 *>(p);
-        if constexpr (NT) __builtin_nontemporal_store(w, q);
-        else *q = w;
+        out.put16(at, w);
     }
 }
 
@@ -242,13 +278,25 @@ constexpr int size_or_zero() {
     else return static_cast<int>(sizeof(T));
 }
 
+// Bit k of F::kConstantInputs (when a functor has it): input k only ever arrives as a kernel-argument constant.
+template <class F, class = void>
+struct ConstantInputs {
+    static constexpr uint32_t mask = 0;
+};
+template <class F>
+struct ConstantInputs<F, std::void_t<decltype(F::kConstantInputs)>> {
+    static constexpr uint32_t mask = F::kConstantInputs;
+};
+
 template <class F>
 struct MapTraits {
     static constexpr int N = F::N;
+    static constexpr uint32_t constant = ConstantInputs<F>::mask;
     static constexpr int so = static_cast<int>(sizeof(typename F::Out));
-    static constexpr int s0 = size_or_zero<typename F::In0>();
-    static constexpr int s1 = size_or_zero<typename F::In1>();
-    static constexpr int s2 = size_or_zero<typename F::In2>();
+    // Sizes of the operands that move through memory (0: none, or a constant).
+    static constexpr int s0 = (constant & 1u) ? 0 : size_or_zero<typename F::In0>();
+    static constexpr int s1 = (constant & 2u) ? 0 : size_or_zero<typename F::In1>();
+    static constexpr int s2 = (constant & 4u) ? 0 : size_or_zero<typename F::In2>();
     static constexpr int cmin(int a, int b) { return (b != 0 && b < a) ? b : a; }
     static constexpr int cmax(int a, int b) { return b > a ? b : a; }
     static constexpr int narrow = cmin(cmin(cmin(so, s0), s1), s2);
@@ -260,7 +308,7 @@ struct MapTraits {
     // different cache lines, which with streaming loads multiplies the traffic.
     static constexpr int V = 16 / wide;
     // Tiles per lane per pass: aim at 64 bytes of the widest operand in flight.
-    static constexpr int U = (V * wide >= 64) ? 1 : 64 / (V * wide);
+    static constexpr int U = HMR_ROWS_U ? HMR_ROWS_U : ((V * wide >= 64) ? 1 : 64 / (V * wide));
 };
 
 template <class F>
@@ -337,11 +385,16 @@ template <class T, int V, bool STREAM = kStreamLoads>
 __device__ __forceinline__ typename Chunk<T, V>::Raw load_chunk(const char *p, bool splat, int &low) {
     using Raw = typename Chunk<T, V>::Raw;
     constexpr int bytes = Chunk<T, V>::bytes;
+    if constexpr (std::is_same_v<T, Unused>) {
+        low = 0;
+        return Unused{};
+    } else {
     // Pointer arithmetic only: an integer-to-pointer cast would lose the global address space.
     low = static_cast<int>(reinterpret_cast<uintptr_t>(p) & static_cast<uintptr_t>(bytes - 1));
     const Raw *q = reinterpret_cast<const Raw *>(splat ? p - low : p);
     if constexpr (STREAM) return __builtin_nontemporal_load(q);
     else return *q;
+    }
 }
 
 // The 32-bit word `wi` of a chunk, chosen with selects.
@@ -362,11 +415,16 @@ __device__ __forceinline__ uint32_t chunk_word(Raw raw, int wi) {
 
 // Turns a loaded chunk into the tile's V elements: as loaded (dense), or V copies of the element
 // at byte offset `low` (splat), or V copies of the constant.
-template <class T, int V>
-__device__ __forceinline__ void unpack_chunk(typename Chunk<T, V>::Raw raw, bool splat, int low, bool is_const,
+// L: what was loaded for the input (Unused for an input that is always a constant).
+template <class T, class L, int V>
+__device__ __forceinline__ void unpack_chunk(typename Chunk<L, V>::Raw raw, bool splat, int low, bool is_const,
                                              uint64_t cbits, T (&r)[V]) {
     if constexpr (std::is_same_v<T, Unused>) {
         return;
+    } else if constexpr (std::is_same_v<L, Unused>) {
+        const T v = from_cbits<T>(cbits);
+#pragma unroll
+        for (int i = 0; i < V; ++i) r[i] = v;
     } else {
         if (!splat) {
             __builtin_memcpy(r, &raw, sizeof(raw));
@@ -412,25 +470,29 @@ __device__ __forceinline__ void read_ragged(T (&r)[V], const char *base, uint64_
 // CACHED: bit k set = input k is loaded through the caches (a broadcast operand, read by many waves); the other
 // inputs stream past them with nontemporal loads. The choice has to be made at compile time: loads that differ
 // only in the hint are folded into one plain load.
-// NTSTORE: nontemporal stores, for outputs far larger than the memory-side cache (16-byte stores only).
-template <class F, bool FLAT, int CACHED = 0, bool NTSTORE = false>
-__global__ void __launch_bounds__(kBlock) map_rows_kernel(RowsArgs<F::N + 1> a) {
+template <class F, bool FLAT, int CACHED = 0>
+__global__ void __launch_bounds__(kRowsBlock) map_rows_kernel(RowsArgs<F::N + 1> a) {
     using T = MapTraits<F>;
     constexpr int V = T::V, U = T::U, N = F::N;
     using Out = typename F::Out;
     using A = typename F::In0;
     using B = typename F::In1;
     using C = typename F::In2;
+    // What is loaded for an input: nothing for one that is always a constant.
+    using LA = std::conditional_t<(T::constant & 1u) != 0, Unused, A>;
+    using LB = std::conditional_t<(T::constant & 2u) != 0, Unused, B>;
+    using LC = std::conditional_t<(T::constant & 4u) != 0, Unused, C>;
     using Off = std::conditional_t<FLAT, int64_t, uint32_t>;
     const F f = make_functor<F>(a.cbits);
+    const OutStores out(a.ptr[0], a.out32 != 0);
     const int64_t tiles = (a.n + V - 1) / V;
     const int64_t whole = a.n / V;  // tiles [0, whole) have all V elements
     const bool c0 = a.const_mask & 2u, c1 = a.const_mask & 4u, c2 = a.const_mask & 8u;
     // "splat": the operand contributes one element per tile (stride 0 inside the tile, or a constant).
     const bool s0 = (a.bcast_mask | a.const_mask) & 2u, s1 = (a.bcast_mask | a.const_mask) & 4u,
                s2 = (a.bcast_mask | a.const_mask) & 8u;
-    for (int64_t base = static_cast<int64_t>(blockIdx.x) * (U * kBlock); base < tiles;
-         base += static_cast<int64_t>(gridDim.x) * (U * kBlock)) {
+    for (int64_t base = static_cast<int64_t>(blockIdx.x) * (U * kRowsBlock); base < tiles;
+         base += static_cast<int64_t>(gridDim.x) * (U * kRowsBlock)) {
         const int64_t t0 = base + threadIdx.x;
         // Element offsets of tile t in each operand.
         auto offsets = [&](int64_t t, Off(&off)[4]) {
@@ -459,24 +521,24 @@ __global__ void __launch_bounds__(kBlock) map_rows_kernel(RowsArgs<F::N + 1> a) 
                 }
             }
         };
-        if (base + U * kBlock <= whole) {
+        if (base + U * kRowsBlock <= whole) {
             // Whole pass: addresses, then all loads, then arithmetic and stores.
-            typename Chunk<A, V>::Raw wa[U];
-            typename Chunk<B, V>::Raw wb[U];
-            typename Chunk<C, V>::Raw wc[U];
+            typename Chunk<LA, V>::Raw wa[U];
+            typename Chunk<LB, V>::Raw wb[U];
+            typename Chunk<LC, V>::Raw wc[U];
             int la[U], lb[U], lc[U];
             Off oo[U];
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 Off off[4];
-                offsets(t0 + static_cast<int64_t>(u) * kBlock, off);
+                offsets(t0 + static_cast<int64_t>(u) * kRowsBlock, off);
                 oo[u] = off[0];
-                wa[u] = load_chunk<A, V, kStreamLoads && !(CACHED & 1)>(a.ptr[1] + static_cast<int64_t>(off[1]) * static_cast<int64_t>(sizeof(A)), s0, la[u]);
+                wa[u] = load_chunk<LA, V, kStreamLoads && !(CACHED & 1)>(a.ptr[1] + static_cast<int64_t>(off[1]) * static_cast<int64_t>(sizeof(A)), s0, la[u]);
                 if constexpr (N >= 2) {
-                    wb[u] = load_chunk<B, V, kStreamLoads && !(CACHED & 2)>(a.ptr[2] + static_cast<int64_t>(off[2]) * static_cast<int64_t>(sizeof(B)), s1, lb[u]);
+                    wb[u] = load_chunk<LB, V, kStreamLoads && !(CACHED & 2)>(a.ptr[2] + static_cast<int64_t>(off[2]) * static_cast<int64_t>(sizeof(B)), s1, lb[u]);
                 }
                 if constexpr (N >= 3) {
-                    wc[u] = load_chunk<C, V, kStreamLoads && !(CACHED & 4)>(a.ptr[3] + static_cast<int64_t>(off[3]) * static_cast<int64_t>(sizeof(C)), s2, lc[u]);
+                    wc[u] = load_chunk<LC, V, kStreamLoads && !(CACHED & 4)>(a.ptr[3] + static_cast<int64_t>(off[3]) * static_cast<int64_t>(sizeof(C)), s2, lc[u]);
                 }
             }
 #pragma unroll
@@ -484,30 +546,33 @@ __global__ void __launch_bounds__(kBlock) map_rows_kernel(RowsArgs<F::N + 1> a) 
                 A ra[V];
                 B rb[V];
                 C rc[V];
-                unpack_chunk<A, V>(wa[u], s0, la[u], c0, a.cbits[1], ra);
-                if constexpr (N >= 2) unpack_chunk<B, V>(wb[u], s1, lb[u], c1, a.cbits[2], rb);
-                if constexpr (N >= 3) unpack_chunk<C, V>(wc[u], s2, lc[u], c2, a.cbits[3], rc);
+                unpack_chunk<A, LA, V>(wa[u], s0, la[u], c0, a.cbits[1], ra);
+                if constexpr (N >= 2) unpack_chunk<B, LB, V>(wb[u], s1, lb[u], c1, a.cbits[2], rb);
+                if constexpr (N >= 3) unpack_chunk<C, LC, V>(wc[u], s2, lc[u], c2, a.cbits[3], rc);
                 Out ro[V];
 #pragma unroll
                 for (int i = 0; i < V; ++i) ro[i] = apply(f, ra[i], rb[i], rc[i]);
-                char *po = a.ptr[0] + static_cast<int64_t>(oo[u]) * static_cast<int64_t>(sizeof(Out));
+                const int64_t at = static_cast<int64_t>(oo[u]) * static_cast<int64_t>(sizeof(Out));
                 if constexpr (V * sizeof(Out) == 2) {
                     if (a.gather) {
                         uint16_t w;
                         __builtin_memcpy(&w, ro, 2);
-                        // Two forms, as the hint is a property of the instruction: a call larger than the
-                        // memory-side cache stores past it (i64 > i64 over 67M elements: 185 -> 176 us).
-                        if (a.gather == 2) store_eight_lanes<true>(po, w);
-                        else store_eight_lanes<false>(po, w);
+                        store_eight_lanes(out, at, w);
                         continue;
                     }
                 }
-                store_tile<Out, V, kStreamStores || NTSTORE>(po, ro);
+                if constexpr (V * sizeof(Out) == 16) {
+                    u32x4 w;
+                    __builtin_memcpy(&w, ro, 16);
+                    out.put16(at, w);
+                } else {
+                    store_tile<Out, V, false>(a.ptr[0] + at, ro);
+                }
             }
         } else {
             // Ragged pass (the last workgroup): tile by tile, partial tiles element by element.
             for (int u = 0; u < U; ++u) {
-                const int64_t t = t0 + static_cast<int64_t>(u) * kBlock;
+                const int64_t t = t0 + static_cast<int64_t>(u) * kRowsBlock;
                 if (t >= tiles) break;
                 const int64_t rem = a.n - t * V;
                 const int valid = rem >= V ? V : static_cast<int>(rem);
@@ -880,6 +945,10 @@ template <class F>
 int pick_variant(const MapCall &c) {
     using T = MapTraits<F>;
     constexpr int sizes[4] = {T::so, T::s0, T::s1, T::s2};
+    // An input the functor declares constant, given as a tensor: only the general kernels read it as one.
+    for (int k = 1; k < c.nops; ++k) {
+        if (((T::constant >> (k - 1)) & 1u) && !c.is_const[k]) return c.ndim <= kFastDims && fits_32(c) ? 2 : 3;
+    }
     // A reversed dimension (negative input stride, hmr_flip only) goes through the general kernels.
     for (int k = 1; k < c.nops; ++k) {
         for (int d = 0; d < c.ndim && !c.is_const[k]; ++d) {
@@ -954,9 +1023,11 @@ RowsArgs<F::N + 1> rows_args(const MapCall &c, int variant) {
     if (T::V * T::so == 2 && reinterpret_cast<uintptr_t>(c.ptr[0]) % 16 == 0) {
         bool whole = variant == 0 || c.size[last] % (8 * T::V) == 0;
         for (int d = 0; whole && variant != 0 && d < last; ++d) whole = (c.stride[0][d] * T::so) % 16 == 0;
-        const int64_t moved = c.n * (T::so + T::s0 + T::s1 + T::s2);
-        a.gather = whole ? (moved > kCacheResidentBytes ? 2u : 1u) : 0u;
+        a.gather = whole ? 1u : 0u;
     }
+    int64_t span = 1;  // elements from the output's first to one past its last
+    for (int d = 0; d < c.ndim; ++d) span += (c.size[d] - 1) * (c.stride[0][d] < 0 ? -c.stride[0][d] : c.stride[0][d]);
+    a.out32 = span * T::so <= kNarrowSpanBytes && !(HMR_BIG_NT && c.n * T::so >= kStreamStoreBytes) ? 1u : 0u;
     if (variant == 0) {
         a.inner = static_cast<uint32_t>(c.n < (int64_t{1} << 31) ? c.n : 0);
         a.nouter = 0;
@@ -1130,7 +1201,7 @@ void launch_map(const MapCall &c, hipStream_t stream) {
     if (variant <= 1) {
         RowsArgs<NOPS> a = rows_args<F>(c, variant);
         int64_t tiles = (c.n + T::V - 1) / T::V;
-        unsigned grid = grid_for(tiles, int64_t{T::U} * kBlock);
+        unsigned grid = grid_for(tiles, int64_t{T::U} * kRowsBlock);
         // Which inputs are broadcast (a zero stride in some dimension). Three patterns get kernels of their own:
         // every input (an outer product), the first one only, the second one only (x + bias, x * scale).
         int reused = 0, inputs = 0;
@@ -1144,41 +1215,27 @@ void launch_map(const MapCall &c, hipStream_t stream) {
         auto run = [&](auto flat) {
             constexpr bool kFlat = decltype(flat)::value;
             if constexpr (F::N >= 2) {
-                // A call whose operands all fit in the memory-side cache together: what the previous kernel left
-                // there (or this one, called again) is found again only by cached loads.
-                constexpr int sizes[4] = {T::so, T::s0, T::s1, T::s2};
-                int64_t bytes = c.n * sizes[0];
-                for (int k = 1; k < NOPS; ++k) {
-                    if (!c.is_const[k] && !(reused & (1 << (k - 1)))) bytes += c.n * sizes[k];
-                }
-                if ((inputs != 0 && reused == inputs) || bytes <= kCacheResidentBytes) {
-                    hipLaunchKernelGGL((map_rows_kernel<F, kFlat, 7>), dim3(grid), dim3(kBlock), 0, stream, a);
+                if (inputs != 0 && reused == inputs) {
+                    hipLaunchKernelGGL((map_rows_kernel<F, kFlat, 7>), dim3(grid), dim3(kRowsBlock), 0, stream, a);
                     return;
                 }
                 if (reused == 1) {
-                    hipLaunchKernelGGL((map_rows_kernel<F, kFlat, 1>), dim3(grid), dim3(kBlock), 0, stream, a);
+                    hipLaunchKernelGGL((map_rows_kernel<F, kFlat, 1>), dim3(grid), dim3(kRowsBlock), 0, stream, a);
                     return;
                 }
                 if (reused == 2) {
-                    hipLaunchKernelGGL((map_rows_kernel<F, kFlat, 2>), dim3(grid), dim3(kBlock), 0, stream, a);
+                    hipLaunchKernelGGL((map_rows_kernel<F, kFlat, 2>), dim3(grid), dim3(kRowsBlock), 0, stream, a);
                     return;
                 }
                 if constexpr (F::N >= 3) {
                     // Two broadcast inputs in front of a streamed one (addr with its input: v1, v2, input).
                     if (reused == 3) {
-                        hipLaunchKernelGGL((map_rows_kernel<F, kFlat, 3>), dim3(grid), dim3(kBlock), 0, stream, a);
+                        hipLaunchKernelGGL((map_rows_kernel<F, kFlat, 3>), dim3(grid), dim3(kRowsBlock), 0, stream, a);
                         return;
                     }
                 }
             }
-            // An output of twice the memory-side cache or more gains nothing from passing through it.
-            if constexpr (T::V * T::so == 16) {
-                if (c.n * T::so >= kStreamStoreBytes) {
-                    hipLaunchKernelGGL((map_rows_kernel<F, kFlat, 0, true>), dim3(grid), dim3(kBlock), 0, stream, a);
-                    return;
-                }
-            }
-            hipLaunchKernelGGL((map_rows_kernel<F, kFlat, 0>), dim3(grid), dim3(kBlock), 0, stream, a);
+            hipLaunchKernelGGL((map_rows_kernel<F, kFlat, 0>), dim3(grid), dim3(kRowsBlock), 0, stream, a);
         };
         if (variant == 0) run(std::true_type{});
         else run(std::false_type{});

@@ -5,7 +5,7 @@
 // by applying the operation's own functor (the one the direct kernels use) to every pattern, so a
 // looked-up result has the direct kernel's bits by construction. The lookup kernel keeps the table
 // in LDS (128 KiB of the 160 KiB a CU has: one 1024-lane workgroup per CU) and streams the tensor
-// past it: 16-byte loads and stores, eight LDS reads per chunk, no arithmetic. What makes this worth
+// past it: 16-byte loads and (write-through) stores, eight LDS reads per chunk, no arithmetic. What makes this worth
 // it is the cost of the exact operations - erf goes through an f64 series of up to forty terms per
 // element - against a kernel that runs at the speed of memory whatever the operation is.
 #pragma once
@@ -69,6 +69,7 @@ __global__ void __launch_bounds__(kTableBlock) map_table_kernel(RowsArgs<2> a, c
     }
     __syncthreads();
     using Off = std::conditional_t<FLAT, int64_t, uint32_t>;
+    const OutStores stores(a.ptr[0], a.out32 != 0);
     const int64_t tiles = (a.n + V - 1) / V;
     const int64_t whole = a.n / V;
     auto offsets = [&](int64_t t, Off &out_off, Off &src_off) {
@@ -128,7 +129,6 @@ __global__ void __launch_bounds__(kTableBlock) map_table_kernel(RowsArgs<2> a, c
                 high_src += idx * static_cast<uint32_t>(a.ostride[1][d]);
             }
             const char *src = a.ptr[1] + static_cast<int64_t>(high_src) * 2;
-            char *out = a.ptr[0] + static_cast<int64_t>(high_out) * 2;
             u32x4 raw[U];
 #pragma unroll
             for (int u = 0; u < U; ++u) {
@@ -138,7 +138,7 @@ __global__ void __launch_bounds__(kTableBlock) map_table_kernel(RowsArgs<2> a, c
             }
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                *reinterpret_cast<u32x4 *>(out + static_cast<int64_t>(low_out[u]) * 2) = lookup(raw[u]);
+                stores.put16((static_cast<int64_t>(high_out) + static_cast<int64_t>(low_out[u])) * 2, lookup(raw[u]));
             }
         }
         return;
@@ -159,7 +159,7 @@ __global__ void __launch_bounds__(kTableBlock) map_table_kernel(RowsArgs<2> a, c
             }
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                *reinterpret_cast<u32x4 *>(a.ptr[0] + static_cast<int64_t>(oo[u]) * 2) = lookup(raw[u]);
+                stores.put16(static_cast<int64_t>(oo[u]) * 2, lookup(raw[u]));
             }
         } else {
             for (int u = 0; u < U; ++u) {

@@ -356,6 +356,7 @@ struct ScalarBinary {
     using In0 = T;
     using In1 = typename Comp<T>::C;
     using In2 = Unused;
+    static constexpr uint32_t kConstantInputs = 2;  // input 1 is never a tensor: its width does not shape the tiles
     using C = typename Comp<T>::C;
     __device__ __forceinline__ T operator()(T a, C s) const {
         const C x = Comp<T>::up(a);

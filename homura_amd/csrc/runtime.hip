@@ -112,6 +112,7 @@ class ContextParts {
     ContextParts(const ContextParts &) = delete;
     ContextParts &operator=(const ContextParts &) = delete;
     ~ContextParts() {
+        if (ctx_ && ctx_->tables != nullptr && hipFree(ctx_->tables) != hipSuccess) (void)hipGetLastError();
         if (ctx_ && ctx_->stream != nullptr) (void)close(ctx_->stream);
     }
 
@@ -274,6 +275,7 @@ hmr_status hmr_context_create(int32_t device, hmr_context_t *out) {
         if (hmr_status s = hmr::bind_reduce_scratch(parts.ctx())) return s;
         parts.ctx().device = device;
         parts.ctx().compute_units = p.multiProcessorCount > 0 ? p.multiProcessorCount : 256;
+        if (hmr_status s = hmr::build_unary_tables(parts.ctx())) return s;
         *out = parts.release();
         return HMR_OK;
     });

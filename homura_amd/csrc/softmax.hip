@@ -238,6 +238,7 @@ struct SoftmaxArgs {
     int64_t nrows;
     int64_t n;
     int64_t so, si;
+    int32_t stream_stores;  // registers plan: nontemporal stores instead of write-through ones
 };
 
 // Contiguous rows held in registers, as loaded (16-byte chunks). G lanes per row, each with C
@@ -250,8 +251,9 @@ struct SoftmaxArgs {
 //
 // WALK = false: the rows form one dimension (row r starts r * stride elements in), which is what a
 // contiguous tensor gives; WALK = true: up to 25 row dimensions, decoded per row.
-// NTSTORE: nontemporal stores, for outputs far larger than the memory-side cache.
-template <class T, int G, int C, bool LOG, bool WALK, bool NTSTORE = false>
+// Stores write through the compute die's L2 (see OutStores in map.hpp), or are nontemporal for outputs far larger
+// than the memory-side cache (`stream_stores`).
+template <class T, int G, int C, bool LOG, bool WALK>
 __global__ void __launch_bounds__(G > kBlock ? G : kBlock) softmax_regs_kernel(SoftmaxArgs a) {
     using M = SoftmaxMath<T>;
     using X = typename M::X;
@@ -266,11 +268,13 @@ __global__ void __launch_bounds__(G > kBlock ? G : kBlock) softmax_regs_kernel(S
     const int64_t groups = (a.nrows + kRowsPerBlock - 1) / kRowsPerBlock;
     const int nvec = static_cast<int>(a.n / V);  // chunks in a row (>= 1)
     for (int64_t g = blockIdx.x; g < groups; g += gridDim.x) {
-        const int64_t row = g * kRowsPerBlock + threadIdx.x / G;
+        // A row belongs to whole waves (G is a multiple of 64): its number is the same in every lane of one.
+        const int64_t row = g * kRowsPerBlock + __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) / G);
         const bool live = row < a.nrows;
         const int64_t r = live ? row : a.nrows - 1;  // idle lanes of the last group redo the last row, without storing
         const T *src = reinterpret_cast<const T *>(a.src) + (WALK ? a.src_rows.offset(r) : r * a.src_rows.stride[0]);
         T *out = reinterpret_cast<T *>(a.out) + (WALK ? a.out_rows.offset(r) : r * a.out_rows.stride[0]);
+        const __amdgpu_buffer_rsrc_t out_row = __builtin_amdgcn_make_buffer_rsrc(out, 0, -1, 0x00020000);
         // Phase 0: one pass over memory.
         u32x4 raw[C];
 #pragma unroll
@@ -374,9 +378,11 @@ __global__ void __launch_bounds__(G > kBlock ? G : kBlock) softmax_regs_kernel(S
                 }
             }
             if (live && tile < nvec) {
-                u32x4 *q = reinterpret_cast<u32x4 *>(reinterpret_cast<char *>(out) + static_cast<uint32_t>(tile) * 16u);
-                if constexpr (kStreamStores || NTSTORE) __builtin_nontemporal_store(M::pack(res), q);
-                else *q = M::pack(res);
+                if (a.stream_stores) {
+                    __builtin_nontemporal_store(M::pack(res), reinterpret_cast<u32x4 *>(reinterpret_cast<char *>(out) + static_cast<uint32_t>(tile) * 16u));
+                } else {
+                    __builtin_amdgcn_raw_buffer_store_b128(M::pack(res), out_row, tile * 16, 0, 17 /* sc0 sc1 */);
+                }
             }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -514,9 +520,7 @@ void launch_softmax(const SoftmaxPlan &p, const SoftmaxArgs &a, bool out_ok, hip
         auto run = [&](auto g, auto c) {
             constexpr int G = decltype(g)::value, C = decltype(c)::value;
             constexpr int kThreads = G > kBlock ? G : kBlock;
-            if (a.src_rows.ndim <= 1 && a.nrows * a.n * static_cast<int64_t>(sizeof(T)) >= kStreamStoreBytes) {
-                hipLaunchKernelGGL((softmax_regs_kernel<T, G, C, LOG, false, true>), blocks(kThreads / G), dim3(kThreads), 0, stream, a);
-            } else if (a.src_rows.ndim <= 1) {
+            if (a.src_rows.ndim <= 1) {
                 hipLaunchKernelGGL((softmax_regs_kernel<T, G, C, LOG, false>), blocks(kThreads / G), dim3(kThreads), 0, stream, a);
             } else {
                 hipLaunchKernelGGL((softmax_regs_kernel<T, G, C, LOG, true>), blocks(kThreads / G), dim3(kThreads), 0, stream, a);
@@ -728,6 +732,7 @@ hmr_status hmr_softmax(hmr_context_t ctx, const hmr_tensor_desc *out_rows, const
         a.n = n;
         a.so = out_stride;
         a.si = src_stride;
+        a.stream_stores = a.nrows * n * elem >= hmr::kStreamStoreBytes ? 1 : 0;
         hmr::SoftmaxPlan plan = hmr::plan_softmax(*src_rows, n, src_stride, a.src_rows);
         bool out_ok = (n == 1 || out_stride == 1) && reinterpret_cast<uintptr_t>(a.out) % 16 == 0;
         for (int d = 0; out_ok && d < a.out_rows.ndim; ++d) out_ok = (a.out_rows.stride[d] * elem) % 16 == 0;

@@ -21,6 +21,31 @@ hmr_status hmr::bind_reduce_scratch(hmr_context &ctx) {
     return HMR_OK;
 }
 
+// The other one (ew_unary.hip): the tables of the 16-bit unary operations. Here a block of the scripted HIP's
+// memory, so that the books show who frees it.
+static bool g_tables_fail = false;
+hmr_status hmr::build_unary_tables(hmr_context &ctx) {
+    if (g_tables_fail) return hmr::fail(HMR_OUT_OF_MEMORY, "hipMalloc(&tables, kTableSlots * kTableBytes): out of memory");
+    void *block = nullptr;
+    if (hipMalloc(&block, 64) != hipSuccess) return hmr::fail(HMR_OUT_OF_MEMORY, "hipMalloc(&tables, kTableSlots * kTableBytes): out of memory");
+    ctx.tables = block;
+    return HMR_OK;
+}
+
+// Large aligned copies and fills leave the plumbing for the kernels (ew_copy.hip, ew_misc.hip); here the calls
+// are counted.
+static int g_kernel_copies = 0, g_kernel_fills = 0;
+static uint64_t g_fill_bits = 0;
+extern "C" hmr_status hmr_copy(hmr_context_t, const hmr_tensor_desc *dst, const hmr_tensor_desc *src) {
+    if (dst->ndim == 1 && src->ndim == 1 && dst->sizes[0] == src->sizes[0] && dst->dtype == src->dtype) ++g_kernel_copies;
+    return HMR_OK;
+}
+extern "C" hmr_status hmr_fill(hmr_context_t, const hmr_tensor_desc *dst, uint64_t bits) {
+    if (dst->ndim == 1) ++g_kernel_fills;
+    g_fill_bits = bits;
+    return HMR_OK;
+}
+
 static int g_failures = 0;
 #define EXPECT(cond)                                                              \
     do {                                                                          \
@@ -116,16 +141,14 @@ static void contexts() {
     {
         hmr_context_t real = nullptr;
         EXPECT(hmr_context_create(0, &real) == HMR_OK && real != nullptr);
-        EXPECT(hmr_test_live_streams() == 1 && M().streams.size() == 1 && M().blocks.empty());
+        EXPECT(hmr_test_live_streams() == 1 && M().streams.size() == 1 && M().blocks.size() == 1);  // its tables
         EXPECT(fake::thread().device == 1 && real->device == 0 && real->compute_units == 256 && real->reduce_scratch != nullptr);
+        EXPECT(real->tables != nullptr);
         EXPECT(hmr_context_synchronize(real) == HMR_OK);
         M().fail_next["hipStreamSynchronize"] = hipErrorLaunchFailure;
         EXPECT(hmr_context_synchronize(real) == HMR_HIP_ERROR && last() == "hipStreamSynchronize(ctx->stream): unspecified launch failure");
         EXPECT(hipGetLastError() == hipSuccess);
         // Destroying frees the tables even when the stream will not go.
-        void *tables = nullptr;
-        EXPECT(hipMalloc(&tables, 64) == hipSuccess);
-        real->tables = tables;
         M().fail_next["hipStreamDestroy"] = hipErrorInvalidHandle;
         EXPECT(hmr_context_destroy(real) == HMR_HIP_ERROR && last() == "hipStreamDestroy(ctx->stream): invalid resource handle");
         EXPECT(M().blocks.empty());
@@ -145,6 +168,12 @@ static void contexts() {
     EXPECT(hmr_context_create(0, &ctx) == HMR_HIP_ERROR && ctx == nullptr);
     EXPECT(hmr_test_live_streams() == live && M().streams.empty() && M().blocks.empty());
     g_bind_fails = false;
+
+    // The tables cannot be had: the stream is given back, nothing stays allocated.
+    g_tables_fail = true;
+    EXPECT(hmr_context_create(0, &ctx) == HMR_OUT_OF_MEMORY && ctx == nullptr);
+    EXPECT(hmr_test_live_streams() == live && M().streams.empty() && M().blocks.empty());
+    g_tables_fail = false;
 }
 
 static void memory() {
@@ -178,6 +207,17 @@ static void memory() {
     EXPECT(hmr_copy_to_host(ctx, host, d, 16) == HMR_OK && host[1] == 2);
     const size_t calls = M().calls.size();
     EXPECT(hmr_copy_device(ctx, d, d, 0) == HMR_OK && M().calls.size() == calls);  // nothing to do, nothing called
+    // A megabyte and more at aligned addresses goes to the kernels: words of eight bytes when they divide the
+    // size, bytes otherwise; an armed failure still comes first.
+    {
+        void *big = reinterpret_cast<void *>(uintptr_t{1} << 40);
+        EXPECT(hmr_copy_device(ctx, big, big, 1 << 20) == HMR_OK && g_kernel_copies == 1);
+        EXPECT(hmr_copy_device(ctx, big, big, (1 << 20) + 3) == HMR_OK && g_kernel_copies == 2);
+        hmr_test_fail_data(1, 1);
+        EXPECT(hmr_copy_device(ctx, big, big, 1 << 20) == HMR_OUT_OF_MEMORY && g_kernel_copies == 2);
+        EXPECT(hmr_memset(ctx, big, 0x5A, 1 << 20) == HMR_OK && g_kernel_fills == 1 && g_fill_bits == UINT64_C(0x5A5A5A5A5A5A5A5A));
+        EXPECT(hmr_memset(ctx, big, 0x5A, (1 << 20) + 1) == HMR_OK && g_kernel_fills == 2 && g_fill_bits == 0x5A);
+    }
     // The launch bracket: an armed failure, a kernel-less call, a launch that HIP refuses.
     hmr_test_fail_data(1, 0);
     bool queued = false;
