@@ -372,9 +372,9 @@ def per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP
     add(None, "addr f32 [8192,8192] without input (beta 0)", 4 * N + 8 * 8192, lambda: mat.addr(v1, v2, 0, -1.5))
     del mat, v1, v2
     xf = residual.reshape([16384, 4096])
-    add(None, "exclusive_cumprod f32 [16384,4096] dim=0 (a thread per column, sequential)", 8 * N,
+    add(None, "exclusive_cumprod f32 [16384,4096] dim=0 (slabs through LDS, a sequential chain per column)", 8 * N,
         lambda: h.exclusive_cumprod(xf, 0, False), 5)
-    add(None, "exclusive_cumprod f32 [16384,4096] dim=1 (a thread per row, sequential)", 8 * N,
+    add(None, "exclusive_cumprod f32 [16384,4096] dim=1 (slabs through LDS, a sequential chain per row)", 8 * N,
         lambda: h.exclusive_cumprod(xf, 1, True), 5)
     del xf
     y = x.reshape([16384, 4096]).softmax(-1)

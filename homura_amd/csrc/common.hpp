@@ -25,6 +25,17 @@ struct hmr_context {
     // input pattern -> its output pattern): allocated and filled by hmr_context_create, read-only afterwards,
     // freed with the context.
     void *tables = nullptr;
+    // Where a position check spread over many workgroups meets (index.hip): the smallest bad position so far and
+    // the count of workgroups that have finished. Device memory behind the tables; the last workgroup of a check
+    // leaves both as it found them (all ones, zero).
+    void *check_state = nullptr;
+    // The mailbox: 16 bytes of pinned host memory the GPU can write. A kernel whose result the caller is about
+    // to read back (the verdict of a position check) stores it there as well as in the caller's device memory;
+    // `mail_src` is that device address while the mailbox holds its current contents, and a read-back of it
+    // (hmr_copy_to_host) waits for the stream and takes the bytes from the mailbox instead of queueing a copy.
+    // Anything else queued on the context forgets the address.
+    void *mailbox = nullptr;
+    const void *mail_src = nullptr;
     // Device address, on this context's GPU, of the library's static block for partial results
     // (hmr_reduce_static). Each GPU holds its own copy of the block at its own address.
     void *reduce_scratch = nullptr;
@@ -52,9 +63,12 @@ hmr_status hip_failure(hipError_t error, const char *what) noexcept;
 // in the context. Called once per context, with its device current (defined beside the block, reduce.hip).
 hmr_status bind_reduce_scratch(hmr_context &ctx);
 
-// Allocates the tables of the 16-bit unary operations on the context's GPU, fills them on its stream and waits
-// for the fills. Called once per context, after its stream exists (defined beside the operations, ew_unary.hip).
+// Allocates the tables of the 16-bit unary operations on the context's GPU (and, behind them, the meeting place
+// of the position checks), fills them on its stream and waits for the fills. Called once per context, after its
+// stream exists (defined beside the operations, ew_unary.hip).
 hmr_status build_unary_tables(hmr_context &ctx);
+// Bytes kept behind the tables for hmr_context::check_state.
+constexpr size_t kCheckStateBytes = 8192;
 
 // ---- one entry point's stay in the library ---------------------------------------------------------------
 
@@ -96,6 +110,7 @@ class Visit {
     // read: that is where a launch that could not be queued shows.
     template <class Queue>
     hmr_status kernels(hmr_context_t ctx, const char *what, Queue queue) {
+        ctx->mail_src = nullptr;  // whatever is queued may write what the mailbox mirrors
         if (hmr_status s = use_device(ctx->device)) return s;
         if (hmr_status s = armed_failure("hipGetLastError()")) return s;
         (void)hipGetLastError();

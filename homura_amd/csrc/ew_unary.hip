@@ -68,7 +68,8 @@ hmr_status build_unary_tables(hmr_context &ctx) {
     Visit v;
     if (hmr_status s = v.use_device(ctx.device)) return s;
     void *block = nullptr;
-    if (hmr_status s = v.hip(hipMalloc(&block, kTableSlots * kTableBytes), "hipMalloc(&tables, kTableSlots * kTableBytes)")) return s;
+    if (hmr_status s = v.hip(hipMalloc(&block, kTableSlots * kTableBytes + kCheckStateBytes), "hipMalloc(&tables, kTableSlots * kTableBytes)")) return s;
+    char *state = static_cast<char *>(block) + kTableSlots * kTableBytes;
     (void)hipGetLastError();
     const auto fill = [&](auto t) {
         using T = typename decltype(t)::type;
@@ -86,12 +87,16 @@ hmr_status build_unary_tables(hmr_context &ctx) {
     fill(TypeTag<f16_t>{});
     fill(TypeTag<bf16_t>{});
     hipError_t ran = hipGetLastError();
+    // The checks' meeting place: no bad position yet (all ones), no workgroup arrived.
+    if (ran == hipSuccess) ran = hipMemsetAsync(state, 0, kCheckStateBytes, ctx.stream);
+    if (ran == hipSuccess) ran = hipMemsetAsync(state, 0xFF, 8, ctx.stream);
     if (ran == hipSuccess) ran = hipStreamSynchronize(ctx.stream);
     if (ran != hipSuccess) {
         (void)hipFree(block);
         return v.hip(ran, "filling the tables of the 16-bit unary operations");
     }
     ctx.tables = block;
+    ctx.check_state = state;
     return HMR_OK;
 }
 

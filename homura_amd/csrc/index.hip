@@ -20,13 +20,76 @@ namespace {
 
 // ---- hmr_index_check ------------------------------------------------------------------------------------
 
-__global__ void check_init_kernel(uint64_t *slot) {
-    slot[0] = ~uint64_t{0};
-    slot[1] = 0;
+// A check is ONE launch. Its workgroups meet in `CheckState` (device memory of the context): every wave that
+// found a bad position lowers `first` (a minimum does not depend on the order they arrive in), every workgroup
+// then counts itself in, and the one that arrives last reads the minimum, looks the value at that position up,
+// publishes both - in the caller's slot and in the context's mailbox (pinned host memory, so that the caller's
+// read-back is a wait for the stream and nothing else) - and leaves the state as it found it.
+//
+// Counting in is two levels deep: an atomic on one address costs some 16 ns however many workgroups issue it
+// (2048 of them on one counter added 33 us to a check of 8.4 M positions), so a workgroup counts itself into one
+// of 32 counters, each on a cache line of its own, and the last one of each counter counts into the top one.
+constexpr int kCheckGroups = 32;
+constexpr unsigned kCheckGrid = 1024;  // workgroups of a check at most (its kernels stride over the rest)
+struct CheckState {
+    unsigned long long first;  // all ones: none
+    char pad0[120];
+    unsigned int top;
+    char pad1[124];
+    struct {
+        unsigned int arrived;
+        char pad[124];
+    } group[kCheckGroups];
+};
+static_assert(sizeof(CheckState) <= kCheckStateBytes, "the context keeps kCheckStateBytes for it");
+
+__device__ __forceinline__ int64_t value_at(const void *index, int is64, const Dims &d, unsigned long long p) {
+    int64_t rest = static_cast<int64_t>(p), off = 0;
+    for (int k = 0; k < d.ndim; ++k) {
+        const int64_t q = rest / d.size[k];
+        off += (rest - q * d.size[k]) * d.stride[0][k];
+        rest = q;
+    }
+    return read_index(index, is64, off);
+}
+
+__device__ __forceinline__ void publish(uint64_t *slot, uint64_t *mailbox, unsigned long long first, int64_t value) {
+    const uint64_t word = first == ~0ull ? 0 : static_cast<uint64_t>(value);
+    slot[0] = first;
+    slot[1] = word;
+    mailbox[0] = first;
+    mailbox[1] = word;
+}
+
+// `first`: the smallest bad position this lane saw. Every lane of the workgroup calls this, once.
+__device__ __forceinline__ void meet(unsigned long long first, CheckState *state, uint64_t *slot, uint64_t *mailbox,
+                                     const void *index, int is64, const Dims &d) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) {
+        const unsigned long long other = (static_cast<unsigned long long>(static_cast<uint32_t>(__shfl_xor(static_cast<int>(first >> 32), m, 64))) << 32) |
+                                         static_cast<uint32_t>(__shfl_xor(static_cast<int>(first), m, 64));
+        first = other < first ? other : first;
+    }
+    if ((threadIdx.x & 63) == 0 && first != ~0ull) atomicMin(&state->first, first);
+    __syncthreads();  // every wave's minimum is out
+    if (threadIdx.x != 0) return;
+    const unsigned mine = blockIdx.x % kCheckGroups;
+    const unsigned members = (gridDim.x - mine + kCheckGroups - 1) / kCheckGroups;
+    const unsigned groups = gridDim.x < kCheckGroups ? gridDim.x : kCheckGroups;
+    // No fences between these: every one of them is an atomic of device scope, carried out where all compute dies
+    // see it; a wave's atomicMin has been acknowledged before the barrier above lets this lane go on, and each
+    // step below is issued only after the one before it has returned its value. (A device-scope fence would write
+    // back and invalidate the die's L2 once per workgroup: a check of 8.4 M positions took 25 us with them, 7 without.)
+    if (atomicAdd(&state->group[mine].arrived, 1u) != members - 1) return;
+    atomicExch(&state->group[mine].arrived, 0u);
+    if (atomicAdd(&state->top, 1u) != groups - 1) return;
+    atomicExch(&state->top, 0u);
+    const unsigned long long found = atomicExch(&state->first, ~0ull);
+    publish(slot, mailbox, found, found == ~0ull ? 0 : value_at(index, is64, d, found));
 }
 
 __global__ void __launch_bounds__(kBlock) check_kernel(const void *index, int is64, Dims d, int64_t n, int64_t low, int64_t high,
-                                                       int has_exempt, int64_t exempt, unsigned long long *slot) {
+                                                       int has_exempt, int64_t exempt, uint64_t *slot, CheckState *state, uint64_t *mailbox) {
     unsigned long long first = ~0ull;
     for (int64_t p = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; p < n; p += static_cast<int64_t>(gridDim.x) * kBlock) {
         int64_t rest = p, off = p * d.stride[0][0];
@@ -42,14 +105,7 @@ __global__ void __launch_bounds__(kBlock) check_kernel(const void *index, int is
         const bool bad = !(v >= low && v < high) && !(has_exempt && v == exempt);
         if (bad && static_cast<unsigned long long>(p) < first) first = static_cast<unsigned long long>(p);
     }
-    // One atomic per wave that found something: the minimum is the same in whatever order they arrive.
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) {
-        const unsigned long long other = (static_cast<unsigned long long>(static_cast<uint32_t>(__shfl_xor(static_cast<int>(first >> 32), m, 64))) << 32) |
-                                         static_cast<uint32_t>(__shfl_xor(static_cast<int>(first), m, 64));
-        first = other < first ? other : first;
-    }
-    if ((threadIdx.x & 63) == 0 && first != ~0ull) atomicMin(slot, first);
+    meet(first, state, slot, mailbox, index, is64, d);
 }
 
 // The same for an index that is one contiguous run: 16 bytes per lane and load, four loads in flight (an
@@ -57,7 +113,8 @@ __global__ void __launch_bounds__(kBlock) check_kernel(const void *index, int is
 // than a tile) come before the first 16-byte boundary; they and the ragged end go to the first workgroup's lanes.
 template <class I>
 __global__ void __launch_bounds__(kBlock) check_flat_kernel(const I *start, int head, int64_t total, int64_t low, int64_t high,
-                                                            int has_exempt, int64_t exempt, unsigned long long *slot) {
+                                                            int has_exempt, int64_t exempt, uint64_t *slot, CheckState *state, uint64_t *mailbox,
+                                                            Dims d) {
     constexpr int V = 16 / static_cast<int>(sizeof(I)), U = 4;
     unsigned long long first = ~0ull;
     const I *index = start + head;  // aligned; position p of the run is index[p - head]
@@ -94,20 +151,14 @@ __global__ void __launch_bounds__(kBlock) check_flat_kernel(const I *start, int 
             if (!(x >= low && x < high) && !(has_exempt && x == exempt) && static_cast<unsigned long long>(p) < first) first = p;
         }
     }
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) {
-        const unsigned long long other = (static_cast<unsigned long long>(static_cast<uint32_t>(__shfl_xor(static_cast<int>(first >> 32), m, 64))) << 32) |
-                                         static_cast<uint32_t>(__shfl_xor(static_cast<int>(first), m, 64));
-        first = other < first ? other : first;
-    }
-    if ((threadIdx.x & 63) == 0 && first != ~0ull) atomicMin(slot, first);
+    meet(first, state, slot, mailbox, start, sizeof(I) == 8, d);
 }
 
-// The whole check in one workgroup, for indices of a few thousand elements (three launches otherwise).
+// The whole check in one workgroup, for indices of a few thousand elements: no meeting, no atomics.
 constexpr int kCheckBlock = 1024;
-constexpr int64_t kCheckSmall = 64 * kCheckBlock;
+constexpr int64_t kCheckSmall = 8 * kCheckBlock;
 __global__ void __launch_bounds__(kCheckBlock) check_small_kernel(const void *index, int is64, Dims d, int64_t n, int64_t low, int64_t high,
-                                                                  int has_exempt, int64_t exempt, uint64_t *slot) {
+                                                                  int has_exempt, int64_t exempt, uint64_t *slot, uint64_t *mailbox) {
     __shared__ unsigned long long firsts[kCheckBlock / 64];
     __shared__ long long values[kCheckBlock / 64];
     unsigned long long first = ~0ull;
@@ -163,21 +214,14 @@ __global__ void __launch_bounds__(kCheckBlock) check_small_kernel(const void *in
                 value = values[w];
             }
         }
-        slot[0] = first;
-        slot[1] = first == ~0ull ? 0 : static_cast<uint64_t>(value);
+        publish(slot, mailbox, first, value);
     }
 }
 
 __global__ void check_value_kernel(const void *index, int is64, Dims d, uint64_t *slot) {
     const uint64_t p = slot[0];
     if (p == ~uint64_t{0}) return;
-    int64_t rest = static_cast<int64_t>(p), off = 0;
-    for (int k = 0; k < d.ndim; ++k) {
-        const int64_t q = rest / d.size[k];
-        off += (rest - q * d.size[k]) * d.stride[0][k];
-        rest = q;
-    }
-    slot[1] = static_cast<uint64_t>(read_index(index, is64, off));
+    slot[1] = static_cast<uint64_t>(value_at(index, is64, d, p));
 }
 
 // ---- hmr_index_select / hmr_gather ---------------------------------------------------------------------
@@ -233,6 +277,7 @@ struct RowsOfTiles {
     const char *src;
     const void *index;
     int32_t is64, nouter, at;  // `at` counts outer dimensions from the innermost outer one
+    int32_t out32;             // nonzero: every byte offset into the output fits 32 bits
     int64_t n_tiles, wrap, index_stride;
     uint32_t tiles_per_row;
     FastDiv tiles_div;
@@ -244,6 +289,7 @@ template <class W>
 __global__ void __launch_bounds__(kBlock) select_rows_kernel(RowsOfTiles a) {
     constexpr int V = 16 / static_cast<int>(sizeof(W));
     constexpr int U = 4;
+    const OutStores stores(a.out, a.out32 != 0);
     const int64_t first = static_cast<int64_t>(blockIdx.x) * (U * kBlock) + threadIdx.x;
     W r[U][V];
     int64_t oo[U];
@@ -275,7 +321,11 @@ __global__ void __launch_bounds__(kBlock) select_rows_kernel(RowsOfTiles a) {
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-        if (valid[u]) store_tile<W, V, false>(a.out + oo[u] * static_cast<int64_t>(sizeof(W)), r[u]);
+        if (valid[u]) {
+            u32x4 w;
+            __builtin_memcpy(&w, r[u], 16);
+            stores.put16(oo[u] * static_cast<int64_t>(sizeof(W)), w);
+        }
     }
 }
 
@@ -619,45 +669,46 @@ hmr_status hmr_index_check(hmr_context_t ctx, const hmr_tensor_desc *index, int6
         const hmr::Dims d = hmr::dims_of(*index, ops, -1);
         const void *base = hmr::first_of(*index);
         const int is64 = index->dtype == HMR_I64;
-        return hmr::queue_on(ctx, "index_check", [&](hipStream_t stream) {
+        hmr::CheckState *state = static_cast<hmr::CheckState *>(ctx->check_state);
+        uint64_t *mailbox = static_cast<uint64_t *>(ctx->mailbox);
+        const hmr_status queued = hmr::queue_on(ctx, "index_check", [&](hipStream_t stream) {
             if (n <= hmr::kCheckSmall) {
                 hipLaunchKernelGGL(hmr::check_small_kernel, dim3(1), dim3(hmr::kCheckBlock), 0, stream, base, is64, d, n, low, high,
-                                   has_exempt, exempt, slot);
+                                   has_exempt, exempt, slot, mailbox);
                 return true;
             }
-            hipLaunchKernelGGL(hmr::check_init_kernel, dim3(1), dim3(1), 0, stream, slot);
-            if (n > 0) {
-                // One contiguous run (after merging: a size-1 dimension's stride does not count)? Its elements
-                // before the first 16-byte boundary are the head.
-                const int elem = is64 ? 8 : 4;
-                const int64_t to_boundary = static_cast<int64_t>((16 - reinterpret_cast<uintptr_t>(base) % 16) % 16) / elem;
-                const int head = static_cast<int>(to_boundary < n ? to_boundary : n);
-                bool flat = reinterpret_cast<uintptr_t>(base) % elem == 0;
-                int64_t run = 1;
-                for (int k = index->ndim - 1; flat && k >= 0; --k) {
-                    flat = index->sizes[k] == 1 || index->strides[k] == run;
-                    run *= index->sizes[k];
-                }
-                if (flat) {
-                    const int64_t per_block = int64_t{4} * hmr::kBlock * (is64 ? 2 : 4);
-                    const unsigned grid = hmr::grid_of((n + per_block - 1) / per_block * hmr::kBlock);
-                    if (is64) {
-                        hipLaunchKernelGGL((hmr::check_flat_kernel<int64_t>), dim3(grid), dim3(hmr::kBlock), 0, stream,
-                                           static_cast<const int64_t *>(base), head, n, low, high, has_exempt, exempt,
-                                           reinterpret_cast<unsigned long long *>(slot));
-                    } else {
-                        hipLaunchKernelGGL((hmr::check_flat_kernel<int32_t>), dim3(grid), dim3(hmr::kBlock), 0, stream,
-                                           static_cast<const int32_t *>(base), head, n, low, high, has_exempt, exempt,
-                                           reinterpret_cast<unsigned long long *>(slot));
-                    }
+            // One contiguous run (after merging: a size-1 dimension's stride does not count)? Its elements
+            // before the first 16-byte boundary are the head.
+            const int elem = is64 ? 8 : 4;
+            const int64_t to_boundary = static_cast<int64_t>((16 - reinterpret_cast<uintptr_t>(base) % 16) % 16) / elem;
+            const int head = static_cast<int>(to_boundary < n ? to_boundary : n);
+            bool flat = reinterpret_cast<uintptr_t>(base) % elem == 0;
+            int64_t run = 1;
+            for (int k = index->ndim - 1; flat && k >= 0; --k) {
+                flat = index->sizes[k] == 1 || index->strides[k] == run;
+                run *= index->sizes[k];
+            }
+            if (flat) {
+                const int64_t per_block = int64_t{4} * hmr::kBlock * (is64 ? 2 : 4);
+                unsigned grid = hmr::grid_of((n + per_block - 1) / per_block * hmr::kBlock);
+                grid = grid < hmr::kCheckGrid ? grid : hmr::kCheckGrid;
+                if (is64) {
+                    hipLaunchKernelGGL((hmr::check_flat_kernel<int64_t>), dim3(grid), dim3(hmr::kBlock), 0, stream,
+                                       static_cast<const int64_t *>(base), head, n, low, high, has_exempt, exempt, slot, state, mailbox, d);
                 } else {
-                    hipLaunchKernelGGL(hmr::check_kernel, dim3(hmr::grid_of(n)), dim3(hmr::kBlock), 0, stream, base, is64, d, n, low, high,
-                                       has_exempt, exempt, reinterpret_cast<unsigned long long *>(slot));
+                    hipLaunchKernelGGL((hmr::check_flat_kernel<int32_t>), dim3(grid), dim3(hmr::kBlock), 0, stream,
+                                       static_cast<const int32_t *>(base), head, n, low, high, has_exempt, exempt, slot, state, mailbox, d);
                 }
-                hipLaunchKernelGGL(hmr::check_value_kernel, dim3(1), dim3(1), 0, stream, base, is64, d, slot);
+            } else {
+                const unsigned all = hmr::grid_of(n);
+                hipLaunchKernelGGL(hmr::check_kernel, dim3(all < hmr::kCheckGrid ? all : hmr::kCheckGrid), dim3(hmr::kBlock), 0, stream, base,
+                                   is64, d, n, low, high, has_exempt, exempt, slot, state, mailbox);
             }
             return true;
         });
+        // The verdict is in the mailbox as well once the kernel has run: a read-back of the slot takes it from there.
+        if (queued == HMR_OK) ctx->mail_src = slot;
+        return queued;
     });
 }
 
@@ -733,6 +784,9 @@ hmr_status hmr_index_select(hmr_context_t ctx, const hmr_tensor_desc *out, const
                     a.n_tiles = n / vec;
                     a.nouter = 0;
                     a.at = -1;
+                    int64_t span = 1;
+                    for (int k = 0; k < out->ndim; ++k) span += (out->sizes[k] - 1) * out->strides[k];
+                    a.out32 = span * elem <= hmr::kNarrowSpanBytes && n * elem < hmr::kStreamStoreBytes ? 1 : 0;
                     for (int k = last - 1; k >= 0; --k) {
                         if (k == dim) a.at = a.nouter;
                         a.div[a.nouter] = hmr::make_fastdiv(static_cast<uint32_t>(out->sizes[k]));

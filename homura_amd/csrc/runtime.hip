@@ -113,6 +113,7 @@ class ContextParts {
     ContextParts &operator=(const ContextParts &) = delete;
     ~ContextParts() {
         if (ctx_ && ctx_->tables != nullptr && hipFree(ctx_->tables) != hipSuccess) (void)hipGetLastError();
+        if (ctx_ && ctx_->mailbox != nullptr && hipHostFree(ctx_->mailbox) != hipSuccess) (void)hipGetLastError();
         if (ctx_ && ctx_->stream != nullptr) (void)close(ctx_->stream);
     }
 
@@ -130,6 +131,14 @@ class ContextParts {
         }
         ctx_->stream = s;
         ++mine().live_streams;
+        return HMR_OK;
+    }
+
+    // The mailbox: pinned host memory that kernels on this GPU may write.
+    hmr_status open_mailbox(Visit &v) {
+        void *box = nullptr;
+        if (hmr_status e = v.hip(hipHostMalloc(&box, 64, hipHostMallocDefault), "hipHostMalloc(&mailbox, 64)")) return e;
+        ctx_->mailbox = box;
         return HMR_OK;
     }
 
@@ -275,6 +284,7 @@ hmr_status hmr_context_create(int32_t device, hmr_context_t *out) {
         if (hmr_status s = hmr::bind_reduce_scratch(parts.ctx())) return s;
         parts.ctx().device = device;
         parts.ctx().compute_units = p.multiProcessorCount > 0 ? p.multiProcessorCount : 256;
+        if (hmr_status s = parts.open_mailbox(v)) return s;
         if (hmr_status s = hmr::build_unary_tables(parts.ctx())) return s;
         *out = parts.release();
         return HMR_OK;
@@ -289,8 +299,10 @@ hmr_status hmr_context_destroy(hmr_context_t ctx) {
         // Both resources go whatever the first one's fate: the first failure is the one reported.
         const hipError_t stream_gone = hmr::ContextParts::close(owned->stream);
         const hipError_t tables_gone = owned->tables != nullptr ? hipFree(owned->tables) : hipSuccess;  // waits for the device
+        const hipError_t mailbox_gone = owned->mailbox != nullptr ? hipHostFree(owned->mailbox) : hipSuccess;
         if (hmr_status s = v.hip(stream_gone, "hipStreamDestroy(ctx->stream)")) return s;
-        return v.hip(tables_gone, "hipFree(ctx->tables)");
+        if (hmr_status s = v.hip(tables_gone, "hipFree(ctx->tables)")) return s;
+        return v.hip(mailbox_gone, "hipHostFree(ctx->mailbox)");
     });
 }
 

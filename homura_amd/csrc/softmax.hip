@@ -1,5 +1,5 @@
-// hmr_softmax / hmr_softmax_workspace / hmr_test_softmax_plan / hmr_exclusive_cumprod
-// (ref: csrc/homura_rocm.h:338-351, csrc/reduce.hip:162-360, 519-608).
+// hmr_softmax / hmr_softmax_workspace / hmr_test_softmax_plan
+// (ref: csrc/homura_rocm.h:338-351, csrc/reduce.hip:162-360, 519-580).
 //
 // What is computed is cpu::softmax (ref: src/backend/cpu/misc.rs:15-51): per row,
 //   max = fold(-inf, v > m ? v : m)      (a NaN never replaces)
@@ -27,6 +27,7 @@
 #include <cmath>
 
 #include "dispatch.hpp"
+#include "lines.hpp"
 #include "reduce.hpp"
 
 namespace hmr {
@@ -432,39 +433,6 @@ struct SoftmaxPlan {
     int tiles = 0;      // registers plan: 128-bit tiles per lane
 };
 
-int64_t walk_pair(const hmr_tensor_desc &out_rows, const hmr_tensor_desc &src_rows, Walk &wo, Walk &ws) {
-    // Merge the row dimensions with respect to both operands, innermost first.
-    int64_t size[HMR_MAX_DIMS], so[HMR_MAX_DIMS], ss[HMR_MAX_DIMS];
-    int n = 0;
-    int64_t count = 1;
-    for (int i = 0; i < src_rows.ndim; ++i) count *= src_rows.sizes[i];
-    wo.ndim = ws.ndim = 0;
-    if (count == 0) return 0;
-    for (int i = 0; i < src_rows.ndim; ++i) {
-        int64_t sz = src_rows.sizes[i];
-        if (sz == 1) continue;
-        int64_t p1 = 0, p2 = 0;
-        if (n > 0 && !__builtin_mul_overflow(out_rows.strides[i], sz, &p1) && p1 == so[n - 1] &&
-            !__builtin_mul_overflow(src_rows.strides[i], sz, &p2) && p2 == ss[n - 1]) {
-            size[n - 1] *= sz;
-            so[n - 1] = out_rows.strides[i];
-            ss[n - 1] = src_rows.strides[i];
-        } else {
-            size[n] = sz;
-            so[n] = out_rows.strides[i];
-            ss[n] = src_rows.strides[i];
-            ++n;
-        }
-    }
-    wo.ndim = ws.ndim = n;
-    for (int i = 0; i < n; ++i) {
-        wo.size[i] = ws.size[i] = size[n - 1 - i];
-        wo.stride[i] = so[n - 1 - i];
-        ws.stride[i] = ss[n - 1 - i];
-    }
-    return count;
-}
-
 // 128-bit chunks of the row a lane keeps: 8 (32 f32 or 16 f64 values, plus their f64 exponentials),
 // or 16 packed chunks (128 values) of a 16-bit type, whose exponentials are not kept.
 constexpr int max_tiles(int elem) { return elem == 2 ? 16 : 8; }
@@ -551,139 +519,6 @@ void launch_softmax(const SoftmaxPlan &p, const SoftmaxArgs &a, bool out_ok, hip
     }
 }
 
-hmr_status check_rows(const hmr_tensor_desc &out_rows, const hmr_tensor_desc &src_rows, int64_t n, int64_t so,
-                      int64_t si, int64_t &nrows) {
-    int64_t m = 0;
-    if (hmr_status s = check_desc(out_rows, nrows)) return s;
-    if (hmr_status s = check_desc(src_rows, m)) return s;
-    bool same = out_rows.ndim == src_rows.ndim;
-    for (int j = 0; same && j < out_rows.ndim; ++j) same = out_rows.sizes[j] == src_rows.sizes[j];
-    if (!same) return fail(HMR_INVALID, "kernel operands have different sizes");
-    if (n < 0 || so < 0 || si < 0) return fail(HMR_INVALID, "invalid row length or stride");
-    return HMR_OK;
-}
-
-// ---- exclusive cumulative product (ref: src/backend/cpu/reduce.rs:227-324) ---------------------------
-//
-// out[k] = the product of the line's elements before k (after k when reversed), accumulated one
-// element at a time in f32 (F16, BF16) or f64 (F32, F64) and rounded to the dtype as it is written;
-// the accumulator is never rounded. Multiplication isn't associative, so a line is one thread's
-// sequential loop, which is what fixes the bits: lines next to each other in memory are read
-// coalesced across the threads, and a line that is itself contiguous is read and written in 16-byte
-// tiles by its thread.
-template <class T>
-struct ProductOf {
-    using A = float;
-    static __device__ __forceinline__ A widen(T x) { return Comp<T>::up(x); }
-    static __device__ __forceinline__ T narrow(A acc) { return Comp<T>::down(acc); }
-};
-template <>
-struct ProductOf<float> {
-    using A = double;
-    static __device__ __forceinline__ A widen(float x) { return static_cast<double>(x); }
-    static __device__ __forceinline__ float narrow(A acc) { return static_cast<float>(acc); }
-};
-template <>
-struct ProductOf<double> {
-    using A = double;
-    static __device__ __forceinline__ A widen(double x) { return x; }
-    static __device__ __forceinline__ double narrow(A acc) { return acc; }
-};
-
-struct CumprodArgs {
-    char *out;
-    const char *src;
-    int64_t nlines, n, so, si;
-    Walk out_lines, src_lines;
-    int32_t reverse;
-};
-
-template <class T, int V>
-__global__ void __launch_bounds__(kBlock) cumprod_kernel(CumprodArgs a) {
-    using P = ProductOf<T>;
-    for (int64_t line = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; line < a.nlines;
-         line += static_cast<int64_t>(gridDim.x) * kBlock) {
-        const T *ps = reinterpret_cast<const T *>(a.src) + a.src_lines.offset(line);
-        T *po = reinterpret_cast<T *>(a.out) + a.out_lines.offset(line);
-        typename P::A acc = 1;
-        // The chain of multiplications is sequential, the memory accesses need not be: kAhead elements (or
-        // tiles: 128 bytes of the thread's own row) are loaded together, multiplied through in
-        // order and written together.
-        constexpr int kAhead = V == 1 ? 32 : 8;
-        if constexpr (V == 1) {
-            int64_t k = 0;
-            for (; k + kAhead <= a.n; k += kAhead) {
-                T x[kAhead];
-#pragma unroll
-                for (int j = 0; j < kAhead; ++j) x[j] = ps[(a.reverse ? a.n - 1 - (k + j) : k + j) * a.si];
-#pragma unroll
-                for (int j = 0; j < kAhead; ++j) {
-                    po[(a.reverse ? a.n - 1 - (k + j) : k + j) * a.so] = P::narrow(acc);
-                    acc = acc * P::widen(x[j]);
-                }
-            }
-            for (; k < a.n; ++k) {
-                const int64_t at = a.reverse ? a.n - 1 - k : k;
-                const T x = ps[at * a.si];  // read before the write: the operands may be one buffer
-                po[at * a.so] = P::narrow(acc);
-                acc = acc * P::widen(x);
-            }
-        } else {
-            const int64_t tiles = a.n / V;
-            auto scan_tile = [&](T(&r)[V], T(&w)[V]) {
-                if (a.reverse) {
-#pragma unroll
-                    for (int i = V - 1; i >= 0; --i) {
-                        w[i] = P::narrow(acc);
-                        acc = acc * P::widen(r[i]);
-                    }
-                } else {
-#pragma unroll
-                    for (int i = 0; i < V; ++i) {
-                        w[i] = P::narrow(acc);
-                        acc = acc * P::widen(r[i]);
-                    }
-                }
-            };
-            int64_t c = 0;
-            for (; c + kAhead <= tiles; c += kAhead) {
-                T r[kAhead][V], w[kAhead][V];
-#pragma unroll
-                for (int j = 0; j < kAhead; ++j) {
-                    load_tile<T, V, false>(reinterpret_cast<const char *>(ps + (a.reverse ? tiles - 1 - (c + j) : c + j) * V), r[j]);
-                }
-#pragma unroll
-                for (int j = 0; j < kAhead; ++j) scan_tile(r[j], w[j]);
-#pragma unroll
-                for (int j = 0; j < kAhead; ++j) {
-                    store_tile<T, V, false>(reinterpret_cast<char *>(po + (a.reverse ? tiles - 1 - (c + j) : c + j) * V), w[j]);
-                }
-            }
-            for (; c < tiles; ++c) {
-                const int64_t at = (a.reverse ? tiles - 1 - c : c) * V;
-                T r[V], w[V];
-                load_tile<T, V, false>(reinterpret_cast<const char *>(ps + at), r);
-                scan_tile(r, w);
-                store_tile<T, V, false>(reinterpret_cast<char *>(po + at), w);
-            }
-        }
-    }
-}
-
-template <class T>
-void launch_cumprod(const CumprodArgs &a, hipStream_t stream) {
-    constexpr int kVec = 16 / static_cast<int>(sizeof(T));
-    bool tiles = a.so == 1 && a.si == 1 && a.n % kVec == 0 && reinterpret_cast<uintptr_t>(a.out) % 16 == 0 &&
-                 reinterpret_cast<uintptr_t>(a.src) % 16 == 0;
-    for (int d = 0; tiles && d < a.src_lines.ndim; ++d) {
-        tiles = a.out_lines.stride[d] % kVec == 0 && a.src_lines.stride[d] % kVec == 0;
-    }
-    const int64_t want = (a.nlines + kBlock - 1) / kBlock;
-    const unsigned grid = static_cast<unsigned>(want < (int64_t{1} << 22) ? want : (int64_t{1} << 22));
-    if (tiles) hipLaunchKernelGGL((cumprod_kernel<T, kVec>), dim3(grid), dim3(kBlock), 0, stream, a);
-    else hipLaunchKernelGGL((cumprod_kernel<T, 1>), dim3(grid), dim3(kBlock), 0, stream, a);
-}
-
 }  // namespace
 }  // namespace hmr
 
@@ -742,30 +577,6 @@ hmr_status hmr_softmax(hmr_context_t ctx, const hmr_tensor_desc *out_rows, const
                 using T = typename decltype(t)::type;
                 if (log != 0) hmr::launch_softmax<T, true>(plan, a, out_ok, stream);
                 else hmr::launch_softmax<T, false>(plan, a, out_ok, stream);
-            });
-        });
-    });
-}
-
-hmr_status hmr_exclusive_cumprod(hmr_context_t ctx, const hmr_tensor_desc *out_lines, const hmr_tensor_desc *src_lines,
-                                 int64_t n, int64_t out_stride, int64_t src_stride, int32_t reverse) {
-    return fenced([&] {
-        int64_t nlines = 0;
-        if (hmr_status s = hmr::check_rows(*out_lines, *src_lines, n, out_stride, src_stride, nlines)) return s;
-        if (nlines == 0 || n == 0) return HMR_OK;
-        hmr::CumprodArgs a{};
-        const int elem = hmr::dtype_size(src_lines->dtype);
-        a.out = static_cast<char *>(out_lines->data) + out_lines->offset * elem;
-        a.src = static_cast<const char *>(src_lines->data) + src_lines->offset * elem;
-        a.nlines = hmr::walk_pair(*out_lines, *src_lines, a.out_lines, a.src_lines);
-        a.n = n;
-        a.so = out_stride;
-        a.si = src_stride;
-        a.reverse = reverse != 0;
-        return hmr::queue_on(ctx, "exclusive_cumprod", [&](hipStream_t stream) {
-            if (out_lines->dtype != src_lines->dtype) return false;
-            return hmr::with_float_type(out_lines->dtype, [&](auto t) {
-                hmr::launch_cumprod<typename decltype(t)::type>(a, stream);
             });
         });
     });

@@ -66,6 +66,7 @@ struct Machine {
     hipError_t count_error = hipSuccess;  // what hipGetDeviceCount reports instead of a count
     std::map<std::string, hipError_t> fail_next;
     std::set<void *> blocks;       // live device allocations
+    std::set<void *> pinned;       // live pinned host allocations
     std::set<FakeStream *> streams;
     std::vector<std::string> calls;  // names of the HIP calls made, in order
 };
@@ -165,6 +166,21 @@ inline hipError_t hipFree(void *p) {
         std::free(p);
     }
     return fake::done("hipFree");
+}
+// Pinned host memory: its own book, so that a leak of it shows.
+constexpr unsigned hipHostMallocDefault = 0;
+inline hipError_t hipHostMalloc(void **p, size_t n, unsigned) {
+    if (fake::armed("hipHostMalloc")) return fake::done("hipHostMalloc");
+    *p = std::calloc(n ? n : 1, 1);
+    fake::machine().pinned.insert(*p);
+    return fake::done("hipHostMalloc");
+}
+inline hipError_t hipHostFree(void *p) {
+    if (p != nullptr) {
+        if (!fake::machine().pinned.erase(p)) return fake::done("hipHostFree", hipErrorInvalidValue);
+        std::free(p);
+    }
+    return fake::done("hipHostFree");
 }
 inline hipError_t hipStreamCreateWithFlags(hipStream_t *s, unsigned) {
     if (fake::armed("hipStreamCreateWithFlags")) return fake::done("hipStreamCreateWithFlags");

@@ -57,7 +57,9 @@ static int g_failures = 0;
 
 static std::string last() { return hmr_last_error(); }
 static fake::Machine &M() { return fake::machine(); }
-static bool clean() { return M().streams.empty() && M().blocks.empty() && hmr_test_live_streams() == 0 && hipGetLastError() == hipSuccess; }
+static bool clean() {
+    return M().streams.empty() && M().blocks.empty() && M().pinned.empty() && hmr_test_live_streams() == 0 && hipGetLastError() == hipSuccess;
+}
 
 static void devices() {
     int32_t n = -1;
@@ -143,7 +145,7 @@ static void contexts() {
         EXPECT(hmr_context_create(0, &real) == HMR_OK && real != nullptr);
         EXPECT(hmr_test_live_streams() == 1 && M().streams.size() == 1 && M().blocks.size() == 1);  // its tables
         EXPECT(fake::thread().device == 1 && real->device == 0 && real->compute_units == 256 && real->reduce_scratch != nullptr);
-        EXPECT(real->tables != nullptr);
+        EXPECT(real->tables != nullptr && real->mailbox != nullptr && M().pinned.size() == 1);
         EXPECT(hmr_context_synchronize(real) == HMR_OK);
         M().fail_next["hipStreamSynchronize"] = hipErrorLaunchFailure;
         EXPECT(hmr_context_synchronize(real) == HMR_HIP_ERROR && last() == "hipStreamSynchronize(ctx->stream): unspecified launch failure");
@@ -151,7 +153,7 @@ static void contexts() {
         // Destroying frees the tables even when the stream will not go.
         M().fail_next["hipStreamDestroy"] = hipErrorInvalidHandle;
         EXPECT(hmr_context_destroy(real) == HMR_HIP_ERROR && last() == "hipStreamDestroy(ctx->stream): invalid resource handle");
-        EXPECT(M().blocks.empty());
+        EXPECT(M().blocks.empty() && M().pinned.empty());
         EXPECT(hmr_test_live_streams() == 1);  // the stream is still there, and still counted
         for (FakeStream *s : M().streams) delete s;  // the fake's books, for what follows
         M().streams.clear();
@@ -172,8 +174,13 @@ static void contexts() {
     // The tables cannot be had: the stream is given back, nothing stays allocated.
     g_tables_fail = true;
     EXPECT(hmr_context_create(0, &ctx) == HMR_OUT_OF_MEMORY && ctx == nullptr);
-    EXPECT(hmr_test_live_streams() == live && M().streams.empty() && M().blocks.empty());
+    EXPECT(hmr_test_live_streams() == live && M().streams.empty() && M().blocks.empty() && M().pinned.empty());
     g_tables_fail = false;
+
+    // Nor the mailbox.
+    M().fail_next["hipHostMalloc"] = hipErrorOutOfMemory;
+    EXPECT(hmr_context_create(0, &ctx) == HMR_OUT_OF_MEMORY && ctx == nullptr && last() == "hipHostMalloc(&mailbox, 64): out of memory");
+    EXPECT(hmr_test_live_streams() == live && M().streams.empty() && M().blocks.empty() && M().pinned.empty());
 }
 
 static void memory() {
@@ -207,6 +214,21 @@ static void memory() {
     EXPECT(hmr_copy_to_host(ctx, host, d, 16) == HMR_OK && host[1] == 2);
     const size_t calls = M().calls.size();
     EXPECT(hmr_copy_device(ctx, d, d, 0) == HMR_OK && M().calls.size() == calls);  // nothing to do, nothing called
+    // A read-back of what the mailbox mirrors is a wait and a host copy; any other transfer forgets the address.
+    {
+        const size_t before = M().calls.size();
+        std::memcpy(ctx->mailbox, "\x11\x22\x33\x44\x55\x66\x77\x88" "ABCDEFGH", 16);
+        ctx->mail_src = d;
+        unsigned char got[16] = {0};
+        EXPECT(hmr_copy_to_host(ctx, got, d, 16) == HMR_OK && got[0] == 0x11 && got[15] == 'H');
+        bool copied = false;
+        for (size_t k = before; k < M().calls.size(); ++k) copied = copied || M().calls[k] == "hipMemcpyAsync";
+        EXPECT(!copied && ctx->mail_src == d);
+        EXPECT(hmr_copy_to_host(ctx, got, d, 8) == HMR_OK && got[7] == 0x88);
+        EXPECT(hmr_copy_from_host(ctx, d, got, 8) == HMR_OK && ctx->mail_src == nullptr);
+        ctx->mail_src = d;
+        EXPECT(hmr_memset(ctx, d, 0, 16) == HMR_OK && ctx->mail_src == nullptr);
+    }
     // A megabyte and more at aligned addresses goes to the kernels: words of eight bytes when they divide the
     // size, bytes otherwise; an armed failure still comes first.
     {

@@ -534,6 +534,34 @@ def test_exclusive_cumprod_of_lines_that_vectorise_and_of_many_lines(dtype):
         h.exclusive_cumprod(h.full([4], 1, DT.I32, GPU), 0, False)
 
 
+@pytest.mark.parametrize("dtype", FLOATS)
+def test_exclusive_cumprod_in_slabs_through_lds(dtype):
+    """Lines of 128 steps and more on 16-byte boundaries go through the slab kernel: lines next to each other in
+    memory (a product along an outer dimension) and lines contiguous along their steps, last slabs that are not
+    whole, workgroups whose last lines do not exist, lines spread over two dimensions, enough workgroups for the
+    short slabs, both directions; zeros, infinities and sign changes on the way. Every line has the CPU's bits."""
+    rng = np.random.default_rng(47)
+    cases = (([300, 72], 0), ([129, 40], 0), ([1000, 16], 0), ([6, 200, 48], 1), ([3, 260, 5, 8], 1),
+             ([90, 264], 1), ([5, 20, 136], 2), ([17, 4096], 1), ([600, 130, 64], 1), ([40000, 128], 1))
+    for shape, dim in cases:
+        v = 1.0 + rng.standard_normal(int(np.prod(shape))) * 0.02
+        v[rng.integers(0, v.size, 30)] = 0.0
+        v[rng.integers(0, v.size, 5)] = np.inf
+        v[rng.integers(0, v.size, 50)] = -1.25
+        x = tensor(from_f64(v, dtype), dtype).reshape(shape)
+        xg = x.to(GPU)
+        for reverse in (False, True):
+            assert_bitwise(h.exclusive_cumprod(xg, dim, reverse), h.exclusive_cumprod(x, dim, reverse),
+                           f"{dtype} {shape} dim {dim} reverse {reverse}")
+    # A view that starts off the first element but on a 16-byte boundary, and one that does not (the thread-per-line kernel).
+    base = tensor(from_f64(1.0 + rng.standard_normal(400 * 80) * 0.02, dtype), dtype).reshape([400, 80])
+    g = base.to(GPU)
+    for cut in (16, 3):
+        x, xg = base.narrow(1, cut, 48).narrow(0, 8, 384), g.narrow(1, cut, 48).narrow(0, 8, 384)
+        for d in (0, 1):
+            assert_bitwise(h.exclusive_cumprod(xg, d, True), h.exclusive_cumprod(x, d, True), f"{dtype} view cut {cut} dim {d}")
+
+
 def test_exclusive_cumprod_through_the_c_abi_in_place_and_its_errors():
     from ctypes import byref
 
@@ -563,5 +591,17 @@ def test_exclusive_cumprod_through_the_c_abi_in_place_and_its_errors():
         other = capi.make_desc(dx.ptr, capi.F32, [rows - 1], [n], 0)
         assert L.hmr_exclusive_cumprod(ctx.handle, byref(lines), byref(other), n, 1, 1, 0) == capi.HMR_INVALID
         capi.check(L.hmr_exclusive_cumprod(ctx.handle, byref(lines), byref(lines), 0, 1, 1, 1))  # nothing to do
+        # In place through the slab kernel too (columns of a [600, 64] matrix, then its rows backwards).
+        big = (1.0 + np.random.default_rng(4).standard_normal((600, 64)) * 0.05).astype(np.float32)
+        db = ctx.upload(big)
+        columns = capi.make_desc(db.ptr, capi.F32, [64], [1], 0)
+        capi.check(L.hmr_exclusive_cumprod(ctx.handle, byref(columns), byref(columns), 600, 64, 64, 0))
+        ctx.synchronize()
+        want = np.empty_like(big)
+        acc = np.ones(64, dtype=np.float64)
+        for k in range(600):
+            want[k] = acc.astype(np.float32)
+            acc = acc * big[k].astype(np.float64)
+        np.testing.assert_array_equal(db.download(np.float32, 600 * 64).reshape(600, 64), want)
     finally:
         ctx.close()
