@@ -85,6 +85,7 @@ hmr_status plan_reduction(const hmr_tensor_desc *out, const hmr_tensor_desc &kep
     a.nout = build_walk(kept, a.kept);
     a.nred = build_walk(red, a.red);
     a.partials = nullptr;
+    a.runs = Runs{};
     p.kind = ReduceKind::Any;
     p.group = 1;
     p.splits = 1;
@@ -113,6 +114,44 @@ hmr_status plan_reduction(const hmr_tensor_desc *out, const hmr_tensor_desc &kep
             if (a.nout * kBlock < kTargetLanes / 2) cut(p, ceil_div(2 * kTargetLanes, a.nout * kBlock), 4096);
         }
         return HMR_OK;
+    }
+    // Rows over several runs: one reduced dimension has stride 1 and holds whole aligned vectors, up to three
+    // others count the runs (whatever their order: a folded range may be walked in any order, and max/min are
+    // told each element's position in the CPU's order).
+    if (a.red.ndim >= 2 && a.red.ndim <= kRunDims + 1 && base_aligned && strides_aligned(a.kept, 0) &&
+        a.nred / vec < (int64_t{1} << 31)) {
+        int inner = -1;
+        for (int d = 0; d < a.red.ndim && inner < 0; ++d) {
+            if (a.red.stride[d] == 1 && a.red.size[d] % vec == 0 && a.red.size[d] * elem >= 256) inner = d;
+        }
+        bool ok = inner >= 0;
+        for (int d = 0; ok && d < a.red.ndim; ++d) ok = d == inner || (a.red.stride[d] * elem) % 16 == 0;
+        if (ok) {
+            Runs &r = a.runs;
+            int64_t pos = 1;
+            r.dims = 0;
+            for (int d = 0; d < a.red.ndim; ++d) {
+                if (d == inner) {
+                    r.length = static_cast<uint32_t>(a.red.size[d]);
+                    r.vectors = make_fastdiv(static_cast<uint32_t>(a.red.size[d] / vec));
+                    r.inner_pos = pos;
+                } else {
+                    r.size[r.dims] = make_fastdiv(static_cast<uint32_t>(a.red.size[d]));
+                    r.stride[r.dims] = a.red.stride[d];
+                    r.pos[r.dims] = pos;
+                    ++r.dims;
+                }
+                pos *= a.red.size[d];
+            }
+            p.kind = ReduceKind::Rows;
+            if (a.nout * kWave >= kTargetLanes / 2 || a.nred <= 2048) {
+                p.group = kWave;
+            } else {
+                p.group = kBlock;
+                if (a.nout * kBlock < kTargetLanes / 2) cut(p, ceil_div(2 * kTargetLanes, a.nout * kBlock), 4096);
+            }
+            return HMR_OK;
+        }
     }
     // Cols: a contiguous run of outputs, one strided reduced dimension (fewer than 2^31 rows: the kernel
     // counts rows in 32 bits).

@@ -329,6 +329,21 @@ __device__ __forceinline__ void put_partial(void *partials, int64_t nout, int64_
 
 // ---- arguments shared by the kernels ----------------------------------------------------------------
 
+// A reduced range made of several contiguous runs (a Rows plan over more than one reduced dimension, one of them
+// with stride 1: the statistics of a batch normalisation over [N, C, L], the sum of a transposed view). The runs
+// are counted over the other reduced dimensions, innermost first; an element's position in the CPU's order of the
+// reduced range (what max/min report) is the sum of its coordinates times `pos`.
+constexpr int kRunDims = 3;
+struct Runs {
+    int32_t dims;               // the other reduced dimensions; 0: the range is one run
+    uint32_t length;            // elements of a run, a multiple of the 16-byte vector
+    FastDiv vectors;            // 16-byte vectors of a run
+    int64_t inner_pos;          // position stride of a run's elements
+    FastDiv size[kRunDims];     // the other dimensions ...
+    int64_t stride[kRunDims];   // ... their strides in elements ...
+    int64_t pos[kRunDims];      // ... and position strides
+};
+
 struct ReduceArgs {
     const char *src;  // address of the source's element (offset)
     Walk kept;        // kept dims, source strides
@@ -338,6 +353,7 @@ struct ReduceArgs {
     int64_t splits;   // slices of the reduced range
     int64_t chunk;    // reduced elements per slice
     void *partials;   // workspace for splits > 1
+    Runs runs;        // Rows plans only
 };
 
 // Sources are read once: every vector load carries the nontemporal hint (a compile-time property of the load;
@@ -466,6 +482,48 @@ __global__ void __launch_bounds__(kBlock) reduce_rows_kernel(ReduceArgs a, Op op
             // Whole vectors: positions begin + (lane + k*G)*V.
             const int64_t nvec = (end - begin) / V;
             int64_t k = lane;
+            if (a.runs.dims > 0) {
+                // Several runs: vector number -> (run, vector inside it) by a 32-bit division, the run's start
+                // and its first position from its coordinates. Slices are whole vectors, runs too.
+                const uint32_t v0 = static_cast<uint32_t>(begin / V);
+                auto locate = [&](uint32_t v, int64_t &at, int64_t &pos) {
+                    uint32_t run = divide(v, a.runs.vectors);
+                    const uint32_t inside = (v - run * a.runs.vectors.div) * V;
+                    at = inside;
+                    pos = inside * a.runs.inner_pos;
+                    for (int d = 0; d < a.runs.dims; ++d) {
+                        const uint32_t q = divide(run, a.runs.size[d]);
+                        const int64_t c = run - q * a.runs.size[d].div;
+                        run = q;
+                        at += c * a.runs.stride[d];
+                        pos += c * a.runs.pos[d];
+                    }
+                };
+                for (; k + (U - 1) * G < nvec; k += U * G) {
+                    T r[U][V];
+                    int64_t pos[U];
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        int64_t at;
+                        locate(v0 + static_cast<uint32_t>(k + u * G), at, pos[u]);
+                        load_stream<T, V>(reinterpret_cast<const char *>(p + at), r[u]);
+                    }
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+#pragma unroll
+                        for (int i = 0; i < V; ++i) op.lane_add(state, r[u][i], pos[u] + i * a.runs.inner_pos, ctx);
+                    }
+                }
+                for (; k < nvec; k += G) {
+                    T r[V];
+                    int64_t at, pos;
+                    locate(v0 + static_cast<uint32_t>(k), at, pos);
+                    load_stream<T, V>(reinterpret_cast<const char *>(p + at), r);
+#pragma unroll
+                    for (int i = 0; i < V; ++i) op.lane_add(state, r[i], pos + i * a.runs.inner_pos, ctx);
+                }
+                k = nvec;  // nothing ragged: the range is whole runs
+            }
             for (; k + (U - 1) * G < nvec; k += U * G) {
                 T r[U][V];
 #pragma unroll
@@ -484,8 +542,10 @@ __global__ void __launch_bounds__(kBlock) reduce_rows_kernel(ReduceArgs a, Op op
 #pragma unroll
                 for (int i = 0; i < V; ++i) op.lane_add(state, r[i], begin + k * V + i, ctx);
             }
-            // Ragged end of the range (fewer than V elements).
-            for (int64_t r = begin + nvec * V + lane; r < end; r += G) op.lane_add(state, p[r], r, ctx);
+            // Ragged end of the range (fewer than V elements; one run only).
+            if (a.runs.dims == 0) {
+                for (int64_t r = begin + nvec * V + lane; r < end; r += G) op.lane_add(state, p[r], r, ctx);
+            }
         }
         Acc acc = wave_fold(op, op.lane_done(state));
         if constexpr (WAVES == 4) {

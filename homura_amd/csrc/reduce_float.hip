@@ -20,7 +20,7 @@ bool launch_float_reduce(int op, int dtype, const ReducePlan &plan, void *partia
 
 // Rows plan, one slice, and a row that fits G lanes x 16 tiles of 16 bytes: registers.
 static int var_row_tiles(const ReducePlan &plan, int elem) {
-    if (plan.kind != ReduceKind::Rows || plan.splits != 1) return 0;
+    if (plan.kind != ReduceKind::Rows || plan.splits != 1 || plan.args.runs.dims != 0) return 0;
     const int64_t vec = 16 / elem;
     if (plan.args.nred % vec != 0) return 0;  // the register kernel takes whole 16-byte chunks
     const int64_t per = (plan.args.nred + vec * plan.group - 1) / (vec * plan.group);
@@ -44,7 +44,16 @@ bool launch_var_single_pass(int dtype, const ReducePlan &plan, void *partials, v
             return;
         }
         const int tiles = var_row_tiles(plan, static_cast<int>(sizeof(T)));
-        if (tiles == 0) return;
+        if (tiles == 0) {
+            // Rows that do not fit the registers - made of several runs, or cut into slices -: the same one pass
+            // of shifted sums (every lane about its own first element, merged by Chan's formula) instead of two
+            // passes over memory; f64 results keep the two passes, as for columns.
+            if (plan.kind == ReduceKind::Rows && (plan.args.runs.dims != 0 || plan.splits > 1) && !std::is_same_v<T, double>) {
+                launch_reduce(plan, partials, MomentsFold<T>{}, sink, stream);
+                done = true;
+            }
+            return;
+        }
         ReduceArgs a = plan.args;
         a.splits = 1;
         a.chunk = a.nred;

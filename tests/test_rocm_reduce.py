@@ -382,13 +382,44 @@ PLAN_SHAPES = [
     ([8192, 2048], [0], 16, True),          # long columns in few tiles: 1024-lane workgroups, four row groups
     ([6, 700, 96], [1], 16, True),          # columns under an outer kept dimension
     ([5000, 20], [1], 1, False),            # short rows: a lane per output
-    ([9, 2, 3000], [0, 2], 256, True),      # two reduced dimensions: any layout, 256 lanes
+    ([9, 2, 3000], [0, 2], 256, True),      # two reduced dimensions, the inner one contiguous: rows made of runs, cut
+    ([64, 40, 512], [0, 2], 256, True),     # ... the statistics of a batch normalisation
+    ([8, 3000, 64], [0, 2], 64, False),     # ... a wave per output, runs of 256 bytes
+    ([3, 5, 7, 256], [0, 1, 3], 256, False),  # ... three reduced dimensions (the outer two merge)
+    ([3, 5, 4, 6, 128], [0, 2, 4], 64, False),  # ... which do not merge
     ([70, 600, 70], [0, 2], 256, False),    # ... without slices
     ([7, 9, 11], [0, 2], 64, False),        # ... a wave per output
     ([100000, 3], [0], 256, True),          # narrow outputs: too few columns for the column kernel
     ([5, 1], [1], 1, False),
     ([(1 << 22) + 1000, 2], [1], 1, False),  # more outputs than one pass of the grid
 ]
+
+
+def test_reductions_over_runs_report_positions_in_the_cpus_order():
+    """A reduced range whose contiguous dimension is not its innermost one (a transposed or permuted view folded as
+    a whole, or along two of its dimensions) is walked run by run, in memory order; extremes must still report the
+    first position in the view's own row-major order, ties, signed zeros and NaNs included."""
+    rng = np.random.default_rng(77)
+    for dtype in (DT.F32, DT.BF16, DT.F64, DT.I32):
+        for shape, order in (([300, 256], [1, 0]), ([12, 64, 96], [1, 0, 2]), ([12, 64, 96], [2, 0, 1]), ([5, 6, 7, 128], [2, 3, 0, 1])):
+            n = prod(shape)
+            letters = rng.choice([-1.0, 0.0, -0.0, 1.0, np.nan], n, p=[0.3, 0.2, 0.2, 0.28, 0.02])
+            if dtype == DT.I32:
+                x = tensor(rng.integers(-3, 4, n).astype(np.int32), dtype, shape)
+            else:
+                x = tensor(from_f64(letters, dtype), dtype, shape)
+            v, vg = x.permute(order), x.to(GPU).permute(order)
+            what = f"{dtype} {shape} permuted {order}"
+            for name in ("argmax", "argmin", "max", "min"):
+                assert_bitwise(getattr(vg, name)(), getattr(v, name)(), f"{name} of {what}")
+            y = finite(DT.F32, n, 20, 900).reshape(shape) if dtype != DT.I32 else x
+            w, wg = y.permute(order), y.to(GPU).permute(order)
+            c = w.sum()
+            if dtype == DT.I32:
+                assert_bitwise(wg.sum(), c, f"sum of {what}")
+            else:
+                check_sum(wg.sum(), c, w.to(DT.F64).abs().sum(), n, False, f"sum of {what}")
+                check_sum(wg.mean(), w.mean(), w.to(DT.F64).abs().sum(), n, True, f"mean of {what}")
 
 
 def test_ties_and_nans_pick_the_cpus_position():
