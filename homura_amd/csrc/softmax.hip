@@ -425,13 +425,556 @@ __global__ void __launch_bounds__(kBlock) softmax_stream_kernel(SoftmaxArgs a) {
     }
 }
 
+// ---- few long rows: a row cut across workgroups ----------------------------------------------------------
+//
+// A contiguous row too long for the registers of one workgroup, or so few rows that a workgroup per row leaves
+// most of the GPU idle, is cut into slices of C chunks per lane of a 256-lane workgroup. Two launches
+// (ref: csrc/reduce.hip:314-360 plans the same split): the first leaves every slice's maximum and the sum of
+// its exponentials about that maximum in the workspace; the second folds a row's slices - in slice order, so
+// the result does not depend on which workgroup ran when - into the row's maximum and sum, and writes its own
+// slice. A slice made of -inf only contributes nothing (and a row made of nothing else comes out NaN, as on
+// the CPU). KEEP: the first launch reads through the caches, so that the second finds a source of up to a
+// couple of hundred megabytes in the memory-side cache; larger sources stream both times.
+// exp(t), t <= 0, for moving a sum of exponentials to a higher maximum: to the accuracy the sums themselves have
+// (F64 rows: the library's exp; everything else is judged in f32 or less, and the polynomial's 2^-36 is plenty).
+template <class X>
+__device__ __forceinline__ double rescale(double t) {
+    if constexpr (std::is_same_v<X, double>) return exp(t);
+    else return exp_neg_f64(t);
+}
+
+struct SlicePartial {
+    double max, sum;
+};
+
+struct SliceArgs {
+    char *out;
+    const char *src;
+    Walk out_rows, src_rows;
+    int64_t nrows, n;
+    int64_t slices;  // per row
+    SlicePartial *partials;  // [row][slice]
+    int32_t stream_stores;
+};
+
+// exp(x - mx) summed over the V elements of one chunk, as the registers kernel sums them.
+template <class T, bool LOG>
+__device__ __forceinline__ double chunk_sum(const u32x4 &raw, typename SoftmaxMath<T>::X mx) {
+    using M = SoftmaxMath<T>;
+    using X = typename M::X;
+    using E = typename M::E;
+    constexpr int V = 16 / static_cast<int>(sizeof(T));
+    X x[V];
+    M::unpack(raw, x);
+    // An element of -inf adds nothing, also about a maximum of -inf (where exp(-inf + inf) would say NaN): a
+    // part of a row may be -inf throughout while the row is not. A NaN adds itself whatever the maximum.
+    const X low = -__builtin_huge_valf();
+    if constexpr (std::is_same_v<E, double>) {
+        double sum = 0.0;
+#pragma unroll
+        for (int i = 0; i < V; ++i) sum += x[i] == low ? 0.0 : M::ex(x[i], mx);
+        return sum;
+    } else {
+        E e[V];
+#pragma unroll
+        for (int i = 0; i < V; ++i) e[i] = x[i] == low ? 0.0f : M::ex(x[i], mx);
+        float part = ((e[0] + e[1]) + (e[2] + e[3])) + ((e[4] + e[5]) + (e[6] + e[7]));
+        double sum = 0.0;
+        if constexpr (LOG) {
+            // The terms that are exactly 1 are counted, not added (see the registers kernel).
+            if (part >= 1.0f) {
+                float ones = 0.0f;
+#pragma unroll
+                for (int i = 0; i < V; ++i) {
+                    const bool one = e[i] == 1.0f;
+                    ones += one ? 1.0f : 0.0f;
+                    e[i] = one ? 0.0f : e[i];
+                }
+                part = ((e[0] + e[1]) + (e[2] + e[3])) + ((e[4] + e[5]) + (e[6] + e[7]));
+                sum = static_cast<double>(ones);
+            }
+        }
+        return sum + static_cast<double>(part);
+    }
+}
+
+template <class T, int C, bool LOG, bool KEEP>
+__global__ void __launch_bounds__(kBlock) softmax_slice_stats_kernel(SliceArgs a) {
+    using M = SoftmaxMath<T>;
+    using X = typename M::X;
+    using MaxFold = std::conditional_t<std::is_same_v<X, float>, MaxOpF, MaxOp>;
+    constexpr int V = 16 / static_cast<int>(sizeof(T));
+    __shared__ double lds[kBlock / kWave];
+    const int64_t row = blockIdx.x / a.slices, slice = blockIdx.x - row * a.slices;
+    const int lane = threadIdx.x;
+    const int64_t nvec = a.n / V, first = slice * (C * kBlock);
+    const char *src = a.src + a.src_rows.offset(row) * static_cast<int64_t>(sizeof(T));
+    u32x4 raw[C];
+    bool inside[C];
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+        const int64_t tile = first + c * kBlock + lane;
+        inside[c] = tile < nvec;
+        const u32x4 *q = reinterpret_cast<const u32x4 *>(src + (inside[c] ? tile : nvec - 1) * 16);
+        if constexpr (KEEP) raw[c] = *q;
+        else raw[c] = __builtin_nontemporal_load(q);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    X mx = -__builtin_huge_valf();
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+        X x[V];
+        M::unpack(raw[c], x);
+        X m = -__builtin_huge_valf();
+#pragma unroll
+        for (int i = 0; i < V; i += 2) m = max3(m, x[i], x[i + 1]);
+        mx = inside[c] && m > mx ? m : mx;
+    }
+    mx = row_fold<kBlock>(MaxFold{}, mx, reinterpret_cast<X *>(lds));
+    double sum = 0.0;
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+        forget(raw[c]);
+        const double part = chunk_sum<T, LOG>(raw[c], mx);
+        sum += inside[c] ? part : 0.0;
+    }
+    sum = row_fold<kBlock>(SumOp{}, sum, lds);
+    if (lane == 0) a.partials[blockIdx.x] = SlicePartial{static_cast<double>(mx), sum};
+}
+
+template <class T, int C, bool LOG>
+__global__ void __launch_bounds__(kBlock) softmax_slice_write_kernel(SliceArgs a) {
+    using M = SoftmaxMath<T>;
+    using X = typename M::X;
+    using E = typename M::E;
+    constexpr int V = 16 / static_cast<int>(sizeof(T));
+    __shared__ double lds[kBlock / kWave];
+    const int64_t row = blockIdx.x / a.slices, slice = blockIdx.x - row * a.slices;
+    const int lane = threadIdx.x;
+    const int64_t nvec = a.n / V, first = slice * (C * kBlock);
+    const char *src = a.src + a.src_rows.offset(row) * static_cast<int64_t>(sizeof(T));
+    char *out = a.out + a.out_rows.offset(row) * static_cast<int64_t>(sizeof(T));
+    u32x4 raw[C];
+    bool inside[C];
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+        const int64_t tile = first + c * kBlock + lane;
+        inside[c] = tile < nvec;
+        raw[c] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + (inside[c] ? tile : nvec - 1) * 16));
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // The row's maximum and sum from its slices': a lane folds slices lane, lane + 256, ... in that order, then
+    // the lanes fold in a fixed tree.
+    const SlicePartial *mine = a.partials + row * a.slices;
+    double top = -__builtin_huge_val();
+    for (int64_t j = lane; j < a.slices; j += kBlock) top = mine[j].max > top ? mine[j].max : top;
+    top = row_fold<kBlock>(MaxOp{}, top, lds);
+    double sum = 0.0;
+    for (int64_t j = lane; j < a.slices; j += kBlock) {
+        const SlicePartial part = mine[j];
+        // A slice of -inf only has sum 0 and stays out (its scale would be exp(-inf - top), or NaN for a row of
+        // -inf only, which comes out NaN below without it).
+        if (part.sum != 0.0) sum += part.sum * rescale<X>(part.max - top);
+    }
+    sum = row_fold<kBlock>(SumOp{}, sum, lds);
+    if (top == -__builtin_huge_val()) sum = __builtin_nan("");  // a row of -inf only: NaN, as exp(-inf - -inf) makes it
+    const X mx = static_cast<X>(top);
+    const E scale = LOG ? M::lg(sum) : M::scale(sum);
+    const __amdgpu_buffer_rsrc_t out_row = __builtin_amdgcn_make_buffer_rsrc(out, 0, -1, 0x00020000);
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+        const int64_t tile = first + c * kBlock + lane;
+        X x[V];
+        M::unpack(raw[c], x);
+        decltype(M::logsoft(x[0], mx, scale)) res[V];
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+            if constexpr (LOG) {
+                res[i] = M::logsoft(x[i], mx, scale);
+            } else if constexpr (M::kKeep) {
+                res[i] = M::soft(x[i], mx, M::ex(x[i], mx), scale);
+            } else {
+                res[i] = M::soft(x[i], mx, E(0), scale);
+            }
+        }
+        if (inside[c]) {
+            // A row's bytes may pass 4 GiB: the buffer form (32-bit offsets) serves rows below that.
+            if (a.stream_stores) __builtin_nontemporal_store(M::pack(res), reinterpret_cast<u32x4 *>(out + tile * 16));
+            else __builtin_amdgcn_raw_buffer_store_b128(M::pack(res), out_row, static_cast<int>(tile * 16), 0, 17 /* sc0 sc1 */);
+        }
+    }
+}
+
+// ---- rows that run across memory: a softmax along an outer dimension ----------------------------------
+//
+// The rows' elements lie `si` apart and the rows themselves next to each other (softmax over dim 0 of a
+// matrix, over the channels of [N, C, H, W]). A lane owns V adjacent rows - one 16-byte vector per position -
+// and the workgroup's lanes split in 8 across (128 bytes of every position; 16 or 32 across were no faster) times
+// RG row groups that take the positions in turn. Two passes over the source: the first keeps, per row, a running
+// maximum and the sum of exponentials about it (when the maximum rises the sum is rescaled), folded across the
+// row groups in a fixed order; the second writes. The second pass finds the tile in the memory-side cache when
+// the tiles in flight fit it.
+struct ColsArgs {
+    char *out;
+    const char *src;
+    Walk out_outer, src_outer;  // the row dimensions outside the contiguous run
+    int64_t inner;              // rows in the contiguous run
+    int64_t tiles_per_run;      // tiles of kColsAcross * V rows in it
+    int64_t n, so, si;
+    int64_t tiles;
+};
+
+constexpr int kColsAcross = 8;
+
+// (max, sum about it) of a row part; merging rescales the side with the lower maximum.
+template <class X>
+struct Running {
+    X m;
+    double s;
+};
+template <class X>
+__device__ __forceinline__ Running<X> merge(Running<X> a, Running<X> b) {
+    const X m = b.m > a.m ? b.m : a.m;
+    // A side that holds nothing yet (sum 0: no element, or -inf only) stays out: its scale may be exp(-inf + inf).
+    const double sa = a.s != 0.0 ? a.s * rescale<X>(static_cast<double>(a.m) - static_cast<double>(m)) : 0.0;
+    const double sb = b.s != 0.0 ? b.s * rescale<X>(static_cast<double>(b.m) - static_cast<double>(m)) : 0.0;
+    return Running<X>{m, sa + sb};
+}
+
+template <class T, int BLOCK, bool LOG>
+__global__ void __launch_bounds__(BLOCK) softmax_cols_kernel(ColsArgs a) {
+    using M = SoftmaxMath<T>;
+    using X = typename M::X;
+    using E = typename M::E;
+    constexpr int V = 16 / static_cast<int>(sizeof(T));
+    constexpr int RG = BLOCK / kColsAcross;   // row groups
+    constexpr int kWaves = BLOCK / kWave;
+    constexpr int kGroupsPerWave = kWave / kColsAcross;
+    constexpr int U = 4;                      // positions in flight per lane
+    __shared__ X lds_m[kWaves][kColsAcross * V];
+    __shared__ double lds_s[kWaves][kColsAcross * V];
+    const int across = threadIdx.x % kColsAcross, rg = threadIdx.x / kColsAcross;
+    const X kLow = -__builtin_huge_valf();
+    for (int64_t tile = blockIdx.x; tile < a.tiles; tile += gridDim.x) {
+        const int64_t run = tile / a.tiles_per_run, in_run = tile - run * a.tiles_per_run;
+        const int64_t row0 = (in_run * kColsAcross + across) * V;  // this lane's first row inside the run
+        const bool live = row0 < a.inner;
+        const int64_t r = live ? row0 : 0;
+        const T *src = reinterpret_cast<const T *>(a.src) + a.src_outer.offset(run) + r;
+        T *out = reinterpret_cast<T *>(a.out) + a.out_outer.offset(run) + r;
+        // Pass 1.
+        Running<X> state[V];
+#pragma unroll
+        for (int i = 0; i < V; ++i) state[i] = Running<X>{kLow, 0.0};
+        for (int64_t k0 = rg; k0 < a.n; k0 += static_cast<int64_t>(U) * RG) {
+            u32x4 raw[U];
+            bool valid[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int64_t k = k0 + static_cast<int64_t>(u) * RG;
+                valid[u] = k < a.n;
+                raw[u] = *reinterpret_cast<const u32x4 *>(src + (valid[u] ? k : k0) * a.si);
+            }
+            X x[U][V];
+#pragma unroll
+            for (int u = 0; u < U; ++u) M::unpack(raw[u], x[u]);
+            bool rose = false;
+            X top[V];
+#pragma unroll
+            for (int i = 0; i < V; ++i) {
+                X m = state[i].m;
+#pragma unroll
+                for (int u = 0; u < U; ++u) m = valid[u] && x[u][i] > m ? x[u][i] : m;
+                top[i] = m;
+                rose |= m != state[i].m && state[i].s != 0.0;
+            }
+            // Rescaling is rare after a row's first positions: the whole wave skips it when no lane needs it.
+            if (__builtin_amdgcn_ballot_w64(rose) != 0) {
+#pragma unroll
+                for (int i = 0; i < V; ++i) {
+                    if (state[i].s != 0.0) state[i].s *= rescale<X>(static_cast<double>(state[i].m) - static_cast<double>(top[i]));
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < V; ++i) {
+                state[i].m = top[i];
+                // An element of -inf adds nothing, also while the running maximum is -inf (exp(-inf + inf) would
+                // say NaN): the end of the pass sees a row that holds nothing else. A NaN adds itself.
+                if constexpr (std::is_same_v<E, double>) {
+                    double add = 0.0;
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        const double e = M::ex(x[u][i], top[i]);
+                        add += valid[u] && x[u][i] != kLow ? e : 0.0;
+                    }
+                    state[i].s += add;
+                } else {
+                    // Halves: the batch's terms meet in f32, one f64 addition per batch; for log_softmax the
+                    // terms that are exactly 1 are counted instead of added (see the registers kernel).
+                    float e[U], ones = 0.0f;
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        e[u] = valid[u] && x[u][i] != kLow ? M::ex(x[u][i], top[i]) : 0.0f;
+                        if constexpr (LOG) {
+                            const bool one = e[u] == 1.0f;
+                            ones += one ? 1.0f : 0.0f;
+                            e[u] = one ? 0.0f : e[u];
+                        }
+                    }
+                    static_assert(U == 4, "the pairwise sum below");
+                    state[i].s += static_cast<double>((e[0] + e[1]) + (e[2] + e[3]));
+                    if constexpr (LOG) state[i].s += static_cast<double>(ones);
+                }
+            }
+        }
+        // The row groups meet in two rounds, each by shuffles inside a wave (lanes 8, 16, 32 apart hold the same
+        // rows) and through LDS across the waves, in a fixed order: first the rows' maxima; then every lane moves
+        // its own sums to them - the only exponentials of the meeting, one per row and lane - and the sums add up.
+        X mx[V];
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+            X m = state[i].m;
+#pragma unroll
+            for (int step = kColsAcross; step < kWave; step <<= 1) {
+                const X other = shfl_xor_any(m, step);
+                m = other > m ? other : m;
+            }
+            mx[i] = m;
+        }
+        __syncthreads();  // the last tile's readers are done
+        if ((threadIdx.x % kWave) < kColsAcross) {
+#pragma unroll
+            for (int i = 0; i < V; ++i) lds_m[threadIdx.x / kWave][across * V + i] = mx[i];
+        }
+        __syncthreads();
+        double total[V];
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+            X m = lds_m[0][across * V + i];
+#pragma unroll
+            for (int w = 1; w < kWaves; ++w) {
+                const X other = lds_m[w][across * V + i];
+                m = other > m ? other : m;
+            }
+            mx[i] = m;
+            // Sums of nothing (no element yet, or -inf only) stay 0: their scale may be exp(-inf + inf).
+            double s = state[i].s;
+            if (s != 0.0 && state[i].m != m) s *= rescale<X>(static_cast<double>(state[i].m) - static_cast<double>(m));
+#pragma unroll
+            for (int step = kColsAcross; step < kWave; step <<= 1) s += shfl_xor_any(s, step);
+            total[i] = s;
+        }
+        if ((threadIdx.x % kWave) < kColsAcross) {
+#pragma unroll
+            for (int i = 0; i < V; ++i) lds_s[threadIdx.x / kWave][across * V + i] = total[i];
+        }
+        __syncthreads();
+        E scale[V];
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+            double sum = lds_s[0][across * V + i];
+#pragma unroll
+            for (int w = 1; w < kWaves; ++w) sum += lds_s[w][across * V + i];
+            if (mx[i] == kLow) sum = __builtin_nan("");  // a row of -inf only
+            scale[i] = LOG ? M::lg(sum) : M::scale(sum);
+        }
+        (void)kGroupsPerWave;
+        // Pass 2.
+        for (int64_t k0 = rg; k0 < a.n; k0 += static_cast<int64_t>(U) * RG) {
+            u32x4 raw[U];
+            bool valid[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int64_t k = k0 + static_cast<int64_t>(u) * RG;
+                valid[u] = k < a.n;
+                raw[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + (valid[u] ? k : k0) * a.si));
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                X x[V];
+                M::unpack(raw[u], x);
+                decltype(M::logsoft(x[0], mx[0], scale[0])) res[V];
+#pragma unroll
+                for (int i = 0; i < V; ++i) {
+                    if constexpr (LOG) res[i] = M::logsoft(x[i], mx[i], scale[i]);
+                    else if constexpr (M::kKeep) res[i] = M::soft(x[i], mx[i], M::ex(x[i], mx[i]), scale[i]);
+                    else res[i] = M::soft(x[i], mx[i], E(0), scale[i]);
+                }
+                const int64_t k = k0 + static_cast<int64_t>(u) * RG;
+                if (valid[u] && live) __builtin_nontemporal_store(M::pack(res), reinterpret_cast<u32x4 *>(out + k * a.so));
+            }
+        }
+    }
+}
+
+// The same rows when every lane's share of the positions fits its registers (C positions per lane, one 16-byte
+// vector of V rows each): read once, all loads in flight together, written from the registers. The streaming
+// form above pays the memory's latency once per batch of four positions and reads the source twice.
+template <class T, int BLOCK, int C, bool LOG>
+__global__ void __launch_bounds__(BLOCK) softmax_cols_regs_kernel(ColsArgs a) {
+    using M = SoftmaxMath<T>;
+    using X = typename M::X;
+    using E = typename M::E;
+    constexpr int V = 16 / static_cast<int>(sizeof(T));
+    constexpr int RG = BLOCK / kColsAcross;
+    constexpr int kWaves = BLOCK / kWave;
+    __shared__ X lds_m[kWaves][kColsAcross * V];
+    __shared__ double lds_s[kWaves][kColsAcross * V];
+    const int across = threadIdx.x % kColsAcross, rg = threadIdx.x / kColsAcross;
+    const X kLow = -__builtin_huge_valf();
+    for (int64_t tile = blockIdx.x; tile < a.tiles; tile += gridDim.x) {
+        const int64_t run = tile / a.tiles_per_run, in_run = tile - run * a.tiles_per_run;
+        const int64_t row0 = (in_run * kColsAcross + across) * V;
+        const bool live = row0 < a.inner;
+        const int64_t r = live ? row0 : 0;
+        const T *src = reinterpret_cast<const T *>(a.src) + a.src_outer.offset(run) + r;
+        T *out = reinterpret_cast<T *>(a.out) + a.out_outer.offset(run) + r;
+        u32x4 raw[C];
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const int64_t k = rg + static_cast<int64_t>(c) * RG;
+            raw[c] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + (k < a.n ? k : 0) * a.si));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // The rows' maxima: this lane's positions, the wave's row groups (lanes kColsAcross and more apart hold
+        // the same rows), the waves through LDS. A position past the end re-read the row's first one.
+        X mx[V];
+#pragma unroll
+        for (int i = 0; i < V; ++i) mx[i] = kLow;
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            X x[V];
+            M::unpack(raw[c], x);
+#pragma unroll
+            for (int i = 0; i < V; ++i) mx[i] = x[i] > mx[i] ? x[i] : mx[i];
+        }
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+#pragma unroll
+            for (int step = kColsAcross; step < kWave; step <<= 1) {
+                const X other = shfl_xor_any(mx[i], step);
+                mx[i] = other > mx[i] ? other : mx[i];
+            }
+        }
+        __syncthreads();  // the last tile's readers are done
+        if ((threadIdx.x % kWave) < kColsAcross) {
+#pragma unroll
+            for (int i = 0; i < V; ++i) lds_m[threadIdx.x / kWave][across * V + i] = mx[i];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+            X m = lds_m[0][across * V + i];
+#pragma unroll
+            for (int w = 1; w < kWaves; ++w) {
+                const X other = lds_m[w][across * V + i];
+                m = other > m ? other : m;
+            }
+            mx[i] = m;
+        }
+        // The sums about them, as the CPU forms them (exp(x - max), so a row of -inf only or one holding +inf or a
+        // NaN comes out NaN by itself).
+        double sum[V];
+#pragma unroll
+        for (int i = 0; i < V; ++i) sum[i] = 0.0;
+        if constexpr (std::is_same_v<E, double>) {
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+                X x[V];
+                forget(raw[c]);
+                M::unpack(raw[c], x);
+                const bool valid = rg + static_cast<int64_t>(c) * RG < a.n;
+#pragma unroll
+                for (int i = 0; i < V; ++i) sum[i] += valid ? M::ex(x[i], mx[i]) : 0.0;
+            }
+        } else {
+            // Halves: four positions' terms meet in f32, then one f64 addition; for log_softmax the terms that are
+            // exactly 1 are counted instead of added (see the rows kernel).
+            static_assert(std::is_same_v<E, double> || C % 4 == 0 || C < 4, "positions are summed four at a time");
+            constexpr int kQuad = C < 4 ? C : 4;
+#pragma unroll
+            for (int c0 = 0; c0 < C; c0 += kQuad) {
+                float e[kQuad][V];
+#pragma unroll
+                for (int j = 0; j < kQuad; ++j) {
+                    X x[V];
+                    forget(raw[c0 + j]);
+                    M::unpack(raw[c0 + j], x);
+                    const bool valid = rg + static_cast<int64_t>(c0 + j) * RG < a.n;
+#pragma unroll
+                    for (int i = 0; i < V; ++i) e[j][i] = valid ? M::ex(x[i], mx[i]) : 0.0f;
+                }
+#pragma unroll
+                for (int i = 0; i < V; ++i) {
+                    float ones = 0.0f, part = 0.0f;
+                    if constexpr (LOG) {
+#pragma unroll
+                        for (int j = 0; j < kQuad; ++j) {
+                            const bool one = e[j][i] == 1.0f;
+                            ones += one ? 1.0f : 0.0f;
+                            e[j][i] = one ? 0.0f : e[j][i];
+                        }
+                    }
+                    if constexpr (kQuad == 4) part = (e[0][i] + e[1][i]) + (e[2][i] + e[3][i]);
+                    else {
+#pragma unroll
+                        for (int j = 0; j < kQuad; ++j) part += e[j][i];
+                    }
+                    sum[i] += static_cast<double>(part);
+                    if constexpr (LOG) sum[i] += static_cast<double>(ones);
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+#pragma unroll
+            for (int step = kColsAcross; step < kWave; step <<= 1) sum[i] += shfl_xor_any(sum[i], step);
+        }
+        if ((threadIdx.x % kWave) < kColsAcross) {
+#pragma unroll
+            for (int i = 0; i < V; ++i) lds_s[threadIdx.x / kWave][across * V + i] = sum[i];
+        }
+        __syncthreads();
+        E scale[V];
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+            double total = lds_s[0][across * V + i];
+#pragma unroll
+            for (int w = 1; w < kWaves; ++w) total += lds_s[w][across * V + i];
+            scale[i] = LOG ? M::lg(total) : M::scale(total);
+        }
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            X x[V];
+            forget(raw[c]);
+            M::unpack(raw[c], x);
+            decltype(M::logsoft(x[0], mx[0], scale[0])) res[V];
+#pragma unroll
+            for (int i = 0; i < V; ++i) {
+                if constexpr (LOG) res[i] = M::logsoft(x[i], mx[i], scale[i]);
+                else if constexpr (M::kKeep) res[i] = M::soft(x[i], mx[i], M::ex(x[i], mx[i]), scale[i]);
+                else res[i] = M::soft(x[i], mx[i], E(0), scale[i]);
+            }
+            const int64_t k = rg + static_cast<int64_t>(c) * RG;
+            if (k < a.n && live) __builtin_nontemporal_store(M::pack(res), reinterpret_cast<u32x4 *>(out + k * a.so));
+        }
+    }
+}
+
 // ---- plan -----------------------------------------------------------------------------------------
 
 struct SoftmaxPlan {
-    bool regs = false;  // registers plan (else streaming)
-    int group = kWave;  // lanes per row
-    int tiles = 0;      // registers plan: 128-bit tiles per lane
+    bool regs = false;   // registers plan
+    bool split = false;  // rows cut across workgroups (two launches, a workspace)
+    bool cols = false;   // rows that run across memory, neighbours adjacent
+    int group = kWave;   // lanes per row (registers, streaming), per slice (split) or per workgroup (cols)
+    int tiles = 0;       // registers and split plans: 128-bit tiles per lane
+    int64_t slices = 0;  // split plan: slices of a row
 };
+
+// Chunks per lane of a slice of the split plan, and the smallest row it is worth cutting.
+constexpr int slice_tiles(int elem) { return elem == 2 ? 16 : 8; }
+constexpr int64_t kSplitRowBytes = int64_t{256} << 10;
 
 // 128-bit chunks of the row a lane keeps: 8 (32 f32 or 16 f64 values, plus their f64 exponentials),
 // or 16 packed chunks (128 values) of a 16-bit type, whose exponentials are not kept.
@@ -444,6 +987,8 @@ SoftmaxPlan plan_softmax(const hmr_tensor_desc &src_rows, int64_t n, int64_t si,
     SoftmaxPlan p;
     const int elem = dtype_size(src_rows.dtype);
     const int vec = 16 / elem;
+    int64_t nrows = 1;
+    for (int d = 0; d < ws.ndim; ++d) nrows *= ws.size[d];
     bool aligned = (n == 1 || si == 1) &&
                    reinterpret_cast<uintptr_t>(static_cast<char *>(src_rows.data) + src_rows.offset * elem) % 16 == 0;
     for (int d = 0; aligned && d < ws.ndim; ++d) aligned = (ws.stride[d] * elem) % 16 == 0;
@@ -467,8 +1012,35 @@ SoftmaxPlan plan_softmax(const hmr_tensor_desc &src_rows, int64_t n, int64_t si,
                 p.regs = true;
                 p.group = g;
                 p.tiles = per <= 1 ? 1 : (per <= 2 ? 2 : (per <= 4 ? 4 : (per <= 8 ? 8 : 16)));
-                return p;
+                break;
             }
+        }
+        // Cut the rows when they do not fit the registers of a workgroup, or when whole rows would leave most of
+        // the GPU without work (fewer than 64 workgroups' worth) and a row is long enough to share.
+        const int64_t per_slice = int64_t{slice_tiles(elem)} * kBlock;
+        const int64_t slices = (tiles + per_slice - 1) / per_slice;
+        const bool few = p.regs && nrows * p.group < 64 * kBlock && n * elem >= kSplitRowBytes;
+        if ((!p.regs || few) && slices >= 2 && nrows * slices < (int64_t{1} << 31)) {
+            p.regs = false;
+            p.split = true;
+            p.group = kBlock;
+            p.tiles = slice_tiles(elem);
+            p.slices = slices;
+            return p;
+        }
+        if (p.regs) return p;
+    }
+    // Rows across memory with their neighbours adjacent: whole 16-byte vectors of V rows at every position.
+    if (n >= 2 && si != 1 && ws.ndim >= 1 && ws.stride[0] == 1 && ws.size[0] % vec == 0 && (si * elem) % 16 == 0 &&
+        reinterpret_cast<uintptr_t>(static_cast<char *>(src_rows.data) + src_rows.offset * elem) % 16 == 0) {
+        bool outer = true;
+        for (int d = 1; outer && d < ws.ndim; ++d) outer = (ws.stride[d] * elem) % 16 == 0;
+        if (outer) {
+            p.cols = true;
+            // Lanes of a workgroup: 8 across times as many row groups as give a lane sixteen positions or fewer
+            // (the rows are then read once, into registers); 1024 lanes stream longer rows twice.
+            p.group = n <= 16 * (kBlock / kColsAcross) ? kBlock : (n <= 16 * (512 / kColsAcross) ? 512 : 1024);
+            return p;
         }
     }
     p.regs = false;
@@ -478,8 +1050,88 @@ SoftmaxPlan plan_softmax(const hmr_tensor_desc &src_rows, int64_t n, int64_t si,
 }
 
 template <class T, bool LOG>
-void launch_softmax(const SoftmaxPlan &p, const SoftmaxArgs &a, bool out_ok, hipStream_t stream) {
+void launch_split(const SoftmaxPlan &p, const SoftmaxArgs &a, void *workspace, hipStream_t stream) {
+    SliceArgs s{};
+    s.out = a.out;
+    s.src = a.src;
+    s.out_rows = a.out_rows;
+    s.src_rows = a.src_rows;
+    if (s.src_rows.ndim == 0) {  // one row
+        s.src_rows.ndim = s.out_rows.ndim = 1;
+        s.src_rows.size[0] = s.out_rows.size[0] = 1;
+        s.src_rows.stride[0] = s.out_rows.stride[0] = 0;
+    }
+    s.nrows = a.nrows;
+    s.n = a.n;
+    s.slices = p.slices;
+    s.partials = static_cast<SlicePartial *>(workspace);
+    // Nontemporal stores for outputs far larger than the memory-side cache, and for rows whose bytes pass what
+    // the buffer form of the store addresses.
+    s.stream_stores = a.stream_stores || a.n * static_cast<int64_t>(sizeof(T)) >= kNarrowSpanBytes ? 1 : 0;
+    constexpr int C = slice_tiles(static_cast<int>(sizeof(T)));
+    const dim3 grid(static_cast<unsigned>(a.nrows * p.slices));
+    // A source that the memory-side cache can hold is read through the caches the first time.
+    if (a.nrows * a.n * static_cast<int64_t>(sizeof(T)) <= (int64_t{192} << 20)) {
+        hipLaunchKernelGGL((softmax_slice_stats_kernel<T, C, LOG, true>), grid, dim3(kBlock), 0, stream, s);
+    } else {
+        hipLaunchKernelGGL((softmax_slice_stats_kernel<T, C, LOG, false>), grid, dim3(kBlock), 0, stream, s);
+    }
+    hipLaunchKernelGGL((softmax_slice_write_kernel<T, C, LOG>), grid, dim3(kBlock), 0, stream, s);
+}
+
+template <class T, bool LOG>
+void launch_cols(const SoftmaxPlan &p, const SoftmaxArgs &a, hipStream_t stream) {
+    constexpr int V = 16 / static_cast<int>(sizeof(T));
+    ColsArgs c{};
+    c.out = a.out;
+    c.src = a.src;
+    c.inner = a.src_rows.size[0];
+    c.tiles_per_run = (c.inner + kColsAcross * V - 1) / (kColsAcross * V);
+    c.n = a.n;
+    c.so = a.so;
+    c.si = a.si;
+    // The walks over the runs: the row dimensions past the first (one run: a single step of stride 0).
+    c.src_outer.ndim = c.out_outer.ndim = a.src_rows.ndim > 1 ? a.src_rows.ndim - 1 : 1;
+    c.src_outer.size[0] = c.out_outer.size[0] = 1;
+    c.src_outer.stride[0] = c.out_outer.stride[0] = 0;
+    for (int d = 1; d < a.src_rows.ndim; ++d) {
+        c.src_outer.size[d - 1] = c.out_outer.size[d - 1] = a.src_rows.size[d];
+        c.src_outer.stride[d - 1] = a.src_rows.stride[d];
+        c.out_outer.stride[d - 1] = a.out_rows.stride[d];
+    }
+    c.tiles = c.tiles_per_run * (a.nrows / c.inner);
     const int64_t cap = 1 << 20;
+    const dim3 grid(static_cast<unsigned>(c.tiles < cap ? c.tiles : cap));
+    // Positions per lane: when they fit sixteen registers' worth of vectors the rows are read once.
+    auto with_block = [&](auto block_tag) {
+        constexpr int BLOCK = decltype(block_tag)::value;
+        const int64_t per = (c.n + BLOCK / kColsAcross - 1) / (BLOCK / kColsAcross);
+        auto regs = [&](auto chunks) {
+            hipLaunchKernelGGL((softmax_cols_regs_kernel<T, BLOCK, decltype(chunks)::value, LOG>), grid, dim3(BLOCK), 0, stream, c);
+        };
+        if constexpr (BLOCK <= 512) {
+            if (per <= 4) return regs(IntTag<4>{});
+            if (per <= 8) return regs(IntTag<8>{});
+            if (per <= 16 && sizeof(T) <= 4) return regs(IntTag<16>{});
+        }
+        hipLaunchKernelGGL((softmax_cols_kernel<T, BLOCK, LOG>), grid, dim3(BLOCK), 0, stream, c);
+    };
+    if (p.group == 1024) with_block(IntTag<1024>{});
+    else if (p.group == 512) with_block(IntTag<512>{});
+    else with_block(IntTag<kBlock>{});
+}
+
+template <class T, bool LOG>
+void launch_softmax(const SoftmaxPlan &p, const SoftmaxArgs &a, bool out_ok, bool out_cols, void *workspace, hipStream_t stream) {
+    const int64_t cap = 1 << 20;
+    if (p.split && out_ok) {
+        launch_split<T, LOG>(p, a, workspace, stream);
+        return;
+    }
+    if (p.cols && out_cols) {
+        launch_cols<T, LOG>(p, a, stream);
+        return;
+    }
     auto blocks = [&](int rows_per_block) {
         int64_t b = (a.nrows + rows_per_block - 1) / rows_per_block;
         return dim3(static_cast<unsigned>(b < cap ? (b < 1 ? 1 : b) : cap));
@@ -511,7 +1163,7 @@ void launch_softmax(const SoftmaxPlan &p, const SoftmaxArgs &a, bool out_ok, hip
         else with_tiles(IntTag<1024>{});
         return;
     }
-    const int group = p.regs ? (a.n <= 4096 ? kWave : kBlock) : p.group;
+    const int group = p.regs || p.split || p.cols ? (a.n <= 4096 ? kWave : kBlock) : p.group;
     if (group == kWave) {
         hipLaunchKernelGGL((softmax_stream_kernel<T, kWave, LOG>), blocks(kBlock / kWave), dim3(kBlock), 0, stream, a);
     } else {
@@ -530,7 +1182,13 @@ hmr_status hmr_softmax_workspace(const hmr_tensor_desc *src_rows, int64_t n, int
     return fenced([&] {
         int64_t nrows = 0;
         if (hmr_status s = hmr::check_rows(*src_rows, *src_rows, n, 0, src_stride, nrows)) return s;
-        *bytes = 0;  // no plan of this library cuts a row across workgroups
+        *bytes = 0;
+        if (nrows == 0 || n == 0) return HMR_OK;
+        hmr::Walk wo, ws;
+        hmr::walk_pair(*src_rows, *src_rows, wo, ws);
+        const hmr::SoftmaxPlan p = hmr::plan_softmax(*src_rows, n, src_stride, ws);
+        // A split plan keeps a (maximum, sum) pair per slice of every row.
+        if (p.split) *bytes = nrows * p.slices * static_cast<int64_t>(sizeof(hmr::SlicePartial));
         return HMR_OK;
     });
 }
@@ -543,9 +1201,9 @@ hmr_status hmr_test_softmax_plan(const hmr_tensor_desc *src_rows, int64_t n, int
         hmr::Walk wo, ws;
         hmr::walk_pair(*src_rows, *src_rows, wo, ws);
         hmr::SoftmaxPlan p = hmr::plan_softmax(*src_rows, n, src_stride, ws);
-        *split = 0;
+        *split = p.split ? 1 : 0;
         *group = p.group;
-        *cache = p.regs ? p.tiles * (16 / hmr::dtype_size(src_rows->dtype)) : 0;
+        *cache = p.regs || p.split ? p.tiles * (16 / hmr::dtype_size(src_rows->dtype)) : 0;
         return HMR_OK;
     });
 }
@@ -553,8 +1211,6 @@ hmr_status hmr_test_softmax_plan(const hmr_tensor_desc *src_rows, int64_t n, int
 hmr_status hmr_softmax(hmr_context_t ctx, const hmr_tensor_desc *out_rows, const hmr_tensor_desc *src_rows, int64_t n,
                        int64_t out_stride, int64_t src_stride, int32_t log, void *workspace,
                        int64_t workspace_bytes) {
-    (void)workspace;
-    (void)workspace_bytes;
     return fenced([&] {
         int64_t nrows = 0;
         if (hmr_status s = hmr::check_rows(*out_rows, *src_rows, n, out_stride, src_stride, nrows)) return s;
@@ -571,12 +1227,20 @@ hmr_status hmr_softmax(hmr_context_t ctx, const hmr_tensor_desc *out_rows, const
         hmr::SoftmaxPlan plan = hmr::plan_softmax(*src_rows, n, src_stride, a.src_rows);
         bool out_ok = (n == 1 || out_stride == 1) && reinterpret_cast<uintptr_t>(a.out) % 16 == 0;
         for (int d = 0; out_ok && d < a.out_rows.ndim; ++d) out_ok = (a.out_rows.stride[d] * elem) % 16 == 0;
+        // The output of a column plan: laid out like the source's rows (neighbours adjacent, everything aligned).
+        bool out_cols = plan.cols && a.out_rows.ndim >= 1 && a.out_rows.stride[0] == 1 && (out_stride * elem) % 16 == 0 &&
+                        reinterpret_cast<uintptr_t>(a.out) % 16 == 0;
+        for (int d = 1; out_cols && d < a.out_rows.ndim; ++d) out_cols = (a.out_rows.stride[d] * elem) % 16 == 0;
+        if (plan.split && out_ok) {
+            const int64_t need = nrows * plan.slices * static_cast<int64_t>(sizeof(hmr::SlicePartial));
+            if (workspace == nullptr || workspace_bytes < need) return hmr::fail(HMR_INVALID, "softmax: the workspace is too small");
+        }
         return hmr::queue_on(ctx, "softmax", [&](hipStream_t stream) {
             if (out_rows->dtype != src_rows->dtype) return false;
             return hmr::with_float_type(out_rows->dtype, [&](auto t) {
                 using T = typename decltype(t)::type;
-                if (log != 0) hmr::launch_softmax<T, true>(plan, a, out_ok, stream);
-                else hmr::launch_softmax<T, false>(plan, a, out_ok, stream);
+                if (log != 0) hmr::launch_softmax<T, true>(plan, a, out_ok, out_cols, workspace, stream);
+                else hmr::launch_softmax<T, false>(plan, a, out_ok, out_cols, workspace, stream);
             });
         });
     });

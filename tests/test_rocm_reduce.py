@@ -480,22 +480,61 @@ def test_every_plan_folds_each_element_once():
 
 
 SOFTMAX_PLAN_SHAPES = [
-    ([700, 200], 1, DT.F32, 64, 4), ([64, 1024], 1, DT.F32, 64, 16), ([64, 2048], 1, DT.F32, 128, 16), ([16, 4096], 1, DT.F32, 256, 16),
-    ([8, 32000], 1, DT.BF16, 256, 128), ([4, 100000], 1, DT.BF16, 1024, 128), ([5, 8192], 1, DT.F16, 64, 128),
-    ([8, 32768], 1, DT.F32, 1024, 32), ([3, 70000], 1, DT.F32, 256, 0),
-    ([2048, 9], 0, DT.F32, 64, 0), ([40, 8, 1000], 1, DT.F16, 64, 0),
+    ([700, 200], 1, DT.F32, False, 64, 4), ([64, 1024], 1, DT.F32, False, 64, 16), ([64, 2048], 1, DT.F32, False, 128, 16),
+    ([16, 4096], 1, DT.F32, False, 256, 16), ([8, 32000], 1, DT.BF16, False, 256, 128), ([4, 100000], 1, DT.BF16, False, 1024, 128),
+    ([5, 8192], 1, DT.F16, False, 64, 128), ([8, 32768], 1, DT.F32, False, 1024, 32),
+    # rows cut across workgroups: too long for a workgroup's registers, or too few to fill the GPU whole
+    ([3, 70000], 1, DT.F32, True, 256, 32), ([2, 300000], 1, DT.F64, True, 256, 16), ([4, 131072], 1, DT.BF16, True, 256, 128),
+    ([1, 1 << 20], 1, DT.F16, True, 256, 128),
+    # rows across memory, neighbours adjacent: 256- and 512-lane workgroups keep a lane's sixteen positions or fewer
+    # in registers, 1024 lanes stream longer rows
+    ([600, 64], 0, DT.F32, False, 512, 0), ([40, 8, 1000], 1, DT.F16, False, 256, 0), ([3, 700, 5, 8], 1, DT.F64, False, 512, 0),
+    ([3000, 32], 0, DT.BF16, False, 1024, 0), ([500, 40], 0, DT.F32, False, 256, 0),
+    # neither: streamed
+    ([2048, 9], 0, DT.F32, False, 64, 0), ([5000, 6], 0, DT.BF16, False, 256, 0),
 ]
 
 
 def test_softmax_plans_cover_every_path():
-    """(lanes per row, elements a lane keeps in registers; 0 = streamed)."""
-    for shape, dim, dtype, group, cache in SOFTMAX_PLAN_SHAPES:
+    """(rows cut across workgroups; lanes per row, slice or workgroup; elements a lane keeps in registers, 0 = streamed)."""
+    for shape, dim, dtype, cut, group, cache in SOFTMAX_PLAN_SHAPES:
         x = finite(dtype, prod(shape), 2, 500 + shape[0]).reshape(shape)
         split, p_group, p_cache = h.softmax_plan(x.to(GPU), dim)
-        assert (split, p_group, p_cache) == (False, group, cache), f"{shape} dim {dim}: {(split, p_group, p_cache)}"
+        assert (split, p_group, p_cache) == (cut, group, cache), f"{shape} dim {dim}: {(split, p_group, p_cache)}"
         for log in (False, True):
             c = x.log_softmax(dim) if log else x.softmax(dim)
             g = x.to(GPU).log_softmax(dim) if log else x.to(GPU).softmax(dim)
+            check_softmax(g, c, x.to(DT.F64), dim, log, f"{dtype} {shape} dim {dim} log {log}")
+
+
+@pytest.mark.parametrize("dtype", FLOATS)
+def test_softmax_of_cut_rows_and_of_rows_across_memory_with_special_values(dtype):
+    """The two plans whose rows meet through partial results: rows holding a NaN, +inf, -inf only, -inf in whole
+    slices / whole stretches of positions, one dominating element, and ordinary rows beside them, come out as the
+    CPU has them (all NaN; exact zeros or -inf for masked entries; within the class otherwise)."""
+    rng = np.random.default_rng(91)
+    inf, nan = np.inf, np.nan
+    for shape, dim in (([10, 70000], 1), ([1200, 48], 0), ([3, 600, 40], 1)):
+        v = rng.standard_normal(int(np.prod(shape))).reshape(shape) * 2.0
+        rows = np.moveaxis(v, dim, -1).reshape(-1, shape[dim])   # a view: writes go to v
+        rows = np.moveaxis(v, dim, -1)
+        flat = rows.reshape(-1, shape[dim]) if rows.flags["C_CONTIGUOUS"] else None
+        cases = np.moveaxis(v, dim, -1).reshape(-1, shape[dim]).copy()
+        cases[0, 5] = nan
+        cases[1, 7] = inf
+        cases[2, :] = -inf
+        cases[3, : shape[dim] // 2] = -inf           # whole leading slices masked
+        cases[4, shape[dim] // 3:] = -inf            # whole trailing slices masked
+        cases[5, :] = -30.0
+        cases[5, shape[dim] - 3] = 40.0              # one element dominates
+        cases[6, ::2] = -inf
+        cases[7, 0] = -inf
+        back = np.moveaxis(cases.reshape(np.moveaxis(v, dim, -1).shape), -1, dim)
+        x = tensor(from_f64(np.ascontiguousarray(back).reshape(-1), dtype), dtype, shape)
+        xg = x.to(GPU)
+        for log in (False, True):
+            c = x.log_softmax(dim) if log else x.softmax(dim)
+            g = xg.log_softmax(dim) if log else xg.softmax(dim)
             check_softmax(g, c, x.to(DT.F64), dim, log, f"{dtype} {shape} dim {dim} log {log}")
 
 
