@@ -377,6 +377,28 @@ def per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP
     add(None, "exclusive_cumprod f32 [16384,4096] dim=1 (slabs through LDS, a sequential chain per row)", 8 * N,
         lambda: h.exclusive_cumprod(xf, 1, True), 5)
     del xf
+    # Softmax plans beyond rows that fit a workgroup's registers, and reductions over two dimensions (inputs and
+    # results in rotation, as for the configs' rows).
+    cols32 = residual.reshape([4096, 16384])
+    hbm(None, "softmax(dim=0) f32 [4096,16384] (rows across memory: running maxima, two passes)", 8 * N, (cols32,),
+        lambda t: t.softmax(0), 4 * N, 4 * N, 10)
+    hbm(None, "log_softmax(dim=0) f32 [4096,16384]", 8 * N, (cols32,), lambda t: t.log_softmax(0), 4 * N, 4 * N, 10)
+    del cols32
+    cols16 = h.full([4, 8, 2048, 4096], 0, DT.BF16, GPU).copy_(x.reshape([1, 8, 2048, 4096]).expand([4, 8, 2048, 4096])).reshape([64, 1024, 4096])
+    hbm(None, "softmax(dim=1) bf16 [64,1024,4096] (rows across memory, read once into registers)", 16 * N, (cols16,),
+        lambda t: t.softmax(1), 8 * N, 8 * N, 5)
+    del cols16
+    long_rows = residual.narrow(0, 0, 4).reshape([8, 4194304])
+    hbm(None, "softmax(dim=1) f32 [8,4194304] (rows cut across workgroups: two launches)", 4 * N, (long_rows,),
+        lambda t: t.softmax(1), 2 * N, 2 * N, 20)
+    del long_rows
+    stats = residual.reshape([64, 256, 4096])
+    hbm(None, "sum over (0,2) f32 [64,256,4096] (rows made of runs)", 4 * N, (stats,), lambda t: t.sum_dim([0, 2], False), 4 * N, 0, 30)
+    hbm(None, "var(unbiased) over (0,2) f32 [64,256,4096]", 4 * N, (stats,), lambda t: t.var_dim([0, 2], 1, False), 4 * N, 0, 30)
+    del stats
+    turned = residual.reshape([16384, 4096])
+    hbm(None, "sum of all elements of a transposed view f32 [16384,4096].T", 4 * N, (turned,), lambda t: t.transpose(0, 1).sum(), 4 * N, 0, 30)
+    del turned
     y = x.reshape([16384, 4096]).softmax(-1)
     gy = t2.reshape([16384, 4096])
     add(None, "softmax backward bf16 [16384,4096] (7 kernels: 2 casts, mul, sum, sub, mul, cast)", 2 * N * (3 + 3 + 6 + 2 + 4 + 6 + 3),

@@ -62,6 +62,8 @@ hmr_status hip_failure(hipError_t error, const char *what) noexcept;
 // Looks up where the static block of hmr_reduce_static lives on the current device and keeps the address
 // in the context. Called once per context, with its device current (defined beside the block, reduce.hip).
 hmr_status bind_reduce_scratch(hmr_context &ctx);
+// Gives the static block back if `ctx` is the context that holds it (hmr_context_destroy).
+void release_reduce_scratch(const hmr_context &ctx) noexcept;
 
 // Allocates the tables of the 16-bit unary operations on the context's GPU (and, behind them, the meeting place
 // of the position checks), fills them on its stream and waits for the fills. Called once per context, after its

@@ -1,6 +1,7 @@
 // Reduction plans and the entry points hmr_reduce_workspace, hmr_reduce, hmr_var, hmr_arg_reduce,
 // hmr_test_reduce_plan (ref: csrc/homura_rocm.h:297-336, csrc/reduce.hip:133-170, 432-517).
 #include <algorithm>
+#include <mutex>
 
 #include "reduce_plan.hpp"
 
@@ -153,9 +154,9 @@ hmr_status plan_reduction(const hmr_tensor_desc *out, const hmr_tensor_desc &kep
             return HMR_OK;
         }
     }
-    // Cols: a contiguous run of outputs, one strided reduced dimension (fewer than 2^31 rows: the kernel
-    // counts rows in 32 bits).
-    if (a.red.ndim == 1 && a.nred < (int64_t{1} << 31) && a.kept.ndim >= 1 && a.kept.stride[0] == 1 &&
+    // Cols: a contiguous run of outputs, one strided reduced dimension (fewer than 2^31 - 2^16 rows: the kernel
+    // counts rows in 32 bits, and steps past the last one by the rows of all its slices' row groups at most).
+    if (a.red.ndim == 1 && a.nred < (int64_t{1} << 31) - (int64_t{1} << 16) && a.kept.ndim >= 1 && a.kept.stride[0] == 1 &&
         a.kept.size[0] >= 32 && base_aligned && (a.red.stride[0] * elem) % 16 == 0 && strides_aligned(a.kept, 1)) {
         p.kind = ReduceKind::Cols;
         p.rstride = a.red.stride[0];
@@ -256,6 +257,30 @@ hmr_status run_reduce(hmr_context_t ctx, int32_t op, const hmr_tensor_desc *out,
 
 }  // namespace
 
+namespace {
+// The block belongs to one context per GPU at a time: the first one that stages partial results in it, until
+// that context is destroyed. Two contexts have two streams, and their kernels would overwrite each other's
+// partial results.
+std::mutex owners_lock;
+constexpr int kMaxDevices = 64;
+const hmr_context *owners[kMaxDevices];
+
+hmr_status claim_reduce_scratch(const hmr_context *ctx) {
+    if (ctx->device < 0 || ctx->device >= kMaxDevices) return fail(HMR_INVALID, "hmr_reduce_static: device out of range");
+    std::lock_guard<std::mutex> lock(owners_lock);
+    if (owners[ctx->device] == nullptr) owners[ctx->device] = ctx;
+    if (owners[ctx->device] == ctx) return HMR_OK;
+    return fail(HMR_INVALID, "hmr_reduce_static: the static block of rocm:" + std::to_string(ctx->device) +
+                                 " is in use by another context; call hmr_reduce with a workspace");
+}
+}  // namespace
+
+void release_reduce_scratch(const hmr_context &ctx) noexcept {
+    if (ctx.device < 0 || ctx.device >= kMaxDevices) return;
+    std::lock_guard<std::mutex> lock(owners_lock);
+    if (owners[ctx.device] == &ctx) owners[ctx.device] = nullptr;
+}
+
 hmr_status bind_reduce_scratch(hmr_context &ctx) {
     void *address = nullptr;
     const hipError_t found = hipGetSymbolAddress(&address, HIP_SYMBOL(::scratch));
@@ -307,6 +332,7 @@ hmr_status hmr_reduce(hmr_context_t ctx, int32_t op, const hmr_tensor_desc *out,
 hmr_status hmr_reduce_static(hmr_context_t ctx, int32_t op, const hmr_tensor_desc *out, const hmr_tensor_desc *kept,
                              const hmr_tensor_desc *red) {
     return fenced([&] {
+        if (ctx == nullptr) return hmr::fail(HMR_INVALID, "hmr_reduce_static: null context");
         hmr::ReducePlan p;
         if (hmr_status s = hmr::plan_reduction(out, *kept, *red, p)) return s;
         const int64_t need = hmr::partial_bytes(p, false);
@@ -315,6 +341,9 @@ hmr_status hmr_reduce_static(hmr_context_t ctx, int32_t op, const hmr_tensor_des
                                               " bytes of partial results, the library's block holds " +
                                               std::to_string(HMR_REDUCE_STATIC_BYTES) +
                                               "; call hmr_reduce with a workspace");
+        }
+        if (need > 0) {
+            if (hmr_status s = hmr::claim_reduce_scratch(ctx)) return s;
         }
         // Every partial result the second kernel reads is written by the first one of the same call, so
         // what an earlier call left in the block needs no clearing.

@@ -296,6 +296,7 @@ hmr_status hmr_context_destroy(hmr_context_t ctx) {
         if (ctx == nullptr) return HMR_OK;
         if (hmr_status s = v.use_device(ctx->device)) return s;
         const std::unique_ptr<hmr_context> owned(ctx);
+        hmr::release_reduce_scratch(*owned);
         // Both resources go whatever the first one's fate: the first failure is the one reported.
         const hipError_t stream_gone = hmr::ContextParts::close(owned->stream);
         const hipError_t tables_gone = owned->tables != nullptr ? hipFree(owned->tables) : hipSuccess;  // waits for the device

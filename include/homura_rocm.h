@@ -270,9 +270,11 @@ hmr_status hmr_reduce(hmr_context_t ctx, int32_t op, const hmr_tensor_desc *out,
  * to pass: the partial results go to HMR_REDUCE_STATIC_BYTES of device memory that the library's
  * code object holds on every GPU it runs on, bound when the context is created. Same results as
  * hmr_reduce, bit for bit. HMR_INVALID, with nothing queued, when the reduction's plan needs more
- * than that (hmr_reduce_workspace reports the need). Allocates nothing. Every call on a GPU uses
- * that GPU's one block: calls on the same GPU must not overlap (two contexts, two threads), or their
- * partial results race. */
+ * than that (hmr_reduce_workspace reports the need). Allocates nothing. A GPU's block belongs to one
+ * context at a time - the first that stages partial results in it, until that context is destroyed -
+ * and another context of the same GPU is refused with HMR_INVALID (two contexts have two streams,
+ * whose kernels would overwrite each other's partial results). Calls on the owning context run on its
+ * one stream, in order; as for every entry point, one thread at a time calls into a context. */
 #define HMR_REDUCE_STATIC_BYTES (8 * 1024 * 1024)
 hmr_status hmr_reduce_static(hmr_context_t ctx, int32_t op, const hmr_tensor_desc *out,
                              const hmr_tensor_desc *kept, const hmr_tensor_desc *red);

@@ -21,6 +21,9 @@ hmr_status hmr::bind_reduce_scratch(hmr_context &ctx) {
     return HMR_OK;
 }
 
+static int g_released = 0;
+void hmr::release_reduce_scratch(const hmr_context &) noexcept { ++g_released; }
+
 // The other one (ew_unary.hip): the tables of the 16-bit unary operations. Here a block of the scripted HIP's
 // memory, so that the books show who frees it.
 static bool g_tables_fail = false;
@@ -152,7 +155,9 @@ static void contexts() {
         EXPECT(hipGetLastError() == hipSuccess);
         // Destroying frees the tables even when the stream will not go.
         M().fail_next["hipStreamDestroy"] = hipErrorInvalidHandle;
+        const int released = g_released;
         EXPECT(hmr_context_destroy(real) == HMR_HIP_ERROR && last() == "hipStreamDestroy(ctx->stream): invalid resource handle");
+        EXPECT(g_released == released + 1);  // the static reduction block goes back with the context
         EXPECT(M().blocks.empty() && M().pinned.empty());
         EXPECT(hmr_test_live_streams() == 1);  // the stream is still there, and still counted
         for (FakeStream *s : M().streams) delete s;  // the fake's books, for what follows

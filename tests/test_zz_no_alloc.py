@@ -131,3 +131,40 @@ def test_a_plan_beyond_the_block_is_refused_and_queues_nothing(ctx):
     bad = capi.make_desc(out.ptr, capi.I64, [nout + 1], [1])
     assert L.hmr_reduce_static(ctx.handle, capi.REDUCE["sum"], byref(bad), byref(kept), byref(red)) == capi.HMR_INVALID
     assert L.hmr_last_error().decode() == "a reduction's output is not contiguous with its sizes"
+
+
+def test_the_block_belongs_to_one_context_per_gpu(ctx):
+    """A second context of the same GPU (another stream) is refused while the first one holds the block, with
+    nothing queued, and takes it over once the first is destroyed; a null context is refused, not followed."""
+    rows, cols = 4096, 2048
+    src = ctx.upload(np.arange(rows * cols, dtype=np.int32) % 7)
+    kept, red, nout = matrix_reduction(src, capi.I32, rows, cols, 0)
+    assert workspace_bytes(kept, red) > 0, "this shape is meant to stage partial results"
+    out = ctx.malloc(nout * 8)
+    o = capi.make_desc(out.ptr, capi.I64, [nout], [1])
+    capi.check(L.hmr_reduce_static(ctx.handle, capi.REDUCE["sum"], byref(o), byref(kept), byref(red)))
+    ctx.synchronize()
+    want = out.download(np.int64, nout)
+    other = capi.Context(0)
+    try:
+        capi.check(L.hmr_memset(other.handle, out.ptr, 0x5C, nout * 8))
+        other.synchronize()
+        assert L.hmr_reduce_static(other.handle, capi.REDUCE["sum"], byref(o), byref(kept), byref(red)) == capi.HMR_INVALID
+        assert L.hmr_last_error().decode() == ("hmr_reduce_static: the static block of rocm:0 is in use by another context; "
+                                               "call hmr_reduce with a workspace")
+        other.synchronize()
+        assert (out.download(np.uint8, nout * 8) == 0x5C).all()
+        # A reduction that stages nothing needs no block and runs on any context.
+        kept1, red1, nout1 = matrix_reduction(src, capi.I32, 64, 512, 1)
+        assert workspace_bytes(kept1, red1) == 0
+        small = capi.make_desc(out.ptr, capi.I64, [nout1], [1])
+        capi.check(L.hmr_reduce_static(other.handle, capi.REDUCE["sum"], byref(small), byref(kept1), byref(red1)))
+        other.synchronize()
+    finally:
+        other.close()
+    assert L.hmr_reduce_static(None, capi.REDUCE["sum"], byref(o), byref(kept), byref(red)) == capi.HMR_INVALID
+    assert L.hmr_last_error().decode() == "hmr_reduce_static: null context"
+    # The owner is still the owner.
+    capi.check(L.hmr_reduce_static(ctx.handle, capi.REDUCE["sum"], byref(o), byref(kept), byref(red)))
+    ctx.synchronize()
+    assert np.array_equal(out.download(np.int64, nout), want)
