@@ -487,9 +487,9 @@ SOFTMAX_PLAN_SHAPES = [
     ([3, 70000], 1, DT.F32, True, 256, 32), ([2, 300000], 1, DT.F64, True, 256, 16), ([4, 131072], 1, DT.BF16, True, 256, 128),
     ([1, 1 << 20], 1, DT.F16, True, 256, 128),
     # rows across memory, neighbours adjacent: 256- and 512-lane workgroups keep a lane's sixteen positions or fewer
-    # in registers, 1024 lanes stream longer rows
+    # in registers, longer rows stream through 512 lanes
     ([600, 64], 0, DT.F32, False, 512, 0), ([40, 8, 1000], 1, DT.F16, False, 256, 0), ([3, 700, 5, 8], 1, DT.F64, False, 512, 0),
-    ([3000, 32], 0, DT.BF16, False, 1024, 0), ([500, 40], 0, DT.F32, False, 256, 0),
+    ([3000, 32], 0, DT.BF16, False, 512, 0), ([500, 40], 0, DT.F32, False, 256, 0),
     # neither: streamed
     ([2048, 9], 0, DT.F32, False, 64, 0), ([5000, 6], 0, DT.BF16, False, 256, 0),
 ]
