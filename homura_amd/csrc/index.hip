@@ -156,7 +156,7 @@ __global__ void __launch_bounds__(kBlock) check_flat_kernel(const I *start, int 
 
 // The whole check in one workgroup, for indices of a few thousand elements: no meeting, no atomics.
 constexpr int kCheckBlock = 1024;
-constexpr int64_t kCheckSmall = 8 * kCheckBlock;
+constexpr int64_t kCheckSmall = 16 * kCheckBlock;
 __global__ void __launch_bounds__(kCheckBlock) check_small_kernel(const void *index, int is64, Dims d, int64_t n, int64_t low, int64_t high,
                                                                   int has_exempt, int64_t exempt, uint64_t *slot, uint64_t *mailbox) {
     __shared__ unsigned long long firsts[kCheckBlock / 64];

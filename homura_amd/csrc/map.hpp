@@ -41,16 +41,11 @@
 namespace hmr {
 
 constexpr int kBlock = 256;      // 4 waves of 64
-#ifndef HMR_ROWS_BLOCK
-#define HMR_ROWS_BLOCK 64
-#endif
-#ifndef HMR_ROWS_U
-#define HMR_ROWS_U 2
-#endif
-#ifndef HMR_BIG_NT
-#define HMR_BIG_NT 1
-#endif
-constexpr int kRowsBlock = HMR_ROWS_BLOCK;  // lanes of a workgroup of the rows kernel
+// The rows kernel: one wave a workgroup, two tiles a lane. With inputs and results both coming from and going to
+// HBM (several buffer sets in rotation), many small workgroups keep more independent streams in flight than
+// 256-lane workgroups of four tiles a lane did: a 268 MB x + bias went from 72 to 77 % of the peak rate.
+constexpr int kRowsBlock = 64;
+constexpr int kRowsTiles = 2;
 constexpr int kFastDims = 6;     // merged dimensions the 32-bit kernels take
 constexpr int kMaxOperands = 4;  // output + 3 inputs
 // The vector kernels mark their 128-bit accesses nontemporal (see load_tile). The hint has to be
@@ -307,8 +302,8 @@ struct MapTraits {
     // 128 contiguous bytes (16 bytes of the narrowest operand) makes each 128-bit load touch 64
     // different cache lines, which with streaming loads multiplies the traffic.
     static constexpr int V = 16 / wide;
-    // Tiles per lane per pass: aim at 64 bytes of the widest operand in flight.
-    static constexpr int U = HMR_ROWS_U ? HMR_ROWS_U : ((V * wide >= 64) ? 1 : 64 / (V * wide));
+    // Tiles per lane per pass.
+    static constexpr int U = kRowsTiles;
 };
 
 template <class F>
@@ -1027,7 +1022,7 @@ RowsArgs<F::N + 1> rows_args(const MapCall &c, int variant) {
     }
     int64_t span = 1;  // elements from the output's first to one past its last
     for (int d = 0; d < c.ndim; ++d) span += (c.size[d] - 1) * (c.stride[0][d] < 0 ? -c.stride[0][d] : c.stride[0][d]);
-    a.out32 = span * T::so <= kNarrowSpanBytes && !(HMR_BIG_NT && c.n * T::so >= kStreamStoreBytes) ? 1u : 0u;
+    a.out32 = span * T::so <= kNarrowSpanBytes && !(c.n * T::so >= kStreamStoreBytes) ? 1u : 0u;
     if (variant == 0) {
         a.inner = static_cast<uint32_t>(c.n < (int64_t{1} << 31) ? c.n : 0);
         a.nouter = 0;

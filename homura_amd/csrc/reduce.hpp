@@ -254,6 +254,18 @@ struct MomentsFold {
         l.s2 += d * d;
         l.n += 1.0;
     }
+    // A whole vector of the row: the shift is settled once for the vector, not once per element.
+    template <int V>
+    __device__ __forceinline__ void lane_add_vector(Lane &l, const T (&x)[V]) const {
+        l.k = l.n == 0.0 ? Conv<T>::to_f64(x[0]) : l.k;
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+            const double d = Conv<T>::to_f64(x[i]) - l.k;
+            l.s1 += d;
+            l.s2 += d * d;
+        }
+        l.n += static_cast<double>(V);
+    }
     __device__ __forceinline__ Acc lane_done(const Lane &l) const {
         if (l.n == 0.0) return Acc{0.0, 0.0, 0.0};
         return Acc{l.n, l.k + l.s1 / l.n, l.s2 - l.s1 * l.s1 / l.n};
@@ -458,6 +470,24 @@ __global__ void __launch_bounds__(kBlock) combine_kernel(ReduceArgs a, Op op, Si
 
 // Contiguous rows, each starting 16-byte aligned. WAVES = 1: a wave per row, four rows per
 // workgroup. WAVES = 4: a workgroup per row (or per row slice when splits > 1).
+// The V elements of one vector into a lane's state: through the op's own vector form when it has one (the
+// elements' positions do not matter to such an op), else one by one with positions `pos + i * step`.
+template <class Op, class = void>
+struct HasVectorAdd : std::false_type {};
+template <class Op>
+struct HasVectorAdd<Op, std::void_t<decltype(&Op::template lane_add_vector<2>)>> : std::true_type {};
+
+template <class Op, int V>
+__device__ __forceinline__ void add_vector(const Op &op, typename Op::Lane &state, const typename Op::In (&x)[V], int64_t pos,
+                                           int64_t step, typename Op::Ctx ctx) {
+    if constexpr (HasVectorAdd<Op>::value) {
+        op.template lane_add_vector<V>(state, x);
+    } else {
+#pragma unroll
+        for (int i = 0; i < V; ++i) op.lane_add(state, x[i], pos + i * step, ctx);
+    }
+}
+
 template <class Op, class Sink, int WAVES>
 __global__ void __launch_bounds__(kBlock) reduce_rows_kernel(ReduceArgs a, Op op, Sink sink) {
     using T = typename Op::In;
@@ -510,8 +540,7 @@ __global__ void __launch_bounds__(kBlock) reduce_rows_kernel(ReduceArgs a, Op op
                     }
 #pragma unroll
                     for (int u = 0; u < U; ++u) {
-#pragma unroll
-                        for (int i = 0; i < V; ++i) op.lane_add(state, r[u][i], pos[u] + i * a.runs.inner_pos, ctx);
+                        add_vector<Op, V>(op, state, r[u], pos[u], a.runs.inner_pos, ctx);
                     }
                 }
                 for (; k < nvec; k += G) {
@@ -519,8 +548,7 @@ __global__ void __launch_bounds__(kBlock) reduce_rows_kernel(ReduceArgs a, Op op
                     int64_t at, pos;
                     locate(v0 + static_cast<uint32_t>(k), at, pos);
                     load_stream<T, V>(reinterpret_cast<const char *>(p + at), r);
-#pragma unroll
-                    for (int i = 0; i < V; ++i) op.lane_add(state, r[i], pos + i * a.runs.inner_pos, ctx);
+                    add_vector<Op, V>(op, state, r, pos, a.runs.inner_pos, ctx);
                 }
                 k = nvec;  // nothing ragged: the range is whole runs
             }
@@ -532,15 +560,13 @@ __global__ void __launch_bounds__(kBlock) reduce_rows_kernel(ReduceArgs a, Op op
                 }
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
-#pragma unroll
-                    for (int i = 0; i < V; ++i) op.lane_add(state, r[u][i], begin + (k + u * G) * V + i, ctx);
+                    add_vector<Op, V>(op, state, r[u], begin + (k + u * G) * V, 1, ctx);
                 }
             }
             for (; k < nvec; k += G) {
                 T r[V];
                 load_stream<T, V>(reinterpret_cast<const char *>(p + begin + k * V), r);
-#pragma unroll
-                for (int i = 0; i < V; ++i) op.lane_add(state, r[i], begin + k * V + i, ctx);
+                add_vector<Op, V>(op, state, r, begin + k * V, 1, ctx);
             }
             // Ragged end of the range (fewer than V elements; one run only).
             if (a.runs.dims == 0) {

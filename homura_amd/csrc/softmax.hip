@@ -276,12 +276,17 @@ __global__ void __launch_bounds__(G > kBlock ? G : kBlock) softmax_regs_kernel(S
         const T *src = reinterpret_cast<const T *>(a.src) + (WALK ? a.src_rows.offset(r) : r * a.src_rows.stride[0]);
         T *out = reinterpret_cast<T *>(a.out) + (WALK ? a.out_rows.offset(r) : r * a.out_rows.stride[0]);
         const __amdgpu_buffer_rsrc_t out_row = __builtin_amdgcn_make_buffer_rsrc(out, 0, -1, 0x00020000);
-        // Phase 0: one pass over memory.
+        // Phase 0: one pass over memory. The lane number is made opaque here and again before the stores: what is
+        // derived from it (a chunk's offset, whether it lies inside the row) is then computed where it is used, a few
+        // instructions per chunk, instead of being hoisted out of the loop over rows and kept - two registers per
+        // chunk, which cost the sixteen-chunk form a workgroup per compute unit.
+        int at = lane;
+        asm volatile("" : "+v"(at));
         u32x4 raw[C];
 #pragma unroll
         for (int c = 0; c < C; ++c) {
             // A uniform row pointer plus a 32-bit byte offset per lane: one address register per chunk.
-            const uint32_t tile = static_cast<uint32_t>(c * G + lane);
+            const uint32_t tile = static_cast<uint32_t>(c * G + at);
             const uint32_t t = tile < static_cast<uint32_t>(nvec) ? tile : static_cast<uint32_t>(nvec - 1);
             const u32x4 *q = reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(src) + t * 16u);
             if constexpr (kStreamLoads) raw[c] = __builtin_nontemporal_load(q);
@@ -296,6 +301,7 @@ __global__ void __launch_bounds__(G > kBlock ? G : kBlock) softmax_regs_kernel(S
             M::unpack(raw[c], x);
 #pragma unroll
             for (int i = 0; i < V; i += 2) mx = max3(mx, x[i], x[i + 1]);
+            __builtin_amdgcn_sched_barrier(0);  // a chunk at a time: unpacked ahead, the row would fill the registers
         }
         mx = row_fold<G>(MaxFold{}, mx, reinterpret_cast<X *>(lds));
         // Phase 2: exponentials and their f64 sum.
@@ -307,7 +313,7 @@ __global__ void __launch_bounds__(G > kBlock ? G : kBlock) softmax_regs_kernel(S
             X x[V];
             forget(raw[c]);
             M::unpack(raw[c], x);
-            const bool inside = c * G + lane < nvec;
+            const bool inside = c * G + at < nvec;
             if constexpr (std::is_same_v<E, double>) {
                 // An f64 exponential is some twenty-five instructions. When no lane of the wave holds an
                 // element of this chunk within 708 of the max (a masked span of attention scores, a
@@ -359,9 +365,10 @@ __global__ void __launch_bounds__(G > kBlock ? G : kBlock) softmax_regs_kernel(S
         sum = row_fold<G>(SumOp{}, sum, lds);
         // Phase 3: write once.
         const E scale = LOG ? M::lg(sum) : M::scale(sum);
+        asm volatile("" : "+v"(at));
 #pragma unroll
         for (int c = 0; c < C; ++c) {
-            const int tile = c * G + lane;
+            const int tile = c * G + at;
             X x[V];
             forget(raw[c]);
             M::unpack(raw[c], x);

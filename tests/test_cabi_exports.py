@@ -53,9 +53,18 @@ def test_rust_ffi_list_is_complete():
     assert len(RUST_FFI) == 77 and len(set(RUST_FFI)) == 77
 
 
+# Beside the Rust crate's 77: the stream accessor for harnesses and the reduction that allocates nothing.
+EXTENSIONS = {"hmr_ext_stream", "hmr_reduce_static"}
+
+
+def test_the_library_exports_exactly_the_declared_set():
+    assert exported() == set(RUST_FFI) | EXTENSIONS
+    assert declared_in_headers() == set(RUST_FFI) | EXTENSIONS
+
+
 def test_every_declared_symbol_is_exported():
     declared = declared_in_headers()
-    assert len(declared) >= 78
+    assert len(declared) == 79
     have = exported()
     assert not (declared - have), f"declared in include/*.h but not exported: {sorted(declared - have)}"
     assert not (set(RUST_FFI) - have), f"needed by the Rust crate but not exported: {sorted(set(RUST_FFI) - have)}"
