@@ -15,6 +15,10 @@
 namespace hmr {
 
 constexpr int kTableBlock = 1024;
+#ifndef HMR_TABLE_TILES
+#define HMR_TABLE_TILES 4
+#endif
+constexpr int kTableTiles = HMR_TABLE_TILES;  // chunks a lane has in flight per pass
 constexpr int kTableEntries = 1 << 16;
 constexpr size_t kTableBytes = size_t{kTableEntries} * 2;
 // Below this the direct kernel runs. Measured on bf16, per call with the host's 4 us included: the lookup takes
@@ -56,7 +60,7 @@ struct TableSplit {
 // [8, 32, 2048, 128] a walk over four dimensions per chunk took 46.3 us, none takes 42.3.
 template <bool FLAT, bool SPLIT = false>
 __global__ void __launch_bounds__(kTableBlock) map_table_kernel(RowsArgs<2> a, const uint16_t *table, TableSplit split) {
-    constexpr int V = 8, U = 4;
+    constexpr int V = 8, U = kTableTiles;
     static_assert(!(FLAT && SPLIT), "the split is one of outer dimensions");
     __shared__ uint16_t lut[kTableEntries];
     {
@@ -195,7 +199,7 @@ void launch_table_fill(uint16_t *table, hipStream_t stream) {
 // The split of a launch of `blocks` workgroups over the layout `a` (see TableSplit), low_dims 0 if there is none.
 inline TableSplit table_split(const RowsArgs<2> &a, int64_t tiles, int64_t blocks) {
     TableSplit none{0, 0, make_fastdiv(1)};
-    constexpr int64_t kPass = 4 * kTableBlock;  // chunks of a pass
+    constexpr int64_t kPass = kTableTiles * kTableBlock;  // chunks of a pass
     if (a.nouter < 1 || a.inner % 8 != 0 || tiles % kPass != 0) return none;
     const int64_t per_row = a.inner / 8;
     if (kPass % per_row != 0) return none;
@@ -216,7 +220,7 @@ void launch_table(const MapCall &c, uint16_t *table, hipStream_t stream) {
     const int variant = resolve_variant<F>(c);
     RowsArgs<2> a = rows_args<F>(c, variant);
     const int64_t tiles = (c.n + 7) / 8;
-    int64_t blocks = (tiles + 4 * kTableBlock - 1) / (4 * kTableBlock);
+    int64_t blocks = (tiles + kTableTiles * kTableBlock - 1) / (kTableTiles * kTableBlock);
     if (blocks > c.compute_units) blocks = c.compute_units;  // one resident workgroup per CU, each loops
     const dim3 grid(static_cast<unsigned>(blocks)), block(kTableBlock);
     if (variant == 0) {

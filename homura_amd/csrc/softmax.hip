@@ -254,8 +254,13 @@ struct SoftmaxArgs {
 // contiguous tensor gives; WALK = true: up to 25 row dimensions, decoded per row.
 // Stores write through the compute die's L2 (see OutStores in map.hpp), or are nontemporal for outputs far larger
 // than the memory-side cache (`stream_stores`).
+//
+// log_softmax waits for one f64 logarithm per row - a chain of dependent instructions that a compute unit can only
+// hide behind another workgroup. The 1024-lane form of a 16-bit row with up to four chunks a lane is therefore held
+// to 64 registers (the softmax form needs 60 by itself), so that two workgroups share a compute unit: a
+// [4096, 32000] bf16 log_softmax 123 -> 93 us.
 template <class T, int G, int C, bool LOG, bool WALK>
-__global__ void __launch_bounds__(G > kBlock ? G : kBlock) softmax_regs_kernel(SoftmaxArgs a) {
+__global__ void __launch_bounds__(G > kBlock ? G : kBlock, (LOG && G == 1024 && C <= 4 && sizeof(T) == 2) ? 8 : 1) softmax_regs_kernel(SoftmaxArgs a) {
     using M = SoftmaxMath<T>;
     using X = typename M::X;
     using E = typename M::E;
@@ -364,7 +369,20 @@ __global__ void __launch_bounds__(G > kBlock ? G : kBlock) softmax_regs_kernel(S
         }
         sum = row_fold<G>(SumOp{}, sum, lds);
         // Phase 3: write once.
-        const E scale = LOG ? M::lg(sum) : M::scale(sum);
+        E scale;
+        if constexpr (LOG && G > kBlock) {
+            // The logarithm is an f64 routine of some hundred instructions, the same for the whole row: with
+            // sixteen waves on a row one of them evaluates it and the others take it from LDS.
+            __shared__ E row_scale;
+            if (threadIdx.x < kWave) {
+                const E v = M::lg(sum);
+                if (threadIdx.x == 0) row_scale = v;
+            }
+            __syncthreads();
+            scale = row_scale;
+        } else {
+            scale = LOG ? M::lg(sum) : M::scale(sum);
+        }
         asm volatile("" : "+v"(at));
 #pragma unroll
         for (int c = 0; c < C; ++c) {
@@ -1037,10 +1055,13 @@ SoftmaxPlan plan_softmax(const hmr_tensor_desc &src_rows, int64_t n, int64_t si,
         // Lanes per row and chunks per lane, first fit. 16-bit rows stay packed (4 registers per chunk);
         // wider rows also keep their f64 exponentials (8 more registers per f32 chunk), so they spread over
         // two waves before a lane takes more than four chunks: more resident waves hide the row loads.
+        // 16-bit rows past 16 384 elements go to 1024 lanes rather than to sixteen chunks on each of 256: a
+        // [4096, 32000] bf16 softmax with inputs and results from HBM took 96-97 us that way and takes 90-91
+        // with four chunks on each of 1024 lanes.
         struct Step {
             int group, tiles;
         };
-        static const Step half_steps[] = {{kWave, 16}, {kBlock, 16}, {1024, 16}};
+        static const Step half_steps[] = {{kWave, 16}, {kBlock, 8}, {1024, 16}};
         static const Step wide_steps[] = {{kWave, 4}, {128, 4}, {kBlock, 8}, {1024, 8}};
         const Step *steps = elem == 2 ? half_steps : wide_steps;
         const int nsteps = elem == 2 ? 3 : 4;
@@ -1215,8 +1236,9 @@ void launch_softmax(const SoftmaxPlan &p, const SoftmaxArgs &a, bool out_ok, boo
                 hipLaunchKernelGGL((softmax_regs_kernel<T, G, C, LOG, true>), blocks(kThreads / G), dim3(kThreads), 0, stream, a);
             }
         };
+        const int group = p.group, tiles = p.tiles;
         auto with_tiles = [&](auto g) {
-            switch (p.tiles) {
+            switch (tiles) {
                 case 1: run(g, IntTag<1>{}); break;
                 case 2: run(g, IntTag<2>{}); break;
                 case 4: run(g, IntTag<4>{}); break;
@@ -1226,9 +1248,9 @@ void launch_softmax(const SoftmaxPlan &p, const SoftmaxArgs &a, bool out_ok, boo
                     break;
             }
         };
-        if (p.group == kWave) with_tiles(IntTag<kWave>{});
-        else if (p.group == 128) with_tiles(IntTag<128>{});
-        else if (p.group == kBlock) with_tiles(IntTag<kBlock>{});
+        if (group == kWave) with_tiles(IntTag<kWave>{});
+        else if (group == 128) with_tiles(IntTag<128>{});
+        else if (group == kBlock) with_tiles(IntTag<kBlock>{});
         else with_tiles(IntTag<1024>{});
         return;
     }
