@@ -15,10 +15,11 @@
 namespace hmr {
 
 constexpr int kTableBlock = 1024;
-#ifndef HMR_TABLE_TILES
-#define HMR_TABLE_TILES 4
-#endif
-constexpr int kTableTiles = HMR_TABLE_TILES;  // chunks a lane has in flight per pass
+// Chunks a lane has in flight per pass: four over views (a pass is then whole 4 KiB runs of the output, see
+// TableSplit), one over a contiguous tensor, where a 134 MB -> 134 MB lookup from and to HBM took 47.8 us with four,
+// 47.2 with two and 45.8 with one (50.2 with eight).
+constexpr int kTableTiles = 4;
+constexpr int kTableTilesFlat = 1;
 constexpr int kTableEntries = 1 << 16;
 constexpr size_t kTableBytes = size_t{kTableEntries} * 2;
 // Below this the direct kernel runs. Measured on bf16, per call with the host's 4 us included: the lookup takes
@@ -60,7 +61,7 @@ struct TableSplit {
 // [8, 32, 2048, 128] a walk over four dimensions per chunk took 46.3 us, none takes 42.3.
 template <bool FLAT, bool SPLIT = false>
 __global__ void __launch_bounds__(kTableBlock) map_table_kernel(RowsArgs<2> a, const uint16_t *table, TableSplit split) {
-    constexpr int V = 8, U = kTableTiles;
+    constexpr int V = 8, U = FLAT ? kTableTilesFlat : kTableTiles;
     static_assert(!(FLAT && SPLIT), "the split is one of outer dimensions");
     __shared__ uint16_t lut[kTableEntries];
     {
@@ -220,7 +221,8 @@ void launch_table(const MapCall &c, uint16_t *table, hipStream_t stream) {
     const int variant = resolve_variant<F>(c);
     RowsArgs<2> a = rows_args<F>(c, variant);
     const int64_t tiles = (c.n + 7) / 8;
-    int64_t blocks = (tiles + kTableTiles * kTableBlock - 1) / (kTableTiles * kTableBlock);
+    const int64_t per_pass = int64_t{variant == 0 ? kTableTilesFlat : kTableTiles} * kTableBlock;
+    int64_t blocks = (tiles + per_pass - 1) / per_pass;
     if (blocks > c.compute_units) blocks = c.compute_units;  // one resident workgroup per CU, each loops
     const dim3 grid(static_cast<unsigned>(blocks)), block(kTableBlock);
     if (variant == 0) {
