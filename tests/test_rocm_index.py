@@ -432,3 +432,36 @@ def test_a_contiguous_index_off_the_16_byte_boundary_is_checked_like_any_other()
                     with pytest.raises(h.HomuraError) as e:
                         g.index_select(0, index.to(GPU))
                     assert str(e.value) == str(c.value), what
+
+
+def test_the_first_bad_position_is_found_at_every_index_length():
+    """Index lengths on both sides of the limits at which the position check changes form (one workgroup up to 16 384
+    positions, a grid that meets at a counter beyond; whole 16-byte vectors or a ragged end), contiguous and every
+    other element of a longer buffer: a bad value at the front, in the middle and at the very end, with a later bad
+    value behind it that must not win, gives the CPU's message; a valid index the CPU's rows. Two checks in a row on
+    one context also show that the counters of the first are back at rest."""
+    x = tensor(values(DT.F32, 40 * 2, 11), DT.F32, [40, 2])
+    g = x.to(GPU)
+    lengths = (1, 2, 63, 64, 1023, 1024, 1025, 8191, 8192, 8193, 16383, 16384, 16385, 16400, 40000, 262147)
+    for dtype in (DT.I32, DT.I64):
+        for n in lengths:
+            for strided in (False, True):
+                picks = random_positions(n * (2 if strided else 1), 40, n % 13 + (7 if strided else 0))
+                for bad_at in (None, 0, n // 2, n - 1):
+                    v = picks.copy()
+                    step = 2 if strided else 1
+                    if bad_at is not None:
+                        v[bad_at * step] = 40 + bad_at % 3
+                        if bad_at + 1 < n:
+                            v[(n - 1) * step] = -9   # a later one must not win
+                    whole = ints(v, [len(v)], dtype)
+                    view = (lambda t: t.reshape([n, 2]).select(1, 0)) if strided else (lambda t: t)   # a view made on the device
+                    what = f"{dtype} n {n} strided {strided} bad at {bad_at}"
+                    if bad_at is None:
+                        assert_same(g.index_select(0, view(whole.to(GPU))), x.index_select(0, view(whole)), what)
+                        continue
+                    with pytest.raises(h.HomuraError) as c:
+                        x.index_select(0, view(whole))
+                    with pytest.raises(h.HomuraError) as e:
+                        g.index_select(0, view(whole.to(GPU)))
+                    assert str(e.value) == str(c.value), what
