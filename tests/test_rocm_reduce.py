@@ -538,6 +538,22 @@ def test_softmax_of_cut_rows_and_of_rows_across_memory_with_special_values(dtype
             check_softmax(g, c, x.to(DT.F64), dim, log, f"{dtype} {shape} dim {dim} log {log}")
 
 
+def test_softmax_across_memory_when_the_positions_lie_megabytes_apart():
+    """A column softmax over a narrow strip of a very wide matrix: 600 positions 4 MiB apart. The registers form
+    addresses with 32-bit offsets from a tile's first element and must leave such a view to the streaming form, whose
+    pointers are 64-bit; the result is the CPU's either way."""
+    n, width, keep = 600, 1 << 20, 64
+    strip = finite(DT.F32, n * keep, 4, 77).reshape([n, keep])
+    wide_cpu = h.full([n, width], 0.0, DT.F32, "cpu")
+    wide_cpu.narrow(1, 128, keep).copy_(strip)
+    wide_gpu = wide_cpu.to(GPU)
+    x, xg = wide_cpu.narrow(1, 128, keep), wide_gpu.narrow(1, 128, keep)
+    for log in (False, True):
+        c = x.log_softmax(0) if log else x.softmax(0)
+        g = xg.log_softmax(0) if log else xg.softmax(0)
+        check_softmax(g, c, strip.to(DT.F64), 0, log, f"strip of [{n}, {width}] log {log}")
+
+
 def test_results_repeat_from_run_to_run():
     """ref: tests/rocm_reduce.rs:797-811"""
     x = finite(DT.F32, 1 << 20, 30, 600).reshape([1024, 1024]).to(GPU)
