@@ -29,13 +29,15 @@ struct hmr_context {
     // the count of workgroups that have finished. Device memory behind the tables; the last workgroup of a check
     // leaves both as it found them (all ones, zero).
     void *check_state = nullptr;
-    // The mailbox: 16 bytes of pinned host memory the GPU can write. A kernel whose result the caller is about
-    // to read back (the verdict of a position check) stores it there as well as in the caller's device memory;
-    // `mail_src` is that device address while the mailbox holds its current contents, and a read-back of it
-    // (hmr_copy_to_host) waits for the stream and takes the bytes from the mailbox instead of queueing a copy.
-    // Anything else queued on the context forgets the address.
+    // The mailbox: pinned host memory the GPU can write (three words in use). A kernel whose result the caller is
+    // about to read back (the verdict of a position check) stores it there as well as in the caller's device
+    // memory, and after it the ticket the launch was given (`mail_ticket`, counted up per check); `mail_src` is
+    // that device address while the mailbox holds its current contents, and a read-back of it (hmr_copy_to_host)
+    // watches the mailbox for the ticket - briefly, then it waits for the stream like any copy - and takes the
+    // bytes from there instead of queueing a copy. Anything else queued on the context forgets the address.
     void *mailbox = nullptr;
     const void *mail_src = nullptr;
+    uint64_t mail_ticket = 0;
     // Device address, on this context's GPU, of the library's static block for partial results
     // (hmr_reduce_static). Each GPU holds its own copy of the block at its own address.
     void *reduce_scratch = nullptr;

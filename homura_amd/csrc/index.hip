@@ -53,17 +53,20 @@ __device__ __forceinline__ int64_t value_at(const void *index, int is64, const D
     return read_index(index, is64, off);
 }
 
-__device__ __forceinline__ void publish(uint64_t *slot, uint64_t *mailbox, unsigned long long first, int64_t value) {
+// The verdict goes to the caller's slot and to the mailbox; the ticket follows it there with release order at
+// system scope, so that a host thread that sees the ticket sees the verdict.
+__device__ __forceinline__ void publish(uint64_t *slot, uint64_t *mailbox, unsigned long long first, int64_t value, uint64_t ticket) {
     const uint64_t word = first == ~0ull ? 0 : static_cast<uint64_t>(value);
     slot[0] = first;
     slot[1] = word;
-    mailbox[0] = first;
-    mailbox[1] = word;
+    __hip_atomic_store(&mailbox[0], static_cast<uint64_t>(first), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    __hip_atomic_store(&mailbox[1], word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    __hip_atomic_store(&mailbox[2], ticket, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
 // `first`: the smallest bad position this lane saw. Every lane of the workgroup calls this, once.
 __device__ __forceinline__ void meet(unsigned long long first, CheckState *state, uint64_t *slot, uint64_t *mailbox,
-                                     const void *index, int is64, const Dims &d) {
+                                     uint64_t ticket, const void *index, int is64, const Dims &d) {
 #pragma unroll
     for (int m = 32; m >= 1; m >>= 1) {
         const unsigned long long other = (static_cast<unsigned long long>(static_cast<uint32_t>(__shfl_xor(static_cast<int>(first >> 32), m, 64))) << 32) |
@@ -85,11 +88,11 @@ __device__ __forceinline__ void meet(unsigned long long first, CheckState *state
     if (atomicAdd(&state->top, 1u) != groups - 1) return;
     atomicExch(&state->top, 0u);
     const unsigned long long found = atomicExch(&state->first, ~0ull);
-    publish(slot, mailbox, found, found == ~0ull ? 0 : value_at(index, is64, d, found));
+    publish(slot, mailbox, found, found == ~0ull ? 0 : value_at(index, is64, d, found), ticket);
 }
 
 __global__ void __launch_bounds__(kBlock) check_kernel(const void *index, int is64, Dims d, int64_t n, int64_t low, int64_t high,
-                                                       int has_exempt, int64_t exempt, uint64_t *slot, CheckState *state, uint64_t *mailbox) {
+                                                       int has_exempt, int64_t exempt, uint64_t *slot, CheckState *state, uint64_t *mailbox, uint64_t ticket) {
     unsigned long long first = ~0ull;
     for (int64_t p = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; p < n; p += static_cast<int64_t>(gridDim.x) * kBlock) {
         int64_t rest = p, off = p * d.stride[0][0];
@@ -105,7 +108,7 @@ __global__ void __launch_bounds__(kBlock) check_kernel(const void *index, int is
         const bool bad = !(v >= low && v < high) && !(has_exempt && v == exempt);
         if (bad && static_cast<unsigned long long>(p) < first) first = static_cast<unsigned long long>(p);
     }
-    meet(first, state, slot, mailbox, index, is64, d);
+    meet(first, state, slot, mailbox, ticket, index, is64, d);
 }
 
 // The same for an index that is one contiguous run: 16 bytes per lane and load, four loads in flight (an
@@ -113,7 +116,7 @@ __global__ void __launch_bounds__(kBlock) check_kernel(const void *index, int is
 // than a tile) come before the first 16-byte boundary; they and the ragged end go to the first workgroup's lanes.
 template <class I>
 __global__ void __launch_bounds__(kBlock) check_flat_kernel(const I *start, int head, int64_t total, int64_t low, int64_t high,
-                                                            int has_exempt, int64_t exempt, uint64_t *slot, CheckState *state, uint64_t *mailbox,
+                                                            int has_exempt, int64_t exempt, uint64_t *slot, CheckState *state, uint64_t *mailbox, uint64_t ticket,
                                                             Dims d) {
     constexpr int V = 16 / static_cast<int>(sizeof(I)), U = 4;
     unsigned long long first = ~0ull;
@@ -151,14 +154,14 @@ __global__ void __launch_bounds__(kBlock) check_flat_kernel(const I *start, int 
             if (!(x >= low && x < high) && !(has_exempt && x == exempt) && static_cast<unsigned long long>(p) < first) first = p;
         }
     }
-    meet(first, state, slot, mailbox, start, sizeof(I) == 8, d);
+    meet(first, state, slot, mailbox, ticket, start, sizeof(I) == 8, d);
 }
 
 // The whole check in one workgroup, for indices of a few thousand elements: no meeting, no atomics.
 constexpr int kCheckBlock = 1024;
 constexpr int64_t kCheckSmall = 16 * kCheckBlock;
 __global__ void __launch_bounds__(kCheckBlock) check_small_kernel(const void *index, int is64, Dims d, int64_t n, int64_t low, int64_t high,
-                                                                  int has_exempt, int64_t exempt, uint64_t *slot, uint64_t *mailbox) {
+                                                                  int has_exempt, int64_t exempt, uint64_t *slot, uint64_t *mailbox, uint64_t ticket) {
     __shared__ unsigned long long firsts[kCheckBlock / 64];
     __shared__ long long values[kCheckBlock / 64];
     unsigned long long first = ~0ull;
@@ -214,7 +217,7 @@ __global__ void __launch_bounds__(kCheckBlock) check_small_kernel(const void *in
                 value = values[w];
             }
         }
-        publish(slot, mailbox, first, value);
+        publish(slot, mailbox, first, value, ticket);
     }
 }
 
@@ -671,10 +674,11 @@ hmr_status hmr_index_check(hmr_context_t ctx, const hmr_tensor_desc *index, int6
         const int is64 = index->dtype == HMR_I64;
         hmr::CheckState *state = static_cast<hmr::CheckState *>(ctx->check_state);
         uint64_t *mailbox = static_cast<uint64_t *>(ctx->mailbox);
+        const uint64_t ticket = ++ctx->mail_ticket;
         const hmr_status queued = hmr::queue_on(ctx, "index_check", [&](hipStream_t stream) {
             if (n <= hmr::kCheckSmall) {
                 hipLaunchKernelGGL(hmr::check_small_kernel, dim3(1), dim3(hmr::kCheckBlock), 0, stream, base, is64, d, n, low, high,
-                                   has_exempt, exempt, slot, mailbox);
+                                   has_exempt, exempt, slot, mailbox, ticket);
                 return true;
             }
             // One contiguous run (after merging: a size-1 dimension's stride does not count)? Its elements
@@ -694,15 +698,15 @@ hmr_status hmr_index_check(hmr_context_t ctx, const hmr_tensor_desc *index, int6
                 grid = grid < hmr::kCheckGrid ? grid : hmr::kCheckGrid;
                 if (is64) {
                     hipLaunchKernelGGL((hmr::check_flat_kernel<int64_t>), dim3(grid), dim3(hmr::kBlock), 0, stream,
-                                       static_cast<const int64_t *>(base), head, n, low, high, has_exempt, exempt, slot, state, mailbox, d);
+                                       static_cast<const int64_t *>(base), head, n, low, high, has_exempt, exempt, slot, state, mailbox, ticket, d);
                 } else {
                     hipLaunchKernelGGL((hmr::check_flat_kernel<int32_t>), dim3(grid), dim3(hmr::kBlock), 0, stream,
-                                       static_cast<const int32_t *>(base), head, n, low, high, has_exempt, exempt, slot, state, mailbox, d);
+                                       static_cast<const int32_t *>(base), head, n, low, high, has_exempt, exempt, slot, state, mailbox, ticket, d);
                 }
             } else {
                 const unsigned all = hmr::grid_of(n);
                 hipLaunchKernelGGL(hmr::check_kernel, dim3(all < hmr::kCheckGrid ? all : hmr::kCheckGrid), dim3(hmr::kBlock), 0, stream, base,
-                                   is64, d, n, low, high, has_exempt, exempt, slot, state, mailbox);
+                                   is64, d, n, low, high, has_exempt, exempt, slot, state, mailbox, ticket);
             }
             return true;
         });

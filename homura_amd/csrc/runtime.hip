@@ -138,6 +138,7 @@ class ContextParts {
     hmr_status open_mailbox(Visit &v) {
         void *box = nullptr;
         if (hmr_status e = v.hip(hipHostMalloc(&box, 64, hipHostMallocDefault), "hipHostMalloc(&mailbox, 64)")) return e;
+        std::memset(box, 0, 64);
         ctx_->mailbox = box;
         return HMR_OK;
     }

@@ -230,6 +230,21 @@ static void memory() {
         for (size_t k = before; k < M().calls.size(); ++k) copied = copied || M().calls[k] == "hipMemcpyAsync";
         EXPECT(!copied && ctx->mail_src == d);
         EXPECT(hmr_copy_to_host(ctx, got, d, 8) == HMR_OK && got[7] == 0x88);
+        // With a ticket out, the read-back watches the mailbox for it: once it is there no HIP call is made at
+        // all; while it is not, the read-back falls back to the wait on the stream after a tenth of a millisecond.
+        ctx->mail_ticket = 7;
+        static_cast<uint64_t *>(ctx->mailbox)[2] = 7;
+        auto waits_since = [&](size_t from) {
+            size_t n = 0;
+            for (size_t k = from; k < M().calls.size(); ++k) n += M().calls[k] == "hipStreamSynchronize" || M().calls[k] == "hipMemcpyAsync";
+            return n;
+        };
+        size_t mark = M().calls.size();
+        EXPECT(hmr_copy_to_host(ctx, got, d, 16) == HMR_OK && got[8] == 'A' && waits_since(mark) == 0);
+        ctx->mail_ticket = 8;
+        mark = M().calls.size();
+        EXPECT(hmr_copy_to_host(ctx, got, d, 16) == HMR_OK && waits_since(mark) == 1);
+        ctx->mail_ticket = 0;
         EXPECT(hmr_copy_from_host(ctx, d, got, 8) == HMR_OK && ctx->mail_src == nullptr);
         ctx->mail_src = d;
         EXPECT(hmr_memset(ctx, d, 0, 16) == HMR_OK && ctx->mail_src == nullptr);
