@@ -12,6 +12,7 @@
 //           (target << 32 | position), the words are sorted by target with a stable radix sort (sort.hpp;
 //           positions ascend on input, so each target's stay in order), and the first word of each target
 //           sums its run in order. Targets run in parallel; index_add also spreads a slice over the lanes.
+#include "mail.hpp"
 #include "index.hpp"
 #include "sort.hpp"
 
@@ -53,15 +54,12 @@ __device__ __forceinline__ int64_t value_at(const void *index, int is64, const D
     return read_index(index, is64, off);
 }
 
-// The verdict goes to the caller's slot and to the mailbox; the ticket follows it there with release order at
-// system scope, so that a host thread that sees the ticket sees the verdict.
+// The verdict goes to the caller's slot and to the mailbox (mail.hpp).
 __device__ __forceinline__ void publish(uint64_t *slot, uint64_t *mailbox, unsigned long long first, int64_t value, uint64_t ticket) {
     const uint64_t word = first == ~0ull ? 0 : static_cast<uint64_t>(value);
     slot[0] = first;
     slot[1] = word;
-    __hip_atomic_store(&mailbox[0], static_cast<uint64_t>(first), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-    __hip_atomic_store(&mailbox[1], word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-    __hip_atomic_store(&mailbox[2], ticket, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    post(mailbox, ticket, static_cast<uint64_t>(first), word);
 }
 
 // `first`: the smallest bad position this lane saw. Every lane of the workgroup calls this, once.

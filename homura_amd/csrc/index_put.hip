@@ -9,6 +9,7 @@
 //   masks       the true elements are counted per tile of 4096, the tiles' counts are scanned by one workgroup
 //               (the total is left where the host reads it), and a second pass over the mask writes the
 //               coordinates of the k-th true element, k = the tile's offset + the rank inside the tile.
+#include "mail.hpp"
 #include "index.hpp"
 
 namespace hmr {
@@ -175,7 +176,7 @@ __global__ void __launch_bounds__(kBlock) mask_count_kernel(const uint8_t *mask,
 // eight adjacent counts per step.
 constexpr int kScanBlock = 1024;
 constexpr int kScanPer = 8;
-__global__ void __launch_bounds__(kScanBlock) mask_scan_kernel(uint64_t *counts, int64_t tiles) {
+__global__ void __launch_bounds__(kScanBlock) mask_scan_kernel(uint64_t *counts, int64_t tiles, uint64_t *mailbox, uint64_t ticket) {
     __shared__ uint64_t lds[kScanBlock / 64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x / 64;
     uint64_t carry = 0;
@@ -210,7 +211,11 @@ __global__ void __launch_bounds__(kScanBlock) mask_scan_kernel(uint64_t *counts,
         carry += total;
         __syncthreads();
     }
-    if (threadIdx.x == 0) counts[tiles] = carry;
+    // The total also goes to the mailbox: the host reads it back at once, to size the result.
+    if (threadIdx.x == 0) {
+        counts[tiles] = carry;
+        post(mailbox, ticket, carry, 0);
+    }
 }
 
 // Division by the mask's sizes (innermost first) for positions below 2^31.
@@ -406,15 +411,21 @@ hmr_status hmr_mask_count(hmr_context_t ctx, const hmr_tensor_desc *mask, void *
         uint64_t *counts = static_cast<uint64_t *>(workspace);
         const bool flat = hmr::mask_is_flat(*mask);
         const int64_t cap = int64_t{1} << 20;
-        return hmr::queue_on(ctx, "mask_count", [&](hipStream_t stream) {
+        if (ctx == nullptr) return fail(HMR_INVALID, "mask_count: null context");
+        uint64_t *mailbox = static_cast<uint64_t *>(ctx->mailbox);
+        const uint64_t ticket = ++ctx->mail_ticket;
+        const hmr_status queued = hmr::queue_on(ctx, "mask_count", [&](hipStream_t stream) {
             if (tiles > 0) {
                 const dim3 grid(static_cast<unsigned>(tiles < cap ? tiles : cap));
                 if (flat) hipLaunchKernelGGL((hmr::mask_count_kernel<true>), grid, dim3(hmr::kBlock), 0, stream, base, d, n, tiles, counts);
                 else hipLaunchKernelGGL((hmr::mask_count_kernel<false>), grid, dim3(hmr::kBlock), 0, stream, base, d, n, tiles, counts);
             }
-            hipLaunchKernelGGL(hmr::mask_scan_kernel, dim3(1), dim3(hmr::kScanBlock), 0, stream, counts, tiles);
+            hipLaunchKernelGGL(hmr::mask_scan_kernel, dim3(1), dim3(hmr::kScanBlock), 0, stream, counts, tiles, mailbox, ticket);
             return true;
         });
+        // The total is in the mailbox as well once the scan has run: a read-back of that word takes it from there.
+        if (queued == HMR_OK) ctx->mail_src = counts + tiles;
+        return queued;
     });
 }
 

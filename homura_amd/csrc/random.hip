@@ -9,6 +9,7 @@
 // are bound by the stores (uniform, integers) or by the f64 transcendentals (normal).
 #include <cmath>
 
+#include "mail.hpp"
 #include "ew_common.hpp"
 #include "normal_math.hpp"
 
@@ -237,7 +238,7 @@ __global__ void __launch_bounds__(kBlock) int_count_kernel(uint64_t *counts, int
 // counts; the lanes' sums are scanned with shuffles inside a wave and through LDS across the waves.
 constexpr int kScanThreads = 1024;
 __global__ void __launch_bounds__(kScanThreads) int_scan_kernel(const uint64_t *counts, uint64_t *offsets, uint64_t *total,
-                                                                int64_t tiles) {
+                                                                int64_t tiles, uint64_t *mailbox, uint64_t ticket) {
     __shared__ uint64_t wave_sum[kScanThreads / 64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int64_t per = (tiles + kScanThreads - 1) / kScanThreads;
@@ -259,7 +260,11 @@ __global__ void __launch_bounds__(kScanThreads) int_scan_kernel(const uint64_t *
         running += w < wave ? wave_sum[w] : 0;
         all += wave_sum[w];
     }
-    if (threadIdx.x == 0) *total = all;
+    // The batch's count also goes to the mailbox (mail.hpp): the host reads it back at once.
+    if (threadIdx.x == 0) {
+        *total = all;
+        post(mailbox, ticket, all, 0);
+    }
     for (int64_t t = first; t < last; ++t) {
         offsets[t] = running;
         running += counts[t];
@@ -383,7 +388,9 @@ hmr_status hmr_random_int(hmr_context_t ctx, const hmr_tensor_desc *out, uint64_
         const int64_t tiles = (nblocks + HMR_RANDOM_INT_TILE - 1) / HMR_RANDOM_INT_TILE;
         if (threshold != 0 && tiles > (int64_t{1} << 31) - 1) return hmr::fail(HMR_INVALID, "random_int: too many blocks in one batch");
         if (blocks == 0 && threshold == 0) return HMR_OK;
-        return hmr::queue_on(ctx, "random_int", [&](hipStream_t stream) {
+        uint64_t *mailbox = static_cast<uint64_t *>(ctx->mailbox);
+        const uint64_t ticket = ++ctx->mail_ticket;
+        const hmr_status queued = hmr::queue_on(ctx, "random_int", [&](hipStream_t stream) {
             int64_t *po = reinterpret_cast<int64_t *>(first);
             if (threshold == 0) {
                 if (n == 0) return true;
@@ -398,13 +405,19 @@ hmr_status hmr_random_int(hmr_context_t ctx, const hmr_tensor_desc *out, uint64_
                 hipLaunchKernelGGL(hmr::int_count_kernel, dim3(static_cast<unsigned>(groups)), dim3(hmr::kBlock), 0, stream, counts,
                                    po, n, nblocks, seed, offset, low, hmr::make_modulus(range), threshold);
             }
-            hipLaunchKernelGGL(hmr::int_scan_kernel, dim3(1), dim3(hmr::kScanThreads), 0, stream, counts, offsets, total, groups);
+            hipLaunchKernelGGL(hmr::int_scan_kernel, dim3(1), dim3(hmr::kScanThreads), 0, stream, counts, offsets, total, groups, mailbox, ticket);
             if (groups > 0 && n > 0) {
                 hipLaunchKernelGGL(hmr::int_write_kernel, dim3(static_cast<unsigned>(groups)), dim3(hmr::kBlock), 0, stream, po, n,
                                    offsets, nblocks, seed, offset, low, hmr::make_modulus(range), threshold, total);
             }
             return true;
         });
+        // A batch that rejects leaves its count in the mailbox as well, for the read-back that follows.
+        if (queued == HMR_OK && threshold != 0) {
+            const int64_t count_tiles = (static_cast<int64_t>(blocks) + HMR_RANDOM_INT_TILE - 1) / HMR_RANDOM_INT_TILE;
+            ctx->mail_src = static_cast<uint64_t *>(workspace) + 2 * count_tiles;
+        }
+        return queued;
     });
 }
 
