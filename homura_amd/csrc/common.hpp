@@ -35,6 +35,8 @@ struct hmr_context {
     // that device address while the mailbox holds its current contents, and a read-back of it (hmr_copy_to_host)
     // watches the mailbox for the ticket - briefly, then it waits for the stream like any copy - and takes the
     // bytes from there instead of queueing a copy. Anything else queued on the context forgets the address.
+    // Like the rest of a context these are the submitting thread's: the caller serialises its submissions per
+    // device (the reference's execution mutex), and a read-back follows its check on the same thread.
     void *mailbox = nullptr;
     const void *mail_src = nullptr;
     uint64_t mail_ticket = 0;
@@ -114,6 +116,7 @@ class Visit {
     // read: that is where a launch that could not be queued shows.
     template <class Queue>
     hmr_status kernels(hmr_context_t ctx, const char *what, Queue queue) {
+        if (ctx == nullptr) return fail(HMR_INVALID, std::string(what) + ": null context");
         ctx->mail_src = nullptr;  // whatever is queued may write what the mailbox mirrors
         if (hmr_status s = use_device(ctx->device)) return s;
         if (hmr_status s = armed_failure("hipGetLastError()")) return s;

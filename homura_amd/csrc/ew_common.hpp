@@ -17,6 +17,7 @@ hmr_status run_map(hmr_context_t ctx, const char *what, int count, const hmr_ten
     MapCall call;
     if (hmr_status s = prepare_map(call, count, descs, bits, negative_inputs)) return s;
     if (call.n == 0) return HMR_OK;
+    if (ctx == nullptr) return fail(HMR_INVALID, std::string(what) + ": null context");
     call.compute_units = ctx->compute_units;
     if (hmr_status s = before(call)) return s;
     return queue_on(ctx, what, [&](hipStream_t stream) { return pick(call, stream); });

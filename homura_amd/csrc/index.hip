@@ -670,6 +670,7 @@ hmr_status hmr_index_check(hmr_context_t ctx, const hmr_tensor_desc *index, int6
         const hmr::Dims d = hmr::dims_of(*index, ops, -1);
         const void *base = hmr::first_of(*index);
         const int is64 = index->dtype == HMR_I64;
+        if (ctx == nullptr) return fail(HMR_INVALID, "index_check: null context");
         hmr::CheckState *state = static_cast<hmr::CheckState *>(ctx->check_state);
         uint64_t *mailbox = static_cast<uint64_t *>(ctx->mailbox);
         const uint64_t ticket = ++ctx->mail_ticket;

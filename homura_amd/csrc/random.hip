@@ -388,6 +388,7 @@ hmr_status hmr_random_int(hmr_context_t ctx, const hmr_tensor_desc *out, uint64_
         const int64_t tiles = (nblocks + HMR_RANDOM_INT_TILE - 1) / HMR_RANDOM_INT_TILE;
         if (threshold != 0 && tiles > (int64_t{1} << 31) - 1) return hmr::fail(HMR_INVALID, "random_int: too many blocks in one batch");
         if (blocks == 0 && threshold == 0) return HMR_OK;
+        if (ctx == nullptr) return hmr::fail(HMR_INVALID, "random_int: null context");
         uint64_t *mailbox = static_cast<uint64_t *>(ctx->mailbox);
         const uint64_t ticket = ++ctx->mail_ticket;
         const hmr_status queued = hmr::queue_on(ctx, "random_int", [&](hipStream_t stream) {

@@ -141,3 +141,14 @@ def test_out_of_scope_entry_points_fail_loudly():
     rc = lib.hmr_max_pool2d_check(None, None, None, None, None, None, None, None)
     assert rc == 2
     assert lib.hmr_last_error() == b"hmr_max_pool2d_check: not built in this library"
+
+
+def test_a_null_context_is_refused_before_anything_is_touched():
+    """Every launch goes through one bracket, which refuses a null context with a message (no GPU needed: nothing is
+    queued and no HIP call is made)."""
+    from ctypes import byref
+    d = capi.make_desc(0x1000, capi.F32, (16,), (1,))
+    assert capi.lib.hmr_fill(None, byref(d), 0) == capi.HMR_INVALID
+    assert b"null context" in capi.lib.hmr_last_error()
+    assert capi.lib.hmr_unary(None, 0, byref(d), byref(d)) == capi.HMR_INVALID
+    assert b"null context" in capi.lib.hmr_last_error()
