@@ -1,6 +1,6 @@
 #!/usr/bin/env python3
 """Applies to a homura checkout the handful of edits that let its `rocm` feature run on an MI355X through this
-library (the same edits INTEGRATION.md describes):
+library:
 
     python homura_amd/integration/apply_to_homura.py /path/to/homura          # edit in place
     python homura_amd/integration/apply_to_homura.py /path/to/homura --check  # only verify that every anchor is there
@@ -14,7 +14,7 @@ library (the same edits INTEGRATION.md describes):
                                    BinaryOp::BitwiseAnd / Tensor::bitwise_and (HMR_BINARY_BITWISE_AND = 15, appended)
 
 Every edit is anchored on one line of the file as homura has it; the script stops, changing nothing, when an anchor is
-missing or not unique (a newer homura: apply the edit by hand, INTEGRATION.md says what it is). Afterwards:
+missing or not unique (a newer homura: apply the edit by hand; EDITS below holds each one in full). Afterwards:
 
     HOMURA_ROCM_PREBUILT=/path/to/homura_amd/lib HOMURA_OFFLOAD_ARCH=gfx950 cargo build --features rocm
 """
