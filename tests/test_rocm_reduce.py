@@ -554,6 +554,34 @@ def test_softmax_across_memory_when_the_positions_lie_megabytes_apart():
         check_softmax(g, c, strip.to(DT.F64), 0, log, f"strip of [{n}, {width}] log {log}")
 
 
+@pytest.mark.parametrize("dtype", [DT.BF16, DT.F32])
+def test_softmax_on_both_sides_of_every_plan_boundary(dtype):
+    """Row lengths and position counts one below, at and one vector past the sizes at which the plans change form
+    (64 / 256 / 1024 lanes a row, rows cut across workgroups; 256 / 512 lanes and the streaming form for rows across
+    memory), a row count that leaves the last workgroup partly idle, and a softmax along an expanded dimension."""
+    vec = 8 if dtype == DT.BF16 else 4
+    row_lengths = [1024 * vec - vec, 1024 * vec, 1024 * vec + vec, 2048 * vec, 2048 * vec + vec, 16384, 16384 + vec,
+                   32768, 32768 + vec, 4096 * vec * 4 + vec]
+    for n in row_lengths:
+        x = finite(dtype, 5 * n, 3, 900 + n % 97).reshape([5, n])
+        for log in (False, True):
+            c = x.log_softmax(1) if log else x.softmax(1)
+            g = x.to(GPU).log_softmax(1) if log else x.to(GPU).softmax(1)
+            check_softmax(g, c, x.to(DT.F64), 1, log, f"{dtype} rows of {n} log {log}")
+    for n in (255, 256, 257, 511, 512, 513, 1023, 1024, 1025, 2050):
+        x = finite(dtype, n * 72, 3, 950 + n % 89).reshape([n, 72])
+        for log in (False, True):
+            c = x.log_softmax(0) if log else x.softmax(0)
+            g = x.to(GPU).log_softmax(0) if log else x.to(GPU).softmax(0)
+            check_softmax(g, c, x.to(DT.F64), 0, log, f"{dtype} {n} positions across memory log {log}")
+    # Every position of a row is the same element: a uniform distribution, exactly 1 / n where that is representable.
+    one = finite(dtype, 64, 3, 77).reshape([1, 64])
+    for n in (8, 300, 1500):
+        x = one.expand([n, 64])
+        c, g = x.softmax(0), one.to(GPU).expand([n, 64]).softmax(0)
+        check_softmax(g, c, x.contiguous().to(DT.F64), 0, False, f"{dtype} expanded to {n} positions")
+
+
 def test_results_repeat_from_run_to_run():
     """ref: tests/rocm_reduce.rs:797-811"""
     x = finite(DT.F32, 1 << 20, 30, 600).reshape([1024, 1024]).to(GPU)
