@@ -333,6 +333,43 @@ def test_variances_down_columns_whose_first_row_is_an_outlier():
                          what=f"{dtype} var [{rows}, {cols}] down columns, first row an outlier")
 
 
+def test_variances_over_runs_and_of_cut_rows_with_special_values_and_outliers():
+    """The one-pass moments of rows made of runs (several reduced dimensions) and of rows cut across workgroups: an
+    output whose elements hold a NaN or an infinity is NaN and its neighbours are not touched; a first element far
+    from the mean, or a mean far from zero, stays within the class 4 n eps v."""
+    for dtype in (DT.F32, DT.BF16, DT.F16):
+        for shape, dims in (([6, 40, 1024], (0, 2)), ([3, 4, 24, 512], (0, 1, 3)), ([4, 300000], (1,)), ([2, 8, 65536], (0, 2))):
+            kept = [d for d in range(len(shape)) if d not in dims]
+            n = int(np.prod([shape[d] for d in dims]))
+            base = to_f64(array(finite(dtype, int(np.prod(shape)), 2, 860 + shape[-1] % 50)), dtype).reshape(shape)
+            # One row per output: the kept dimensions first, the reduced ones flattened behind them.
+            flat = np.moveaxis(base, kept, list(range(len(kept)))).reshape(int(np.prod([shape[d] for d in kept])), n).copy()
+            flat[0, 0] *= 2.0 ** (9 if dtype == DT.F16 else 30)          # first element an outlier
+            if flat.shape[0] > 1:
+                flat[1, :] += 100.0                                       # a mean far from zero
+            if flat.shape[0] > 2:
+                flat[2, n // 3] = np.nan
+            if flat.shape[0] > 3:
+                flat[3, n - 1] = np.inf
+            # Rebuild the tensor in its own layout from the edited rows.
+            moved_shape = [shape[d] for d in kept] + [shape[d] for d in dims]
+            full = flat.reshape(moved_shape)
+            order = kept + list(dims)
+            inverse = [order.index(d) for d in range(len(shape))]
+            data = np.ascontiguousarray(np.transpose(full, inverse))
+            x = tensor(from_f64(data.reshape(-1), dtype), dtype, shape)
+            g = x.to(GPU)
+            for correction in (0, 1):
+                c = x.var_dim(list(dims), correction, False)
+                v64 = f64(x.to(DT.F64).var_dim(list(dims), correction, False))
+                with np.errstate(all="ignore"):
+                    delta = np.nan_to_num(4.0 * n * EPS * v64, nan=0.0, posinf=0.0)
+                check_within(g.var_dim(list(dims), correction, False), c, extra=delta, what=f"{dtype} var {shape} over {dims}")
+                if flat.shape[0] > 3:
+                    assert np.isnan(f64(c).reshape(-1)[2]) and np.isnan(f64(c).reshape(-1)[3])
+                    assert np.isfinite(f64(c).reshape(-1)[0]) and np.isfinite(f64(c).reshape(-1)[1])
+
+
 def test_softmax_extreme_rows_match_the_cpu():
     """ref: tests/rocm_reduce.rs:615-653; plus the KAT of ref: tests/m0_boundaries.rs:468-480."""
     inf, nan = math.inf, math.nan
