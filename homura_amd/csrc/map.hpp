@@ -698,20 +698,35 @@ struct TiledArgs {
     int32_t ostride[NOPS][kFastDims - 2];
 };
 
-// The tile of a workgroup and the element offsets of its outer coordinates. Tiles are numbered along `a`
-// first, and the tile along `b` is shifted by the one along `a`: workgroups that run at the same time then
-// differ in both coordinates. With a power-of-two pitch, tiles that differ in one coordinate only read (or
-// write) pieces a multiple of that pitch apart, which land on few memory channels: an f32 [8192, 8192]
-// transposition took 115-131 us in either plain order and 92 us in this one.
-template <int N, class Args>
+// The tile of a workgroup and the element offsets of its outer coordinates. Which tiles run at the same time
+// decides what the memory sees. Numbered along one dimension, the tiles in flight differ in one coordinate only,
+// and with a power-of-two pitch their pieces lie a multiple of that pitch apart, on few memory channels: an f32
+// [8192, 8192] transposition took 115-131 us in either plain order. Two orders avoid that:
+//   BAND == 0  the tile along `b` is shifted by the one along `a` (a diagonal): 92 us for that kernel. The pieces in
+//              flight are scattered one per row, which suits the shorter runs of 1- and 2-byte elements.
+//   BAND > 0   bands of BAND tiles along `b`; within a band along `b` first (shifted as above), then along `a`: the
+//              512 workgroups in flight cover 64 x 8 tiles, kilobytes of every row they touch on both sides. For
+//              4- and 8-byte elements (512-byte runs) this is 3 % slower on f32 [8192, 8192] and 23-24 % faster on
+//              [8320, 8064], [32768, 2048] and i64 [8320, 8064], within 4 % elsewhere.
+template <int N, int BAND, class Args>
 __device__ __forceinline__ void which_tile(const Args &a, uint32_t &ta, uint32_t &tb, int64_t (&base)[4]) {
     uint32_t rest = blockIdx.x;
     uint32_t q = divide(rest, a.tiles_a);
     ta = rest - q * a.tiles_a.div;
     rest = q;
     q = divide(rest, a.tiles_b);
-    const uint32_t shifted = rest - q * a.tiles_b.div + ta;
-    tb = shifted - divide(shifted, a.tiles_b) * a.tiles_b.div;
+    if constexpr (BAND > 0) {
+        const uint32_t t = (rest - q * a.tiles_b.div) * a.tiles_a.div + ta;  // the tile's number in its plane
+        const uint32_t per_band = BAND * a.tiles_a.div;
+        const uint32_t band = t / per_band, within = t - band * per_band;
+        const uint32_t start = band * BAND;
+        const uint32_t width = a.tiles_b.div - start < BAND ? a.tiles_b.div - start : BAND;  // the last band may be narrower
+        ta = within / width;
+        tb = start + (within - ta * width + ta) % width;
+    } else {
+        const uint32_t shifted = rest - q * a.tiles_b.div + ta;
+        tb = shifted - divide(shifted, a.tiles_b) * a.tiles_b.div;
+    }
     rest = q;
     for (int d = 0; d < a.nouter; ++d) {
         q = divide(rest, a.div[d]);
@@ -744,7 +759,7 @@ __global__ void __launch_bounds__(kBlock) map_tiled_kernel(TiledArgs<F::N + 1> a
     const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
     uint32_t ta, tb;
     int64_t base[4] = {0, 0, 0, 0};
-    which_tile<N>(a, ta, tb, base);
+    which_tile<N, 0>(a, ta, tb, base);
     const uint32_t a0 = ta * S, b0 = tb * S;
     // Phase 1: the turned inputs, lanes along b.
     auto park = [&](auto &tile, int k, auto zero) {
@@ -808,8 +823,8 @@ __global__ void __launch_bounds__(kBlock) map_tiled_kernel(TiledArgs<F::N + 1> a
     }
 }
 
-// The same transposition with 16-byte accesses on both sides, for whole aligned tiles of operands that all have
-// the output's element size and exactly one input turned. A tile is TA x TB elements; it lies in LDS as the
+// The same transposition with 16-byte accesses on both sides, for aligned operands that all have the output's
+// element size, exactly one input turned and both dimensions a multiple of 16 bytes. A tile is TA x TB elements; it lies in LDS as the
 // turned input has it, rows along `a` of 16-byte slots along `b`, slot s of row r at s ^ (r / V): the 16-byte
 // writes of phase 1 spread over all banks, and so do the element reads of phase 2, whose lanes take V
 // consecutive rows each at one column. 512 lanes; all loads of a phase are issued before their first use.
@@ -842,17 +857,22 @@ __global__ void __launch_bounds__(Tiled16Traits<F>::kThreads) map_tiled16_kernel
     const F f = make_functor<F>(a.cbits);
     uint32_t ta, tb;
     int64_t base[4] = {0, 0, 0, 0};
-    which_tile<N>(a, ta, tb, base);
+    which_tile<N, (E >= 4 ? 8 : 0)>(a, ta, tb, base);
     const uint32_t a0 = ta * TA, b0 = tb * TB;
     const int turned = (a.turned_mask & 2u) ? 1 : 2;
     {
         constexpr int kRows = TT::kRows1, kPasses = TT::kPasses1;
         const int row = threadIdx.x / kSlots, slot = threadIdx.x % kSlots;
-        const char *src = a.ptr[turned] + (base[turned] + static_cast<int64_t>(a0) * a.stride_a[turned] + b0) * E;
+        // The last tiles along either dimension may reach past the tensor, by whole 16-byte slots: those slots
+        // load the tensor's last row or last slot again (no branch around a load, whose join would wait for it)
+        // and are not stored.
+        const uint32_t bb = b0 + slot * V < a.size_b ? b0 + slot * V : a.size_b - V;
+        const char *src = a.ptr[turned] + (base[turned] + bb) * E;
         u32x4 v[kPasses];
 #pragma unroll
         for (int j = 0; j < kPasses; ++j) {
-            const u32x4 *p = reinterpret_cast<const u32x4 *>(src + static_cast<int64_t>(j * kRows + row) * a.stride_a[turned] * E) + slot;
+            const uint32_t aa = a0 + j * kRows + row < a.size_a ? a0 + j * kRows + row : a.size_a - 1;
+            const u32x4 *p = reinterpret_cast<const u32x4 *>(src + static_cast<int64_t>(aa) * a.stride_a[turned] * E);
             v[j] = NT ? __builtin_nontemporal_load(p) : *p;
         }
 #pragma unroll
@@ -873,7 +893,9 @@ __global__ void __launch_bounds__(Tiled16Traits<F>::kThreads) map_tiled16_kernel
 #pragma unroll
                 for (int i = 0; i < V; ++i) r[i] = from_cbits<X>(a.cbits[k]);
             } else if (k != turned) {
-                const char *p = a.ptr[k] + (base[k] + static_cast<int64_t>(b0 + j * kRows + row) * a.stride_b[k] + a0 + lane_a * V) * E;
+                const uint32_t bb = b0 + j * kRows + row < a.size_b ? b0 + j * kRows + row : a.size_b - 1;
+                const uint32_t aa = a0 + lane_a * V < a.size_a ? a0 + lane_a * V : a.size_a - V;
+                const char *p = a.ptr[k] + (base[k] + static_cast<int64_t>(bb) * a.stride_b[k] + aa) * E;
                 load_tile<X, V, NT>(p, r);
             }
         }
@@ -907,7 +929,7 @@ __global__ void __launch_bounds__(Tiled16Traits<F>::kThreads) map_tiled16_kernel
             else ro[i] = f(xa[j][i]);
         }
         char *po = a.ptr[0] + (base[0] + static_cast<int64_t>(b0 + j * kRows + row) * a.stride_b[0] + a0 + lane_a * V) * E;
-        store_tile<Out, V, NT>(po, ro);
+        if (b0 + j * kRows + row < a.size_b && a0 + lane_a * V < a.size_a) store_tile<Out, V, NT>(po, ro);
     }
 }
 
@@ -1110,7 +1132,7 @@ bool tiled_applies(const MapCall &c, int &b) {
 }
 
 // Whether a call that tiled_applies accepted (with `b`) can take the 16-byte form: one input turned, the others
-// running with the output, whole tiles, every access aligned.
+// running with the output, both dimensions whole 16-byte slots, every access aligned.
 template <class F>
 bool tiled16_applies(const MapCall &c, int b) {
     using TT = Tiled16Traits<F>;
@@ -1118,7 +1140,9 @@ bool tiled16_applies(const MapCall &c, int b) {
         return false;
     } else {
         const int a = c.ndim - 1;
-        if (c.size[a] % TT::TA != 0 || c.size[b] % TT::TB != 0) return false;
+        // Whole 16-byte slots along both dimensions (the last tiles may be partly empty), and enough of them.
+        if (c.size[a] % TT::V != 0 || c.size[b] % TT::V != 0) return false;
+        if (c.size[a] < TT::TA / 2 || c.size[b] < TT::TB / 2) return false;
         int turned = 0;
         for (int k = 0; k < c.nops; ++k) {
             if (c.is_const[k]) continue;

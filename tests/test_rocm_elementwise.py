@@ -573,10 +573,11 @@ def test_transposed_operands_through_tiles_of_two_dimensions():
 
     for dtype in (DT.U8, DT.Bool, DT.BF16, DT.F16, DT.F32, DT.I32, DT.I64, DT.F64):
         wide = dtype in (DT.U8, DT.Bool, DT.BF16, DT.F16)
-        # The last two of each list are whole tiles of the 16-byte form (64 x 64 elements of 8 bytes, 128 x 128 of
-        # 4, 256 x 128 of 2, 256 x 256 of 1).
-        sizes = ([(64, 64), (70, 33), (129, 65), (257, 100), (128, 256), (384, 128)] if not wide else
-                 [(128, 128), (140, 65), (257, 130), (64, 300), (256, 512), (768, 256)])
+        # The last four of each list take the 16-byte form: two of whole tiles (64 x 64 elements of 8 bytes,
+        # 128 x 128 of 4, 256 x 128 of 2, 256 x 256 of 1) and two of whole 16-byte slots whose last tiles are partly
+        # empty along one dimension or both.
+        sizes = ([(64, 64), (70, 33), (129, 65), (257, 100), (128, 256), (384, 128), (132, 260), (392, 68)] if not wide else
+                 [(128, 128), (140, 65), (257, 130), (64, 300), (256, 512), (768, 256), (272, 400), (784, 144)])
         for rows, cols in sizes:
             (a, ga), (b, gb) = both(dtype, [rows, cols], 91), both(dtype, [cols, rows], 92)
             at, gat = a.transpose(0, 1), ga.transpose(0, 1)  # [cols, rows], contiguous along dimension 0
@@ -609,7 +610,7 @@ def test_transposed_operands_through_tiles_of_two_dimensions():
         w, gw = b.narrow(0, 5, 170).narrow(1, 11, 150), gb.narrow(0, 5, 170).narrow(1, 11, 150)
         assert_bitwise(gv.add(gw), v.add(w), f"{dtype} offset view transposed + offset view")
         # Writes into a transposed or permuted view: the output is the operand that runs along another dimension.
-        for rows, cols in ((70, 33), (128, 256), (257, 130), (384, 128)):
+        for rows, cols in ((70, 33), (128, 256), (257, 130), (384, 128), (264, 136)):
             (d, gd), (src, gsrc) = both(dtype, [rows, cols], 103), both(dtype, [cols, rows], 104)
             d.transpose(0, 1).copy_(src)
             gd.transpose(0, 1).copy_(gsrc)
@@ -633,6 +634,7 @@ def test_transposed_operands_through_tiles_of_two_dimensions():
             assert_bitwise(gv.neg(), v.neg(), f"{dtype} neg of whole tiles at ({r0}, {c0}) transposed")
         for shape, perm in (([5, 70, 140], [2, 0, 1]), ([5, 70, 140], [1, 2, 0]), ([5, 70, 140], [2, 1, 0]),
                             ([3, 128, 256], [2, 0, 1]), ([3, 128, 256], [1, 2, 0]), ([2, 256, 3, 128], [2, 0, 3, 1]),
+                            ([3, 136, 264], [2, 0, 1]), ([3, 136, 264], [1, 2, 0]), ([2, 264, 3, 136], [2, 0, 3, 1]),
                             ([3, 66, 2, 130], [0, 3, 2, 1]), ([2, 129, 3, 2, 70], [4, 2, 0, 3, 1]),
                             ([2, 2, 65, 2, 3, 131], [5, 0, 3, 1, 4, 2])):
             (a, ga) = both(dtype, shape, 100)
