@@ -431,12 +431,12 @@ def per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP
     add(None, "scatter_add f32 [16384,512] into [16384,4096] dim 1 (copy, check, ordered sums line by line in LDS)",
         8 * N + (4 + 4 + 8) * 16384 * 512, lambda: mat.scatter_add(1, cols, vals), 3)
     # A boolean mask over the f32 matrix, 60 % true: the coordinates (count, scan, write; two i64 per true element),
-    # then the selected elements (positions, one element per pick).
+    # then the selected elements (the mask is the only index: one i64 position per true element, one element per pick).
     keep = tensor((words(0x5EED0602, N) % np.uint64(5) < 3).astype(np.uint8), DT.Bool, [16384, 4096], GPU)
     kept = int((words(0x5EED0602, N) % np.uint64(5) < 3).sum())
     add(None, "mask coordinates bool [16384,4096], 60 % true (count, scan, coordinates)", 2 * N + 16 * kept,
         lambda: keep.mask_coordinates(), 5)
-    add(None, "x[mask] f32 [16384,4096], 60 % true (coordinates, check, positions, picks)", 2 * N + 88 * kept,
+    add(None, "x[mask] f32 [16384,4096], 60 % true (count, scan, positions in the flattened mask, picks)", 2 * N + 24 * kept,
         lambda: mat.index_tensors([keep]), 3)
     del mat, cols, vals, keep
     shape = [8, 2048, 4096]

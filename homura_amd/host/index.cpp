@@ -199,6 +199,8 @@ class AdvancedIndex {
         if (count > nd) {
             throw Error("too many indices for tensor of dimension " + std::to_string(nd) + " (got " + std::to_string(count) + ")");
         }
+        size_t defined_indices = 0;
+        for (const auto &t : indices) defined_indices += t ? 1 : 0;
         std::vector<std::optional<Coords>> slots;
         for (const auto &t : indices) {
             if (!t) {
@@ -219,6 +221,19 @@ class AdvancedIndex {
                                 " does not match the shape of the indexed tensor " + shape_str(shape) + " at index " +
                                 std::to_string(start + j));
                 }
+            }
+            if (defined_indices == 1 && data.layout.is_contiguous()) {
+                // The only index, and its elements lie in order: the coordinates of the flattened mask are the
+                // linear positions in the subspace it covers. They are in range by construction, so neither a
+                // check nor a pass per dimension follows; the slots of the mask's dimensions keep the shape.
+                TensorData flat = data;
+                flat.layout = Layout::contiguous(Shape{data.layout.num_elements()});
+                flat.layout.offset = data.layout.offset;
+                mask_positions_ = on_device(backend::mask_coordinates(flat).front(), device);
+                for (size_t j = 0; j < mask_shape.size(); ++j) {
+                    slots.push_back(Coords{mask_positions_->layout.shape, *mask_positions_});
+                }
+                continue;
             }
             for (const TensorData &values : backend::mask_coordinates(data)) {
                 slots.push_back(Coords{values.layout.shape, on_device(values, device)});
@@ -344,6 +359,7 @@ class AdvancedIndex {
     // Checks every position to be in range along its dimension, the indices in order; with `out`, then writes
     // the linear position in the indexed subspace of every element of the broadcast shape (ref: :241-262).
     void check_and_place(const TensorData *out) const {
+        if (mask_positions_ && out == nullptr) return;  // the coordinates of a mask need no check
         std::vector<TensorData> values;
         for (const Coords &c : coords_) values.push_back(c.values);
         const std::vector<int64_t> sizes(shape_.begin() + first_, shape_.begin() + first_ + coords_.size());
@@ -354,6 +370,7 @@ class AdvancedIndex {
 
     // ref: advanced_index.rs:264-279
     TensorData positions(Device device) const {
+        if (mask_positions_) return *mask_positions_;
         const int64_t n = product(broadcast_, 0, broadcast_.size());
         const TensorData out = Tensor::uninit_on(Shape{n}, DType::I64, device).data();
         TensorData shaped = out;
@@ -377,6 +394,7 @@ class AdvancedIndex {
     Shape shape_;               // the target's shape in that order
     size_t first_ = 0;          // the first indexed dimension in shape_
     std::vector<Coords> coords_;
+    std::optional<TensorData> mask_positions_;  // set when one contiguous mask is the only index: its true elements' positions
     Shape broadcast_;           // what the indices broadcast to
     Shape out_shape_;           // before + broadcast + after
 };
