@@ -438,7 +438,10 @@ def per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP
         lambda: keep.mask_coordinates(), 5)
     add(None, "x[mask] f32 [16384,4096], 60 % true (count, scan, positions in the flattened mask, picks)", 2 * N + 24 * kept,
         lambda: mat.index_tensors([keep]), 3)
-    del mat, cols, vals, keep
+    seven = tensor(np.array([7.0], dtype=np.float32), DT.F32, [], GPU)
+    add(None, "x[mask] = v f32 [16384,4096], one value (count, scan, one select between the value and x)", 10 * N,
+        lambda: mat.index_put_tensors([keep], seven, False), 5)
+    del mat, cols, vals, keep, seven
     shape = [8, 2048, 4096]
     add(None, "rand f32 [8,2048,4096] (Philox on the device, write only)", 4 * N, lambda: h.rand(shape, DT.F32, GPU))
     add(None, "rand bf16 [8,2048,4096]", 2 * N, lambda: h.rand(shape, DT.BF16, GPU))

@@ -872,47 +872,66 @@ void index_overwrite(const TensorData &out, size_t dim, const TensorData &index,
 
 // ref: src/backend/rocm/index.rs:560-612: the count, its read-back and the coordinates in one critical section,
 // so that both passes see the same mask.
-std::vector<TensorData> mask_coordinates(const TensorData &mask) {
-    const size_t nd = mask.layout.shape.size();
-    const int64_t n = mask.layout.num_elements();
-    const Device device = mask.device();
-    auto rows_of = [&](const Tensor &coords) {
-        std::vector<TensorData> rows;
-        for (size_t d = 0; d < nd; ++d) rows.push_back(coords.select(0, static_cast<int64_t>(d)).data());
-        return rows;
-    };
-    if (on_cpu(mask)) {
-        hcb_tensor m = cpu_desc(mask);
-        int64_t count = 0;
-        cpu_check(cpu_backend("mask_coordinates").mask_coordinates(&m, nullptr, &count));
-        Tensor coords = Tensor::uninit_on(Shape{static_cast<int64_t>(nd), count}, DType::I64, device);
-        hcb_tensor o = cpu_desc(coords.data());
-        cpu_check(cpu_backend("mask_coordinates").mask_coordinates(&m, &o, &count));
-        return rows_of(coords);
-    }
-    if (n == 0) return rows_of(Tensor::uninit_on(Shape{static_cast<int64_t>(nd), 0}, DType::I64, device));
-    // Every dimension of the mask, unmerged: the kernel reports coordinates along each.
+namespace {
+
+// The mask as the device kernels take it: every dimension unmerged, the kernel reports coordinates along each.
+hmr_tensor_desc mask_desc(const TensorData &mask) {
     std::vector<MergedDim> dims;
     const Strides strides = walk_strides(mask.layout);
-    for (size_t d = 0; d < nd; ++d) dims.push_back(MergedDim{mask.layout.shape[d], {strides[d]}});
-    const hmr_tensor_desc desc = desc_with_dims("mask_coordinates", mask, mask.layout.offset, dims, 0);
-    int64_t bytes = 0, total_word = 0;
-    expect(hmr_mask_workspace(n, &bytes, &total_word));
-    std::shared_ptr<Storage> ws = workspace(bytes, device);
-    Tensor coords;
-    exec(mask, [&](hmr_context_t ctx) {
-        expect(hmr_mask_count(ctx, &desc, ws->ptr(), bytes));
-        uint64_t count = 0;
-        expect(hmr_copy_to_host(ctx, &count, static_cast<const uint64_t *>(ws->ptr()) + total_word, sizeof count));
-        coords = Tensor::uninit_on(Shape{static_cast<int64_t>(nd), static_cast<int64_t>(count)}, DType::I64, device);
-        const TensorData &out = coords.data();
-        const std::vector<MergedDim> rows{MergedDim{static_cast<int64_t>(nd), {static_cast<int64_t>(count)}},
-                                          MergedDim{static_cast<int64_t>(count), {1}}};
-        const hmr_tensor_desc o = desc_with_dims("mask_coordinates", out, out.layout.offset, rows, 0);
-        expect(hmr_mask_coordinates(ctx, &desc, ws->ptr(), bytes, &o));
-    });
-    return rows_of(coords);
+    for (size_t d = 0; d < mask.layout.shape.size(); ++d) dims.push_back(MergedDim{mask.layout.shape[d], {strides[d]}});
+    return desc_with_dims("mask_coordinates", mask, mask.layout.offset, dims, 0);
 }
+
+}  // namespace
+
+MaskCount mask_count(const TensorData &mask) {
+    MaskCount counted;
+    counted.mask = mask;
+    const int64_t n = mask.layout.num_elements();
+    if (on_cpu(mask)) {
+        hcb_tensor m = cpu_desc(mask);
+        cpu_check(cpu_backend("mask_coordinates").mask_coordinates(&m, nullptr, &counted.count));
+        return counted;
+    }
+    if (n == 0) return counted;
+    const hmr_tensor_desc desc = mask_desc(mask);
+    int64_t total_word = 0;
+    expect(hmr_mask_workspace(n, &counted.workspace_bytes, &total_word));
+    counted.workspace = workspace(counted.workspace_bytes, mask.device());
+    exec(mask, [&](hmr_context_t ctx) {
+        expect(hmr_mask_count(ctx, &desc, counted.workspace->ptr(), counted.workspace_bytes));
+        uint64_t count = 0;
+        expect(hmr_copy_to_host(ctx, &count, static_cast<const uint64_t *>(counted.workspace->ptr()) + total_word, sizeof count));
+        counted.count = static_cast<int64_t>(count);
+    });
+    return counted;
+}
+
+std::vector<TensorData> mask_coordinates(const MaskCount &counted) {
+    const TensorData &mask = counted.mask;
+    const size_t nd = mask.layout.shape.size();
+    const Device device = mask.device();
+    Tensor coords = Tensor::uninit_on(Shape{static_cast<int64_t>(nd), counted.count}, DType::I64, device);
+    if (on_cpu(mask)) {
+        hcb_tensor m = cpu_desc(mask);
+        hcb_tensor o = cpu_desc(coords.data());
+        int64_t count = counted.count;
+        cpu_check(cpu_backend("mask_coordinates").mask_coordinates(&m, &o, &count));
+    } else if (counted.count > 0) {
+        const hmr_tensor_desc desc = mask_desc(mask);
+        const TensorData &out = coords.data();
+        const std::vector<MergedDim> rows{MergedDim{static_cast<int64_t>(nd), {counted.count}}, MergedDim{counted.count, {1}}};
+        const hmr_tensor_desc o = desc_with_dims("mask_coordinates", out, out.layout.offset, rows, 0);
+        exec(mask, [&](hmr_context_t ctx) {
+            expect(hmr_mask_coordinates(ctx, &desc, counted.workspace->ptr(), counted.workspace_bytes, &o));
+        });
+    }
+    std::vector<TensorData> rows;
+    for (size_t d = 0; d < nd; ++d) rows.push_back(coords.select(0, static_cast<int64_t>(d)).data());
+    return rows;
+}
+
+std::vector<TensorData> mask_coordinates(const TensorData &mask) { return mask_coordinates(mask_count(mask)); }
 
 // ref: src/backend/rocm/index.rs:614-668: the indices are checked and, without a position out of range, `out`
 // written, in one critical section.

@@ -464,6 +464,16 @@ void index_overwrite(const TensorData &out, size_t dim, const TensorData &index,
 // The coordinates of the true elements of a bool tensor in row-major order: one I64 vector per dimension, on
 // the mask's device (ref: src/backend/mod.rs:398-403).
 std::vector<TensorData> mask_coordinates(const TensorData &mask);
+// The same in two steps, for a caller that needs the number of true elements first and the coordinates later or
+// not at all: the count, with what the second step needs kept beside it.
+struct MaskCount {
+    TensorData mask;
+    int64_t count = 0;
+    std::shared_ptr<Storage> workspace;  // the device's per-tile offsets
+    int64_t workspace_bytes = 0;
+};
+MaskCount mask_count(const TensorData &mask);
+std::vector<TensorData> mask_coordinates(const MaskCount &counted);
 // The positions of advanced indexing: checks each index, in order, to lie in -size..size for its size in `sizes`
 // and returns the first value out of range as (k, value). Without one, and with `out` (I64, the shape the indices
 // broadcast to), writes the row-major position in the subspace of `sizes` of every element, negative coordinates

@@ -225,14 +225,15 @@ class AdvancedIndex {
             if (defined_indices == 1 && data.layout.is_contiguous()) {
                 // The only index, and its elements lie in order: the coordinates of the flattened mask are the
                 // linear positions in the subspace it covers. They are in range by construction, so neither a
-                // check nor a pass per dimension follows; the slots of the mask's dimensions keep the shape.
+                // check nor a pass per dimension follows. Only the count is taken here: it shapes the result;
+                // the positions are written when a read or a write asks for them.
                 TensorData flat = data;
                 flat.layout = Layout::contiguous(Shape{data.layout.num_elements()});
                 flat.layout.offset = data.layout.offset;
-                mask_positions_ = on_device(backend::mask_coordinates(flat).front(), device);
-                for (size_t j = 0; j < mask_shape.size(); ++j) {
-                    slots.push_back(Coords{mask_positions_->layout.shape, *mask_positions_});
-                }
+                counted_ = backend::mask_count(flat);
+                mask_ = data;
+                // The slots of the mask's dimensions keep the shape; their values are never read.
+                for (size_t j = 0; j < mask_shape.size(); ++j) slots.push_back(Coords{Shape{counted_->count}, flat});
                 continue;
             }
             for (const TensorData &values : backend::mask_coordinates(data)) {
@@ -327,6 +328,18 @@ class AdvancedIndex {
     // copied, the last of repeated positions winning. The work happens on a contiguous copy with the dimensions
     // in the order of perm, which the result sees in the original order (ref: advanced_index.rs:345-387).
     Tensor scatter(const TensorData &target, const TensorData &values, bool accumulate) const {
+        if (mask_ && !accumulate && values.layout.num_elements() == 1) {
+            // One value for every element a mask selects: an element-wise choice between the value and the target,
+            // with the mask broadcast over the dimensions behind it. No positions, no copy of the target first.
+            const Shape &shape = target.layout.shape;
+            TensorData cond = on_device(*mask_, target.device());
+            cond.layout.shape = shape;
+            cond.layout.strides.assign(shape.size(), 0);
+            for (size_t j = 0; j < mask_->layout.shape.size(); ++j) cond.layout.strides[first_ + j] = mask_->layout.strides[j];
+            Tensor out = Tensor::uninit_on(shape, target.dtype, target.device());
+            backend::where_(out.data(), cond, values.expand_to(shape), target);
+            return out;
+        }
         const TensorData work = copy_of(Tensor(permuted(target)));
         if (product(out_shape_, 0, out_shape_.size()) == 0) {
             check_and_place(nullptr);
@@ -359,7 +372,7 @@ class AdvancedIndex {
     // Checks every position to be in range along its dimension, the indices in order; with `out`, then writes
     // the linear position in the indexed subspace of every element of the broadcast shape (ref: :241-262).
     void check_and_place(const TensorData *out) const {
-        if (mask_positions_ && out == nullptr) return;  // the coordinates of a mask need no check
+        if (counted_ && out == nullptr) return;  // the coordinates of a mask need no check
         std::vector<TensorData> values;
         for (const Coords &c : coords_) values.push_back(c.values);
         const std::vector<int64_t> sizes(shape_.begin() + first_, shape_.begin() + first_ + coords_.size());
@@ -370,7 +383,7 @@ class AdvancedIndex {
 
     // ref: advanced_index.rs:264-279
     TensorData positions(Device device) const {
-        if (mask_positions_) return *mask_positions_;
+        if (counted_) return on_device(backend::mask_coordinates(*counted_).front(), device);
         const int64_t n = product(broadcast_, 0, broadcast_.size());
         const TensorData out = Tensor::uninit_on(Shape{n}, DType::I64, device).data();
         TensorData shaped = out;
@@ -394,7 +407,8 @@ class AdvancedIndex {
     Shape shape_;               // the target's shape in that order
     size_t first_ = 0;          // the first indexed dimension in shape_
     std::vector<Coords> coords_;
-    std::optional<TensorData> mask_positions_;  // set when one contiguous mask is the only index: its true elements' positions
+    std::optional<backend::MaskCount> counted_;  // set when one contiguous mask is the only index: its flattening, counted
+    std::optional<TensorData> mask_;             // and the mask itself
     Shape broadcast_;           // what the indices broadcast to
     Shape out_shape_;           // before + broadcast + after
 };

@@ -302,6 +302,54 @@ def test_large_masks_compact_in_order():
             assert_same(g, c, "mask coordinates")
 
 
+def _a_mask_alone(device):
+    """A mask as the only index - over leading dimensions, over all of them, behind full slices, as a view - read,
+    assigned one value, assigned as many values as it selects, and accumulated into: numpy's results. (The host layer
+    takes a contiguous mask that stands alone as linear positions, and one value for all of it as a select.)"""
+    rng = np.random.default_rng(11)
+    for dtype, npdt in ((DT.F32, np.float32), (DT.I64, np.int64), (DT.BF16, np.uint16)):
+        for shape, mshape, start in (([6, 5, 4], [6, 5], 0), ([6, 5, 4], [6], 0), ([6, 5, 4], [6, 5, 4], 0), ([6, 5, 4], [5], 1),
+                                     ([6, 5, 4], [5, 4], 1), ([70, 130], [70, 130], 0), ([9000], [9000], 0)):
+            a = rng.integers(0, 30000, shape).astype(npdt)
+            m = rng.random(mshape) < 0.5
+            x, mt = tensor(a, dtype, shape, device), bools(m).to(device)
+            at = (slice(None),) * start + (m,)
+            idx = [None] * start + [mt]
+            assert np.array_equal(array(x.index_tensors(idx)), a[at]), (dtype, shape, mshape)
+            one = np.array([7], dtype=npdt)
+            for vshape in ([], [1]):
+                got = x.index_put_tensors(idx, tensor(one, dtype, vshape, device), False)
+                want = a.copy()
+                want[at] = one[0]
+                assert np.array_equal(array(got), want), (dtype, shape, mshape, vshape)
+            many = rng.integers(0, 30000, a[at].shape).astype(npdt)
+            got = x.index_put_tensors(idx, tensor(many, dtype, list(many.shape), device), False)
+            want = a.copy()
+            want[at] = many
+            assert np.array_equal(array(got), want), (dtype, shape, mshape, "values")
+            if dtype == DT.I64:
+                got = x.index_put_tensors(idx, tensor(one, dtype, [], device), True)
+                want = a.copy()
+                want[at] += one[0]
+                assert np.array_equal(array(got), want), (dtype, shape, mshape, "accumulate")
+            if len(mshape) == 2:
+                view = bools(np.ascontiguousarray(m.T)).to(device).transpose(0, 1)
+                got = x.index_put_tensors([None] * start + [view], tensor(one, dtype, [], device), False)
+                want = a.copy()
+                want[at] = one[0]
+                assert np.array_equal(array(got), want), (dtype, shape, mshape, "view")
+                assert np.array_equal(array(x.index_tensors([None] * start + [view])), a[at])
+
+
+def test_a_mask_alone_follows_numpy():
+    _a_mask_alone("cpu")
+
+
+@pytest.mark.gpu
+def test_a_mask_alone_follows_numpy_on_the_device():
+    _a_mask_alone(GPU)
+
+
 @pytest.mark.gpu
 def test_overwrites_of_rows_keep_the_last_of_repeated_positions():
     """Rows that copy as 16-byte tiles and rows that don't, many repeats of few positions."""
