@@ -233,8 +233,8 @@ template <class W>
 __global__ void __launch_bounds__(kBlock) pick_kernel(W *out, const W *src, const void *index, int is64, Dims d, int64_t n,
                                                       int64_t wrap) {
     // Four picks per lane, a workgroup apart: their positions are read first, then their elements, then they are
-    // stored (one pick per lane leaves a wave with one dependent pair of loads in flight). The outermost
-    // dimension needs no division.
+    // stored (one pick per lane leaves a wave with one dependent pair of loads in flight; eight were no faster).
+    // The outermost dimension needs no division.
     constexpr int U = 4;
     for (int64_t base = static_cast<int64_t>(blockIdx.x) * (U * kBlock); base < n; base += static_cast<int64_t>(gridDim.x) * (U * kBlock)) {
         int64_t oo[U], so[U], j[U];
@@ -248,7 +248,9 @@ __global__ void __launch_bounds__(kBlock) pick_kernel(W *out, const W *src, cons
             for (int k = 0; k < d.ndim; ++k) {
                 int64_t c = rest;
                 if (k + 1 < d.ndim) {
-                    const int64_t q = rest / d.size[k];
+                    // n is below 2^32 for all but the largest tensors: a 32-bit division is a third of a 64-bit one.
+                    const int64_t q = n <= int64_t{0xFFFFFFFF} ? static_cast<int64_t>(static_cast<uint32_t>(rest) / static_cast<uint32_t>(d.size[k]))
+                                                               : rest / d.size[k];
                     c = rest - q * d.size[k];
                     rest = q;
                 }
@@ -803,7 +805,7 @@ hmr_status hmr_index_select(hmr_context_t ctx, const hmr_tensor_desc *out, const
                 } else {
                     hipLaunchKernelGGL((hmr::pick_kernel<W>), dim3(hmr::grid_of((n + 3) / 4)), dim3(hmr::kBlock), 0, stream,
                                        reinterpret_cast<W *>(hmr::first_of(*out)), reinterpret_cast<const W *>(hmr::first_of(*src)),
-                                       static_cast<const void *>(hmr::first_of(*index)), is64, d, n, wrap);
+                                       static_cast<const void *>(hmr::first_of(*index)), is64, hmr::squeezed(d), n, wrap);
                 }
             });
         });
@@ -851,7 +853,8 @@ hmr_status hmr_gather(hmr_context_t ctx, const hmr_tensor_desc *out, const hmr_t
                 }
                 hipLaunchKernelGGL((hmr::pick_kernel<W>), dim3(hmr::grid_of((n + 3) / 4)), dim3(hmr::kBlock), 0, stream,
                                    reinterpret_cast<W *>(hmr::first_of(*out)), reinterpret_cast<const W *>(hmr::first_of(*src)),
-                                   static_cast<const void *>(hmr::first_of(*index)), index->dtype == HMR_I64 ? 1 : 0, d, n, int64_t{0});
+                                   static_cast<const void *>(hmr::first_of(*index)), index->dtype == HMR_I64 ? 1 : 0, hmr::squeezed(d), n,
+                                   int64_t{0});
             });
         });
     });

@@ -41,6 +41,21 @@ inline Dims dims_of(const hmr_tensor_desc &shape_of, const hmr_tensor_desc *cons
     return d;
 }
 
+// The same walk without the dimensions of one element (their coordinate is always 0), `at` kept whatever its size:
+// the element kernels divide once per dimension and element.
+inline Dims squeezed(const Dims &d) {
+    Dims s{};
+    s.at = -1;
+    for (int k = 0; k < d.ndim; ++k) {
+        if (d.size[k] == 1 && k != d.at) continue;
+        if (k == d.at) s.at = s.ndim;
+        s.size[s.ndim] = d.size[k];
+        for (int o = 0; o < 3; ++o) s.stride[o][s.ndim] = d.stride[o][k];
+        ++s.ndim;
+    }
+    return s;
+}
+
 inline char *first_of(const hmr_tensor_desc &d) { return static_cast<char *>(d.data) + d.offset * dtype_size(d.dtype); }
 
 // The largest offset (in elements) a walk over `sizes` with `strides` reaches.
