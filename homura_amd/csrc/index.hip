@@ -268,7 +268,7 @@ __global__ void __launch_bounds__(kBlock) pick_kernel(W *out, const W *src, cons
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            if (valid[u]) out[oo[u]] = v[u];
+            if (valid[u]) __builtin_nontemporal_store(v[u], out + oo[u]);
         }
     }
 }
