@@ -268,7 +268,10 @@ __global__ void __launch_bounds__(kBlock) pick_kernel(W *out, const W *src, cons
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            if (valid[u]) __builtin_nontemporal_store(v[u], out + oo[u]);
+            if (!valid[u]) continue;
+            // Results too large for the caches to keep for a reader go past them, as everywhere in the library.
+            if (n * static_cast<int64_t>(sizeof(W)) >= kStreamStoreBytes) __builtin_nontemporal_store(v[u], out + oo[u]);
+            else out[oo[u]] = v[u];
         }
     }
 }
