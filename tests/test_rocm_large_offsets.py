@@ -173,6 +173,11 @@ def test_index_ops_on_a_table_of_five_gib():
     got = array(table.index_put_tensors([ids], src, False))
     assert np.array_equal(got, expected)
     del got, expected
+    # Single elements by position, enough of them (every 13th: 412 MB) for the stores that go past the caches.
+    every = np.arange(0, rows * width, 13, dtype=np.int64)
+    got = array(table.reshape([rows * width]).index_select(0, tensor(every, DT.I64, [every.size], GPU)))
+    assert np.array_equal(got, a.reshape(-1)[::13])
+    del got, every
     # gather and scatter_add along the rows: four distinct columns of every row.
     r = np.arange(rows, dtype=np.int64)[:, None]
     cols_np = (r * 7 + np.arange(4, dtype=np.int64)[None, :] * 259) % width
