@@ -118,7 +118,17 @@ struct HalfMath {
     static __device__ __forceinline__ E ex(X x, X mx) { return __builtin_amdgcn_exp2f((x - mx) * kLog2eF); }
     static __device__ __forceinline__ double wide(E e) { return static_cast<double>(e); }
     static __device__ __forceinline__ E scale(double sum) { return 64.0f - __builtin_log2f(static_cast<float>(sum)); }
-    static __device__ __forceinline__ E lg(double sum) { return static_cast<float>(log(sum)); }
+    // The logarithm of a row's sum (1 <= sum, the maximum's own term being 1), for results that are rounded to 8
+    // or 11 bits: f32 arithmetic serves and costs a dozen registers less than the f64 routine, which the rows held
+    // in registers cannot spare. Just above 1 (a row that one element dominates) log(1 + t) must keep the
+    // accuracy of t, which 1 + t in f32 has lost: the series there (t < 2^-6: the next term is below 2^-32 of t),
+    // the hardware's log2 elsewhere (relative error below 2^-17 of a logarithm that is at least 2^-6).
+    static __device__ __forceinline__ E lg(double sum) {
+        const float t = static_cast<float>(sum - 1.0);
+        const float series = t * (1.0f + t * (-0.5f + t * (0.333333343f + t * (-0.25f + t * 0.2f))));
+        const float general = __builtin_amdgcn_logf(static_cast<float>(sum)) * 0.693147182f;
+        return t < 0.015625f ? series : general;  // a NaN sum takes the second and stays NaN
+    }
     static __device__ __forceinline__ float soft(X x, X mx, E, E bias) {  // bias = 64 - log2 sum
         return __builtin_ldexpf(__builtin_amdgcn_exp2f(__builtin_fmaf(x - mx, kLog2eF, bias)), -64);
     }
@@ -231,6 +241,20 @@ __device__ __forceinline__ typename Op::Acc row_fold(const Op &op, typename Op::
     return v;
 }
 
+// A value that every lane of the wave holds alike, moved to scalar registers: it stops costing a vector register
+// for as long as it lives (a row's maximum, sum and scale live across whole phases).
+template <class A>
+__device__ __forceinline__ A uniform(A v) {
+    constexpr int words = static_cast<int>(sizeof(A)) / 4;
+    static_assert(sizeof(A) % 4 == 0, "whole words");
+    uint32_t w[words];
+    __builtin_memcpy(w, &v, sizeof(A));
+#pragma unroll
+    for (int i = 0; i < words; ++i) w[i] = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(w[i])));
+    __builtin_memcpy(&v, w, sizeof(A));
+    return v;
+}
+
 struct SoftmaxArgs {
     char *out;        // element (0,..) of the output rows
     const char *src;  // element (0,..) of the source rows
@@ -308,7 +332,7 @@ __global__ void __launch_bounds__(G > kBlock ? G : kBlock, (LOG && G == 1024 && 
             for (int i = 0; i < V; i += 2) mx = max3(mx, x[i], x[i + 1]);
             __builtin_amdgcn_sched_barrier(0);  // a chunk at a time: unpacked ahead, the row would fill the registers
         }
-        mx = row_fold<G>(MaxFold{}, mx, reinterpret_cast<X *>(lds));
+        mx = uniform(row_fold<G>(MaxFold{}, mx, reinterpret_cast<X *>(lds)));  // a row is whole waves
         // Phase 2: exponentials and their f64 sum.
         double sum = 0.0;
         E ex[kKeep ? C : 1][kKeep ? V : 1];  // chunk c is defined where did[c]
@@ -367,7 +391,7 @@ __global__ void __launch_bounds__(G > kBlock ? G : kBlock, (LOG && G == 1024 && 
             // temporaries.
             __builtin_amdgcn_sched_barrier(0);
         }
-        sum = row_fold<G>(SumOp{}, sum, lds);
+        sum = uniform(row_fold<G>(SumOp{}, sum, lds));
         // Phase 3: write once.
         E scale;
         if constexpr (LOG && G > kBlock) {
@@ -379,9 +403,9 @@ __global__ void __launch_bounds__(G > kBlock ? G : kBlock, (LOG && G == 1024 && 
                 if (threadIdx.x == 0) row_scale = v;
             }
             __syncthreads();
-            scale = row_scale;
+            scale = uniform(row_scale);
         } else {
-            scale = LOG ? M::lg(sum) : M::scale(sum);
+            scale = uniform(LOG ? M::lg(sum) : M::scale(sum));
         }
         asm volatile("" : "+v"(at));
 #pragma unroll
