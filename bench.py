@@ -439,7 +439,7 @@ def per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP
     add(None, "x[mask] f32 [16384,4096], 60 % true (count, scan, positions in the flattened mask, picks)", 2 * N + 24 * kept,
         lambda: mat.index_tensors([keep]), 3)
     seven = tensor(np.array([7.0], dtype=np.float32), DT.F32, [], GPU)
-    add(None, "x[mask] = v f32 [16384,4096], one value (count, scan, one select between the value and x)", 10 * N,
+    add(None, "x[mask] = v f32 [16384,4096], one value (one select between the value and x)", 9 * N,
         lambda: mat.index_put_tensors([keep], seven, False), 5)
     del mat, cols, vals, keep, seven
     shape = [8, 2048, 4096]

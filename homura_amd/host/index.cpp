@@ -177,7 +177,10 @@ class AdvancedIndex {
   public:
     // ref: advanced_index.rs:99-231 (ATen's make_info): index dtypes, then devices, mask shapes, the number of
     // indices, broadcasting, and indices into empty dimensions.
-    AdvancedIndex(const TensorData &target, const std::vector<std::optional<Tensor>> &indices) {
+    // `one_value`: the caller is about to assign a single value without accumulating. A mask that stands alone
+    // then needs neither positions nor its count (one value fits any number of selected elements): the slots of its
+    // dimensions take the mask's size as a stand-in, and scatter() selects.
+    AdvancedIndex(const TensorData &target, const std::vector<std::optional<Tensor>> &indices, bool one_value = false) {
         const Device device = target.device();
         const Shape &shape = target.layout.shape;
         const size_t nd = shape.size();
@@ -230,10 +233,16 @@ class AdvancedIndex {
                 TensorData flat = data;
                 flat.layout = Layout::contiguous(Shape{data.layout.num_elements()});
                 flat.layout.offset = data.layout.offset;
-                counted_ = backend::mask_count(flat);
                 mask_ = data;
+                int64_t count = flat.layout.num_elements();
+                if (one_value) {
+                    select_only_ = true;
+                } else {
+                    counted_ = backend::mask_count(flat);
+                    count = counted_->count;
+                }
                 // The slots of the mask's dimensions keep the shape; their values are never read.
-                for (size_t j = 0; j < mask_shape.size(); ++j) slots.push_back(Coords{Shape{counted_->count}, flat});
+                for (size_t j = 0; j < mask_shape.size(); ++j) slots.push_back(Coords{Shape{count}, flat});
                 continue;
             }
             for (const TensorData &values : backend::mask_coordinates(data)) {
@@ -372,7 +381,7 @@ class AdvancedIndex {
     // Checks every position to be in range along its dimension, the indices in order; with `out`, then writes
     // the linear position in the indexed subspace of every element of the broadcast shape (ref: :241-262).
     void check_and_place(const TensorData *out) const {
-        if (counted_ && out == nullptr) return;  // the coordinates of a mask need no check
+        if (mask_ && out == nullptr) return;  // the coordinates of a mask need no check
         std::vector<TensorData> values;
         for (const Coords &c : coords_) values.push_back(c.values);
         const std::vector<int64_t> sizes(shape_.begin() + first_, shape_.begin() + first_ + coords_.size());
@@ -383,6 +392,7 @@ class AdvancedIndex {
 
     // ref: advanced_index.rs:264-279
     TensorData positions(Device device) const {
+        if (select_only_) throw Error("advanced indexing: the positions of an uncounted mask were asked for");
         if (counted_) return on_device(backend::mask_coordinates(*counted_).front(), device);
         const int64_t n = product(broadcast_, 0, broadcast_.size());
         const TensorData out = Tensor::uninit_on(Shape{n}, DType::I64, device).data();
@@ -409,6 +419,7 @@ class AdvancedIndex {
     std::vector<Coords> coords_;
     std::optional<backend::MaskCount> counted_;  // set when one contiguous mask is the only index: its flattening, counted
     std::optional<TensorData> mask_;             // and the mask itself
+    bool select_only_ = false;                   // the mask was not counted: only scatter()'s select may follow
     Shape broadcast_;           // what the indices broadcast to
     Shape out_shape_;           // before + broadcast + after
 };
@@ -421,7 +432,8 @@ Tensor Tensor::index_tensors(const std::vector<std::optional<Tensor>> &indices) 
 }
 
 Tensor Tensor::index_put_tensors(const std::vector<std::optional<Tensor>> &indices, const Tensor &values, bool accumulate) const {
-    const AdvancedIndex info(d_, indices);
+    const bool one_value = !accumulate && values.num_elements() == 1 && values.num_dims() <= 1;
+    const AdvancedIndex info(d_, indices, one_value);
     info.check_values(d_, values.data());
     return info.scatter(d_, values.data(), accumulate);
 }
