@@ -218,6 +218,66 @@ __global__ void __launch_bounds__(kScanBlock) mask_scan_kernel(uint64_t *counts,
     }
 }
 
+// The same scan by many workgroups, for up to kSpreadTiles tiles: workgroup w owns 256 tiles, adds up every count
+// before them (its lanes take every 256th, sixteen loads at a time; the counts of all earlier tiles are at most
+// 512 KB, which the L2 serves) and scans its own. It reads `raw` and writes `offsets`, two arrays: a workgroup
+// may still be reading counts that another has already replaced by offsets. One launch of some microseconds
+// instead of two dependent passes of one workgroup.
+constexpr int64_t kSpreadTiles = 65536;
+__global__ void __launch_bounds__(kBlock) mask_scan_spread_kernel(const uint64_t *raw, uint64_t *offsets, int64_t tiles, uint64_t *mailbox,
+                                                                  uint64_t ticket) {
+    __shared__ uint64_t lds[kBlock / 64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x / 64;
+    const int64_t first = static_cast<int64_t>(blockIdx.x) * kBlock;
+    auto fold = [&](uint64_t x) {  // the sum over the workgroup, in every lane
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1) {
+            const uint64_t lo = static_cast<uint32_t>(__shfl_xor(static_cast<int>(x), m, 64));
+            const uint64_t hi = static_cast<uint32_t>(__shfl_xor(static_cast<int>(x >> 32), m, 64));
+            x += (hi << 32) | lo;
+        }
+        __syncthreads();
+        if (lane == 0) lds[wave] = x;
+        __syncthreads();
+        uint64_t total = 0;
+        for (int w = 0; w < kBlock / 64; ++w) total += lds[w];
+        return total;
+    };
+    constexpr int kAhead = 16;  // loads in flight per lane: the last workgroup of 65 536 tiles reads 255 counts a lane
+    uint64_t sum = 0;
+    int64_t j = threadIdx.x;
+    for (; j + (kAhead - 1) * kBlock < first; j += kAhead * kBlock) {
+        uint64_t got[kAhead];
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) got[u] = raw[j + u * kBlock];
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) sum += got[u];
+    }
+    for (; j < first; j += kBlock) sum += raw[j];
+    const uint64_t before = fold(sum);
+    // The workgroup's own 256 counts: an inclusive scan along the lanes, then across the waves.
+    const int64_t mine = first + threadIdx.x;
+    const uint64_t v = mine < tiles ? raw[mine] : 0;
+    uint64_t x = v;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const uint64_t lo = static_cast<uint32_t>(__shfl_up(static_cast<int>(x), off, 64));
+        const uint64_t hi = static_cast<uint32_t>(__shfl_up(static_cast<int>(x >> 32), off, 64));
+        if (lane >= off) x += (hi << 32) | lo;
+    }
+    __syncthreads();
+    if (lane == 63) lds[wave] = x;
+    __syncthreads();
+    uint64_t ahead = before;
+    for (int w = 0; w < wave; ++w) ahead += lds[w];
+    if (mine < tiles) offsets[mine] = ahead + x - v;
+    if (mine == tiles - 1) {
+        const uint64_t total = ahead + x;
+        offsets[tiles] = total;
+        post(mailbox, ticket, total, 0);
+    }
+}
+
 // Division by the mask's sizes (innermost first) for positions below 2^31.
 struct MaskDivs {
     FastDiv d[kMaxIndexDims];
@@ -392,7 +452,8 @@ hmr_status hmr_mask_workspace(int64_t n, int64_t *bytes, int64_t *total_word) {
     return fenced([&] {
         if (n < 0) return fail(HMR_INVALID, "mask_workspace: negative size");
         const int64_t tiles = hmr::mask_tiles(n);
-        *bytes = (tiles + 1) * 8;
+        // The tiles' offsets and the total, then the tiles' raw counts where the spread scan wants them apart.
+        *bytes = (tiles + 1 + (tiles <= hmr::kSpreadTiles ? tiles : 0)) * 8;
         *total_word = tiles;
         return HMR_OK;
     });
@@ -404,11 +465,15 @@ hmr_status hmr_mask_count(hmr_context_t ctx, const hmr_tensor_desc *mask, void *
         if (hmr_status s = hmr::check_desc(*mask, n)) return s;
         if (mask->dtype != HMR_BOOL) return fail(HMR_INVALID, "mask_count: the mask is BOOL");
         const int64_t tiles = hmr::mask_tiles(n);
-        if (workspace == nullptr || workspace_bytes < (tiles + 1) * 8) return fail(HMR_INVALID, "mask_count: the workspace is too small");
+        const bool spread = tiles > 0 && tiles <= hmr::kSpreadTiles;
+        if (workspace == nullptr || workspace_bytes < (tiles + 1 + (spread ? tiles : 0)) * 8) {
+            return fail(HMR_INVALID, "mask_count: the workspace is too small");
+        }
         const hmr_tensor_desc *const ops[3] = {mask, nullptr, nullptr};
         const hmr::Dims d = hmr::dims_of(*mask, ops, -1);
         const uint8_t *base = reinterpret_cast<const uint8_t *>(hmr::first_of(*mask));
-        uint64_t *counts = static_cast<uint64_t *>(workspace);
+        uint64_t *offsets = static_cast<uint64_t *>(workspace);
+        uint64_t *counts = spread ? offsets + tiles + 1 : offsets;
         const bool flat = hmr::mask_is_flat(*mask);
         const int64_t cap = int64_t{1} << 20;
         if (ctx == nullptr) return fail(HMR_INVALID, "mask_count: null context");
@@ -420,11 +485,16 @@ hmr_status hmr_mask_count(hmr_context_t ctx, const hmr_tensor_desc *mask, void *
                 if (flat) hipLaunchKernelGGL((hmr::mask_count_kernel<true>), grid, dim3(hmr::kBlock), 0, stream, base, d, n, tiles, counts);
                 else hipLaunchKernelGGL((hmr::mask_count_kernel<false>), grid, dim3(hmr::kBlock), 0, stream, base, d, n, tiles, counts);
             }
-            hipLaunchKernelGGL(hmr::mask_scan_kernel, dim3(1), dim3(hmr::kScanBlock), 0, stream, counts, tiles, mailbox, ticket);
+            if (spread) {
+                hipLaunchKernelGGL(hmr::mask_scan_spread_kernel, dim3(static_cast<unsigned>((tiles + hmr::kBlock - 1) / hmr::kBlock)),
+                                   dim3(hmr::kBlock), 0, stream, counts, offsets, tiles, mailbox, ticket);
+            } else {
+                hipLaunchKernelGGL(hmr::mask_scan_kernel, dim3(1), dim3(hmr::kScanBlock), 0, stream, counts, tiles, mailbox, ticket);
+            }
             return true;
         });
         // The total is in the mailbox as well once the scan has run: a read-back of that word takes it from there.
-        if (queued == HMR_OK) ctx->mail_src = counts + tiles;
+        if (queued == HMR_OK) ctx->mail_src = offsets + tiles;
         return queued;
     });
 }

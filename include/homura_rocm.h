@@ -404,7 +404,8 @@ hmr_status hmr_index_overwrite(hmr_context_t ctx, const hmr_tensor_desc *out,
 /* ref :416-426  cpu::mask_coordinates (misc.rs:128-148) in two calls: hmr_mask_count queues counting
  * the true elements of the BOOL mask (any layout), whose number it leaves at word total_word of the
  * workspace (hmr_mask_workspace bytes for the mask's number of elements: a 64-bit word per tile of
- * 4096 elements and one for the total); hmr_mask_coordinates then writes coordinate d of the k-th
+ * 4096 elements and one for the total, and for masks of up to 65 536 tiles a second word per tile);
+ * hmr_mask_coordinates then writes coordinate d of the k-th
  * true element, in row-major order, to out[d][k] (I64, the mask's rank x the number). */
 hmr_status hmr_mask_workspace(int64_t n, int64_t *bytes, int64_t *total_word);
 hmr_status hmr_mask_count(hmr_context_t ctx, const hmr_tensor_desc *mask, void *workspace,

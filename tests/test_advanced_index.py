@@ -408,11 +408,15 @@ def test_the_c_abi_of_positions_masks_and_overwrites():
         assert L.hmr_index_positions(ctx.handle, byref(F), byref(R), 3, 4, 1) == capi.HMR_INVALID
         assert L.hmr_last_error().decode() == "index_positions: the positions are I64"
         assert L.hmr_index_positions(ctx.handle, byref(O), byref(F), 3, 4, 1) == capi.HMR_INVALID
-        # Masks: a word per tile of 4096 elements and the total after them.
+        # Masks: an offset per tile of 4096 elements and the total after them, then (up to 65 536 tiles) the tiles' raw
+        # counts, which the scan by many workgroups keeps apart from the offsets it writes.
         n = 3 * 4096 + 5
         bytes_, word = c_int64(), c_int64()
         capi.check(L.hmr_mask_workspace(n, byref(bytes_), byref(word)))
-        assert (bytes_.value, word.value) == (5 * 8, 4)
+        assert (bytes_.value, word.value) == ((5 + 4) * 8, 4)
+        big, big_word = c_int64(), c_int64()
+        capi.check(L.hmr_mask_workspace(65537 * 4096, byref(big), byref(big_word)))
+        assert (big.value, big_word.value) == (65538 * 8, 65537)
         m = words(9, n) % np.uint64(4) == 0
         dm = ctx.upload(m.astype(np.uint8))
         ws = ctx.malloc(bytes_.value)
