@@ -5,7 +5,8 @@
 // A pass handles 8 bits. Workgroups take tiles of 2048 words:
 //   count    the tile's digit histogram into hist[digit][tile] (digit-major, so that one exclusive scan of the whole
 //            table gives, for every digit and tile, where the tile's words of that digit go);
-//   scan     the table in chunks of 4096 entries, then the chunks' totals by one workgroup;
+//   scan     the table in chunks of 4096 entries, then the chunks' totals by one workgroup (sorts of up to 16 tiles
+//            skip both: their scatter workgroups add up the small table themselves);
 //   scatter  the tile again: every word's rank among the tile's words of its digit, in input order (waves find
 //            their equal digits with ballots, the counts per round and wave are scanned in LDS), the words placed
 //            in LDS in sorted order, and written out from there so that runs of a digit leave as whole lines.
@@ -143,6 +144,12 @@ static __global__ void __launch_bounds__(kSortScanBlock) scan_totals_kernel(uint
     }
 }
 
+// SELF_SCAN: `hist` is the table as radix_count_kernel left it, of at most kSortSelfTiles tiles, and every workgroup
+// finds its own places in it: thread d adds up digit d's counts over the tiles (the digit's words, and those of the
+// tiles before this one), the digits' sums are scanned over the workgroup. Two launches fewer per pass, which for a
+// sort of some ten thousand words is a third of its time.
+constexpr int kSortSelfTiles = 16;
+template <bool SELF_SCAN>
 static __global__ void __launch_bounds__(kSortThreads) radix_scatter_kernel(const uint64_t *in, uint64_t *out, int64_t n, int shift,
                                                                      const uint32_t *hist, const uint32_t *totals, int64_t tiles) {
     __shared__ uint16_t counts[kSortRounds][kSortWaves][kSortDigits];  // words of a digit in (round, wave), then their prefix
@@ -198,7 +205,28 @@ static __global__ void __launch_bounds__(kSortThreads) radix_scatter_kernel(cons
     for (int w = 0; w < wave; ++w) before += wave_sums[w];
     const int64_t entry = static_cast<int64_t>(threadIdx.x) * tiles + blockIdx.x;
     local_base[threadIdx.x] = before;
-    digit_base[threadIdx.x] = hist[entry] + totals[entry / kSortScanChunk] - before;
+    if constexpr (SELF_SCAN) {
+        uint32_t all = 0, ahead = 0;  // digit threadIdx.x: its words in every tile, and in the tiles before this one
+        for (int t = 0; t < static_cast<int>(tiles); ++t) {
+            const uint32_t c = hist[static_cast<int64_t>(threadIdx.x) * tiles + t];
+            all += c;
+            ahead += t < static_cast<int>(blockIdx.x) ? c : 0u;
+        }
+        uint32_t y = all;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const uint32_t z = static_cast<uint32_t>(__shfl_up(static_cast<int>(y), off, 64));
+            if (lane >= off) y += z;
+        }
+        __syncthreads();  // wave_sums was read above
+        if (lane == 63) wave_sums[wave] = y;
+        __syncthreads();
+        uint32_t smaller = y - all;  // words of smaller digits, in all tiles
+        for (int w = 0; w < wave; ++w) smaller += wave_sums[w];
+        digit_base[threadIdx.x] = smaller + ahead - before;
+    } else {
+        digit_base[threadIdx.x] = hist[entry] + totals[entry / kSortScanChunk] - before;
+    }
     __syncthreads();
 #pragma unroll
     for (int r = 0; r < kSortRounds; ++r) {
@@ -226,10 +254,16 @@ inline uint64_t *sort_words(void *workspace, int64_t n, int key_bits, hipStream_
         const int shift = 32 + done;
         const dim3 grid(static_cast<unsigned>(l.tiles));
         hipLaunchKernelGGL(radix_count_kernel, grid, dim3(kSortThreads), 0, stream, static_cast<const uint64_t *>(a), n, shift, hist, l.tiles);
-        hipLaunchKernelGGL(scan_chunks_kernel, dim3(static_cast<unsigned>(l.chunks)), dim3(kSortThreads), 0, stream, hist, l.entries, totals);
-        hipLaunchKernelGGL(scan_totals_kernel, dim3(1), dim3(kSortScanBlock), 0, stream, totals, l.chunks);
-        hipLaunchKernelGGL(radix_scatter_kernel, grid, dim3(kSortThreads), 0, stream, static_cast<const uint64_t *>(a), b, n, shift,
-                           static_cast<const uint32_t *>(hist), static_cast<const uint32_t *>(totals), l.tiles);
+        if (l.tiles <= kSortSelfTiles) {
+            hipLaunchKernelGGL(radix_scatter_kernel<true>, grid, dim3(kSortThreads), 0, stream, static_cast<const uint64_t *>(a), b, n,
+                               shift, static_cast<const uint32_t *>(hist), static_cast<const uint32_t *>(totals), l.tiles);
+        } else {
+            hipLaunchKernelGGL(scan_chunks_kernel, dim3(static_cast<unsigned>(l.chunks)), dim3(kSortThreads), 0, stream, hist, l.entries,
+                               totals);
+            hipLaunchKernelGGL(scan_totals_kernel, dim3(1), dim3(kSortScanBlock), 0, stream, totals, l.chunks);
+            hipLaunchKernelGGL(radix_scatter_kernel<false>, grid, dim3(kSortThreads), 0, stream, static_cast<const uint64_t *>(a), b, n,
+                               shift, static_cast<const uint32_t *>(hist), static_cast<const uint32_t *>(totals), l.tiles);
+        }
         uint64_t *t = a;
         a = b;
         b = t;
