@@ -447,25 +447,50 @@ __global__ void __launch_bounds__(kBlock) index_runs_tiles_kernel(T *out, const 
     const int lane = threadIdx.x % lanes;
     for (int64_t r = static_cast<int64_t>(blockIdx.x) * per_block + threadIdx.x / lanes; r < m;
          r += static_cast<int64_t>(gridDim.x) * per_block) {
-        const uint64_t target = words[r] >> 32;
+        const uint64_t first = words[r];
+        const uint64_t target = first >> 32;
         if (r > 0 && (words[r - 1] >> 32) == target) continue;
-        for (int64_t t = lane; t < tiles; t += lanes) {
-            T *po = out + static_cast<int64_t>(target) * out_step + t * V;
-            T v[V];
-            typename S::A acc[V];
-            load_tile<T, V, false>(reinterpret_cast<const char *>(po), v);
+        // Two tiles of the row per step, and for each the target's tile and the run's first source tile requested
+        // together: most runs are one row long, and a lane's chain is then the sorted word, these loads, the store
+        // (one tile at a time with the source behind the target it was three round trips per tile).
+        constexpr int U = 2;
+        const int64_t from = static_cast<int64_t>(first & 0xFFFFFFFFu) * src_step;
+        for (int64_t t0 = lane; t0 < tiles; t0 += static_cast<int64_t>(U) * lanes) {
+            T v[U][V], s0[U][V];
+            typename S::A acc[U][V];
 #pragma unroll
-            for (int i = 0; i < V; ++i) acc[i] = S::widen(v[i]);
-            for (int64_t x = r; x < m; ++x) {
-                const uint64_t w = words[x];
-                if ((w >> 32) != target) break;
-                load_tile<T, V, false>(reinterpret_cast<const char *>(src + static_cast<int64_t>(w & 0xFFFFFFFFu) * src_step + t * V), v);
-#pragma unroll
-                for (int i = 0; i < V; ++i) acc[i] = S::add(acc[i], v[i]);
+            for (int u = 0; u < U; ++u) {
+                const int64_t t = t0 + static_cast<int64_t>(u) * lanes < tiles ? t0 + static_cast<int64_t>(u) * lanes : t0;
+                load_tile<T, V, false>(reinterpret_cast<const char *>(out + static_cast<int64_t>(target) * out_step + t * V), v[u]);
+                load_tile<T, V, false>(reinterpret_cast<const char *>(src + from + t * V), s0[u]);
             }
 #pragma unroll
-            for (int i = 0; i < V; ++i) v[i] = S::narrow(acc[i]);
-            store_tile<T, V, false>(reinterpret_cast<char *>(po), v);
+            for (int u = 0; u < U; ++u) {
+#pragma unroll
+                for (int i = 0; i < V; ++i) acc[u][i] = S::add(S::widen(v[u][i]), s0[u][i]);
+            }
+            for (int64_t x = r + 1; x < m; ++x) {
+                const uint64_t w = words[x];
+                if ((w >> 32) != target) break;
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int64_t t = t0 + static_cast<int64_t>(u) * lanes < tiles ? t0 + static_cast<int64_t>(u) * lanes : t0;
+                    load_tile<T, V, false>(reinterpret_cast<const char *>(src + static_cast<int64_t>(w & 0xFFFFFFFFu) * src_step + t * V), s0[u]);
+                }
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+#pragma unroll
+                    for (int i = 0; i < V; ++i) acc[u][i] = S::add(acc[u][i], s0[u][i]);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int64_t t = t0 + static_cast<int64_t>(u) * lanes;
+                if (t >= tiles) continue;
+#pragma unroll
+                for (int i = 0; i < V; ++i) v[u][i] = S::narrow(acc[u][i]);
+                store_tile<T, V, false>(reinterpret_cast<char *>(out + static_cast<int64_t>(target) * out_step + t * V), v[u]);
+            }
         }
     }
 }
