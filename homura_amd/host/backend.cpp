@@ -734,7 +734,7 @@ template <class F>
 void run_checked(const char *kernel, const TensorData &on, const TensorData &index, size_t dim, int64_t size, Bounds bounds,
                  F then) {
     hmr_tensor_desc check{};
-    const bool checks = bounds != Bounds::Valid && own_desc(kernel, index, check);
+    const bool checks = bounds != Bounds::Valid && bounds != Bounds::ValidWrap && own_desc(kernel, index, check);
     std::shared_ptr<Storage> slots = checks ? workspace(16, on.device()) : nullptr;
     exec(on, [&](hmr_context_t ctx) {
         if (checks) {
@@ -753,7 +753,8 @@ void run_checked(const char *kernel, const TensorData &on, const TensorData &ind
 void index_select(const TensorData &out, const TensorData &src, size_t dim, const TensorData &index, Bounds bounds) {
     if (on_cpu(out)) {
         hcb_tensor o = cpu_desc(out), s = cpu_desc(src), i = cpu_desc(index);
-        cpu_check(cpu_backend("index_select").index_select(&o, &s, static_cast<int32_t>(dim), &i, static_cast<int32_t>(bounds)));
+        const Bounds known = bounds == Bounds::ValidWrap ? Bounds::AllowNegative : bounds;  // the CPU kernel checks again
+        cpu_check(cpu_backend("index_select").index_select(&o, &s, static_cast<int32_t>(dim), &i, static_cast<int32_t>(known)));
         return;
     }
     const int64_t size = src.layout.shape[dim];
@@ -775,7 +776,7 @@ void index_select(const TensorData &out, const TensorData &src, size_t dim, cons
         i.ndim = 1;
         i.sizes[0] = d[2].sizes[at];
         i.strides[0] = d[2].strides[at];
-        expect(hmr_index_select(ctx, &d[0], &d[1], &i, at, bounds == Bounds::AllowNegative ? 1 : 0));
+        expect(hmr_index_select(ctx, &d[0], &d[1], &i, at, bounds == Bounds::AllowNegative || bounds == Bounds::ValidWrap ? 1 : 0));
     });
 }
 

@@ -423,7 +423,8 @@ Tensor adam_step(const Tensor &p, const Tensor &grad, std::optional<AdamState> &
 // ---- backend dispatch (ref: src/backend/mod.rs:298-534) ---------------------------------------------
 
 // How the positions of an index tensor are checked (ref: src/backend/mod.rs:360-373).
-enum class Bounds { Valid = 0, NonNegative = 1, AllowNegative = 2 };
+// ValidWrap: checked already to lie in -size..size; negative positions count from the end.
+enum class Bounds { Valid = 0, NonNegative = 1, AllowNegative = 2, ValidWrap = 3 };
 
 // The optimizers' fused steps (ref: src/backend/cpu/mod.rs:509-530).
 struct Fused {

@@ -302,10 +302,24 @@ class AdvancedIndex {
             check_and_place(nullptr);
             return out;
         }
-        const TensorData where = positions(target.device());
-        const int64_t count = where.layout.num_elements();
         const Tensor src = Tensor(permuted(target)).reshape(folded());
         TensorData shaped = out.data();
+        if (coords_.size() == 1 && !mask_ && coords_[0].values.layout.is_contiguous()) {
+            // One index tensor: its elements are the positions along the one indexed dimension, the negative ones
+            // counted from the end, which the row lookup does by itself. The check stays (and its message, which
+            // names the dimension as the caller sees it); the pass that writes positions is not needed.
+            check_and_place(nullptr);
+            TensorData ids = coords_[0].values;
+            const int64_t count = ids.layout.num_elements();
+            const int64_t offset = ids.layout.offset;
+            ids.layout = Layout::contiguous(Shape{count});
+            ids.layout.offset = offset;
+            shaped.layout = Layout::contiguous(Shape{before(), count, after()});
+            backend::index_select(shaped, src.data(), 1, ids, Bounds::ValidWrap);
+            return out;
+        }
+        const TensorData where = positions(target.device());
+        const int64_t count = where.layout.num_elements();
         shaped.layout = Layout::contiguous(Shape{before(), count, after()});
         backend::index_select(shaped, src.data(), 1, where, Bounds::Valid);
         return out;
