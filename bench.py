@@ -417,10 +417,10 @@ def per_op_table(h, timed, tensor, from_f64, normal, uniform, words, DT, GPU, NP
     zeros = h.full([vocab, hidden], 0.0, DT.BF16, GPU)
     add(None, "index_add bf16 16384 rows into [32768,4096] (embedding gradient: copy, check, sort, ordered sums)",
         4 * vocab * hidden + 2 * tokens * hidden + 4 * tokens * hidden, lambda: zeros.index_add(0, ids, grads), 5)
-    # Advanced indexing: the same rows through index tensors (check, positions, rows of tiles) and written back
+    # Advanced indexing: the same rows through an index tensor (check, rows of tiles) and written back
     # (copy of the table, winners per row, the winners' rows).
     add(None, "x[ids] bf16 [32768,4096] by 16384 ids (advanced indexing: check, rows)",
-        4 * tokens * hidden + 24 * tokens, lambda: table.index_tensors([ids]), 10)
+        4 * tokens * hidden + 16 * tokens, lambda: table.index_tensors([ids]), 10)
     add(None, "index_put bf16 16384 rows into [32768,4096] (copy, check, positions, last write wins)",
         4 * vocab * hidden + 4 * tokens * hidden + 24 * tokens, lambda: table.index_put_tensors([ids], grads, False), 5)
     del table, grads, zeros
