@@ -225,15 +225,18 @@ class AdvancedIndex {
                                 std::to_string(start + j));
                 }
             }
-            if (defined_indices == 1 && data.layout.is_contiguous()) {
-                // The only index, and its elements lie in order: the coordinates of the flattened mask are the
+            if (defined_indices == 1) {
+                // The only index: with its elements in order, the coordinates of the flattened mask are the
                 // linear positions in the subspace it covers. They are in range by construction, so neither a
                 // check nor a pass per dimension follows. Only the count is taken here: it shapes the result;
                 // the positions are written when a read or a write asks for them.
-                TensorData flat = data;
-                flat.layout = Layout::contiguous(Shape{data.layout.num_elements()});
-                flat.layout.offset = data.layout.offset;
-                mask_ = data;
+                // (A mask that is a view is laid out in order first, a copy of a byte per element - unless only a
+                // select follows, which walks any layout.)
+                const TensorData dense = one_value || data.layout.is_contiguous() ? data : Tensor(data).contiguous().data();
+                TensorData flat = dense;
+                flat.layout = Layout::contiguous(Shape{dense.layout.num_elements()});
+                flat.layout.offset = dense.layout.offset;
+                mask_ = dense;
                 int64_t count = flat.layout.num_elements();
                 if (one_value) {
                     select_only_ = true;
@@ -355,10 +358,11 @@ class AdvancedIndex {
             // One value for every element a mask selects: an element-wise choice between the value and the target,
             // with the mask broadcast over the dimensions behind it. No positions, no copy of the target first.
             const Shape &shape = target.layout.shape;
-            TensorData cond = on_device(*mask_, target.device());
+            const TensorData moved = on_device(*mask_, target.device());  // any layout: the select walks it
+            TensorData cond = moved;
             cond.layout.shape = shape;
             cond.layout.strides.assign(shape.size(), 0);
-            for (size_t j = 0; j < mask_->layout.shape.size(); ++j) cond.layout.strides[first_ + j] = mask_->layout.strides[j];
+            for (size_t j = 0; j < moved.layout.shape.size(); ++j) cond.layout.strides[first_ + j] = moved.layout.strides[j];
             Tensor out = Tensor::uninit_on(shape, target.dtype, target.device());
             backend::where_(out.data(), cond, values.expand_to(shape), target);
             return out;

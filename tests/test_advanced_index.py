@@ -341,6 +341,25 @@ def _a_mask_alone(device):
                 assert np.array_equal(array(x.index_tensors([None] * start + [view])), a[at])
 
 
+    # Masks that are views: expanded along a dimension, and cut out of a larger one.
+    a = rng.integers(0, 30000, [6, 5, 4]).astype(np.float32)
+    x = tensor(a, DT.F32, [6, 5, 4], device)
+    seven = tensor(np.array([7.0], dtype=np.float32), DT.F32, [], device)
+    row = rng.random([5]) < 0.5
+    wide = rng.random([8, 7]) < 0.5
+    views = [(bools(row.reshape(1, 5)).to(device).expand([6, 5]), np.broadcast_to(row, (6, 5))),
+             (bools(wide).to(device).narrow(0, 1, 6).narrow(1, 2, 5), wide[1:7, 2:7])]
+    for view, m in views:
+        assert np.array_equal(array(x.index_tensors([view])), a[m])
+        want = a.copy()
+        want[m] = 7.0
+        assert np.array_equal(array(x.index_put_tensors([view], seven, False)), want)
+        many = np.arange(int(m.sum()) * 4, dtype=np.float32).reshape(-1, 4)
+        want = a.copy()
+        want[m] = many
+        assert np.array_equal(array(x.index_put_tensors([view], tensor(many, DT.F32, list(many.shape), device), False)), want)
+
+
 def test_a_mask_alone_follows_numpy():
     _a_mask_alone("cpu")
 
